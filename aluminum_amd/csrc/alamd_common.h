@@ -1,0 +1,192 @@
+// Shared host/device helpers of the aluminum_amd library: error reporting,
+// element tag types, the pairwise step of every (type, op) pair and the
+// 128-bit vector load/store helpers.  gfx950 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "aluminum_amd.h"
+
+namespace alamd {
+
+// ---- errors ---------------------------------------------------------------
+
+// Records the message for alamd_last_error() and returns `code`.
+int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+#define ALAMD_HIP(call)                                                        \
+  do {                                                                         \
+    hipError_t e_ = (call);                                                    \
+    if (e_ != hipSuccess)                                                      \
+      return ::alamd::set_error(ALAMD_ERR_HIP, "%s failed: %s", #call,         \
+                                hipGetErrorString(e_));                        \
+  } while (0)
+
+// Number of compute units of the current device (cached per device); < 0 on
+// error (message set).
+int device_cus();
+
+// Checks (dtype, op) as alamd_check_op does, setting the error message.
+int check_type_op(int dtype, int op);
+
+inline bool is_float_dtype(int dt) {
+  return dt == ALAMD_F16 || dt == ALAMD_BF16 || dt == ALAMD_F32 || dt == ALAMD_F64;
+}
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---- element types --------------------------------------------------------
+
+struct f16_t { uint16_t b; };   // IEEE binary16 bit pattern
+struct bf16_t { uint16_t b; };  // bfloat16 bit pattern
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Exact widening of the 16-bit float types.
+__device__ __forceinline__ float widen(f16_t h) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, h.b));
+}
+__device__ __forceinline__ float widen(bf16_t h) {
+  return __uint_as_float(static_cast<uint32_t>(h.b) << 16);
+}
+
+// Round-to-nearest-even narrowing.  A NaN stays a NaN with the quiet bit set.
+template <typename H> __device__ __forceinline__ H narrow(float f);
+template <> __device__ __forceinline__ f16_t narrow<f16_t>(float f) {
+  f16_t r;
+  r.b = __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+  return r;
+}
+template <> __device__ __forceinline__ bf16_t narrow<bf16_t>(float f) {
+  uint32_t u = __float_as_uint(f);
+  bf16_t r;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    r.b = static_cast<uint16_t>((u >> 16) | 0x0040u);
+  } else {
+    u += 0x7fffu + ((u >> 16) & 1u);
+    r.b = static_cast<uint16_t>(u >> 16);
+  }
+  return r;
+}
+
+// ---- the pairwise step ----------------------------------------------------
+//
+// step<T, OP>(in, inout) is one application of an MPI reduction function to
+// one element: the value stored back to inoutvec.  For the native types it
+// is OP(inout, in) with MIN(x, y) = (x < y) ? x : y and MAX(x, y) =
+// (x > y) ? x : y, so a tie or a NaN operand yields `in`; for fp16 / bf16 it
+// is narrow(OP(widen(in), widen(inout))) with std::min / std::max
+// (reference: src/mpi_impl.cpp:61-145), which chooses the same operand.
+
+template <typename T> struct unsigned_of { using type = T; };
+template <> struct unsigned_of<int8_t> { using type = uint8_t; };
+template <> struct unsigned_of<int16_t> { using type = uint16_t; };
+template <> struct unsigned_of<int32_t> { using type = uint32_t; };
+template <> struct unsigned_of<int64_t> { using type = uint64_t; };
+
+template <typename T, int OP> struct Step {
+  // integer types
+  static __device__ __forceinline__ T apply(T in, T inout) {
+    using U = typename unsigned_of<T>::type;
+    if constexpr (OP == ALAMD_SUM) return static_cast<T>(static_cast<U>(static_cast<U>(inout) + static_cast<U>(in)));
+    else if constexpr (OP == ALAMD_PROD) return static_cast<T>(static_cast<U>(static_cast<U>(inout) * static_cast<U>(in)));
+    else if constexpr (OP == ALAMD_MIN) return (inout < in) ? inout : in;
+    else if constexpr (OP == ALAMD_MAX) return (inout > in) ? inout : in;
+    else if constexpr (OP == ALAMD_LOR) return static_cast<T>((inout != 0) || (in != 0));
+    else if constexpr (OP == ALAMD_LAND) return static_cast<T>((inout != 0) && (in != 0));
+    else if constexpr (OP == ALAMD_LXOR) return static_cast<T>((inout != 0) != (in != 0));
+    else if constexpr (OP == ALAMD_BOR) return static_cast<T>(inout | in);
+    else if constexpr (OP == ALAMD_BAND) return static_cast<T>(inout & in);
+    else return static_cast<T>(inout ^ in);
+  }
+};
+
+template <typename F, int OP> __device__ __forceinline__ F fp_step(F in, F inout) {
+  if constexpr (OP == ALAMD_SUM) return inout + in;
+  else if constexpr (OP == ALAMD_PROD) return inout * in;
+  else if constexpr (OP == ALAMD_MIN) return (inout < in) ? inout : in;
+  else return (inout > in) ? inout : in;
+}
+
+template <int OP> struct Step<float, OP> {
+  static __device__ __forceinline__ float apply(float in, float inout) { return fp_step<float, OP>(in, inout); }
+};
+template <int OP> struct Step<double, OP> {
+  static __device__ __forceinline__ double apply(double in, double inout) { return fp_step<double, OP>(in, inout); }
+};
+template <int OP> struct Step<f16_t, OP> {
+  static __device__ __forceinline__ f16_t apply(f16_t in, f16_t inout) {
+    return narrow<f16_t>(fp_step<float, OP>(widen(in), widen(inout)));
+  }
+};
+template <int OP> struct Step<bf16_t, OP> {
+  static __device__ __forceinline__ bf16_t apply(bf16_t in, bf16_t inout) {
+    return narrow<bf16_t>(fp_step<float, OP>(widen(in), widen(inout)));
+  }
+};
+
+// The step applied to every element of a 128-bit vector.
+template <typename T, int OP>
+__device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
+  constexpr int N = 16 / sizeof(T);
+  union U { u32x4 v; T e[N]; __device__ U() {} } a, b;
+  a.v = in;
+  b.v = inout;
+#pragma unroll
+  for (int j = 0; j < N; ++j) b.e[j] = Step<T, OP>::apply(a.e[j], b.e[j]);
+  return b.v;
+}
+
+// ---- streaming loads and stores ---------------------------------------------
+// Every byte on this path is touched once, so loads and stores are marked
+// non-temporal to keep them from displacing each other in L2 / MALL.
+
+__device__ __forceinline__ u32x4 ld_stream(const void *p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+}
+__device__ __forceinline__ void st_stream(void *p, u32x4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
+}
+template <typename T> __device__ __forceinline__ T ld_elem(const void *p) {
+  return *reinterpret_cast<const T *>(p);
+}
+template <typename T> __device__ __forceinline__ void st_elem(void *p, T v) {
+  *reinterpret_cast<T *>(p) = v;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Grid size for a streaming kernel over `work_items` items with `per_block`
+// items per workgroup pass: enough workgroups to cover the work, capped at
+// `waves` workgroups per compute unit.
+unsigned stream_grid(size_t work_items, size_t per_block, int waves);
+
+}  // namespace alamd
+
+// ---- lanes: what one thread handles per access ------------------------------
+namespace alamd {
+
+// VECTOR = true: a 128-bit vector of 16/sizeof(T) elements (needs 16-byte
+// aligned addresses); VECTOR = false: one element.
+template <typename T, bool VECTOR> struct Lane;
+
+template <typename T> struct Lane<T, true> {
+  using V = u32x4;
+  static constexpr int N = 16 / sizeof(T);
+  static __device__ __forceinline__ V ld(const char *base, size_t i) { return ld_stream(base + i * 16); }
+  static __device__ __forceinline__ void st(char *base, size_t i, V v) { st_stream(base + i * 16, v); }
+  template <int OP> static __device__ __forceinline__ V step(V in, V inout) { return step_vec<T, OP>(in, inout); }
+};
+
+template <typename T> struct Lane<T, false> {
+  using V = T;
+  static constexpr int N = 1;
+  static __device__ __forceinline__ V ld(const char *base, size_t i) { return ld_elem<T>(base + i * sizeof(T)); }
+  static __device__ __forceinline__ void st(char *base, size_t i, V v) { st_elem<T>(base + i * sizeof(T), v); }
+  template <int OP> static __device__ __forceinline__ V step(V in, V inout) { return Step<T, OP>::apply(in, inout); }
+};
+
+}  // namespace alamd

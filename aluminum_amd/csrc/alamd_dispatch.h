@@ -1,0 +1,108 @@
+// Run-time (dtype, op) -> compile-time <T, OP> dispatch shared by the kernel
+// translation units.
+#pragma once
+
+#include "alamd_common.h"
+
+namespace alamd {
+
+template <typename T> struct TypeTag { using type = T; };
+template <int OP> struct OpTag { static constexpr int value = OP; };
+
+// Integer ops other than min / max do not depend on signedness, so signed
+// types share the kernels of the unsigned type of the same width.
+template <typename S, typename F> int dispatch_int_op(int op, F &&f) {
+  using U = typename unsigned_of<S>::type;
+  switch (op) {
+  case ALAMD_SUM: return f(TypeTag<U>{}, OpTag<ALAMD_SUM>{});
+  case ALAMD_PROD: return f(TypeTag<U>{}, OpTag<ALAMD_PROD>{});
+  case ALAMD_MIN: return f(TypeTag<S>{}, OpTag<ALAMD_MIN>{});
+  case ALAMD_MAX: return f(TypeTag<S>{}, OpTag<ALAMD_MAX>{});
+  case ALAMD_LOR: return f(TypeTag<U>{}, OpTag<ALAMD_LOR>{});
+  case ALAMD_LAND: return f(TypeTag<U>{}, OpTag<ALAMD_LAND>{});
+  case ALAMD_LXOR: return f(TypeTag<U>{}, OpTag<ALAMD_LXOR>{});
+  case ALAMD_BOR: return f(TypeTag<U>{}, OpTag<ALAMD_BOR>{});
+  case ALAMD_BAND: return f(TypeTag<U>{}, OpTag<ALAMD_BAND>{});
+  case ALAMD_BXOR: return f(TypeTag<U>{}, OpTag<ALAMD_BXOR>{});
+  default: return set_error(ALAMD_ERR_UNSUPPORTED_OP, "Reduction operator not supported");
+  }
+}
+
+template <typename T, typename F> int dispatch_fp_op(int op, F &&f) {
+  switch (op) {
+  case ALAMD_SUM: return f(TypeTag<T>{}, OpTag<ALAMD_SUM>{});
+  case ALAMD_PROD: return f(TypeTag<T>{}, OpTag<ALAMD_PROD>{});
+  case ALAMD_MIN: return f(TypeTag<T>{}, OpTag<ALAMD_MIN>{});
+  case ALAMD_MAX: return f(TypeTag<T>{}, OpTag<ALAMD_MAX>{});
+  default: return set_error(ALAMD_ERR_UNSUPPORTED_OP, "Reduction operator not supported");
+  }
+}
+
+// Calls f(TypeTag<T>, OpTag<OP>) for the kernel types of a float dtype.
+template <typename F> int dispatch_float(int dtype, int op, F &&f) {
+  switch (dtype) {
+  case ALAMD_F16: return dispatch_fp_op<f16_t>(op, f);
+  case ALAMD_BF16: return dispatch_fp_op<bf16_t>(op, f);
+  case ALAMD_F32: return dispatch_fp_op<float>(op, f);
+  case ALAMD_F64: return dispatch_fp_op<double>(op, f);
+  default: return set_error(ALAMD_ERR_UNSUPPORTED_TYPE, "unknown dtype %d", dtype);
+  }
+}
+
+template <typename F> int dispatch_any(int dtype, int op, F &&f) {
+  switch (dtype) {
+  case ALAMD_I8: return dispatch_int_op<int8_t>(op, f);
+  case ALAMD_U8: return dispatch_int_op<uint8_t>(op, f);
+  case ALAMD_I16: return dispatch_int_op<int16_t>(op, f);
+  case ALAMD_U16: return dispatch_int_op<uint16_t>(op, f);
+  case ALAMD_I32: return dispatch_int_op<int32_t>(op, f);
+  case ALAMD_U32: return dispatch_int_op<uint32_t>(op, f);
+  case ALAMD_I64: return dispatch_int_op<int64_t>(op, f);
+  case ALAMD_U64: return dispatch_int_op<uint64_t>(op, f);
+  default: return dispatch_float(dtype, op, f);
+  }
+}
+
+// ---- parameters of the two combine kernel families -------------------------
+
+// Work is a grid of segments (blockIdx.y) x tiles (blockIdx.x).  Segment s
+// covers elements [s*seg_base + min(s, seg_rem), +seg_base + (s < seg_rem)).
+struct SegParams {
+  unsigned long long seg_base;
+  unsigned long long seg_rem;
+  int in_blocked;   // 1: inputs are read at the segment's offset, 0: at 0
+  int out_mode;     // OUT_ALL / OUT_SEG / OUT_OWNER
+  int owner_shift;  // OUT_OWNER: output index is (segment + owner_shift) mod P
+  int nout;         // OUT_ALL: number of outputs written
+};
+enum { OUT_ALL = 0, OUT_SEG = 1, OUT_OWNER = 2 };
+
+// Left fold over a rotated rank sequence.
+struct FoldParams {
+  const char *in[ALAMD_MAX_RANKS];
+  char *out[ALAMD_MAX_RANKS];
+  SegParams seg;
+  int P;
+  int start0;        // first operand of segment s is rank (start0 + s*start_stride) mod P
+  int start_stride;
+  int dir;           // +1: next operand is rank+1, -1: rank-1 (with wrap)
+};
+
+// Balanced pairwise tree over up to 32 slots.  Slot j holds a[j], or
+// step(in = a[j], inout = b[j]) when b[j] is set; slots >= nvalid are empty.
+// Level d = 1,2,4..: slot i (multiple of 2d) = step(in = slot i+d, inout = slot i).
+struct TreeParams {
+  const char *a[32];
+  const char *b[32];
+  char *out[ALAMD_MAX_RANKS];
+  SegParams seg;
+  int P;        // number of ranks (for OUT_OWNER)
+  int nvalid;   // occupied slots
+};
+
+int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op,
+                bool acc_is_in, bool vector, hipStream_t stream);
+int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, int dtype,
+                int op, bool vector, hipStream_t stream);
+
+}  // namespace alamd

@@ -1,0 +1,290 @@
+// Host side of the combine entry points: argument checks, the mapping of a
+// named order onto one of the two kernel families, the Reduce_scatter and
+// Allgather layouts.
+#include <string>
+
+#include "alamd_dispatch.h"
+
+namespace alamd {
+
+namespace {
+
+bool ranges_overlap(const void *a, size_t abytes, const void *b, size_t bbytes) {
+  const uintptr_t x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);
+  return x < y + bbytes && y < x + abytes;
+}
+
+int floor_pow2(int p) { int q = 1; while (2 * q <= p) q *= 2; return q; }
+int ceil_pow2(int p) { int q = 1; while (q < p) q *= 2; return q; }
+
+int bit_reverse(int v, int bits) {
+  int r = 0;
+  for (int b = 0; b < bits; ++b) if (v & (1 << b)) r |= 1 << (bits - 1 - b);
+  return r;
+}
+
+bool order_has_start(int order) { return order == ALAMD_ORDER_PAIRWISE_DESC || order == ALAMD_ORDER_RING; }
+bool order_is_tree(int order) {
+  return order == ALAMD_ORDER_TREE_DBL || order == ALAMD_ORDER_TREE_HALV || order == ALAMD_ORDER_TREE_BINOMIAL;
+}
+bool order_valid(int order) { return order >= ALAMD_ORDER_RANK_ASC && order <= ALAMD_ORDER_TREE_BINOMIAL; }
+
+// Fills the slot tables of a tree order over the P inputs `ins`.
+int build_tree(TreeParams &tp, const void *const *ins, int P, int order) {
+  for (int j = 0; j < 32; ++j) { tp.a[j] = nullptr; tp.b[j] = nullptr; }
+  tp.P = P;
+  if (order == ALAMD_ORDER_TREE_BINOMIAL) {
+    for (int j = 0; j < P; ++j) tp.a[j] = static_cast<const char *>(ins[j]);
+    tp.nvalid = P;
+    return ceil_pow2(P);
+  }
+  const int pof2 = floor_pow2(P), rem = P - pof2;
+  const char *la[32], *lb[32];
+  for (int j = 0; j < pof2; ++j) {
+    if (j < rem) { la[j] = static_cast<const char *>(ins[2 * j]); lb[j] = static_cast<const char *>(ins[2 * j + 1]); }
+    else { la[j] = static_cast<const char *>(ins[j + rem]); lb[j] = nullptr; }
+  }
+  int bits = 0;
+  while ((1 << bits) < pof2) ++bits;
+  for (int k = 0; k < pof2; ++k) {
+    // pairing at distance pof2/2, ..., 1 is the adjacent-pair tree over the
+    // bit-reversed slot order
+    const int src = order == ALAMD_ORDER_TREE_HALV ? bit_reverse(k, bits) : k;
+    tp.a[k] = la[src];
+    tp.b[k] = lb[src];
+  }
+  tp.nvalid = pof2;
+  return pof2;
+}
+
+struct Layout {
+  unsigned nseg;
+  SegParams seg;
+  size_t max_len;
+  int start0, start_stride;  // fold orders
+};
+
+// Launches the fold or tree kernels for `order` over inputs `ins`.
+int launch_order(void *const *outs, const void *const *ins, int P, const Layout &lay, int dtype, int op,
+                 int order, bool vector, hipStream_t stream) {
+  if (!is_float_dtype(dtype)) order = ALAMD_ORDER_RANK_ASC;  // integer ops: every order gives the same bits
+  if (P == 1 && order_is_tree(order)) order = ALAMD_ORDER_RANK_ASC;
+  if (order_is_tree(order)) {
+    if (P > ALAMD_MAX_TREE_RANKS)
+      return set_error(ALAMD_ERR_INVALID_ARG, "tree orders support at most %d ranks (got %d)",
+                       ALAMD_MAX_TREE_RANKS, P);
+    TreeParams tp;
+    const int slots = build_tree(tp, ins, P, order);
+    for (int j = 0; j < ALAMD_MAX_RANKS; ++j) tp.out[j] = static_cast<char *>(outs[j]);
+    tp.seg = lay.seg;
+    return launch_tree(tp, slots, lay.nseg, lay.max_len, dtype, op, vector, stream);
+  }
+  FoldParams fp;
+  for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
+    fp.in[r] = r < P ? static_cast<const char *>(ins[r]) : nullptr;
+    fp.out[r] = static_cast<char *>(outs[r]);
+  }
+  fp.seg = lay.seg;
+  fp.P = P;
+  fp.start0 = lay.start0;
+  fp.start_stride = lay.start_stride;
+  fp.dir = order == ALAMD_ORDER_PAIRWISE_DESC ? -1 : 1;
+  return launch_fold(fp, lay.nseg, lay.max_len, dtype, op, order == ALAMD_ORDER_RING, vector, stream);
+}
+
+__global__ void __launch_bounds__(256) gather_kernel_vec(FoldParams p, size_t nvec, size_t tail_bytes) {
+  // blockIdx.y = source rank q; every destination gets a copy at block q
+  const int q = blockIdx.y;
+  const char *src = p.in[q];
+  const size_t blk_bytes = nvec * 16 + tail_bytes;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (size_t)gridDim.x * 256) {
+    const u32x4 v = ld_stream(src + i * 16);
+    for (int r = 0; r < p.P; ++r) {
+      char *dst = p.out[r] + (size_t)q * blk_bytes;
+      if (dst != src) st_stream(dst + i * 16, v);
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail_bytes) {
+    const size_t i = nvec * 16 + threadIdx.x;
+    const char c = src[i];
+    for (int r = 0; r < p.P; ++r) {
+      char *dst = p.out[r] + (size_t)q * blk_bytes;
+      if (dst != src) dst[i] = c;
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) gather_kernel_bytes(FoldParams p, size_t blk_bytes) {
+  const int q = blockIdx.y;
+  const char *src = p.in[q];
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < blk_bytes; i += (size_t)gridDim.x * 256) {
+    const char c = src[i];
+    for (int r = 0; r < p.P; ++r) {
+      char *dst = p.out[r] + (size_t)q * blk_bytes;
+      if (dst != src) dst[i] = c;
+    }
+  }
+}
+
+int check_common(int P, size_t count, int dtype) {
+  if (P < 1 || P > ALAMD_MAX_RANKS)
+    return set_error(ALAMD_ERR_INVALID_ARG, "number of ranks %d outside [1, %d]", P, ALAMD_MAX_RANKS);
+  if (alamd_dtype_size(dtype) == 0) return set_error(ALAMD_ERR_UNSUPPORTED_TYPE, "unknown dtype %d", dtype);
+  if (count > (size_t)1 << 48) return set_error(ALAMD_ERR_INVALID_ARG, "count too large");
+  return ALAMD_OK;
+}
+
+}  // namespace
+
+}  // namespace alamd
+
+using namespace alamd;
+
+extern "C" {
+
+int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, size_t count, int dtype,
+                  int op, int order, int start, void *stream) {
+  int rc = check_common(P, count, dtype);
+  if (rc) return rc;
+  if ((rc = check_type_op(dtype, op))) return rc;
+  if (!order_valid(order)) return set_error(ALAMD_ERR_INVALID_ALGO, "Invalid algorithm");
+  if (nout < 1 || nout > ALAMD_MAX_RANKS)
+    return set_error(ALAMD_ERR_INVALID_ARG, "number of outputs %d outside [1, %d]", nout, ALAMD_MAX_RANKS);
+  if (start < 0 || start >= P || (start != 0 && !order_has_start(order)))
+    return set_error(ALAMD_ERR_INVALID_ARG, "start rank %d invalid for this order", start);
+  if (!outs || !ins) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
+  if (count == 0) return ALAMD_OK;
+  const size_t es = alamd_dtype_size(dtype), bytes = count * es;
+  bool vector = true;
+  for (int r = 0; r < P; ++r) {
+    if (!ins[r]) return set_error(ALAMD_ERR_INVALID_ARG, "input %d is null", r);
+    vector = vector && aligned16(ins[r]);
+  }
+  void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
+  for (int j = 0; j < nout; ++j) {
+    if (!outs[j]) return set_error(ALAMD_ERR_INVALID_ARG, "output %d is null", j);
+    vector = vector && aligned16(outs[j]);
+    for (int r = 0; r < P; ++r)
+      if (outs[j] != ins[r] && ranges_overlap(outs[j], bytes, ins[r], bytes))
+        return set_error(ALAMD_ERR_OVERLAP, "output %d partially overlaps input %d", j, r);
+    for (int k = 0; k < j; ++k)
+      if (ranges_overlap(outs[j], bytes, outs[k], bytes))
+        return set_error(ALAMD_ERR_OVERLAP, "outputs %d and %d overlap", k, j);
+    out_tab[j] = outs[j];
+  }
+  Layout lay;
+  lay.nseg = 1;
+  lay.seg.seg_base = count;
+  lay.seg.seg_rem = 0;
+  lay.seg.in_blocked = 0;
+  lay.seg.out_mode = OUT_ALL;
+  lay.seg.owner_shift = 0;
+  lay.seg.nout = nout;
+  lay.max_len = count;
+  lay.start0 = start;
+  lay.start_stride = 0;
+  return launch_order(out_tab, ins, P, lay, dtype, op, order, vector, as_stream(stream));
+}
+
+int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, size_t count, int dtype,
+                         int op, int order, void *stream) {
+  int rc = check_common(P, count, dtype);
+  if (rc) return rc;
+  if ((rc = check_type_op(dtype, op))) return rc;
+  if (!order_valid(order)) return set_error(ALAMD_ERR_INVALID_ALGO, "Invalid algorithm");
+  if (!recvs || !sends) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
+  if (count == 0) return ALAMD_OK;
+  const size_t es = alamd_dtype_size(dtype), blk = count * es, total = blk * (size_t)P;
+  bool vector = (blk % 16) == 0, inplace = false;
+  void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
+  for (int r = 0; r < P; ++r) {
+    if (!sends[r] || !recvs[r]) return set_error(ALAMD_ERR_INVALID_ARG, "buffer %d is null", r);
+    vector = vector && aligned16(sends[r]) && aligned16(recvs[r]);
+    out_tab[r] = recvs[r];
+  }
+  for (int b = 0; b < P; ++b) {
+    for (int r = 0; r < P; ++r) {
+      if (recvs[b] == sends[r] && b == r) { inplace = true; continue; }
+      if (ranges_overlap(recvs[b], blk, sends[r], total))
+        return set_error(ALAMD_ERR_OVERLAP, "receive buffer %d overlaps send buffer %d", b, r);
+    }
+    for (int k = 0; k < b; ++k)
+      if (ranges_overlap(recvs[b], blk, recvs[k], blk))
+        return set_error(ALAMD_ERR_OVERLAP, "receive buffers %d and %d overlap", k, b);
+  }
+  Layout lay;
+  lay.seg.seg_base = count;
+  lay.seg.seg_rem = 0;
+  lay.seg.in_blocked = 1;
+  lay.seg.out_mode = OUT_SEG;
+  lay.seg.owner_shift = 0;
+  lay.seg.nout = 1;
+  lay.max_len = count;
+  lay.start0 = 0;
+  lay.start_stride = order_has_start(order) ? 1 : 0;
+  if (!inplace || P == 1) {
+    lay.nseg = (unsigned)P;
+    return launch_order(out_tab, sends, P, lay, dtype, op, order, vector, as_stream(stream));
+  }
+  // In place every result lands on block 0 of its own send buffer, which
+  // block 0's fold still has to read: fold block 0 first (it overwrites only
+  // what its own lanes have read), then the other blocks.
+  lay.nseg = 1;
+  rc = launch_order(out_tab, sends, P, lay, dtype, op, order, vector, as_stream(stream));
+  if (rc) return rc;
+  // blocks 1..P-1: shift the tables by one block
+  const void *in_shift[ALAMD_MAX_RANKS];
+  void *out_shift[ALAMD_MAX_RANKS] = {nullptr};
+  for (int r = 0; r < P; ++r) in_shift[r] = static_cast<const char *>(sends[r]) + blk;
+  for (int b = 1; b < P; ++b) out_shift[b - 1] = recvs[b];
+  lay.nseg = (unsigned)(P - 1);
+  lay.start0 = order_has_start(order) ? 1 : 0;
+  return launch_order(out_shift, in_shift, P, lay, dtype, op, order, vector, as_stream(stream));
+}
+
+int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t count, int dtype,
+                    void *stream) {
+  int rc = check_common(P, count, dtype);
+  if (rc) return rc;
+  if (!recvs || !sends) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
+  if (count == 0) return ALAMD_OK;
+  const size_t es = alamd_dtype_size(dtype), blk = count * es;
+  FoldParams fp;
+  bool vector = (blk % 16) == 0;
+  for (int r = 0; r < ALAMD_MAX_RANKS; ++r) { fp.in[r] = nullptr; fp.out[r] = nullptr; }
+  for (int r = 0; r < P; ++r) {
+    if (!sends[r] || !recvs[r]) return set_error(ALAMD_ERR_INVALID_ARG, "buffer %d is null", r);
+    fp.in[r] = static_cast<const char *>(sends[r]);
+    fp.out[r] = static_cast<char *>(recvs[r]);
+    vector = vector && aligned16(sends[r]) && aligned16(recvs[r]);
+  }
+  for (int r = 0; r < P; ++r) {
+    for (int q = 0; q < P; ++q) {
+      const char *slot = static_cast<const char *>(recvs[r]) + (size_t)q * blk;
+      if (r == q && sends[q] == slot) continue;  // in place
+      if (ranges_overlap(recvs[r], blk * (size_t)P, sends[q], blk))
+        return set_error(ALAMD_ERR_OVERLAP, "receive buffer %d overlaps send buffer %d", r, q);
+    }
+    for (int k = 0; k < r; ++k)
+      if (ranges_overlap(recvs[r], blk * (size_t)P, recvs[k], blk * (size_t)P))
+        return set_error(ALAMD_ERR_OVERLAP, "receive buffers %d and %d overlap", k, r);
+  }
+  fp.P = P;
+  hipStream_t st = as_stream(stream);
+  if (vector) {
+    const size_t nvec = blk / 16;
+    unsigned per = (stream_grid((size_t)-1 / 2, 1, 8) + P - 1) / P;
+    unsigned gx = stream_grid(nvec, 256, 8);
+    if (gx > per) gx = per < 1 ? 1 : per;
+    hipLaunchKernelGGL(gather_kernel_vec, dim3(gx, P, 1), dim3(256, 1, 1), 0, st, fp, nvec, (size_t)0);
+  } else {
+    unsigned per = (stream_grid((size_t)-1 / 2, 1, 8) + P - 1) / P;
+    unsigned gx = stream_grid(blk, 256, 8);
+    if (gx > per) gx = per < 1 ? 1 : per;
+    hipLaunchKernelGGL(gather_kernel_bytes, dim3(gx, P, 1), dim3(256, 1, 1), 0, st, fp, blk);
+  }
+  ALAMD_HIP(hipGetLastError());
+  return ALAMD_OK;
+}
+
+}  // extern "C"

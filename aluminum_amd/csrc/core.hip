@@ -1,0 +1,91 @@
+// Library-wide host code: error text, dtype table, device probe.
+#include <cstdarg>
+#include <cstdio>
+#include <mutex>
+
+#include "alamd_common.h"
+
+namespace alamd {
+
+namespace {
+thread_local char g_err[512] = "";
+std::mutex g_dev_mutex;
+int g_dev_cus[64];
+bool g_dev_known[64];
+}  // namespace
+
+int set_error(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+void clear_error() { g_err[0] = 0; }
+
+int device_cus() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    set_error(ALAMD_ERR_HIP, "hipGetDevice failed: no usable GPU");
+    return -1;
+  }
+  if (dev < 0 || dev >= 64) {
+    set_error(ALAMD_ERR_HIP, "device index %d out of range", dev);
+    return -1;
+  }
+  std::lock_guard<std::mutex> lock(g_dev_mutex);
+  if (!g_dev_known[dev]) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+      set_error(ALAMD_ERR_HIP, "hipGetDeviceProperties failed");
+      return -1;
+    }
+    g_dev_cus[dev] = prop.multiProcessorCount;
+    g_dev_known[dev] = true;
+  }
+  return g_dev_cus[dev];
+}
+
+int check_type_op(int dtype, int op) {
+  if (dtype < 0 || dtype >= ALAMD_NUM_DTYPES)
+    return set_error(ALAMD_ERR_UNSUPPORTED_TYPE, "unknown dtype %d", dtype);
+  if (op < ALAMD_SUM || op > ALAMD_BXOR)
+    return set_error(ALAMD_ERR_UNSUPPORTED_OP, "Reduction operator not supported");
+  if (is_float_dtype(dtype) && op > ALAMD_MAX)
+    return set_error(ALAMD_ERR_UNSUPPORTED_OP, "Reduction operator not supported");
+  return ALAMD_OK;
+}
+
+}  // namespace alamd
+
+extern "C" {
+
+const char *alamd_last_error(void) { return alamd::g_err; }
+
+int alamd_version(void) { return ALAMD_VERSION_MAJOR * 100 + ALAMD_VERSION_MINOR; }
+
+size_t alamd_dtype_size(int dtype) {
+  switch (dtype) {
+  case ALAMD_I8: case ALAMD_U8: return 1;
+  case ALAMD_I16: case ALAMD_U16: case ALAMD_F16: case ALAMD_BF16: return 2;
+  case ALAMD_I32: case ALAMD_U32: case ALAMD_F32: return 4;
+  case ALAMD_I64: case ALAMD_U64: case ALAMD_F64: return 8;
+  default: return 0;
+  }
+}
+
+int alamd_check_op(int dtype, int op) { return alamd::check_type_op(dtype, op); }
+
+int alamd_init(void) {
+  int dev = 0;
+  ALAMD_HIP(hipGetDevice(&dev));
+  hipDeviceProp_t prop;
+  ALAMD_HIP(hipGetDeviceProperties(&prop, dev));
+  if (std::string(prop.gcnArchName).rfind("gfx950", 0) != 0)
+    return alamd::set_error(ALAMD_ERR_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only",
+                            dev, prop.gcnArchName);
+  return alamd::device_cus() > 0 ? ALAMD_OK : ALAMD_ERR_HIP;
+}
+
+}  // extern "C"

@@ -1,0 +1,248 @@
+// Ring reduce-scatter + allgather over P logical ranks held in one GPU's HBM.
+//
+// STEPWISE: one launch per ring step.  In reduce-scatter step t every rank r
+// (blockIdx.y) folds the segment it "receives" from rank r-1 into its own
+// copy; in allgather step t it copies the segment.  A segment is worked
+// through chunk by chunk: a chunk is owned by a fixed group of workgroups.
+// FUSED: the fold kernels walk each segment once in ring order.
+#include "alamd_dispatch.h"
+
+namespace alamd {
+
+namespace {
+
+constexpr int kThreads = 256;
+
+struct RingParams {
+  char *buf[ALAMD_MAX_RANKS];
+  unsigned long long seg_base, seg_rem;
+  unsigned long long chunk_accesses;  // accesses (vectors or elements) per chunk
+  int P;
+  int t;              // ring step
+  unsigned wg_per_chunk;
+};
+
+__device__ __forceinline__ void ring_seg(const RingParams &p, int seg, size_t &off, size_t &len) {
+  const unsigned long long sg = (unsigned long long)seg;
+  off = sg * p.seg_base + (sg < p.seg_rem ? sg : p.seg_rem);
+  len = p.seg_base + (sg < p.seg_rem ? 1u : 0u);
+}
+
+// OP < 0: plain copy (allgather step).
+template <typename T, int OP, bool VECTOR>
+__global__ void __launch_bounds__(kThreads) ring_step_kernel(const RingParams p) {
+  using L = Lane<T, VECTOR>;
+  using V = typename L::V;
+  constexpr int U = 4;
+  constexpr size_t TILE = (size_t)kThreads * U;
+  const int P = p.P, r = blockIdx.y;
+  // reduce-scatter step t receives segment r-t-1, allgather step t segment r-t
+  int seg = (OP >= 0 ? r - p.t - 1 : r - p.t) % P;
+  if (seg < 0) seg += P;
+  const int from = r == 0 ? P - 1 : r - 1;
+  size_t off, len;
+  ring_seg(p, seg, off, len);
+  char *local = p.buf[r] + off * sizeof(T);
+  const char *recv = p.buf[from] + off * sizeof(T);
+
+  const size_t n = len / L::N;
+  const size_t cn = p.chunk_accesses;
+  const size_t nchunks = (n + cn - 1) / cn;
+  const unsigned wgpc = p.wg_per_chunk;
+  const unsigned lane_wg = blockIdx.x % wgpc;
+  for (size_t c = blockIdx.x / wgpc; c < nchunks; c += gridDim.x / wgpc) {
+    const size_t c0 = c * cn, c1 = (c0 + cn < n) ? c0 + cn : n;
+    for (size_t i0 = c0 + (size_t)lane_wg * TILE + threadIdx.x; i0 < c1; i0 += (size_t)wgpc * TILE) {
+      V a[U], b[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const size_t i = i0 + (size_t)u * kThreads;
+        if (i < c1) {
+          a[u] = L::ld(recv, i);
+          if constexpr (OP >= 0) b[u] = L::ld(local, i);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const size_t i = i0 + (size_t)u * kThreads;
+        if (i < c1) {
+          if constexpr (OP >= 0) L::st(local, i, L::template step<(OP >= 0 ? OP : 0)>(a[u], b[u]));
+          else L::st(local, i, a[u]);
+        }
+      }
+    }
+  }
+  if constexpr (VECTOR) {
+    const size_t e = n * L::N + threadIdx.x;
+    if (blockIdx.x == 0 && e < len) {
+      using S = Lane<T, false>;
+      const T a = S::ld(recv, e);
+      if constexpr (OP >= 0) S::st(local, e, S::template step<(OP >= 0 ? OP : 0)>(a, S::ld(local, e)));
+      else S::st(local, e, a);
+    }
+  }
+}
+
+struct RingPlan {
+  RingParams rp;
+  bool vector;
+  unsigned gx;
+  size_t es;
+};
+
+int make_plan(RingPlan &pl, void *const *bufs, int P, size_t count, int dtype, size_t chunk_bytes) {
+  if (P < 1 || P > ALAMD_MAX_RANKS)
+    return set_error(ALAMD_ERR_INVALID_ARG, "number of ranks %d outside [1, %d]", P, ALAMD_MAX_RANKS);
+  pl.es = alamd_dtype_size(dtype);
+  if (pl.es == 0) return set_error(ALAMD_ERR_UNSUPPORTED_TYPE, "unknown dtype %d", dtype);
+  if (!bufs) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
+  if (chunk_bytes == 0 || chunk_bytes % pl.es != 0)
+    return set_error(ALAMD_ERR_INVALID_ARG, "chunk size %zu is not a positive multiple of the element size", chunk_bytes);
+  const size_t bytes = count * pl.es;
+  pl.vector = (count % (size_t)P == 0) && ((count / (size_t)P) * pl.es) % 16 == 0;
+  for (int r = 0; r < ALAMD_MAX_RANKS; ++r) pl.rp.buf[r] = nullptr;
+  for (int r = 0; r < P; ++r) {
+    if (!bufs[r] && count) return set_error(ALAMD_ERR_INVALID_ARG, "buffer %d is null", r);
+    pl.rp.buf[r] = static_cast<char *>(bufs[r]);
+    pl.vector = pl.vector && aligned16(bufs[r]);
+    for (int k = 0; k < r; ++k) {
+      const uintptr_t x = reinterpret_cast<uintptr_t>(bufs[r]), y = reinterpret_cast<uintptr_t>(bufs[k]);
+      if (count && x < y + bytes && y < x + bytes)
+        return set_error(ALAMD_ERR_OVERLAP, "rank buffers %d and %d overlap", k, r);
+    }
+  }
+  pl.rp.P = P;
+  pl.rp.seg_base = count / (size_t)P;
+  pl.rp.seg_rem = count % (size_t)P;
+  pl.rp.t = 0;
+  const size_t access = pl.vector ? 16 : pl.es;
+  size_t cn = chunk_bytes / access;
+  if (cn < 1) cn = 1;
+  pl.rp.chunk_accesses = cn;
+  // workgroups: enough to fill the device across the P rows, a whole number per chunk
+  const size_t seg_max = pl.rp.seg_base + (pl.rp.seg_rem ? 1 : 0);
+  const size_t n = seg_max / (pl.vector ? 16 / pl.es : 1);
+  size_t nchunks = (n + cn - 1) / cn;
+  if (nchunks < 1) nchunks = 1;
+  const size_t tiles_per_chunk = ((cn < n ? cn : (n ? n : 1)) + (size_t)kThreads * 4 - 1) / ((size_t)kThreads * 4);
+  const unsigned row_budget = (stream_grid((size_t)-1 / 2, 1, 8) + P - 1) / P;
+  size_t wgpc = row_budget / nchunks;
+  if (wgpc < 1) wgpc = 1;
+  if (wgpc > tiles_per_chunk) wgpc = tiles_per_chunk;
+  size_t chunk_rows = nchunks;
+  if (chunk_rows * wgpc > row_budget) chunk_rows = row_budget / wgpc ? row_budget / wgpc : 1;
+  pl.rp.wg_per_chunk = (unsigned)wgpc;
+  pl.gx = (unsigned)(chunk_rows * wgpc);
+  return ALAMD_OK;
+}
+
+int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, hipStream_t stream) {
+  const dim3 grid(pl.gx, pl.rp.P, 1), block(kThreads, 1, 1);
+  if (!reduce) {
+    // a copy is type-blind: move bytes as the widest unit the layout allows
+    void (*kern)(const RingParams) = nullptr;
+    if (pl.vector) kern = ring_step_kernel<uint32_t, -1, true>;
+    else switch (pl.es) {
+      case 1: kern = ring_step_kernel<uint8_t, -1, false>; break;
+      case 2: kern = ring_step_kernel<uint16_t, -1, false>; break;
+      case 4: kern = ring_step_kernel<uint32_t, -1, false>; break;
+      default: kern = ring_step_kernel<uint64_t, -1, false>; break;
+    }
+    hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
+    ALAMD_HIP(hipGetLastError());
+    return ALAMD_OK;
+  }
+  return dispatch_any(dtype, op, [&](auto tt, auto ot) -> int {
+    using T = typename decltype(tt)::type;
+    constexpr int OP = decltype(ot)::value;
+    void (*kern)(const RingParams) = pl.vector ? ring_step_kernel<T, OP, true> : ring_step_kernel<T, OP, false>;
+    hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
+    ALAMD_HIP(hipGetLastError());
+    return ALAMD_OK;
+  });
+}
+
+int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool all, bool vector,
+               hipStream_t stream) {
+  FoldParams fp;
+  for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
+    fp.in[r] = r < P ? static_cast<const char *>(bufs[r]) : nullptr;
+    fp.out[r] = r < P ? static_cast<char *>(bufs[r]) : nullptr;
+  }
+  fp.P = P;
+  fp.seg.seg_base = count / (size_t)P;
+  fp.seg.seg_rem = count % (size_t)P;
+  fp.seg.in_blocked = 1;
+  fp.seg.out_mode = all ? OUT_ALL : OUT_OWNER;
+  fp.seg.owner_shift = P - 1;
+  fp.seg.nout = P;
+  fp.start0 = 0;
+  fp.start_stride = 1;
+  fp.dir = 1;
+  const size_t max_len = fp.seg.seg_base + (fp.seg.seg_rem ? 1 : 0);
+  if (max_len == 0) return ALAMD_OK;
+  return launch_fold(fp, (unsigned)P, max_len, dtype, op, true, vector, stream);
+}
+
+}  // namespace
+}  // namespace alamd
+
+using namespace alamd;
+
+extern "C" {
+
+int alamd_ring_segment(size_t count, int P, int s, size_t *offset, size_t *len) {
+  if (P < 1 || s < 0 || s >= P || !offset || !len)
+    return set_error(ALAMD_ERR_INVALID_ARG, "bad ring segment query");
+  const size_t base = count / (size_t)P, rem = count % (size_t)P;
+  *offset = (size_t)s * base + ((size_t)s < rem ? (size_t)s : rem);
+  *len = base + ((size_t)s < rem ? 1 : 0);
+  return ALAMD_OK;
+}
+
+int alamd_ring_reduce_scatter(void *const *bufs, int P, size_t count, int dtype, int op,
+                              size_t chunk_bytes, int mode, void *stream) {
+  RingPlan pl;
+  int rc = make_plan(pl, bufs, P, count, dtype, chunk_bytes);
+  if (rc) return rc;
+  if ((rc = check_type_op(dtype, op))) return rc;
+  if (mode != ALAMD_RING_STEPWISE && mode != ALAMD_RING_FUSED)
+    return set_error(ALAMD_ERR_INVALID_ALGO, "Invalid algorithm");
+  if (count == 0 || P == 1) return ALAMD_OK;
+  if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, P, count, dtype, op, false, pl.vector, as_stream(stream));
+  for (int t = 0; t < P - 1; ++t) {
+    pl.rp.t = t;
+    if ((rc = launch_step(pl, dtype, op, true, as_stream(stream)))) return rc;
+  }
+  return ALAMD_OK;
+}
+
+int alamd_ring_allgather(void *const *bufs, int P, size_t count, int dtype, size_t chunk_bytes,
+                         void *stream) {
+  RingPlan pl;
+  int rc = make_plan(pl, bufs, P, count, dtype, chunk_bytes);
+  if (rc) return rc;
+  if (count == 0 || P == 1) return ALAMD_OK;
+  for (int t = 0; t < P - 1; ++t) {
+    pl.rp.t = t;
+    if ((rc = launch_step(pl, dtype, 0, false, as_stream(stream)))) return rc;
+  }
+  return ALAMD_OK;
+}
+
+int alamd_ring_allreduce(void *const *bufs, int P, size_t count, int dtype, int op, size_t chunk_bytes,
+                         int mode, void *stream) {
+  RingPlan pl;
+  int rc = make_plan(pl, bufs, P, count, dtype, chunk_bytes);
+  if (rc) return rc;
+  if ((rc = check_type_op(dtype, op))) return rc;
+  if (mode != ALAMD_RING_STEPWISE && mode != ALAMD_RING_FUSED)
+    return set_error(ALAMD_ERR_INVALID_ALGO, "Invalid algorithm");
+  if (count == 0 || P == 1) return ALAMD_OK;
+  if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, P, count, dtype, op, true, pl.vector, as_stream(stream));
+  rc = alamd_ring_reduce_scatter(bufs, P, count, dtype, op, chunk_bytes, mode, stream);
+  if (rc) return rc;
+  return alamd_ring_allgather(bufs, P, count, dtype, chunk_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,173 @@
+#!/usr/bin/env python3
+"""Benchmark of the combine hot path on one MI355X.
+
+A step is one pass of alamd_combine over one batch of synthetic input that is
+already resident in HBM: P = 8 logical-rank buffers folded into one output.
+Prints ONE JSON line (see the keys below).  The kernel's own duration is
+measured with events on the stream the kernel runs on; the CPU baseline is the
+reference's MPI-backend host combine (a direct MPI_Allreduce, 4 ranks) timed
+on this box's host cores in the same run.
+"""
+import argparse
+import json
+import os
+import subprocess
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "combine HBM GB/s (% of 8 TB/s peak), P=8 fp32/bf16 sum, 2 GiB buffers"
+HBM_PEAK_GBPS = 8000.0
+
+WORKLOADS = {
+    # name: (dtype, count per rank, op, dist, seed base, order)
+    "c2_f32_sum": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "rank_asc"),
+    "c2_f32_prod": ("f32", 1 << 26, "prod", "uniform_09_11", 1000, "rank_asc"),
+    "c2_f32_sum_tree": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "tree_dbl"),
+    "c2_bf16_sum": ("bf16", 1 << 27, "sum", "normal", 2000, "rank_asc"),
+    "c4_i32_max": ("i32", 1 << 28, "max", "fullrange", 3000, "rank_asc"),
+    "c4_i64_bxor": ("i64", 1 << 28, "bxor", "fullrange", 3000, "rank_asc"),
+    "c4_u8_lxor": ("u8", 1 << 28, "lxor", "bool01", 3000, "rank_asc"),
+}
+P = 8
+
+
+def run_combine_workload(al, torch, name, steps, warmup, check=True):
+    dtype, count, op, dist, seed, order = WORKLOADS[name]
+    es = al.dtype_size(dtype)
+    carrier = al.torch_dtype(dtype)
+    ins = [torch.empty(count, dtype=carrier, device="cuda") for _ in range(P)]
+    out = torch.empty(count, dtype=carrier, device="cuda")
+    for r in range(P):
+        al.fill(ins[r], dist, seed + r, dtype=dtype)
+    torch.cuda.synchronize()
+    for _ in range(warmup):
+        al.combine([out], ins, op, order=order, dtype=dtype)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        al.combine([out], ins, op, order=order, dtype=dtype)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_ms = ev0.elapsed_time(ev1) / steps
+    alg_bytes = (P + 1) * count * es
+    res = {
+        "workload": name, "dtype": dtype, "op": op, "order": order, "P": P, "count": count,
+        "algorithmic_bytes": alg_bytes, "ms_per_step": wall * 1e3 / steps, "kernel_ms": kernel_ms,
+        "gbps_wall": alg_bytes / (wall / steps) * 1e-9, "gbps_kernel": alg_bytes / (kernel_ms * 1e-3) * 1e-9,
+    }
+    if check:
+        # parity spot-check against the CPU oracle on the first and last 2^18 elements
+        import numpy as np
+        import oracle
+        m = 1 << 18
+        np_dt = oracle.NP_CARRIER[dtype]
+        ok = True
+        for lo in (0, count - m):
+            want = oracle.combine_generated(P, m, dtype, op, order, 0, dist, seed, lo)
+            got = out[lo:lo + m].cpu().numpy().view(np_dt)
+            ok = ok and got.tobytes() == want.tobytes()
+        res["parity_vs_oracle"] = bool(ok)
+    del ins, out
+    torch.cuda.empty_cache()
+    return res
+
+
+def cpu_baseline():
+    """The reference's MPI-backend host combine on this box's host cores."""
+    exe = os.path.join(ROOT, "oracle", "mpi_baseline")
+    mpiexec = "/opt/conda/bin/mpiexec"
+    if os.path.exists(exe) and os.path.exists(mpiexec):
+        try:
+            p = subprocess.run([mpiexec, "-n", "4", exe, str(1 << 20), "10", "100"], capture_output=True,
+                               text=True, timeout=120)
+            line = [l for l in p.stdout.splitlines() if l.startswith("{")]
+            if p.returncode == 0 and line:
+                r = json.loads(line[-1])
+                return {"value": r["gbps_median"], "unit": "GB/s", "cores": 4, "kind": "port",
+                        "sample": "MPI_Allreduce(MPI_SUM, MPI_FLOAT) on a dup'd communicator, the call "
+                                  "Al::Allreduce<MPIBackend> forwards to; 4 MPICH ranks on this host, "
+                                  "2^20 elements per rank, uniform[-1,1] seed 1000+rank, 10 warm-up + 100 "
+                                  "timed, median of max-over-ranks; GB/s over (P+1)*n*4 bytes",
+                        "median_ms": r["median_ms"], "min_ms": r["min_ms"],
+                        "host_cpus": os.cpu_count()}
+        except Exception:
+            pass
+    # MPI-free restatement: the oracle's threaded tree combine on the same shape
+    import numpy as np
+    import oracle
+    n, ranks = 1 << 20, 4
+    ins = [oracle.fill(n, "f32", "uniform_pm1", 1000 + r) for r in range(ranks)]
+    ts = []
+    for _ in range(30):
+        t0 = time.perf_counter()
+        oracle.combine(ins, "f32", "sum", "tree_dbl")
+        ts.append(time.perf_counter() - t0)
+    med = sorted(ts)[len(ts) // 2]
+    return {"value": (ranks + 1) * n * 4 / med * 1e-9, "unit": "GB/s", "cores": oracle.num_threads(),
+            "kind": "port", "sample": "MPI-free restatement: CPU oracle TREE_DBL combine, 4 buffers of 2^20 "
+                                      "fp32, median of 30", "median_ms": med * 1e3,
+            "host_cpus": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2_f32_sum", choices=sorted(WORKLOADS))
+    ap.add_argument("--also", default="c2_bf16_sum",
+                    help="comma-separated extra workloads reported under 'also' ('' for none)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the P logical ranks live in one GPU's HBM); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import aluminum_amd as al
+    al.load()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    rc = al.load().alamd_init()
+    if rc:
+        print("bench.py: " + al.load().alamd_last_error().decode(), file=sys.stderr)
+        sys.exit(1)
+
+    main_res = run_combine_workload(al, torch, args.workload, args.steps, args.warmup)
+    also = {}
+    for name in [w for w in args.also.split(",") if w and w != args.workload]:
+        also[name] = run_combine_workload(al, torch, name, max(5, args.steps // 2), max(2, args.warmup // 2))
+
+    out = {
+        "metric": METRIC, "value": main_res["gbps_wall"], "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": main_res["dtype"], "data": "synthetic",
+        "config": {"workload": "C2 single-GPU P-way combine: P=8 logical-rank fp32 buffers of 2^26 elements "
+                               "(2 GiB in, 256 MiB out), ReductionOperator::sum, order %s" % main_res["order"]
+                   if args.workload == "c2_f32_sum" else args.workload,
+                   "P": P, "count_per_rank": main_res["count"], "op": main_res["op"], "order": main_res["order"],
+                   "entry_point": "alamd_combine"},
+        "pct_of_hbm_peak": 100.0 * main_res["gbps_wall"] / HBM_PEAK_GBPS,
+        "parity_vs_oracle": main_res.get("parity_vs_oracle"),
+        "roofline": {"bound": "hbm", "achieved": main_res["gbps_kernel"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": main_res["gbps_kernel"] / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "fold_kernel<float, sum, P=8>", "kernel_ms": main_res["kernel_ms"],
+                     "algorithmic_bytes": main_res["algorithmic_bytes"]},
+        "also": also,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

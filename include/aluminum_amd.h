@@ -1,0 +1,263 @@
+/*
+ * aluminum_amd - MI355X (gfx950) on-device combine engine for the
+ * Al::Allreduce / Reduce_scatter / Allgather hot path of Aluminum.
+ *
+ * C ABI.  No C++ or HIP types cross this boundary: streams are passed as
+ * `void *` (a hipStream_t; NULL is the default stream), buffers as device
+ * pointers.  Every call that takes a stream only enqueues work on it and
+ * returns; buffers are caller-owned and must stay valid until the stream has
+ * passed the call (reference contract: docs/comm.rst:18, docs/index.rst:33-40).
+ * Calls return ALAMD_OK or a negative-free small error code; the message of
+ * the last error on the calling thread is alamd_last_error().  The library is
+ * thread-compatible: concurrent calls are fine as long as they do not share a
+ * stream or output buffers.
+ *
+ * The reference has no C ABI; its boundary is a compile-time backend policy
+ * class (include/aluminum/ht_impl.hpp:125-1111).  The header-only C++ shim
+ * include/aluminum_amd/Al.hpp maps that class interface onto the functions
+ * below, turning error codes into Al::al_exception.
+ */
+#ifndef ALUMINUM_AMD_H
+#define ALUMINUM_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ALAMD_VERSION_MAJOR 0
+#define ALAMD_VERSION_MINOR 1
+
+/* Largest number of logical ranks one call can combine. */
+#define ALAMD_MAX_RANKS 64
+/* Largest number of logical ranks under the tree orders. */
+#define ALAMD_MAX_TREE_RANKS 32
+
+typedef enum {
+  ALAMD_OK = 0,
+  ALAMD_ERR_INVALID_ARG = 1,     /* null pointer, bad count, bad rank count        */
+  ALAMD_ERR_UNSUPPORTED_OP = 2,  /* "Reduction operator not supported"
+                                    (include/aluminum/mpi/utils.hpp:192-194)       */
+  ALAMD_ERR_UNSUPPORTED_TYPE = 3,
+  ALAMD_ERR_INVALID_ALGO = 4,    /* "Invalid algorithm" (ht_impl.hpp:156-158)      */
+  ALAMD_ERR_OVERLAP = 5,         /* partially overlapping buffers
+                                    (include/aluminum/debug_helpers.hpp:117-135)   */
+  ALAMD_ERR_HIP = 6,             /* a HIP runtime call failed                      */
+  ALAMD_ERR_TIMEOUT = 7,         /* a bounded wait expired                         */
+  ALAMD_ERR_UNSUPPORTED = 8      /* feature not available on this device           */
+} alamd_status;
+
+/* Element types: the arithmetic types of mpi::TypeMap<T>
+ * (include/aluminum/mpi/utils.hpp:43-67) by width and signedness, plus the
+ * two 16-bit float types of include/aluminum/datatypes.hpp:37-56. */
+typedef enum {
+  ALAMD_I8 = 0, ALAMD_U8 = 1, ALAMD_I16 = 2, ALAMD_U16 = 3, ALAMD_I32 = 4,
+  ALAMD_U32 = 5, ALAMD_I64 = 6, ALAMD_U64 = 7, ALAMD_F16 = 8, ALAMD_BF16 = 9,
+  ALAMD_F32 = 10, ALAMD_F64 = 11, ALAMD_NUM_DTYPES = 12
+} alamd_dtype;
+
+/* Numerically identical to Al::ReductionOperator
+ * (include/aluminum/base.hpp:103-105), so the C++ shim casts.  avg is
+ * rejected with ALAMD_ERR_UNSUPPORTED_OP exactly as the reference's MPI and
+ * host-transfer backends reject it. */
+typedef enum {
+  ALAMD_SUM = 0, ALAMD_PROD = 1, ALAMD_MIN = 2, ALAMD_MAX = 3, ALAMD_LOR = 4,
+  ALAMD_LAND = 5, ALAMD_LXOR = 6, ALAMD_BOR = 7, ALAMD_BAND = 8, ALAMD_BXOR = 9,
+  ALAMD_AVG = 10
+} alamd_op;
+
+/* Named combine orders.  One pairwise step is always
+ *   result = OP(inout, in)
+ * with the operand roles of an MPI reduction function (for fp16 / bf16:
+ * src/mpi_impl.cpp:61-145); the order names which operand plays which role
+ * and in what sequence the P contributions meet.
+ *   RANK_ASC       acc = x0; acc = step(in = x_k, inout = acc), k = 1..P-1
+ *   PAIRWISE_DESC  acc = x_s; acc = step(in = x_{s-k}, inout = acc)  (wrap)
+ *   RING           acc = x_s; acc = step(in = acc, inout = x_{s+k})  (wrap)
+ *   TREE_BINOMIAL  distance 1,2,4..: x_i = step(in = x_{i+d}, inout = x_i)
+ *                  for every i that is a multiple of 2d with i+d < P
+ *   TREE_DBL       the first 2*(P - 2^k) ranks fold pairwise
+ *                  (step(in = x_{2j}, inout = x_{2j+1})), the 2^k survivors
+ *                  then pair at distance 1,2,4,...
+ *   TREE_HALV      the same pre-fold, survivors pair at distance 2^k/2,...,1
+ * With MPICH 3.3.2 on one host the reference's MPI backend produces
+ * TREE_BINOMIAL (Allreduce up to 2048 bytes), TREE_DBL (larger Allreduce),
+ * TREE_HALV (Reduce_scatter below 512 KiB in total) and PAIRWISE_DESC with
+ * s = receiving rank (larger Reduce_scatter). */
+typedef enum {
+  ALAMD_ORDER_RANK_ASC = 0,
+  ALAMD_ORDER_TREE_DBL = 1,
+  ALAMD_ORDER_TREE_HALV = 2,
+  ALAMD_ORDER_PAIRWISE_DESC = 3,
+  ALAMD_ORDER_RING = 4,
+  ALAMD_ORDER_TREE_BINOMIAL = 5
+} alamd_order;
+
+/* ---- library ---------------------------------------------------------- */
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char *alamd_last_error(void);
+/* major * 100 + minor */
+int alamd_version(void);
+/* Bytes per element, 0 for an unknown dtype. */
+size_t alamd_dtype_size(int dtype);
+/* ALAMD_OK if `op` is defined for `dtype`
+ * (include/aluminum/mpi/utils.hpp:169-269: every op but avg for the native
+ * types; sum, prod, min, max for fp16 / bf16; MPI defines the logical and
+ * bitwise ops for integers only). */
+int alamd_check_op(int dtype, int op);
+/* Selects nothing and allocates nothing; checks that the current device is a
+ * gfx950 and caches its compute-unit count.  Optional: every entry point
+ * performs it on first use.  (Replaces internal::cuda::init,
+ * src/cuda/cuda.cpp:52-78.) */
+int alamd_init(void);
+
+/* ---- combine: the element-wise fold of P rank contributions ----------- */
+
+/* outs[j][i] = fold over r of ins[r][i], i in [0, count), for each of the
+ * `nout` output buffers.  This is the arithmetic the reference delegates to
+ * MPI_Iallreduce on a pinned host copy
+ * (include/aluminum/ht/allreduce.hpp:41-79) or to MPI_Allreduce
+ * (include/aluminum/mpi/allreduce.hpp:38-44); nout = 1 is a Reduce
+ * (include/aluminum/ht/reduce.hpp:72-82), nout = P an Allreduce over P
+ * logical ranks.  An output may be identical to an input (in-place), but
+ * must not overlap one partially.  `start` is the rank s of the orders that
+ * have one and must be 0 otherwise. */
+int alamd_combine(void *const *outs, int nout, const void *const *ins, int P,
+                  size_t count, int dtype, int op, int order, int start,
+                  void *stream);
+
+/* Reduce_scatter over P logical ranks: sends[r] holds P*count elements;
+ * recvs[b] receives count elements, the fold of block b of every sends[r],
+ * with start = b for the orders that have one.  In-place form
+ * (recvs[b] == sends[b]) puts the result at the start of the buffer.
+ * Replaces MPI_Ireduce_scatter_block on the host copy
+ * (include/aluminum/ht/reduce_scatter.hpp:45-74; layout docs/comm.rst:284-285). */
+int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P,
+                         size_t count, int dtype, int op, int order,
+                         void *stream);
+
+/* Allgather over P logical ranks: recvs[r][q*count + i] = sends[q][i].
+ * In-place form: sends[q] == recvs[q] + q*count elements
+ * (include/aluminum/ht/allgather.hpp:48-81; docs/comm.rst:152). */
+int alamd_allgather(void *const *recvs, const void *const *sends, int P,
+                    size_t count, int dtype, void *stream);
+
+/* ---- ring reduce-scatter + allgather over P logical ranks ------------- */
+
+typedef enum {
+  /* one launch per ring step; every byte a real ring moves is moved */
+  ALAMD_RING_STEPWISE = 0,
+  /* one launch; each segment is folded in registers in ring order and
+   * written once to every rank (same bits, fewer bytes) */
+  ALAMD_RING_FUSED = 1
+} alamd_ring_mode;
+
+/* In place on bufs[0..P-1], each `count` elements.  Segment s is
+ * [s*q + min(s, m), ...) with q = count / P, m = count % P, and the first m
+ * segments one element longer.  Reduce-scatter step t = 0..P-2: rank r
+ * receives segment (r-t-1) mod P from rank r-1 and applies
+ * local = step(in = received, inout = local); afterwards rank r holds the
+ * fully reduced segment (r+1) mod P.  Allgather step t: rank r receives
+ * segment (r-t) mod P from rank r-1.  Segments move in chunks of
+ * `chunk_bytes` (a multiple of the element size; the chunk is the unit of
+ * work of one workgroup pass and does not change any bit of the result).
+ * The reference names the algorithm (mpi_impl.hpp:83-90 `mpi_ring`) but
+ * carries no implementation of it. */
+int alamd_ring_allreduce(void *const *bufs, int P, size_t count, int dtype,
+                         int op, size_t chunk_bytes, int mode, void *stream);
+int alamd_ring_reduce_scatter(void *const *bufs, int P, size_t count, int dtype,
+                              int op, size_t chunk_bytes, int mode, void *stream);
+int alamd_ring_allgather(void *const *bufs, int P, size_t count, int dtype,
+                         size_t chunk_bytes, void *stream);
+/* Offset and length (in elements) of ring segment s. */
+int alamd_ring_segment(size_t count, int P, int s, size_t *offset, size_t *len);
+
+/* ---- halo faces -------------------------------------------------------- */
+
+/* A 3-D grid, x fastest: interior dims[0] x dims[1] x dims[2], halo width
+ * `halo` on all six sides, allocation (dims[d] + 2*halo) per axis.  Faces:
+ * 0 -x, 1 +x, 2 -y, 3 +y, 4 -z, 5 +z; a face excludes edges and corners and
+ * its buffer keeps the grid's index order (x fastest).  pack copies the
+ * interior boundary slab of each selected face into its send buffer; unpack
+ * copies each receive buffer into the ghost slab of its face.  `face_mask`
+ * selects faces (bit f); bufs[f] is ignored for unselected faces.  All
+ * selected faces are handled by one launch.  These produce the contiguous
+ * buffers that Al::ext::Put moves (include/aluminum/mpi_cuda/rma_ipc.hpp:287-301,
+ * test/test_rma_halo_exchange.cpp:171-197); the reference itself has no
+ * strided faces. */
+int alamd_halo_pack(void *const bufs[6], const void *grid, const size_t dims[3],
+                    size_t halo, size_t elem_size, unsigned face_mask, void *stream);
+int alamd_halo_unpack(void *grid, const void *const bufs[6], const size_t dims[3],
+                      size_t halo, size_t elem_size, unsigned face_mask, void *stream);
+/* Elements in the buffer of `face`. */
+size_t alamd_halo_face_elems(const size_t dims[3], size_t halo, int face);
+
+/* ---- stream flags ------------------------------------------------------ */
+
+/* One int32 synchronisation word in pinned, device-mapped host memory on its
+ * own 128-byte line (include/aluminum/cuda/sync_memory.hpp:46-60). */
+typedef struct alamd_flag alamd_flag;
+
+typedef enum {
+  ALAMD_FLAG_AUTO = 0,   /* stream memory operation if the device has them  */
+  ALAMD_FLAG_MEMOP = 1,  /* hipStreamWaitValue32 / hipStreamWriteValue32    */
+  ALAMD_FLAG_KERNEL = 2  /* single-lane spin kernel / store kernel          */
+} alamd_flag_mode;
+
+int alamd_flag_create(alamd_flag **flag, int32_t initial);
+int alamd_flag_destroy(alamd_flag *flag);
+/* Host address of the word. */
+volatile int32_t *alamd_flag_host_ptr(alamd_flag *flag);
+/* 1 if stream memory operations are usable on the current device
+ * (internal::cuda::stream_memory_operations_supported, src/cuda/cuda.cpp:52-88). */
+int alamd_stream_memops_supported(void);
+/* Blocks `stream` until the word equals `value`
+ * (launch_wait_kernel / spin_wait_kernel, src/cuda/helper_kernels.cu:42-71;
+ * GPUWait::wait, src/cuda/gpu_wait.cpp:64-70).  In ALAMD_FLAG_KERNEL mode
+ * `max_spins` bounds the number of polls (0 = unbounded, as the reference);
+ * a wait that gives up stores 1 to the word returned by
+ * alamd_flag_timed_out(). */
+int alamd_stream_wait_flag(void *stream, alamd_flag *flag, int32_t value,
+                           int mode, uint64_t max_spins);
+/* Has `stream` store `value` into the word when it gets there
+ * (GPUStatusFlag::record, src/cuda/gpu_status_flag.cpp:65-82). */
+int alamd_stream_write_flag(void *stream, alamd_flag *flag, int32_t value, int mode);
+/* Host-side atomic store / load (GPUWait::signal, src/cuda/gpu_wait.cpp:72-74;
+ * GPUStatusFlag::query, src/cuda/gpu_status_flag.cpp:84-87). */
+int alamd_flag_signal(alamd_flag *flag, int32_t value);
+int32_t alamd_flag_query(alamd_flag *flag);
+/* 1 if a bounded kernel wait on this flag has expired since creation. */
+int alamd_flag_timed_out(alamd_flag *flag);
+
+/* ---- test and bench support -------------------------------------------- */
+
+/* Input distributions of the counter-based generator. */
+typedef enum {
+  ALAMD_DIST_UNIFORM_PM1 = 0, ALAMD_DIST_UNIFORM_09_11 = 1, ALAMD_DIST_UNIFORM_01 = 2,
+  ALAMD_DIST_FULLRANGE = 3, ALAMD_DIST_BOOL01 = 4, ALAMD_DIST_NORMAL = 5,
+  ALAMD_DIST_SMALLINT = 6
+} alamd_dist;
+
+/* dst[i] = value of element (idx0 + i) of stream `seed` under `dist`: a pure
+ * integer hash followed by correctly rounded fp64 operations, so a host
+ * implementation of the same formula yields the same bits.  (Stands in for
+ * gen_data, test/test_utils.hpp:157-256, whose libstdc++ distributions are
+ * not reproducible on a device.) */
+int alamd_fill(void *dst, size_t count, int dtype, int dist, uint64_t seed,
+               uint64_t idx0, void *stream);
+/* The library's own fp32 -> fp16 / bf16 narrowing and the exact widening,
+ * as used inside the combine kernels (exposed so that all 2^32 inputs can be
+ * checked). */
+int alamd_narrow_f32(void *dst16, const float *src, size_t count, int dtype, void *stream);
+int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void *stream);
+/* dst[i] = src[i] for `bytes` bytes with the same load / store path as the
+ * combine kernels: the practical 1-read + 1-write bandwidth ceiling. */
+int alamd_copy(void *dst, const void *src, size_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,636 @@
+/*
+ * CPU oracle for the Aluminum combine hot path.  TEST INFRASTRUCTURE ONLY:
+ * the checker for the GPU library, never a fallback for it.  See oracle.h for
+ * what each function restates and what pins it.
+ */
+#include "oracle.h"
+
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ------------------------------------------------------------------------ */
+/* dtype table                                                              */
+/* ------------------------------------------------------------------------ */
+
+size_t alo_dtype_size(int dtype) {
+  switch (dtype) {
+  case ALO_I8: case ALO_U8: return 1;
+  case ALO_I16: case ALO_U16: case ALO_F16: case ALO_BF16: return 2;
+  case ALO_I32: case ALO_U32: case ALO_F32: return 4;
+  case ALO_I64: case ALO_U64: case ALO_F64: return 8;
+  default: return 0;
+  }
+}
+
+static int is_float_dtype(int dtype) {
+  return dtype == ALO_F16 || dtype == ALO_BF16 || dtype == ALO_F32 ||
+         dtype == ALO_F64;
+}
+
+/* include/aluminum/mpi/utils.hpp:169-233: the generic map accepts sum..bxor
+ * and throws on avg; the __half / bfloat specialisations accept only
+ * sum, prod, min, max.  MPI itself defines the logical and bitwise ops for
+ * integer types only, so fp32/fp64 with them is an error at the MPI call. */
+int alo_check_op(int dtype, int op) {
+  if (alo_dtype_size(dtype) == 0) return 2;
+  if (op < ALO_SUM || op > ALO_BXOR) return 1;
+  if (is_float_dtype(dtype) && op > ALO_MAX) return 1;
+  return 0;
+}
+
+int alo_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+
+void alo_set_num_threads(int n) {
+#ifdef _OPENMP
+  if (n > 0) omp_set_num_threads(n);
+#else
+  (void)n;
+#endif
+}
+
+/* ------------------------------------------------------------------------ */
+/* 16-bit float conversions                                                 */
+/* ------------------------------------------------------------------------ */
+
+static inline uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float bits_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* __bfloat162float: the bf16 pattern is the top half of the fp32 pattern. */
+float alo_bf16_to_f32(uint16_t h) { return bits_f32((uint32_t)h << 16); }
+
+/* __float2bfloat16 (src/mpi_impl.cpp:110): round to nearest, ties to even.
+ * A NaN stays a NaN: quiet bit set, upper payload bits kept. */
+uint16_t alo_f32_to_bf16(float f) {
+  uint32_t u = f32_bits(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+/* __half2float: exact widening, subnormals normalised. */
+float alo_f16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  if (exp == 0x1fu) return bits_f32(sign | 0x7f800000u | (man << 13));
+  if (exp == 0) {
+    if (man == 0) return bits_f32(sign);
+    int e = -1;
+    do { man <<= 1; e++; } while (!(man & 0x400u));
+    man &= 0x3ffu;
+    return bits_f32(sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13));
+  }
+  return bits_f32(sign | ((exp + 127 - 15) << 23) | (man << 13));
+}
+
+/* __float2half (src/mpi_impl.cpp:66): round to nearest, ties to even, with
+ * gradual underflow and overflow to infinity. */
+uint16_t alo_f32_to_f16(float f) {
+  uint32_t u = f32_bits(f);
+  uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+  uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) /* NaN: quiet, keep upper payload */
+    return (uint16_t)(sign | 0x7e00u | ((a >> 13) & 0x3ffu));
+  if (a >= 0x47800000u) { /* |f| >= 65536 (incl. inf) -> inf; 65520..65536 handled below */
+    return (uint16_t)(sign | 0x7c00u);
+  }
+  if (a >= 0x38800000u) { /* normal half range: |f| >= 2^-14 */
+    uint32_t r = a - 0x38000000u; /* rebias exponent by 112 */
+    uint32_t lsb = (r >> 13) & 1u;
+    r += 0xfffu + lsb;
+    return (uint16_t)(sign | (r >> 13)); /* may carry into exponent / infinity: correct */
+  }
+  if (a < 0x33000000u) return sign; /* |f| < 2^-25 -> 0 (2^-25 itself ties to even 0 below) */
+  {
+    /* subnormal half: value = man * 2^-24 */
+    uint32_t e = a >> 23;               /* 102..112 */
+    uint32_t m = (a & 0x7fffffu) | 0x800000u;
+    uint32_t shift = 126u - e;          /* 14..24 : m >> shift gives units of 2^-24 */
+    uint32_t q = m >> shift;
+    uint32_t rem = m & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1u);
+    if (rem > half || (rem == half && (q & 1u))) q++;
+    return (uint16_t)(sign | q);
+  }
+}
+
+void alo_f32_to_bf16_array(uint16_t *dst, const float *src, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) dst[i] = alo_f32_to_bf16(src[i]);
+}
+void alo_f32_to_f16_array(uint16_t *dst, const float *src, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) dst[i] = alo_f32_to_f16(src[i]);
+}
+void alo_bf16_to_f32_array(float *dst, const uint16_t *src, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) dst[i] = alo_bf16_to_f32(src[i]);
+}
+void alo_f16_to_f32_array(float *dst, const uint16_t *src, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; i++) dst[i] = alo_f16_to_f32(src[i]);
+}
+
+/* ------------------------------------------------------------------------ */
+/* Counter-based input generator                                            */
+/* ------------------------------------------------------------------------ */
+
+#define ALO_GAMMA 0x9E3779B97F4A7C15ull
+
+static inline uint64_t fin64(uint64_t z) {
+  z ^= z >> 30; z *= 0xBF58476D1CE4E5B9ull;
+  z ^= z >> 27; z *= 0x94D049BB133111EBull;
+  z ^= z >> 31;
+  return z;
+}
+
+uint64_t alo_mix64(uint64_t seed, uint64_t idx) {
+  return fin64(fin64(seed + ALO_GAMMA) + (idx + 1) * ALO_GAMMA);
+}
+
+/* Sum of the twelve 16-bit fields of three chained 64-bit words. */
+static inline uint32_t ih12_sum(uint64_t b0) {
+  uint64_t b1 = fin64(b0 + ALO_GAMMA), b2 = fin64(b1 + ALO_GAMMA);
+  uint32_t s = 0;
+  for (int k = 0; k < 4; k++) {
+    s += (uint32_t)((b0 >> (16 * k)) & 0xffffu);
+    s += (uint32_t)((b1 >> (16 * k)) & 0xffffu);
+    s += (uint32_t)((b2 >> (16 * k)) & 0xffffu);
+  }
+  return s;
+}
+
+/* Real-valued draws are made in fp64 (every operation below is a single
+ * correctly rounded IEEE operation, so host and device agree bit for bit) and
+ * narrowed once, round-to-nearest-even, for the narrower types.  The uniform
+ * draws keep full significands at every magnitude, so that different
+ * summation orders really do round differently. */
+static inline double gen_f64(uint64_t bits, int dist) {
+  switch (dist) {
+  case ALO_DIST_UNIFORM_09_11: {
+    double u = (double)(bits >> 11) * 0x1p-53; /* exact */
+    double t = u * 0.2;                        /* rounded product */
+    return 0.9 + t;                            /* rounded sum, no fma */
+  }
+  case ALO_DIST_UNIFORM_01: return (double)(bits >> 11) * 0x1p-53;
+  case ALO_DIST_BOOL01: return (double)(bits >> 63);
+  case ALO_DIST_NORMAL: return (double)ih12_sum(bits) * 0x1p-16 - 6.0;
+  case ALO_DIST_SMALLINT: return (double)((int)(bits >> 60) - 8);
+  default:
+    /* one rounding (int64 -> fp64, nearest-even), then an exact scaling */
+    return (double)(int64_t)bits * 0x1p-63;
+  }
+}
+
+static inline float gen_f32(uint64_t bits, int dist) {
+  return (float)gen_f64(bits, dist);
+}
+
+static inline uint64_t gen_int(uint64_t bits, int dist, int is_signed) {
+  switch (dist) {
+  case ALO_DIST_FULLRANGE: return bits;
+  case ALO_DIST_BOOL01: return bits >> 63;
+  default:
+    return is_signed ? (uint64_t)((int64_t)(bits >> 60) - 8) : (bits >> 60);
+  }
+}
+
+static void fill_range(void *dst, size_t n, int dtype, int dist, uint64_t seed,
+                       uint64_t idx0) {
+  for (size_t i = 0; i < n; i++) {
+    uint64_t bits = alo_mix64(seed, idx0 + i);
+    switch (dtype) {
+    case ALO_I8: ((int8_t *)dst)[i] = (int8_t)gen_int(bits, dist, 1); break;
+    case ALO_U8: ((uint8_t *)dst)[i] = (uint8_t)gen_int(bits, dist, 0); break;
+    case ALO_I16: ((int16_t *)dst)[i] = (int16_t)gen_int(bits, dist, 1); break;
+    case ALO_U16: ((uint16_t *)dst)[i] = (uint16_t)gen_int(bits, dist, 0); break;
+    case ALO_I32: ((int32_t *)dst)[i] = (int32_t)gen_int(bits, dist, 1); break;
+    case ALO_U32: ((uint32_t *)dst)[i] = (uint32_t)gen_int(bits, dist, 0); break;
+    case ALO_I64: ((int64_t *)dst)[i] = (int64_t)gen_int(bits, dist, 1); break;
+    case ALO_U64: ((uint64_t *)dst)[i] = gen_int(bits, dist, 0); break;
+    case ALO_F16: ((uint16_t *)dst)[i] = alo_f32_to_f16(gen_f32(bits, dist)); break;
+    case ALO_BF16: ((uint16_t *)dst)[i] = alo_f32_to_bf16(gen_f32(bits, dist)); break;
+    case ALO_F32: ((float *)dst)[i] = gen_f32(bits, dist); break;
+    case ALO_F64: ((double *)dst)[i] = gen_f64(bits, dist); break;
+    default: break;
+    }
+  }
+}
+
+void alo_fill(void *dst, size_t n, int dtype, int dist, uint64_t seed,
+              uint64_t idx0) {
+  const size_t es = alo_dtype_size(dtype);
+  const size_t tile = 1u << 14;
+  const size_t ntiles = (n + tile - 1) / tile;
+  if (es == 0) return;
+#pragma omp parallel for schedule(static)
+  for (size_t t = 0; t < ntiles; t++) {
+    size_t lo = t * tile, len = n - lo < tile ? n - lo : tile;
+    fill_range((char *)dst + lo * es, len, dtype, dist, seed, idx0 + lo);
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* The pairwise step: inout[i] = in[i] OP inout[i]                          */
+/* ------------------------------------------------------------------------ */
+
+/* Integers.  a = invec element, b = inoutvec element.  Sum and product wrap
+ * (computed unsigned so the oracle itself has no undefined behaviour). */
+#define DEF_INT_STEP(NAME, T)                                                   \
+  static int step_##NAME(T *b, const T *a, size_t n, int op) {                  \
+    size_t i;                                                                   \
+    switch (op) {                                                               \
+    case ALO_SUM: for (i = 0; i < n; i++) b[i] = (T)((uint64_t)a[i] + (uint64_t)b[i]); break; \
+    case ALO_PROD: for (i = 0; i < n; i++) b[i] = (T)((uint64_t)a[i] * (uint64_t)b[i]); break; \
+    case ALO_MIN: for (i = 0; i < n; i++) b[i] = (b[i] < a[i]) ? b[i] : a[i]; break; \
+    case ALO_MAX: for (i = 0; i < n; i++) b[i] = (b[i] > a[i]) ? b[i] : a[i]; break; \
+    case ALO_LOR: for (i = 0; i < n; i++) b[i] = (T)(a[i] || b[i]); break;      \
+    case ALO_LAND: for (i = 0; i < n; i++) b[i] = (T)(a[i] && b[i]); break;     \
+    case ALO_LXOR: for (i = 0; i < n; i++) b[i] = (T)((a[i] && !b[i]) || (!a[i] && b[i])); break; \
+    case ALO_BOR: for (i = 0; i < n; i++) b[i] = (T)(a[i] | b[i]); break;       \
+    case ALO_BAND: for (i = 0; i < n; i++) b[i] = (T)(a[i] & b[i]); break;      \
+    case ALO_BXOR: for (i = 0; i < n; i++) b[i] = (T)(a[i] ^ b[i]); break;      \
+    default: return 1;                                                          \
+    }                                                                           \
+    return 0;                                                                   \
+  }
+
+DEF_INT_STEP(i8, int8_t)
+DEF_INT_STEP(u8, uint8_t)
+DEF_INT_STEP(i16, int16_t)
+DEF_INT_STEP(u16, uint16_t)
+DEF_INT_STEP(i32, int32_t)
+DEF_INT_STEP(u32, uint32_t)
+DEF_INT_STEP(i64, int64_t)
+DEF_INT_STEP(u64, uint64_t)
+
+/* fp32 / fp64: the MPI predefined ops, inoutvec[i] = OP(inoutvec[i], invec[i]):
+ * MIN(x, y) is (x < y) ? x : y and MAX(x, y) is (x > y) ? x : y, so a tie or a
+ * NaN on either side yields the invec element. */
+#define DEF_FP_STEP(NAME, T)                                                    \
+  static int step_##NAME(T *b, const T *a, size_t n, int op) {                  \
+    size_t i;                                                                   \
+    switch (op) {                                                               \
+    case ALO_SUM: for (i = 0; i < n; i++) b[i] = a[i] + b[i]; break;            \
+    case ALO_PROD: for (i = 0; i < n; i++) b[i] = a[i] * b[i]; break;           \
+    case ALO_MIN: for (i = 0; i < n; i++) b[i] = (b[i] < a[i]) ? b[i] : a[i]; break; \
+    case ALO_MAX: for (i = 0; i < n; i++) b[i] = (b[i] > a[i]) ? b[i] : a[i]; break; \
+    default: return 1;                                                          \
+    }                                                                           \
+    return 0;                                                                   \
+  }
+
+DEF_FP_STEP(f32, float)
+DEF_FP_STEP(f64, double)
+
+/* fp16 / bf16: src/mpi_impl.cpp:61-145.  std::min(x, y) is (y < x) ? y : x
+ * and std::max(x, y) is (x < y) ? y : x, called with x = float(invec[i]),
+ * y = float(inoutvec[i]); the chosen fp32 value is narrowed again. */
+#define DEF_H_STEP(NAME, WIDEN, NARROW)                                         \
+  static int step_##NAME(uint16_t *b, const uint16_t *a, size_t n, int op) {    \
+    size_t i;                                                                   \
+    switch (op) {                                                               \
+    case ALO_SUM: for (i = 0; i < n; i++) b[i] = NARROW(WIDEN(a[i]) + WIDEN(b[i])); break; \
+    case ALO_PROD: for (i = 0; i < n; i++) b[i] = NARROW(WIDEN(a[i]) * WIDEN(b[i])); break; \
+    case ALO_MIN: for (i = 0; i < n; i++) { float x = WIDEN(a[i]), y = WIDEN(b[i]); b[i] = NARROW((y < x) ? y : x); } break; \
+    case ALO_MAX: for (i = 0; i < n; i++) { float x = WIDEN(a[i]), y = WIDEN(b[i]); b[i] = NARROW((x < y) ? y : x); } break; \
+    default: return 1;                                                          \
+    }                                                                           \
+    return 0;                                                                   \
+  }
+
+DEF_H_STEP(f16, alo_f16_to_f32, alo_f32_to_f16)
+DEF_H_STEP(bf16, alo_bf16_to_f32, alo_f32_to_bf16)
+
+static int step_serial(void *inout, const void *in, size_t n, int dtype, int op) {
+  switch (dtype) {
+  case ALO_I8: return step_i8((int8_t *)inout, (const int8_t *)in, n, op);
+  case ALO_U8: return step_u8((uint8_t *)inout, (const uint8_t *)in, n, op);
+  case ALO_I16: return step_i16((int16_t *)inout, (const int16_t *)in, n, op);
+  case ALO_U16: return step_u16((uint16_t *)inout, (const uint16_t *)in, n, op);
+  case ALO_I32: return step_i32((int32_t *)inout, (const int32_t *)in, n, op);
+  case ALO_U32: return step_u32((uint32_t *)inout, (const uint32_t *)in, n, op);
+  case ALO_I64: return step_i64((int64_t *)inout, (const int64_t *)in, n, op);
+  case ALO_U64: return step_u64((uint64_t *)inout, (const uint64_t *)in, n, op);
+  case ALO_F16: return step_f16((uint16_t *)inout, (const uint16_t *)in, n, op);
+  case ALO_BF16: return step_bf16((uint16_t *)inout, (const uint16_t *)in, n, op);
+  case ALO_F32: return step_f32((float *)inout, (const float *)in, n, op);
+  case ALO_F64: return step_f64((double *)inout, (const double *)in, n, op);
+  default: return 2;
+  }
+}
+
+#define ALO_TILE 4096u
+
+int alo_step(void *inout, const void *in, size_t n, int dtype, int op) {
+  const size_t es = alo_dtype_size(dtype);
+  int rc = alo_check_op(dtype, op);
+  if (rc) return rc;
+  const size_t ntiles = (n + ALO_TILE - 1) / ALO_TILE;
+#pragma omp parallel for schedule(static)
+  for (size_t t = 0; t < ntiles; t++) {
+    size_t lo = t * ALO_TILE, len = n - lo < ALO_TILE ? n - lo : ALO_TILE;
+    step_serial((char *)inout + lo * es, (const char *)in + lo * es, len, dtype, op);
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Named orders as schedules of pairwise steps                              */
+/* ------------------------------------------------------------------------ */
+
+static int floor_pow2(int p) { int q = 1; while (2 * q <= p) q *= 2; return q; }
+
+int alo_schedule(int P, int order, int start, int *pairs, int *result) {
+  int np = 0;
+  if (P < 1 || P > 1024) return -1;
+  if (start < 0 || start >= P) return -1;
+  switch (order) {
+  case ALO_ORDER_RANK_ASC:
+    for (int k = 1; k < P; k++) { pairs[2 * np] = 0; pairs[2 * np + 1] = k; np++; }
+    *result = 0;
+    return np;
+  case ALO_ORDER_PAIRWISE_DESC:
+    /* rank s keeps its own block as inoutvec and folds in the block received
+     * from rank s-1, s-2, ... */
+    for (int k = 1; k < P; k++) {
+      pairs[2 * np] = start; pairs[2 * np + 1] = (start - k + P) % P; np++;
+    }
+    *result = start;
+    return np;
+  case ALO_ORDER_RING: {
+    /* the partial travels: rank s+k receives it (invec) and folds it into
+     * its own contribution (inoutvec) */
+    int cur = start;
+    for (int k = 1; k < P; k++) {
+      int nxt = (start + k) % P;
+      pairs[2 * np] = nxt; pairs[2 * np + 1] = cur; np++;
+      cur = nxt;
+    }
+    *result = cur;
+    return np;
+  }
+  case ALO_ORDER_TREE_BINOMIAL:
+    /* binomial reduce to rank 0: at distance d every rank that is a multiple
+     * of 2d folds in the partial of rank+d, if that rank exists */
+    for (int d = 1; d < P; d *= 2)
+      for (int i = 0; i + d < P; i += 2 * d) {
+        pairs[2 * np] = i; pairs[2 * np + 1] = i + d; np++;
+      }
+    *result = 0;
+    return np;
+  case ALO_ORDER_TREE_DBL:
+  case ALO_ORDER_TREE_HALV: {
+    /* Non-power-of-two P: the first 2*rem ranks fold pairwise (even rank
+     * sends to the odd rank above it, which keeps the result), leaving a
+     * power-of-two set of survivors. */
+    int pof2 = floor_pow2(P), rem = P - pof2;
+    int *L = (int *)malloc(sizeof(int) * (size_t)pof2);
+    if (!L) return -1;
+    for (int j = 0; j < rem; j++) {
+      pairs[2 * np] = 2 * j + 1; pairs[2 * np + 1] = 2 * j; np++;
+      L[j] = 2 * j + 1;
+    }
+    for (int j = rem; j < pof2; j++) L[j] = j + rem;
+    if (order == ALO_ORDER_TREE_DBL) {
+      for (int d = 1; d < pof2; d *= 2)
+        for (int i = 0; i + d < pof2; i += 2 * d) {
+          pairs[2 * np] = L[i]; pairs[2 * np + 1] = L[i + d]; np++;
+        }
+    } else {
+      for (int d = pof2 / 2; d >= 1; d /= 2)
+        for (int i = 0; i < d; i++) {
+          pairs[2 * np] = L[i]; pairs[2 * np + 1] = L[i + d]; np++;
+        }
+    }
+    *result = L[0];
+    free(L);
+    return np;
+  }
+  default:
+    return -1;
+  }
+}
+
+/* Run a schedule over P tiles held in `slots` (each `len` elements). */
+static void run_schedule(char **slots, const int *pairs, int np, size_t len,
+                         int dtype, int op) {
+  for (int k = 0; k < np; k++)
+    step_serial(slots[pairs[2 * k]], slots[pairs[2 * k + 1]], len, dtype, op);
+}
+
+static int combine_impl(void *out, const void *const *in, int P, size_t n,
+                        int dtype, int op, int order, int start, int generated,
+                        int dist, uint64_t seed_base, uint64_t idx0) {
+  const size_t es = alo_dtype_size(dtype);
+  int rc = alo_check_op(dtype, op);
+  if (rc) return rc;
+  int *pairs = (int *)malloc(sizeof(int) * 2 * (size_t)(P > 1 ? P : 1));
+  int result = 0;
+  if (!pairs) return 3;
+  int np = alo_schedule(P, order, start, pairs, &result);
+  if (np < 0) { free(pairs); return 4; }
+  const size_t ntiles = (n + ALO_TILE - 1) / ALO_TILE;
+  int fail = 0;
+#pragma omp parallel
+  {
+    char *tiles = (char *)malloc((size_t)P * ALO_TILE * es);
+    char **slots = (char **)malloc(sizeof(char *) * (size_t)P);
+    if (!tiles || !slots) {
+#pragma omp atomic write
+      fail = 1;
+    } else {
+      for (int r = 0; r < P; r++) slots[r] = tiles + (size_t)r * ALO_TILE * es;
+#pragma omp for schedule(static)
+      for (size_t t = 0; t < ntiles; t++) {
+        size_t lo = t * ALO_TILE, len = n - lo < ALO_TILE ? n - lo : ALO_TILE;
+        for (int r = 0; r < P; r++) {
+          if (generated)
+            fill_range(slots[r], len, dtype, dist, seed_base + (uint64_t)r, idx0 + lo);
+          else
+            memcpy(slots[r], (const char *)in[r] + lo * es, len * es);
+        }
+        run_schedule(slots, pairs, np, len, dtype, op);
+        memcpy((char *)out + lo * es, slots[result], len * es);
+      }
+    }
+    free(tiles);
+    free(slots);
+  }
+  free(pairs);
+  return fail ? 3 : 0;
+}
+
+int alo_combine(void *out, const void *const *in, int P, size_t n, int dtype,
+                int op, int order, int start) {
+  return combine_impl(out, in, P, n, dtype, op, order, start, 0, 0, 0, 0);
+}
+
+int alo_combine_generated(void *out, int P, size_t n, int dtype, int op,
+                          int order, int start, int dist, uint64_t seed_base,
+                          uint64_t idx0) {
+  return combine_impl(out, NULL, P, n, dtype, op, order, start, 1, dist,
+                      seed_base, idx0);
+}
+
+int alo_reduce_scatter(void *const *recv, const void *const *send, int P,
+                       size_t count, int dtype, int op, int order) {
+  const size_t es = alo_dtype_size(dtype);
+  int rc = alo_check_op(dtype, op);
+  if (rc) return rc;
+  const void **blk = (const void **)malloc(sizeof(void *) * (size_t)P);
+  if (!blk) return 3;
+  for (int b = 0; b < P && rc == 0; b++) {
+    for (int r = 0; r < P; r++) blk[r] = (const char *)send[r] + (size_t)b * count * es;
+    rc = alo_combine(recv[b], blk, P, count, dtype, op, order, b);
+  }
+  free(blk);
+  return rc;
+}
+
+int alo_allgather(void *const *recv, const void *const *send, int P,
+                  size_t count, int dtype) {
+  const size_t es = alo_dtype_size(dtype);
+  if (es == 0) return 2;
+  for (int r = 0; r < P; r++)
+    for (int q = 0; q < P; q++) {
+      char *dst = (char *)recv[r] + (size_t)q * count * es;
+      if (dst != (const char *)send[q]) memmove(dst, send[q], count * es);
+    }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Ring reduce-scatter + allgather, moved literally chunk by chunk           */
+/* ------------------------------------------------------------------------ */
+
+void alo_ring_segment(size_t n, int P, int s, size_t *offset, size_t *len) {
+  size_t base = n / (size_t)P, rem = n % (size_t)P;
+  *offset = (size_t)s * base + ((size_t)s < rem ? (size_t)s : rem);
+  *len = base + ((size_t)s < rem ? 1 : 0);
+}
+
+int alo_ring_reduce_scatter(void *const *bufs, int P, size_t n, int dtype,
+                            int op, size_t chunk_elems) {
+  const size_t es = alo_dtype_size(dtype);
+  int rc = alo_check_op(dtype, op);
+  if (rc) return rc;
+  if (P < 1 || chunk_elems == 0) return 4;
+  char *wire = (char *)malloc(chunk_elems * es);
+  if (!wire) return 3;
+  for (int t = 0; t < P - 1; t++)
+    for (int r = 0; r < P; r++) {
+      int seg = ((r - t - 1) % P + P) % P, from = (r - 1 + P) % P;
+      size_t off, len;
+      alo_ring_segment(n, P, seg, &off, &len);
+      for (size_t c = 0; c < len; c += chunk_elems) {
+        size_t m = len - c < chunk_elems ? len - c : chunk_elems;
+        memcpy(wire, (const char *)bufs[from] + (off + c) * es, m * es); /* the message */
+        alo_step((char *)bufs[r] + (off + c) * es, wire, m, dtype, op);
+      }
+    }
+  free(wire);
+  return 0;
+}
+
+int alo_ring_allgather(void *const *bufs, int P, size_t n, int dtype,
+                       size_t chunk_elems) {
+  const size_t es = alo_dtype_size(dtype);
+  if (es == 0) return 2;
+  if (P < 1 || chunk_elems == 0) return 4;
+  /* after the reduce-scatter rank r owns segment (r+1) mod P; at step t it
+   * receives segment (r-t) mod P from rank r-1 */
+  for (int t = 0; t < P - 1; t++)
+    for (int r = 0; r < P; r++) {
+      int seg = ((r - t) % P + P) % P, from = (r - 1 + P) % P;
+      size_t off, len;
+      alo_ring_segment(n, P, seg, &off, &len);
+      for (size_t c = 0; c < len; c += chunk_elems) {
+        size_t m = len - c < chunk_elems ? len - c : chunk_elems;
+        memcpy((char *)bufs[r] + (off + c) * es,
+               (const char *)bufs[from] + (off + c) * es, m * es);
+      }
+    }
+  return 0;
+}
+
+int alo_ring_allreduce(void *const *bufs, int P, size_t n, int dtype, int op,
+                       size_t chunk_elems) {
+  int rc = alo_ring_reduce_scatter(bufs, P, n, dtype, op, chunk_elems);
+  if (rc) return rc;
+  return alo_ring_allgather(bufs, P, n, dtype, chunk_elems);
+}
+
+/* ------------------------------------------------------------------------ */
+/* Halo faces                                                               */
+/* ------------------------------------------------------------------------ */
+
+/* Box of a face in allocation coordinates: lo[d] .. lo[d]+ext[d]. */
+static int halo_box(size_t nx, size_t ny, size_t nz, size_t h, int face,
+                    int ghost, size_t lo[3], size_t ext[3]) {
+  size_t n[3] = {nx, ny, nz};
+  if (face < 0 || face > 5) return 1;
+  int axis = face / 2, plus = face % 2;
+  for (int d = 0; d < 3; d++) { lo[d] = h; ext[d] = n[d]; }
+  ext[axis] = h;
+  if (ghost) lo[axis] = plus ? h + n[axis] : 0;
+  else lo[axis] = plus ? n[axis] : h;
+  return 0;
+}
+
+size_t alo_halo_face_elems(size_t nx, size_t ny, size_t nz, size_t h, int face) {
+  size_t lo[3], ext[3];
+  if (halo_box(nx, ny, nz, h, face, 0, lo, ext)) return 0;
+  return ext[0] * ext[1] * ext[2];
+}
+
+static int halo_copy(void *grid, void *buf, size_t nx, size_t ny, size_t nz,
+                     size_t h, int face, size_t es, int unpack) {
+  size_t lo[3], ext[3];
+  if (halo_box(nx, ny, nz, h, face, unpack, lo, ext)) return 1;
+  if (h > nx || h > ny || h > nz) return 1;
+  const size_t sx = nx + 2 * h, sy = ny + 2 * h;
+  size_t k = 0;
+  for (size_t z = 0; z < ext[2]; z++)
+    for (size_t y = 0; y < ext[1]; y++)
+      for (size_t x = 0; x < ext[0]; x++, k++) {
+        size_t g = ((lo[2] + z) * sy + (lo[1] + y)) * sx + (lo[0] + x);
+        if (unpack) memcpy((char *)grid + g * es, (char *)buf + k * es, es);
+        else memcpy((char *)buf + k * es, (char *)grid + g * es, es);
+      }
+  return 0;
+}
+
+int alo_halo_pack(void *buf, const void *grid, size_t nx, size_t ny, size_t nz,
+                  size_t h, int face, size_t elem_size) {
+  return halo_copy((void *)grid, buf, nx, ny, nz, h, face, elem_size, 0);
+}
+
+int alo_halo_unpack(void *grid, const void *buf, size_t nx, size_t ny,
+                    size_t nz, size_t h, int face, size_t elem_size) {
+  return halo_copy(grid, (void *)buf, nx, ny, nz, h, face, elem_size, 1);
+}
+
+/* ------------------------------------------------------------------------ */
+
+uint64_t alo_checksum(const void *buf, size_t nbytes) {
+  const unsigned char *p = (const unsigned char *)buf;
+  uint64_t h = 0xcbf29ce484222325ull;
+  size_t i = 0;
+  for (; i + 8 <= nbytes; i += 8) {
+    uint64_t w;
+    memcpy(&w, p + i, 8);
+    h = fin64(h ^ w) + ALO_GAMMA;
+  }
+  for (; i < nbytes; i++) h = (h ^ p[i]) * 0x100000001b3ull;
+  return h;
+}

@@ -1,0 +1,212 @@
+/*
+ * Golden-vector generator for the host combine that the reference performs.
+ *
+ * The reference's MPI backend forwards Al::Allreduce / Al::Reduce_scatter
+ * straight to the MPI library (include/aluminum/mpi/allreduce.hpp:38-44,
+ * include/aluminum/mpi/reduce_scatter.hpp:40-46), so the values it produces
+ * are those of MPI_Allreduce / MPI_Reduce_scatter_block in the MPI it was
+ * built with.  This program makes exactly those calls against the image's
+ * MPICH and prints one JSON document (inputs and outputs as hex strings) that
+ * is committed next to it as a fixture.  It runs nothing from the reference.
+ *
+ * Build and run: see make_mpich_golden.sh.
+ */
+#include <mpi.h>
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../../oracle/oracle.h"
+
+static int rank_, P_;
+
+static const char *dt_name[] = {"i8", "u8", "i16", "u16", "i32", "u32", "i64",
+                                "u64", "f16", "bf16", "f32", "f64"};
+static const char *op_name[] = {"sum", "prod", "min", "max", "lor", "land",
+                                "lxor", "bor", "band", "bxor"};
+
+static MPI_Datatype mpi_type(int dt) {
+  switch (dt) {
+  case ALO_I8: return MPI_SIGNED_CHAR;
+  case ALO_U8: return MPI_UNSIGNED_CHAR;
+  case ALO_I16: return MPI_SHORT;
+  case ALO_U16: return MPI_UNSIGNED_SHORT;
+  case ALO_I32: return MPI_INT;
+  case ALO_U32: return MPI_UNSIGNED;
+  case ALO_I64: return MPI_LONG;
+  case ALO_U64: return MPI_UNSIGNED_LONG;
+  case ALO_F32: return MPI_FLOAT;
+  case ALO_F64: return MPI_DOUBLE;
+  default: return MPI_DATATYPE_NULL;
+  }
+}
+
+static MPI_Op mpi_op(int op) {
+  static MPI_Op t[10];
+  t[0] = MPI_SUM; t[1] = MPI_PROD; t[2] = MPI_MIN; t[3] = MPI_MAX; t[4] = MPI_LOR;
+  t[5] = MPI_LAND; t[6] = MPI_LXOR; t[7] = MPI_BOR; t[8] = MPI_BAND; t[9] = MPI_BXOR;
+  return t[op];
+}
+
+static void print_hex(const unsigned char *p, size_t nbytes) {
+  putchar('"');
+  for (size_t i = 0; i < nbytes; i++) printf("%02x", p[i]);
+  putchar('"');
+}
+
+static int first_case = 1;
+
+/* Gather `nbytes` from every rank to rank 0 and print as a JSON list. */
+static void emit_list(const char *key, const void *mine, size_t nbytes) {
+  unsigned char *all = NULL;
+  if (rank_ == 0) all = (unsigned char *)malloc(nbytes * (size_t)P_);
+  MPI_Gather(mine, (int)nbytes, MPI_BYTE, all, (int)nbytes, MPI_BYTE, 0, MPI_COMM_WORLD);
+  if (rank_ == 0) {
+    printf(", \"%s\": [", key);
+    for (int r = 0; r < P_; r++) {
+      if (r) printf(", ");
+      print_hex(all + (size_t)r * nbytes, nbytes);
+    }
+    printf("]");
+    free(all);
+  }
+}
+
+static void emit_sums(const char *key, const void *mine, size_t nbytes) {
+  unsigned long long cs = alo_checksum(mine, nbytes), *all = NULL;
+  if (rank_ == 0) all = (unsigned long long *)malloc(sizeof(*all) * (size_t)P_);
+  MPI_Gather(&cs, 1, MPI_UNSIGNED_LONG_LONG, all, 1, MPI_UNSIGNED_LONG_LONG, 0, MPI_COMM_WORLD);
+  if (rank_ == 0) {
+    printf(", \"%s\": [", key);
+    for (int r = 0; r < P_; r++) printf("%s\"%016llx\"", r ? ", " : "", all[r]);
+    printf("]");
+    free(all);
+  }
+}
+
+static void head(const char *coll, int dt, int op, size_t n, int dist,
+                 unsigned long long seed, const char *note) {
+  if (rank_ != 0) return;
+  printf("%s\n  {\"coll\": \"%s\", \"P\": %d, \"dtype\": \"%s\", \"op\": \"%s\", "
+         "\"n\": %zu, \"dist\": %d, \"seed_base\": %llu, \"note\": \"%s\"",
+         first_case ? "" : ",", coll, P_, dt_name[dt], op_name[op], n, dist, seed, note);
+}
+
+static void tail(void) {
+  if (rank_ == 0) { printf("}"); fflush(stdout); }
+  first_case = 0;
+}
+
+/* Special values planted over the start of a float buffer (P = 2 only):
+ * element i of rank 0 meets element i of rank 1.  NaN against numbers on
+ * either side, signed-zero ties both ways, infinities, denormals. */
+static void plant_specials(void *buf, size_t n, int dt) {
+  static const unsigned r0[] = {0x7fc00000u, 0xbf800000u, 0x7fc00000u, 0x00000000u, 0x80000000u,
+                                0x7f800000u, 0xff800000u, 0x00000001u, 0x80000001u, 0x3f800000u,
+                                0x7f7fffffu, 0x00800000u, 0x00000000u, 0x80000000u, 0x7f800000u,
+                                0x00400000u};
+  static const unsigned r1[] = {0x7f800000u, 0x7fc00000u, 0x7fc00000u, 0x80000000u, 0x00000000u,
+                                0xff800000u, 0x7f800000u, 0x80000001u, 0x00000001u, 0x3f800000u,
+                                0x7f7fffffu, 0x00800001u, 0x00000000u, 0x80000000u, 0x7f800000u,
+                                0x00400000u};
+  const size_t cnt = sizeof(r0) / sizeof(r0[0]);
+  for (size_t i = 0; i < n && i < cnt; i++) {
+    unsigned u = rank_ == 0 ? r0[i] : r1[i];
+    float f;
+    memcpy(&f, &u, 4);
+    if (dt == ALO_F32) ((float *)buf)[i] = f;
+    else ((double *)buf)[i] = (double)f; /* exact widening keeps the class */
+  }
+}
+
+static void case_allreduce(int dt, int op, size_t n, int dist, int specials,
+                           const char *note) {
+  const unsigned long long seed = 1000;
+  size_t es = alo_dtype_size(dt);
+  void *in = malloc(n * es), *out = malloc(n * es);
+  alo_fill(in, n, dt, dist, seed + (unsigned long long)rank_, 0);
+  if (specials) plant_specials(in, n, dt);
+  MPI_Allreduce(in, out, (int)n, mpi_type(dt), mpi_op(op), MPI_COMM_WORLD);
+  head("allreduce", dt, op, n, dist, seed, note);
+  emit_list("in", in, n * es);
+  emit_list("out", out, n * es);
+  tail();
+  free(in); free(out);
+}
+
+/* count = elements per rank; send buffer holds P*count. */
+static void case_reduce_scatter(int dt, int op, size_t count, int dist, int full,
+                                const char *note) {
+  const unsigned long long seed = 1000;
+  size_t es = alo_dtype_size(dt), n = count * (size_t)P_;
+  void *in = malloc(n * es), *out = malloc(count * es);
+  alo_fill(in, n, dt, dist, seed + (unsigned long long)rank_, 0);
+  MPI_Reduce_scatter_block(in, out, (int)count, mpi_type(dt), mpi_op(op), MPI_COMM_WORLD);
+  head("reduce_scatter", dt, op, count, dist, seed, note);
+  if (full) {
+    emit_list("in", in, n * es);
+    emit_list("out", out, count * es);
+  } else {
+    emit_sums("out_checksum", out, count * es);
+    emit_list("out_head", out, 8 * es);
+  }
+  tail();
+  free(in); free(out);
+}
+
+int main(int argc, char **argv) {
+  MPI_Init(&argc, &argv);
+  MPI_Comm_rank(MPI_COMM_WORLD, &rank_);
+  MPI_Comm_size(MPI_COMM_WORLD, &P_);
+  alo_set_num_threads(1);
+  int big = argc > 1 && !strcmp(argv[1], "big");
+
+  if (rank_ == 0) {
+    char ver[MPI_MAX_LIBRARY_VERSION_STRING];
+    int len;
+    MPI_Get_library_version(ver, &len);
+    for (char *c = ver; *c; c++) if (*c == '\n' || *c == '\t' || *c == '"') *c = ' ';
+    ver[60] = 0;
+    printf("{\"mpi\": \"%s\", \"P\": %d, \"cases\": [", ver, P_);
+  }
+
+  /* fp sum / prod: 16 elements (<= 2048 bytes) and just over 2048 bytes. */
+  const int fdt[2] = {ALO_F32, ALO_F64};
+  for (int d = 0; d < 2; d++) {
+    const size_t nlong = 2048 / alo_dtype_size(fdt[d]) + 8;
+    case_allreduce(fdt[d], ALO_SUM, 16, ALO_DIST_UNIFORM_PM1, 0, "short message");
+    case_allreduce(fdt[d], ALO_SUM, nlong, ALO_DIST_UNIFORM_PM1, 0, "long message");
+    case_allreduce(fdt[d], ALO_PROD, 16, ALO_DIST_UNIFORM_09_11, 0, "short message");
+    case_allreduce(fdt[d], ALO_PROD, nlong, ALO_DIST_UNIFORM_09_11, 0, "long message");
+    case_allreduce(fdt[d], ALO_MIN, 48, ALO_DIST_UNIFORM_PM1, 0, "");
+    case_allreduce(fdt[d], ALO_MAX, 48, ALO_DIST_UNIFORM_PM1, 0, "");
+    if (P_ == 2) { /* the two-operand step, special values, seen from both ranks */
+      for (int op = ALO_SUM; op <= ALO_MAX; op++)
+        case_allreduce(fdt[d], op, 48, ALO_DIST_UNIFORM_PM1, 1, "specials");
+    }
+    case_reduce_scatter(fdt[d], ALO_SUM, 8, ALO_DIST_UNIFORM_PM1, 1, "short message");
+    if (big) /* >= 512 KiB in total selects the pairwise exchange */
+      case_reduce_scatter(fdt[d], ALO_SUM, (size_t)(1u << 20) / (size_t)P_ / alo_dtype_size(fdt[d]) + 64,
+                          ALO_DIST_UNIFORM_PM1, 0, "long message");
+  }
+
+  /* integer types: every op, full-range bits (logical ops see arbitrary
+   * nonzero values as true) and {0,1} inputs. */
+  if (P_ == 2 || P_ == 5) {
+    for (int dt = ALO_I8; dt <= ALO_U64; dt++)
+      for (int op = ALO_SUM; op <= ALO_BXOR; op++) {
+        case_allreduce(dt, op, 12, ALO_DIST_FULLRANGE, 0, "");
+        if (op >= ALO_LOR && op <= ALO_LXOR)
+          case_allreduce(dt, op, 12, ALO_DIST_BOOL01, 0, "");
+        if (op == ALO_SUM || op == ALO_PROD)
+          case_allreduce(dt, op, 12, ALO_DIST_SMALLINT, 0, "");
+      }
+    case_reduce_scatter(ALO_I32, ALO_SUM, 8, ALO_DIST_FULLRANGE, 1, "");
+    case_reduce_scatter(ALO_U64, ALO_BXOR, 8, ALO_DIST_FULLRANGE, 1, "");
+  }
+
+  if (rank_ == 0) printf("\n]}\n");
+  MPI_Finalize();
+  return 0;
+}

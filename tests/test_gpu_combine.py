@@ -1,0 +1,192 @@
+"""GPU parity of alamd_combine / reduce_scatter / allgather against the CPU
+oracle, through the C ABI.  Bit-exact for every type; two NaNs compare equal
+whatever their payload."""
+import numpy as np
+import pytest
+
+import oracle
+from util import (ALL_DTYPES, FLOAT_DTYPES, INT_DTYPES, ORDERS, assert_bits_equal, dev_empty,
+                  ops_of, to_dev, to_host)
+
+pytestmark = pytest.mark.gpu
+
+DIST_FOR = {"sum": "uniform_pm1", "prod": "uniform_09_11", "min": "uniform_pm1", "max": "uniform_pm1",
+            "lor": "bool01", "land": "bool01", "lxor": "bool01", "bor": "fullrange",
+            "band": "fullrange", "bxor": "fullrange"}
+
+
+def make_inputs(P, n, dtype, op, seed=1000):
+    dist = DIST_FOR[op]
+    if dtype in INT_DTYPES and op in ("sum", "prod", "min", "max"):
+        dist = "fullrange"
+    return [oracle.fill(n, dtype, dist, seed + r) for r in range(P)]
+
+
+def run_combine(al, ins, dtype, op, order, start=0, nout=1):
+    import torch
+    d_ins = [to_dev(a) for a in ins]
+    outs = [dev_empty(ins[0].size, ins[0].dtype) for _ in range(nout)]
+    al.combine(outs, d_ins, op, order=order, start=start, dtype=dtype, count=ins[0].size)
+    torch.cuda.synchronize()
+    return [to_host(o, ins[0].dtype) for o in outs]
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_combine_all_ops_orders(al, dtype):
+    for op in ops_of(dtype):
+        for P in (1, 2, 3, 5, 8):
+            orders = ORDERS if dtype in FLOAT_DTYPES else ("rank_asc", "tree_halv")
+            for order in orders:
+                for n in (1, 37, 4099):
+                    start = (P - 1) // 2 if order in ("pairwise_desc", "ring") else 0
+                    ins = make_inputs(P, n, dtype, op)
+                    want = oracle.combine(ins, dtype, op, order, start)
+                    got = run_combine(al, ins, dtype, op, order, start)[0]
+                    assert_bits_equal(got, want, dtype, "%s %s P=%d %s n=%d" % (dtype, op, P, order, n))
+
+
+@pytest.mark.parametrize("dtype", ("f32", "bf16", "i32"))
+@pytest.mark.parametrize("P", (4, 6, 7, 8, 13, 16, 31, 32))
+def test_combine_many_ranks(al, dtype, P):
+    n = 5000
+    for order in ORDERS:
+        ins = make_inputs(P, n, dtype, "sum")
+        start = P // 3 if order in ("pairwise_desc", "ring") else 0
+        want = oracle.combine(ins, dtype, "sum", order, start)
+        got = run_combine(al, ins, dtype, "sum", order, start)[0]
+        assert_bits_equal(got, want, dtype, "%s P=%d %s" % (dtype, P, order))
+
+
+def test_combine_64_ranks_fold(al):
+    ins = make_inputs(64, 3001, "f32", "sum")
+    for order, start in (("rank_asc", 0), ("ring", 17), ("pairwise_desc", 40)):
+        want = oracle.combine(ins, "f32", "sum", order, start)
+        got = run_combine(al, ins, "f32", "sum", order, start)[0]
+        assert_bits_equal(got, want, "f32", order)
+
+
+def test_combine_allreduce_outputs_and_inplace(al):
+    import torch
+    P, n = 8, 100003
+    ins = make_inputs(P, n, "f32", "sum")
+    want = oracle.combine(ins, "f32", "sum", "tree_dbl")
+    outs = run_combine(al, ins, "f32", "sum", "tree_dbl", nout=P)
+    for o in outs:
+        assert_bits_equal(o, want, "f32", "allreduce outputs")
+    # in place: every rank's buffer is both its contribution and its result
+    bufs = [to_dev(a) for a in ins]
+    al.combine(bufs, bufs, "sum", order="tree_dbl")
+    torch.cuda.synchronize()
+    for b in bufs:
+        assert_bits_equal(to_host(b, np.float32), want, "f32", "in-place allreduce")
+
+
+def test_combine_unaligned_pointers(al):
+    import torch
+    P, n = 4, 10007
+    ins = make_inputs(P, n, "f32", "sum")
+    want = oracle.combine(ins, "f32", "sum", "rank_asc")
+    base = [to_dev(np.concatenate([np.zeros(1, np.float32), a])) for a in ins]
+    views = [b[1:] for b in base]  # 4-byte aligned only
+    out = dev_empty(n + 1, np.float32)
+    al.combine([out[1:]], views, "sum", dtype="f32", count=n)
+    torch.cuda.synchronize()
+    assert_bits_equal(to_host(out, np.float32)[1:], want, "f32", "unaligned")
+
+
+@pytest.mark.parametrize("dtype", ("f32", "f64", "bf16", "f16"))
+def test_combine_special_values(al, dtype):
+    # NaN, infinities, signed zeros, denormals and ties on every side
+    f32 = np.array([np.nan, -1.0, np.nan, 0.0, -0.0, np.inf, -np.inf, 1e-45, -1e-45, 1.0,
+                    3.4028235e38, 1.1754944e-38, 0.0, -0.0, np.inf, 5.877472e-39, 65504.0, 1e-8],
+                   dtype=np.float32)
+    rng = np.random.default_rng(7)
+    P = 4
+    cols = [f32[rng.permutation(f32.size)] for _ in range(P)]
+    # every pair of specials meets somewhere
+    grid = [np.concatenate([np.repeat(f32, f32.size), c]) if r == 0 else
+            np.concatenate([np.tile(f32, f32.size), c]) if r == 1 else
+            np.concatenate([np.full(f32.size ** 2, f32[(3 * r) % f32.size], np.float32), c])
+            for r, c in enumerate(cols)]
+    if dtype == "f32":
+        ins = grid
+    elif dtype == "f64":
+        ins = [g.astype(np.float64) for g in grid]
+    elif dtype == "bf16":
+        ins = [oracle.f32_to_bf16(g) for g in grid]
+    else:
+        ins = [oracle.f32_to_f16(g) for g in grid]
+    for op in ("sum", "prod", "min", "max"):
+        for order, start in (("rank_asc", 0), ("tree_dbl", 0), ("tree_halv", 0), ("ring", 1),
+                             ("pairwise_desc", 2), ("tree_binomial", 0)):
+            want = oracle.combine(ins, dtype, op, order, start)
+            got = run_combine(al, ins, dtype, op, order, start)[0]
+            assert_bits_equal(got, want, dtype, "%s %s %s" % (dtype, op, order))
+
+
+@pytest.mark.parametrize("dtype", ("f32", "bf16", "u8", "i64"))
+@pytest.mark.parametrize("order", ("rank_asc", "tree_halv", "pairwise_desc", "ring"))
+def test_reduce_scatter(al, dtype, order):
+    import torch
+    for P in (1, 2, 5, 8):
+        for count in (1, 24, 1000, 4096):
+            sends = make_inputs(P, P * count, dtype, "sum")
+            want = oracle.reduce_scatter(sends, dtype, "sum", order)
+            d_sends = [to_dev(a) for a in sends]
+            recvs = [dev_empty(count, sends[0].dtype) for _ in range(P)]
+            al.reduce_scatter(recvs, d_sends, "sum", order=order, dtype=dtype, count=count)
+            torch.cuda.synchronize()
+            for r in range(P):
+                assert_bits_equal(to_host(recvs[r], sends[0].dtype), want[r], dtype,
+                                  "reduce_scatter %s P=%d count=%d rank %d" % (order, P, count, r))
+            # in place: the result replaces the start of each send buffer
+            al.reduce_scatter(d_sends, d_sends, "sum", order=order, dtype=dtype, count=count)
+            torch.cuda.synchronize()
+            for r in range(P):
+                assert_bits_equal(to_host(d_sends[r], sends[0].dtype)[:count], want[r], dtype,
+                                  "in-place reduce_scatter %s P=%d count=%d rank %d" % (order, P, count, r))
+
+
+@pytest.mark.parametrize("dtype", ("u8", "bf16", "f32", "f64"))
+def test_allgather(al, dtype):
+    import torch
+    for P in (1, 3, 8):
+        for count in (1, 5, 1024, 4099):
+            sends = make_inputs(P, count, dtype, "bxor" if dtype == "u8" else "sum")
+            want = oracle.allgather(sends, dtype)
+            d_sends = [to_dev(a) for a in sends]
+            recvs = [dev_empty(count * P, sends[0].dtype) for _ in range(P)]
+            al.allgather(recvs, d_sends, dtype=dtype, count=count)
+            torch.cuda.synchronize()
+            for r in range(P):
+                assert_bits_equal(to_host(recvs[r], sends[0].dtype), want[r], dtype, "allgather")
+            # in place: each rank's slice already sits at its rank offset
+            bufs = [to_dev(np.zeros(count * P, sends[0].dtype)) for _ in range(P)]
+            for r in range(P):
+                bufs[r][r * count:(r + 1) * count].copy_(d_sends[r])
+            views = [bufs[r][r * count:(r + 1) * count] for r in range(P)]
+            al.allgather(bufs, views, dtype=dtype, count=count)
+            torch.cuda.synchronize()
+            for r in range(P):
+                assert_bits_equal(to_host(bufs[r], sends[0].dtype), want[r], dtype, "in-place allgather")
+
+
+def test_errors(al):
+    import torch
+    a = [to_dev(np.zeros(16, np.float32)) for _ in range(2)]
+    out = [dev_empty(16, np.float32)]
+    with pytest.raises(al.AlError, match="Reduction operator not supported"):
+        al.combine(out, a, "avg")
+    with pytest.raises(al.AlError, match="Reduction operator not supported"):
+        al.combine(out, a, "band")
+    with pytest.raises(al.AlError, match="Invalid algorithm"):
+        al.combine(out, a, "sum", order=17)
+    big = to_dev(np.zeros(40, np.float32))
+    with pytest.raises(al.AlError) as e:
+        al.combine([big[4:20]], [big[0:16], big[20:36]], "sum", dtype="f32", count=16)
+    assert e.value.code == 5
+    with pytest.raises(al.AlError):
+        al.combine(out, [a[0]] * 65, "sum")
+    # zero-length is a no-op
+    al.combine(out, a, "sum", count=0)
+    torch.cuda.synchronize()
