@@ -139,14 +139,13 @@ int make_plan(RingPlan &pl, void *const *bufs, int P, size_t count, int dtype, s
 int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, hipStream_t stream) {
   const dim3 grid(pl.gx, pl.rp.P, 1), block(kThreads, 1, 1);
   if (!reduce) {
-    // a copy is type-blind: move bytes as the widest unit the layout allows
+    // a copy only needs the element size
     void (*kern)(const RingParams) = nullptr;
-    if (pl.vector) kern = ring_step_kernel<uint32_t, -1, true>;
-    else switch (pl.es) {
-      case 1: kern = ring_step_kernel<uint8_t, -1, false>; break;
-      case 2: kern = ring_step_kernel<uint16_t, -1, false>; break;
-      case 4: kern = ring_step_kernel<uint32_t, -1, false>; break;
-      default: kern = ring_step_kernel<uint64_t, -1, false>; break;
+    switch (pl.es) {
+    case 1: kern = pl.vector ? ring_step_kernel<uint8_t, -1, true> : ring_step_kernel<uint8_t, -1, false>; break;
+    case 2: kern = pl.vector ? ring_step_kernel<uint16_t, -1, true> : ring_step_kernel<uint16_t, -1, false>; break;
+    case 4: kern = pl.vector ? ring_step_kernel<uint32_t, -1, true> : ring_step_kernel<uint32_t, -1, false>; break;
+    default: kern = pl.vector ? ring_step_kernel<uint64_t, -1, true> : ring_step_kernel<uint64_t, -1, false>; break;
     }
     hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
     ALAMD_HIP(hipGetLastError());

@@ -81,7 +81,8 @@ float alo_f16_to_f32(uint16_t h) {
   uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
   uint32_t exp = (h >> 10) & 0x1fu;
   uint32_t man = h & 0x3ffu;
-  if (exp == 0x1fu) return bits_f32(sign | 0x7f800000u | (man << 13));
+  if (exp == 0x1fu) /* inf, or NaN made quiet as a hardware conversion does */
+    return bits_f32(sign | 0x7f800000u | (man ? 0x00400000u : 0u) | (man << 13));
   if (exp == 0) {
     if (man == 0) return bits_f32(sign);
     int e = -1;
