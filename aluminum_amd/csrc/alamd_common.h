@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <type_traits>
 
 #include "aluminum_amd.h"
 
@@ -60,15 +61,17 @@ template <> __device__ __forceinline__ f16_t narrow<f16_t>(float f) {
   r.b = __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
   return r;
 }
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+// Two fp32 values to a packed pair of bf16 with the hardware conversion
+// (v_cvt_pk_bf16_f32: nearest-even, NaN stays NaN).
+__device__ __forceinline__ uint32_t narrow_bf16x2(float lo, float hi) {
+  const f32x2_t f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
 template <> __device__ __forceinline__ bf16_t narrow<bf16_t>(float f) {
-  uint32_t u = __float_as_uint(f);
   bf16_t r;
-  if ((u & 0x7fffffffu) > 0x7f800000u) {
-    r.b = static_cast<uint16_t>((u >> 16) | 0x0040u);
-  } else {
-    u += 0x7fffu + ((u >> 16) & 1u);
-    r.b = static_cast<uint16_t>(u >> 16);
-  }
+  r.b = static_cast<uint16_t>(narrow_bf16x2(f, 0.0f) & 0xffffu);
   return r;
 }
 
@@ -131,13 +134,26 @@ template <int OP> struct Step<bf16_t, OP> {
 // The step applied to every element of a 128-bit vector.
 template <typename T, int OP>
 __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
-  constexpr int N = 16 / sizeof(T);
-  union U { u32x4 v; T e[N]; __device__ U() {} } a, b;
-  a.v = in;
-  b.v = inout;
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    // two elements per dword: widen by shift / mask, one fp32 operation each,
+    // narrow the pair with one packed conversion
+    u32x4 r;
 #pragma unroll
-  for (int j = 0; j < N; ++j) b.e[j] = Step<T, OP>::apply(a.e[j], b.e[j]);
-  return b.v;
+    for (int j = 0; j < 4; ++j) {
+      const float a_lo = __uint_as_float(in[j] << 16), a_hi = __uint_as_float(in[j] & 0xffff0000u);
+      const float b_lo = __uint_as_float(inout[j] << 16), b_hi = __uint_as_float(inout[j] & 0xffff0000u);
+      r[j] = narrow_bf16x2(fp_step<float, OP>(a_lo, b_lo), fp_step<float, OP>(a_hi, b_hi));
+    }
+    return r;
+  } else {
+    constexpr int N = 16 / sizeof(T);
+    union U { u32x4 v; T e[N]; __device__ U() {} } a, b;
+    a.v = in;
+    b.v = inout;
+#pragma unroll
+    for (int j = 0; j < N; ++j) b.e[j] = Step<T, OP>::apply(a.e[j], b.e[j]);
+    return b.v;
+  }
 }
 
 // ---- streaming loads and stores ---------------------------------------------

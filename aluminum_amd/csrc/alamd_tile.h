@@ -1,0 +1,41 @@
+// Tile access through buffer instructions.
+//
+// A workgroup owns one tile of THREADS*U 128-bit vectors per stream; each wave
+// covers U KiB of it contiguously (lane l of wave w touches bytes
+// w*U*1024 + u*1024 + l*16, u = 0..U-1).  The buffer descriptor is rebuilt per
+// tile from a uniform base address, so the per-lane offset never changes and
+// the address arithmetic stays in scalar registers; the descriptor's record
+// count makes the hardware drop out-of-range lanes, which is the guard for a
+// partial last tile.  Loads carry the non-temporal hint (every byte is read
+// once), stores are written through (sc0 sc1) so that dirty lines do not
+// gather in L2 and drain in bursts between the reads.
+#pragma once
+
+#include "alamd_common.h"
+
+namespace alamd {
+
+constexpr int kAuxLoadStream = 2;    // nt
+constexpr int kAuxStoreStream = 17;  // sc0 | sc1
+constexpr unsigned kRsrcFlags = 0x00020000u;
+
+template <int U, int THREADS> struct Tile {
+  static constexpr size_t BYTES = (size_t)THREADS * U * 16;
+  unsigned vo;
+  __device__ __forceinline__ Tile() {
+    const unsigned lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    vo = wave * (U * 1024u) + lane * 16u;
+  }
+  // Descriptor over [base, base + nbytes); nbytes <= BYTES.
+  static __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc(const char *base, int nbytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base), 0, nbytes, kRsrcFlags);
+  }
+  __device__ __forceinline__ u32x4 load(__amdgpu_buffer_rsrc_t r, int u) const {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, vo + (unsigned)u * 1024u, 0, kAuxLoadStream);
+  }
+  __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, int u, u32x4 v) const {
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, vo + (unsigned)u * 1024u, 0, kAuxStoreStream);
+  }
+};
+
+}  // namespace alamd

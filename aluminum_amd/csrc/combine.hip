@@ -4,6 +4,7 @@
 #include <string>
 
 #include "alamd_dispatch.h"
+#include "alamd_tile.h"
 
 namespace alamd {
 
@@ -92,25 +93,26 @@ int launch_order(void *const *outs, const void *const *ins, int P, const Layout 
   return launch_fold(fp, lay.nseg, lay.max_len, dtype, op, order == ALAMD_ORDER_RING, vector, stream);
 }
 
-__global__ void __launch_bounds__(256) gather_kernel_vec(FoldParams p, size_t nvec, size_t tail_bytes) {
+constexpr int kGatherU = 8, kGatherThreads = 128;
+__global__ void __launch_bounds__(kGatherThreads) gather_kernel_vec(FoldParams p, size_t blk_bytes) {
   // blockIdx.y = source rank q; every destination gets a copy at block q
+  using TL = Tile<kGatherU, kGatherThreads>;
+  const TL tl;
   const int q = blockIdx.y;
   const char *src = p.in[q];
-  const size_t blk_bytes = nvec * 16 + tail_bytes;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (size_t)gridDim.x * 256) {
-    const u32x4 v = ld_stream(src + i * 16);
-    for (int r = 0; r < p.P; ++r) {
-      char *dst = p.out[r] + (size_t)q * blk_bytes;
-      if (dst != src) st_stream(dst + i * 16, v);
-    }
-  }
-  if (blockIdx.x == 0 && threadIdx.x < tail_bytes) {
-    const size_t i = nvec * 16 + threadIdx.x;
-    const char c = src[i];
-    for (int r = 0; r < p.P; ++r) {
-      char *dst = p.out[r] + (size_t)q * blk_bytes;
-      if (dst != src) dst[i] = c;
-    }
+  const size_t tb = (size_t)blockIdx.x * TL::BYTES;
+  if (tb >= blk_bytes) return;
+  const int nrec = blk_bytes - tb > TL::BYTES ? (int)TL::BYTES : (int)(blk_bytes - tb);
+  const auto rs = TL::rsrc(src + tb, nrec);
+  u32x4 v[kGatherU];
+#pragma unroll
+  for (int u = 0; u < kGatherU; ++u) v[u] = tl.load(rs, u);
+  for (int r = 0; r < p.P; ++r) {
+    char *dst = p.out[r] + (size_t)q * blk_bytes;
+    if (dst == src) continue;
+    const auto rd = TL::rsrc(dst + tb, nrec);
+#pragma unroll
+    for (int u = 0; u < kGatherU; ++u) tl.store(rd, u, v[u]);
   }
 }
 
@@ -272,11 +274,10 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
   fp.P = P;
   hipStream_t st = as_stream(stream);
   if (vector) {
-    const size_t nvec = blk / 16;
-    unsigned per = (stream_grid((size_t)-1 / 2, 1, 8) + P - 1) / P;
-    unsigned gx = stream_grid(nvec, 256, 8);
-    if (gx > per) gx = per < 1 ? 1 : per;
-    hipLaunchKernelGGL(gather_kernel_vec, dim3(gx, P, 1), dim3(256, 1, 1), 0, st, fp, nvec, (size_t)0);
+    const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
+    const size_t tiles = (blk + tile - 1) / tile;
+    if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
+    hipLaunchKernelGGL(gather_kernel_vec, dim3((unsigned)tiles, P, 1), dim3(kGatherThreads, 1, 1), 0, st, fp, blk);
   } else {
     unsigned per = (stream_grid((size_t)-1 / 2, 1, 8) + P - 1) / P;
     unsigned gx = stream_grid(blk, 256, 8);

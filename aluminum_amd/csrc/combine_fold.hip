@@ -1,14 +1,17 @@
 // The fold kernels: out[i] = (((x_s . x_s+-1) . x_s+-2) ...)[i] over P rank
 // contributions resident in HBM.  Bandwidth-bound: every input byte is read
-// once with 128-bit non-temporal loads, all P loads of a lane are issued
-// before the first use, and the result is written once per output.
+// once, every output byte written once.
+//
+// Vector path (all buffers 16-byte aligned): one workgroup per tile, all loads
+// of a lane issued before the first use, buffer instructions with per-tile
+// descriptors (see alamd_tile.h).  Element path (any alignment): one element
+// per access, grid-stride.
 #include "alamd_dispatch.h"
+#include "alamd_tile.h"
 
 namespace alamd {
 
 namespace {
-
-constexpr int kThreads = 256;
 
 __device__ __forceinline__ void seg_range(const SegParams &s, unsigned seg, size_t &off, size_t &len) {
   const unsigned long long sg = seg;
@@ -31,85 +34,38 @@ __device__ __forceinline__ int next_rank(int idx, int dir, int P) {
   return idx;
 }
 
-// One tile: U accesses per thread, spaced one workgroup apart so that every
-// wave-wide access is a run of contiguous 128-bit vectors.
-template <typename T, int OP, bool ACC_IS_IN, bool VECTOR, int PT, int U, bool GUARD>
-__device__ __forceinline__ void fold_tile(const FoldParams &p, int P, int s, size_t in_bytes,
-                                          int j0, int nj, size_t out_bytes, size_t i0, size_t n) {
-  using L = Lane<T, VECTOR>;
-  using V = typename L::V;
-  V acc[U];
-  bool act[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u) act[u] = !GUARD || (i0 + (size_t)u * kThreads < n);
-
-  if constexpr (PT > 0) {
-    V x[PT][U];
-    int idx = s;
-#pragma unroll
-    for (int k = 0; k < PT; ++k) {
-      const char *pk = p.in[idx] + in_bytes;
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (act[u]) x[k][u] = L::ld(pk, i0 + (size_t)u * kThreads);
-      idx = next_rank(idx, p.dir, PT);
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (!act[u]) continue;
-      acc[u] = x[0][u];
-#pragma unroll
-      for (int k = 1; k < PT; ++k)
-        acc[u] = ACC_IS_IN ? L::template step<OP>(acc[u], x[k][u]) : L::template step<OP>(x[k][u], acc[u]);
-    }
-  } else {
-    constexpr int B = 4;  // loads in flight per access between uses
-    int idx = s;
-    {
-      const char *p0 = p.in[idx] + in_bytes;
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (act[u]) acc[u] = L::ld(p0, i0 + (size_t)u * kThreads);
-    }
-    for (int k = 1; k < P; k += B) {
-      V x[B][U];
-      int id = idx;
-#pragma unroll
-      for (int b = 0; b < B; ++b) {
-        if (k + b < P) {
-          id = next_rank(id, p.dir, P);
-          const char *pk = p.in[id] + in_bytes;
-#pragma unroll
-          for (int u = 0; u < U; ++u)
-            if (act[u]) x[b][u] = L::ld(pk, i0 + (size_t)u * kThreads);
-        }
-      }
-#pragma unroll
-      for (int b = 0; b < B; ++b) {
-        if (k + b < P) {
-#pragma unroll
-          for (int u = 0; u < U; ++u)
-            if (act[u])
-              acc[u] = ACC_IS_IN ? L::template step<OP>(acc[u], x[b][u]) : L::template step<OP>(x[b][u], acc[u]);
-        }
-      }
-      idx = id;
-    }
+// The fold of one element position, one element per access.
+template <typename T, int OP, bool ACC_IS_IN>
+__device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, size_t in_bytes, int j0, int nj,
+                                          size_t out_bytes, size_t e) {
+  int idx = s;
+  T acc = ld_elem<T>(p.in[idx] + in_bytes + e * sizeof(T));
+  for (int k = 1; k < P; ++k) {
+    idx = next_rank(idx, p.dir, P);
+    const T x = ld_elem<T>(p.in[idx] + in_bytes + e * sizeof(T));
+    acc = ACC_IS_IN ? Step<T, OP>::apply(acc, x) : Step<T, OP>::apply(x, acc);
   }
-
-  for (int j = j0; j < j0 + nj; ++j) {
-    char *po = p.out[j] + out_bytes;
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      if (act[u]) L::st(po, i0 + (size_t)u * kThreads, acc[u]);
-  }
+  for (int j = j0; j < j0 + nj; ++j) st_elem<T>(p.out[j] + out_bytes + e * sizeof(T), acc);
 }
 
-template <typename T, int OP, bool ACC_IS_IN, bool VECTOR, int PT>
-__global__ void __launch_bounds__(kThreads) fold_kernel(const FoldParams p) {
-  using L = Lane<T, VECTOR>;
-  constexpr int U = VECTOR ? 2 : 4;
-  constexpr size_t TILE = (size_t)kThreads * U;
+// Tile shape per element type: narrow arithmetic types spend many more ALU
+// operations per byte, so they keep fewer loads in flight per lane and more
+// waves resident to overlap arithmetic with memory.
+template <typename T, int OP> struct Shape {
+  static constexpr bool heavy = sizeof(T) <= 2 && OP <= ALAMD_MAX;
+  static constexpr int U = heavy ? 4 : 8;
+  static constexpr int THREADS = heavy ? 256 : 128;
+};
+
+// amdgpu_waves_per_eu(1, 2): the loads in flight are the point of this kernel;
+// the register allocator must not trade them away for more resident waves.
+template <typename T, int OP, bool ACC_IS_IN, int PT>
+__global__ void __launch_bounds__((Shape<T, OP>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
+fold_vec_kernel(const FoldParams p) {
+  constexpr int U = Shape<T, OP>::U, THREADS = Shape<T, OP>::THREADS;
+  constexpr int N = 16 / sizeof(T);
+  using TL = Tile<U, THREADS>;
+  const TL tl;
   const int P = PT ? PT : p.P;
   const unsigned seg = blockIdx.y;
   size_t off, len;
@@ -121,22 +77,87 @@ __global__ void __launch_bounds__(kThreads) fold_kernel(const FoldParams p) {
   size_t out_bytes;
   out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
 
-  const size_t n = len / L::N;  // accesses in this segment
-  const size_t ntiles = (n + TILE - 1) / TILE;
-  for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    const size_t i0 = t * TILE + threadIdx.x;
-    if ((t + 1) * TILE <= n)
-      fold_tile<T, OP, ACC_IS_IN, VECTOR, PT, U, false>(p, P, s, in_bytes, j0, nj, out_bytes, i0, n);
-    else
-      fold_tile<T, OP, ACC_IS_IN, VECTOR, PT, U, true>(p, P, s, in_bytes, j0, nj, out_bytes, i0, n);
+  const size_t vec_bytes = (len / N) * 16;
+  const size_t tb = (size_t)blockIdx.x * TL::BYTES;
+  if (tb < vec_bytes) {
+    const size_t rem = vec_bytes - tb;
+    const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
+    u32x4 acc[U];
+    if constexpr (PT > 0) {
+      u32x4 x[PT][U];
+      int idx = s;
+#pragma unroll
+      for (int k = 0; k < PT; ++k) {
+        const auto r = TL::rsrc(p.in[idx] + in_bytes + tb, nrec);
+#pragma unroll
+        for (int u = 0; u < U; ++u) x[k][u] = tl.load(r, u);
+        idx = next_rank(idx, p.dir, PT);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        acc[u] = x[0][u];
+#pragma unroll
+        for (int k = 1; k < PT; ++k)
+          acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[k][u]) : step_vec<T, OP>(x[k][u], acc[u]);
+      }
+    } else {
+      constexpr int B = 4;  // streams in flight between uses
+      int idx = s;
+      {
+        const auto r = TL::rsrc(p.in[idx] + in_bytes + tb, nrec);
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc[u] = tl.load(r, u);
+      }
+      for (int k = 1; k < P; k += B) {
+        u32x4 x[B][U];
+        int id = idx;
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+          if (k + b < P) {
+            id = next_rank(id, p.dir, P);
+            const auto r = TL::rsrc(p.in[id] + in_bytes + tb, nrec);
+#pragma unroll
+            for (int u = 0; u < U; ++u) x[b][u] = tl.load(r, u);
+          }
+        }
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+          if (k + b < P) {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+              acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[b][u]) : step_vec<T, OP>(x[b][u], acc[u]);
+          }
+        }
+        idx = id;
+      }
+    }
+    for (int j = j0; j < j0 + nj; ++j) {
+      const auto r = TL::rsrc(p.out[j] + out_bytes + tb, nrec);
+#pragma unroll
+      for (int u = 0; u < U; ++u) tl.store(r, u, acc[u]);
+    }
   }
+  // the len % N trailing elements, one per thread of the first workgroup
+  const size_t e = (len / N) * N + threadIdx.x;
+  if (blockIdx.x == 0 && e < len) fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
+}
 
-  if constexpr (VECTOR) {
-    // the len % N trailing elements, one per thread of the first workgroup
-    const size_t e = n * L::N + threadIdx.x;
-    if (blockIdx.x == 0 && e < len)
-      fold_tile<T, OP, ACC_IS_IN, false, 0, 1, false>(p, P, s, in_bytes, j0, nj, out_bytes, e, len);
-  }
+constexpr int kElemThreads = 256;
+
+template <typename T, int OP, bool ACC_IS_IN>
+__global__ void __launch_bounds__(kElemThreads) fold_elem_kernel(const FoldParams p) {
+  const int P = p.P;
+  const unsigned seg = blockIdx.y;
+  size_t off, len;
+  seg_range(p.seg, seg, off, len);
+  const size_t off_bytes = off * sizeof(T);
+  const size_t in_bytes = p.seg.in_blocked ? off_bytes : 0;
+  const int s = (p.start0 + (int)seg * p.start_stride) % P;
+  int j0, nj;
+  size_t out_bytes;
+  out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
+  for (size_t e = (size_t)blockIdx.x * kElemThreads + threadIdx.x; e < len; e += (size_t)gridDim.x * kElemThreads)
+    fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
 }
 
 }  // namespace
@@ -159,27 +180,32 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
     constexpr bool FP_MINMAX = (std::is_same<T, float>::value || std::is_same<T, double>::value ||
                                 std::is_same<T, f16_t>::value || std::is_same<T, bf16_t>::value) &&
                                (OP == ALAMD_MIN || OP == ALAMD_MAX);
-    const size_t per_access = vector ? 16 / sizeof(T) : 1;
-    const size_t tile = (size_t)kThreads * (vector ? 2 : 4) * per_access;
-    unsigned gx = stream_grid(max_len, tile, 8);
-    if (nseg > 1) {
-      unsigned per_seg = (stream_grid((size_t)-1 / 2, 1, 8) + nseg - 1) / nseg;
-      if (per_seg < 1) per_seg = 1;
-      if (gx > per_seg) gx = per_seg;
-    }
-    dim3 grid(gx, nseg, 1), block(kThreads, 1, 1);
     void (*kern)(const FoldParams) = nullptr;
+    dim3 grid, block;
     if (vector) {
+      const size_t tile_elems = Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES / sizeof(T);
+      const size_t tiles = (max_len + tile_elems - 1) / tile_elems;
+      if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
+      grid = dim3((unsigned)(tiles ? tiles : 1), nseg, 1);
+      block = dim3(Shape<T, OP>::THREADS, 1, 1);
       if (p.P == 8) {
-        if constexpr (FP_MINMAX) kern = roles ? fold_kernel<T, OP, true, true, 8> : fold_kernel<T, OP, false, true, 8>;
-        else kern = fold_kernel<T, OP, false, true, 8>;
+        if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 8> : fold_vec_kernel<T, OP, false, 8>;
+        else kern = fold_vec_kernel<T, OP, false, 8>;
       } else {
-        if constexpr (FP_MINMAX) kern = roles ? fold_kernel<T, OP, true, true, 0> : fold_kernel<T, OP, false, true, 0>;
-        else kern = fold_kernel<T, OP, false, true, 0>;
+        if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 0> : fold_vec_kernel<T, OP, false, 0>;
+        else kern = fold_vec_kernel<T, OP, false, 0>;
       }
     } else {
-      if constexpr (FP_MINMAX) kern = roles ? fold_kernel<T, OP, true, false, 0> : fold_kernel<T, OP, false, false, 0>;
-      else kern = fold_kernel<T, OP, false, false, 0>;
+      unsigned gx = stream_grid(max_len, (size_t)kElemThreads * 4, 8);
+      if (nseg > 1) {
+        unsigned per_seg = (stream_grid((size_t)-1 / 2, 1, 8) + nseg - 1) / nseg;
+        if (per_seg < 1) per_seg = 1;
+        if (gx > per_seg) gx = per_seg;
+      }
+      grid = dim3(gx, nseg, 1);
+      block = dim3(kElemThreads, 1, 1);
+      if constexpr (FP_MINMAX) kern = roles ? fold_elem_kernel<T, OP, true> : fold_elem_kernel<T, OP, false>;
+      else kern = fold_elem_kernel<T, OP, false>;
     }
     hipLaunchKernelGGL(kern, grid, block, 0, stream, p);
     ALAMD_HIP(hipGetLastError());

@@ -2,6 +2,7 @@
 // registers.  Used for floating-point types under the TREE_* orders, where
 // the pairing decides the rounding; integer types never need it.
 #include "alamd_dispatch.h"
+#include "alamd_tile.h"
 
 namespace alamd {
 
@@ -15,60 +16,49 @@ __device__ __forceinline__ void seg_range(const SegParams &s, unsigned seg, size
   len = s.seg_base + (sg < s.seg_rem ? 1u : 0u);
 }
 
-template <typename T, int OP, int SLOTS, bool VECTOR, int U, bool GUARD>
-__device__ __forceinline__ void tree_tile(const TreeParams &p, size_t in_bytes, int j0, int nj,
-                                          size_t out_bytes, size_t i0, size_t n) {
-  using L = Lane<T, VECTOR>;
-  using V = typename L::V;
+// The tree over one element position, one element per access.
+template <typename T, int OP, int SLOTS>
+__device__ __forceinline__ void tree_elem(const TreeParams &p, size_t in_bytes, int j0, int nj,
+                                          size_t out_bytes, size_t e) {
   const int nvalid = p.nvalid;
-  bool act[U];
+  T v[SLOTS];
 #pragma unroll
-  for (int u = 0; u < U; ++u) act[u] = !GUARD || (i0 + (size_t)u * kThreads < n);
-
-  V v[SLOTS][U];
+  for (int j = 0; j < SLOTS; ++j)
+    if (j < nvalid) v[j] = ld_elem<T>(p.a[j] + in_bytes + e * sizeof(T));
 #pragma unroll
-  for (int j = 0; j < SLOTS; ++j) {
-    if (j < nvalid) {
-      const char *pa = p.a[j] + in_bytes;
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (act[u]) v[j][u] = L::ld(pa, i0 + (size_t)u * kThreads);
-    }
-  }
-  // pre-folded slots: the odd rank keeps step(in = even rank, inout = odd rank)
-#pragma unroll
-  for (int j = 0; j < SLOTS; ++j) {
-    if (j < nvalid && p.b[j] != nullptr) {
-      const char *pb = p.b[j] + in_bytes;
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        if (act[u]) v[j][u] = L::template step<OP>(v[j][u], L::ld(pb, i0 + (size_t)u * kThreads));
-    }
-  }
+  for (int j = 0; j < SLOTS; ++j)
+    if (j < nvalid && p.b[j] != nullptr)
+      v[j] = Step<T, OP>::apply(v[j], ld_elem<T>(p.b[j] + in_bytes + e * sizeof(T)));
 #pragma unroll
   for (int d = 1; d < SLOTS; d *= 2) {
 #pragma unroll
-    for (int i = 0; i + d < SLOTS; i += 2 * d) {
-      if (i + d < nvalid) {
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-          if (act[u]) v[i][u] = L::template step<OP>(v[i + d][u], v[i][u]);
-      }
-    }
+    for (int i = 0; i + d < SLOTS; i += 2 * d)
+      if (i + d < nvalid) v[i] = Step<T, OP>::apply(v[i + d], v[i]);
   }
-  for (int j = j0; j < j0 + nj; ++j) {
-    char *po = p.out[j] + out_bytes;
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-      if (act[u]) L::st(po, i0 + (size_t)u * kThreads, v[0][u]);
-  }
+  for (int j = j0; j < j0 + nj; ++j) st_elem<T>(p.out[j] + out_bytes + e * sizeof(T), v[0]);
 }
 
-template <typename T, int OP, int SLOTS, bool VECTOR>
-__global__ void __launch_bounds__(kThreads) tree_kernel(const TreeParams p) {
-  using L = Lane<T, VECTOR>;
-  constexpr int U = VECTOR ? (SLOTS <= 8 ? 2 : 1) : (SLOTS <= 8 ? 4 : 2);
-  constexpr size_t TILE = (size_t)kThreads * U;
+template <typename T, int OP, int SLOTS> struct TreeShape {
+  static constexpr bool heavy = sizeof(T) <= 2;
+  static constexpr int budget = heavy ? 32 : 64;  // 128-bit loads in flight per lane
+  static constexpr int U = budget / SLOTS >= 8 ? (heavy ? 4 : 8) : (budget / SLOTS >= 1 ? budget / SLOTS : 1);
+  static constexpr int THREADS = U == 8 ? 128 : 256;
+};
+
+__device__ __forceinline__ void tree_out_select(const TreeParams &p, unsigned seg, size_t off_bytes,
+                                                size_t in_bytes, int &j0, int &nj, size_t &out_bytes) {
+  if (p.seg.out_mode == OUT_ALL) { j0 = 0; nj = p.seg.nout; out_bytes = in_bytes; }
+  else if (p.seg.out_mode == OUT_SEG) { j0 = (int)seg; nj = 1; out_bytes = 0; }
+  else { j0 = ((int)seg + p.seg.owner_shift) % p.P; nj = 1; out_bytes = off_bytes; }
+}
+
+template <typename T, int OP, int SLOTS>
+__global__ void __launch_bounds__((TreeShape<T, OP, SLOTS>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
+tree_vec_kernel(const TreeParams p) {
+  constexpr int U = TreeShape<T, OP, SLOTS>::U, THREADS = TreeShape<T, OP, SLOTS>::THREADS;
+  constexpr int N = 16 / sizeof(T);
+  using TL = Tile<U, THREADS>;
+  const TL tl;
   const unsigned seg = blockIdx.y;
   size_t off, len;
   seg_range(p.seg, seg, off, len);
@@ -76,27 +66,86 @@ __global__ void __launch_bounds__(kThreads) tree_kernel(const TreeParams p) {
   const size_t in_bytes = p.seg.in_blocked ? off_bytes : 0;
   int j0, nj;
   size_t out_bytes;
-  if (p.seg.out_mode == OUT_ALL) { j0 = 0; nj = p.seg.nout; out_bytes = in_bytes; }
-  else if (p.seg.out_mode == OUT_SEG) { j0 = (int)seg; nj = 1; out_bytes = 0; }
-  else { j0 = ((int)seg + p.seg.owner_shift) % p.P; nj = 1; out_bytes = off_bytes; }
+  tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
+  const int nvalid = p.nvalid;
 
-  const size_t n = len / L::N;
-  const size_t ntiles = (n + TILE - 1) / TILE;
-  for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    const size_t i0 = t * TILE + threadIdx.x;
-    if ((t + 1) * TILE <= n) tree_tile<T, OP, SLOTS, VECTOR, U, false>(p, in_bytes, j0, nj, out_bytes, i0, n);
-    else tree_tile<T, OP, SLOTS, VECTOR, U, true>(p, in_bytes, j0, nj, out_bytes, i0, n);
+  const size_t vec_bytes = (len / N) * 16;
+  const size_t tb = (size_t)blockIdx.x * TL::BYTES;
+  if (tb < vec_bytes) {
+    const size_t rem = vec_bytes - tb;
+    const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
+    u32x4 v[SLOTS][U];
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j) {
+      if (j < nvalid) {
+        const auto r = TL::rsrc(p.a[j] + in_bytes + tb, nrec);
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[j][u] = tl.load(r, u);
+      }
+    }
+    // pre-folded slots: the odd rank keeps step(in = even rank, inout = odd rank)
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j) {
+      if (j < nvalid && p.b[j] != nullptr) {
+        const auto r = TL::rsrc(p.b[j] + in_bytes + tb, nrec);
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[j][u] = step_vec<T, OP>(v[j][u], tl.load(r, u));
+      }
+    }
+#pragma unroll
+    for (int d = 1; d < SLOTS; d *= 2) {
+#pragma unroll
+      for (int i = 0; i + d < SLOTS; i += 2 * d) {
+        if (i + d < nvalid) {
+#pragma unroll
+          for (int u = 0; u < U; ++u) v[i][u] = step_vec<T, OP>(v[i + d][u], v[i][u]);
+        }
+      }
+    }
+    for (int j = j0; j < j0 + nj; ++j) {
+      const auto r = TL::rsrc(p.out[j] + out_bytes + tb, nrec);
+#pragma unroll
+      for (int u = 0; u < U; ++u) tl.store(r, u, v[0][u]);
+    }
   }
-  if constexpr (VECTOR) {
-    const size_t e = n * L::N + threadIdx.x;
-    if (blockIdx.x == 0 && e < len)
-      tree_tile<T, OP, SLOTS, false, 1, false>(p, in_bytes, j0, nj, out_bytes, e, len);
-  }
+  const size_t e = (len / N) * N + threadIdx.x;
+  if (blockIdx.x == 0 && e < len) tree_elem<T, OP, SLOTS>(p, in_bytes, j0, nj, out_bytes, e);
 }
 
 template <typename T, int OP, int SLOTS>
-void (*pick_tree(bool vector))(const TreeParams) {
-  return vector ? tree_kernel<T, OP, SLOTS, true> : tree_kernel<T, OP, SLOTS, false>;
+__global__ void __launch_bounds__(kThreads) tree_elem_kernel(const TreeParams p) {
+  const unsigned seg = blockIdx.y;
+  size_t off, len;
+  seg_range(p.seg, seg, off, len);
+  const size_t off_bytes = off * sizeof(T);
+  const size_t in_bytes = p.seg.in_blocked ? off_bytes : 0;
+  int j0, nj;
+  size_t out_bytes;
+  tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
+  for (size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x; e < len; e += (size_t)gridDim.x * kThreads)
+    tree_elem<T, OP, SLOTS>(p, in_bytes, j0, nj, out_bytes, e);
+}
+
+template <typename T, int OP, int SLOTS>
+int launch_tree_slots(const TreeParams &p, unsigned nseg, size_t max_len, bool vector, hipStream_t stream) {
+  if (vector) {
+    using S = TreeShape<T, OP, SLOTS>;
+    const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
+    const size_t tiles = (max_len + tile_elems - 1) / tile_elems;
+    if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
+    hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS>), dim3((unsigned)(tiles ? tiles : 1), nseg, 1),
+                       dim3(S::THREADS, 1, 1), 0, stream, p);
+  } else {
+    unsigned gx = stream_grid(max_len, (size_t)kThreads * 4, 8);
+    if (nseg > 1) {
+      unsigned per_seg = (stream_grid((size_t)-1 / 2, 1, 8) + nseg - 1) / nseg;
+      if (per_seg < 1) per_seg = 1;
+      if (gx > per_seg) gx = per_seg;
+    }
+    hipLaunchKernelGGL((tree_elem_kernel<T, OP, SLOTS>), dim3(gx, nseg, 1), dim3(kThreads, 1, 1), 0, stream, p);
+  }
+  ALAMD_HIP(hipGetLastError());
+  return ALAMD_OK;
 }
 
 }  // namespace
@@ -106,27 +155,14 @@ int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, i
   return dispatch_float(dtype, op, [&](auto tt, auto ot) -> int {
     using T = typename decltype(tt)::type;
     constexpr int OP = decltype(ot)::value;
-    const size_t per_access = vector ? 16 / sizeof(T) : 1;
-    const int u = vector ? (slots <= 8 ? 2 : 1) : (slots <= 8 ? 4 : 2);
-    const size_t tile = (size_t)kThreads * (size_t)u * per_access;
-    unsigned gx = stream_grid(max_len, tile, 8);
-    if (nseg > 1) {
-      unsigned per_seg = (stream_grid((size_t)-1 / 2, 1, 8) + nseg - 1) / nseg;
-      if (per_seg < 1) per_seg = 1;
-      if (gx > per_seg) gx = per_seg;
-    }
-    void (*kern)(const TreeParams) = nullptr;
     switch (slots) {
-    case 2: kern = pick_tree<T, OP, 2>(vector); break;
-    case 4: kern = pick_tree<T, OP, 4>(vector); break;
-    case 8: kern = pick_tree<T, OP, 8>(vector); break;
-    case 16: kern = pick_tree<T, OP, 16>(vector); break;
-    case 32: kern = pick_tree<T, OP, 32>(vector); break;
+    case 2: return launch_tree_slots<T, OP, 2>(p, nseg, max_len, vector, stream);
+    case 4: return launch_tree_slots<T, OP, 4>(p, nseg, max_len, vector, stream);
+    case 8: return launch_tree_slots<T, OP, 8>(p, nseg, max_len, vector, stream);
+    case 16: return launch_tree_slots<T, OP, 16>(p, nseg, max_len, vector, stream);
+    case 32: return launch_tree_slots<T, OP, 32>(p, nseg, max_len, vector, stream);
     default: return set_error(ALAMD_ERR_INVALID_ARG, "tree combine: bad slot count %d", slots);
     }
-    hipLaunchKernelGGL(kern, dim3(gx, nseg, 1), dim3(kThreads, 1, 1), 0, stream, p);
-    ALAMD_HIP(hipGetLastError());
-    return ALAMD_OK;
   });
 }
 

@@ -1,6 +1,7 @@
 // Test and bench support: the counter-based input generator, the exposed
 // 16-bit float conversions, and a plain streaming copy.
 #include "alamd_common.h"
+#include "alamd_tile.h"
 
 namespace alamd {
 
@@ -92,20 +93,20 @@ __global__ void __launch_bounds__(256) widen_kernel(float *dst, const uint16_t *
   }
 }
 
-__global__ void __launch_bounds__(256) copy_kernel_vec(char *dst, const char *src, size_t nvec) {
-  constexpr int U = 4;
-  constexpr size_t TILE = 256 * U;
-  const size_t ntiles = (nvec + TILE - 1) / TILE;
-  for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    const size_t i0 = t * TILE + threadIdx.x;
-    u32x4 v[U];
+constexpr int kCopyU = 8, kCopyThreads = 128;
+__global__ void __launch_bounds__(kCopyThreads) copy_kernel_vec(char *dst, const char *src, size_t vec_bytes) {
+  using TL = Tile<kCopyU, kCopyThreads>;
+  const TL tl;
+  const size_t tb = (size_t)blockIdx.x * TL::BYTES;
+  if (tb >= vec_bytes) return;
+  const int nrec = vec_bytes - tb > TL::BYTES ? (int)TL::BYTES : (int)(vec_bytes - tb);
+  const auto rs = TL::rsrc(src + tb, nrec);
+  const auto rd = TL::rsrc(dst + tb, nrec);
+  u32x4 v[kCopyU];
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-      if (i0 + (size_t)u * 256 < nvec) v[u] = ld_stream(src + (i0 + (size_t)u * 256) * 16);
+  for (int u = 0; u < kCopyU; ++u) v[u] = tl.load(rs, u);
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-      if (i0 + (size_t)u * 256 < nvec) st_stream(dst + (i0 + (size_t)u * 256) * 16, v[u]);
-  }
+  for (int u = 0; u < kCopyU; ++u) tl.store(rd, u, v[u]);
 }
 
 __global__ void __launch_bounds__(256) copy_kernel_bytes(char *dst, const char *src, size_t n) {
@@ -168,9 +169,11 @@ int alamd_copy(void *dst, const void *src, size_t bytes, void *stream) {
   if (bytes == 0) return ALAMD_OK;
   if (!dst || !src) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer");
   if (aligned16(dst) && aligned16(src) && bytes % 16 == 0) {
-    const size_t nvec = bytes / 16;
-    const unsigned grid = stream_grid(nvec, 256 * 4, 8);
-    hipLaunchKernelGGL(copy_kernel_vec, dim3(grid), dim3(256), 0, as_stream(stream), (char *)dst, (const char *)src, nvec);
+    const size_t tile = Tile<kCopyU, kCopyThreads>::BYTES;
+    const size_t tiles = (bytes + tile - 1) / tile;
+    if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "copy too large for one launch");
+    hipLaunchKernelGGL(copy_kernel_vec, dim3((unsigned)tiles), dim3(kCopyThreads), 0, as_stream(stream), (char *)dst,
+                       (const char *)src, bytes);
   } else {
     const unsigned grid = stream_grid(bytes, 256 * 16, 8);
     hipLaunchKernelGGL(copy_kernel_bytes, dim3(grid), dim3(256), 0, as_stream(stream), (char *)dst, (const char *)src, bytes);

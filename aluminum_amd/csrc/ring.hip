@@ -6,6 +6,7 @@
 // through chunk by chunk: a chunk is owned by a fixed group of workgroups.
 // FUSED: the fold kernels walk each segment once in ring order.
 #include "alamd_dispatch.h"
+#include "alamd_tile.h"
 
 namespace alamd {
 
@@ -19,7 +20,8 @@ struct RingParams {
   unsigned long long chunk_accesses;  // accesses (vectors or elements) per chunk
   int P;
   int t;              // ring step
-  unsigned wg_per_chunk;
+  unsigned wg_per_chunk;    // element path: workgroups that share one chunk
+  unsigned tiles_per_chunk; // vector path: workgroups (tiles) per chunk
 };
 
 __device__ __forceinline__ void ring_seg(const RingParams &p, int seg, size_t &off, size_t &len) {
@@ -28,11 +30,9 @@ __device__ __forceinline__ void ring_seg(const RingParams &p, int seg, size_t &o
   len = p.seg_base + (sg < p.seg_rem ? 1u : 0u);
 }
 
-// OP < 0: plain copy (allgather step).
-template <typename T, int OP, bool VECTOR>
-__global__ void __launch_bounds__(kThreads) ring_step_kernel(const RingParams p) {
-  using L = Lane<T, VECTOR>;
-  using V = typename L::V;
+// Element path (any alignment).  OP < 0: plain copy (allgather step).
+template <typename T, int OP>
+__global__ void __launch_bounds__(kThreads) ring_step_elem_kernel(const RingParams p) {
   constexpr int U = 4;
   constexpr size_t TILE = (size_t)kThreads * U;
   const int P = p.P, r = blockIdx.y;
@@ -44,42 +44,72 @@ __global__ void __launch_bounds__(kThreads) ring_step_kernel(const RingParams p)
   ring_seg(p, seg, off, len);
   char *local = p.buf[r] + off * sizeof(T);
   const char *recv = p.buf[from] + off * sizeof(T);
-
-  const size_t n = len / L::N;
-  const size_t cn = p.chunk_accesses;
+  const size_t n = len, cn = p.chunk_accesses;
   const size_t nchunks = (n + cn - 1) / cn;
   const unsigned wgpc = p.wg_per_chunk;
   const unsigned lane_wg = blockIdx.x % wgpc;
   for (size_t c = blockIdx.x / wgpc; c < nchunks; c += gridDim.x / wgpc) {
     const size_t c0 = c * cn, c1 = (c0 + cn < n) ? c0 + cn : n;
     for (size_t i0 = c0 + (size_t)lane_wg * TILE + threadIdx.x; i0 < c1; i0 += (size_t)wgpc * TILE) {
-      V a[U], b[U];
+      T a[U], b[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const size_t i = i0 + (size_t)u * kThreads;
         if (i < c1) {
-          a[u] = L::ld(recv, i);
-          if constexpr (OP >= 0) b[u] = L::ld(local, i);
+          a[u] = ld_elem<T>(recv + i * sizeof(T));
+          if constexpr (OP >= 0) b[u] = ld_elem<T>(local + i * sizeof(T));
         }
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const size_t i = i0 + (size_t)u * kThreads;
         if (i < c1) {
-          if constexpr (OP >= 0) L::st(local, i, L::template step<(OP >= 0 ? OP : 0)>(a[u], b[u]));
-          else L::st(local, i, a[u]);
+          if constexpr (OP >= 0) st_elem<T>(local + i * sizeof(T), Step<T, (OP >= 0 ? OP : 0)>::apply(a[u], b[u]));
+          else st_elem<T>(local + i * sizeof(T), a[u]);
         }
       }
     }
   }
-  if constexpr (VECTOR) {
-    const size_t e = n * L::N + threadIdx.x;
-    if (blockIdx.x == 0 && e < len) {
-      using S = Lane<T, false>;
-      const T a = S::ld(recv, e);
-      if constexpr (OP >= 0) S::st(local, e, S::template step<(OP >= 0 ? OP : 0)>(a, S::ld(local, e)));
-      else S::st(local, e, a);
-    }
+}
+
+// Vector path: a chunk is a run of tiles_per_chunk tiles; no tile crosses a
+// chunk boundary.  OP < 0: plain copy.
+constexpr int kRingU = 8;
+template <typename T, int OP>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4)))
+ring_step_vec_kernel(const RingParams p) {
+  using TL = Tile<kRingU, kThreads>;
+  const TL tl;
+  const int P = p.P, r = blockIdx.y;
+  int seg = (OP >= 0 ? r - p.t - 1 : r - p.t) % P;
+  if (seg < 0) seg += P;
+  const int from = r == 0 ? P - 1 : r - 1;
+  size_t off, len;
+  ring_seg(p, seg, off, len);
+  char *local = p.buf[r] + off * sizeof(T);
+  const char *recv = p.buf[from] + off * sizeof(T);
+  const size_t seg_bytes = len * sizeof(T);  // a multiple of 16 on this path
+  const size_t chunk_bytes = (size_t)p.chunk_accesses * 16;
+  const size_t c = blockIdx.x / p.tiles_per_chunk, ti = blockIdx.x % p.tiles_per_chunk;
+  const size_t c0 = c * chunk_bytes;
+  if (c0 >= seg_bytes) return;
+  const size_t c1 = c0 + chunk_bytes < seg_bytes ? c0 + chunk_bytes : seg_bytes;
+  const size_t tb = c0 + ti * TL::BYTES;
+  if (tb >= c1) return;
+  const int nrec = c1 - tb > TL::BYTES ? (int)TL::BYTES : (int)(c1 - tb);
+  const auto rr = TL::rsrc(recv + tb, nrec);
+  const auto rl = TL::rsrc(local + tb, nrec);
+  u32x4 a[kRingU], b[kRingU];
+#pragma unroll
+  for (int u = 0; u < kRingU; ++u) a[u] = tl.load(rr, u);
+  if constexpr (OP >= 0) {
+#pragma unroll
+    for (int u = 0; u < kRingU; ++u) b[u] = tl.load(rl, u);
+#pragma unroll
+    for (int u = 0; u < kRingU; ++u) tl.store(rl, u, step_vec<T, (OP >= 0 ? OP : 0)>(a[u], b[u]));
+  } else {
+#pragma unroll
+    for (int u = 0; u < kRingU; ++u) tl.store(rl, u, a[u]);
   }
 }
 
@@ -132,7 +162,15 @@ int make_plan(RingPlan &pl, void *const *bufs, int P, size_t count, int dtype, s
   size_t chunk_rows = nchunks;
   if (chunk_rows * wgpc > row_budget) chunk_rows = row_budget / wgpc ? row_budget / wgpc : 1;
   pl.rp.wg_per_chunk = (unsigned)wgpc;
+  pl.rp.tiles_per_chunk = 1;
   pl.gx = (unsigned)(chunk_rows * wgpc);
+  if (pl.vector) {
+    const size_t tile_vecs = Tile<kRingU, kThreads>::BYTES / 16;
+    const size_t tpc = ((cn < n ? cn : (n ? n : 1)) + tile_vecs - 1) / tile_vecs;
+    if (nchunks * tpc > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "too many chunks for one launch");
+    pl.rp.tiles_per_chunk = (unsigned)tpc;
+    pl.gx = (unsigned)(nchunks * tpc);
+  }
   return ALAMD_OK;
 }
 
@@ -142,10 +180,10 @@ int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, hipStream_t 
     // a copy only needs the element size
     void (*kern)(const RingParams) = nullptr;
     switch (pl.es) {
-    case 1: kern = pl.vector ? ring_step_kernel<uint8_t, -1, true> : ring_step_kernel<uint8_t, -1, false>; break;
-    case 2: kern = pl.vector ? ring_step_kernel<uint16_t, -1, true> : ring_step_kernel<uint16_t, -1, false>; break;
-    case 4: kern = pl.vector ? ring_step_kernel<uint32_t, -1, true> : ring_step_kernel<uint32_t, -1, false>; break;
-    default: kern = pl.vector ? ring_step_kernel<uint64_t, -1, true> : ring_step_kernel<uint64_t, -1, false>; break;
+    case 1: kern = pl.vector ? ring_step_vec_kernel<uint8_t, -1> : ring_step_elem_kernel<uint8_t, -1>; break;
+    case 2: kern = pl.vector ? ring_step_vec_kernel<uint16_t, -1> : ring_step_elem_kernel<uint16_t, -1>; break;
+    case 4: kern = pl.vector ? ring_step_vec_kernel<uint32_t, -1> : ring_step_elem_kernel<uint32_t, -1>; break;
+    default: kern = pl.vector ? ring_step_vec_kernel<uint64_t, -1> : ring_step_elem_kernel<uint64_t, -1>; break;
     }
     hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
     ALAMD_HIP(hipGetLastError());
@@ -154,7 +192,7 @@ int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, hipStream_t 
   return dispatch_any(dtype, op, [&](auto tt, auto ot) -> int {
     using T = typename decltype(tt)::type;
     constexpr int OP = decltype(ot)::value;
-    void (*kern)(const RingParams) = pl.vector ? ring_step_kernel<T, OP, true> : ring_step_kernel<T, OP, false>;
+    void (*kern)(const RingParams) = pl.vector ? ring_step_vec_kernel<T, OP> : ring_step_elem_kernel<T, OP>;
     hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;
