@@ -52,7 +52,7 @@ __device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, siz
 // operations per byte, so they keep fewer loads in flight per lane and more
 // waves resident to overlap arithmetic with memory.
 template <typename T, int OP> struct Shape {
-  static constexpr bool heavy = sizeof(T) <= 2 && OP <= ALAMD_MAX;
+  static constexpr bool heavy = sizeof(T) == 1 && OP <= ALAMD_MAX;
   static constexpr int U = heavy ? 4 : 8;
   static constexpr int THREADS = heavy ? 256 : 128;
 };
@@ -93,11 +93,14 @@ fold_vec_kernel(const FoldParams p) {
         for (int u = 0; u < U; ++u) x[k][u] = tl.load(r, u);
         idx = next_rank(idx, p.dir, PT);
       }
+      // stream-major, the order the loads were issued in (they return in
+      // order): every accumulator advances as soon as a stream has arrived
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        acc[u] = x[0][u];
+      for (int u = 0; u < U; ++u) acc[u] = x[0][u];
 #pragma unroll
-        for (int k = 1; k < PT; ++k)
+      for (int k = 1; k < PT; ++k) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
           acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[k][u]) : step_vec<T, OP>(x[k][u], acc[u]);
       }
     } else {

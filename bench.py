@@ -30,8 +30,20 @@ WORKLOADS = {
     "c4_i32_max": ("i32", 1 << 28, "max", "fullrange", 3000, "rank_asc"),
     "c4_i64_bxor": ("i64", 1 << 28, "bxor", "fullrange", 3000, "rank_asc"),
     "c4_u8_lxor": ("u8", 1 << 28, "lxor", "bool01", 3000, "rank_asc"),
+    # size / type probes
+    "f32_sum_2p28": ("f32", 1 << 28, "sum", "uniform_pm1", 1000, "rank_asc"),
+    "i32_max_2p26": ("i32", 1 << 26, "max", "fullrange", 3000, "rank_asc"),
+    "f16_sum": ("f16", 1 << 27, "sum", "normal", 2000, "rank_asc"),
+    "i8_sum": ("i8", 1 << 28, "sum", "fullrange", 3000, "rank_asc"),
+    "i16_min": ("i16", 1 << 27, "min", "fullrange", 3000, "rank_asc"),
+    "f64_sum": ("f64", 1 << 25, "sum", "uniform_pm1", 1000, "rank_asc"),
 }
 P = 8
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
+# the same counter's reading for the 1 GiB copy kernel (profiles/fold_vec_kernel_f32_sum_P8_c2.md).
+MEASURED_TRAFFIC = {"c2_f32_sum": 2415955967}
+KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false, 8>"}
 
 
 def run_combine_workload(al, torch, name, steps, warmup, check=True):
@@ -76,6 +88,28 @@ def run_combine_workload(al, torch, name, steps, warmup, check=True):
     del ins, out
     torch.cuda.empty_cache()
     return res
+
+
+def run_copy_calibration(al, torch, steps, warmup):
+    """A plain 1-read + 1-write copy of 1 GiB through alamd_copy: the reference
+    point that hardware-counter readings of the combine kernel are scaled by."""
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda")
+    dst = torch.empty(n, dtype=torch.uint8, device="cuda")
+    al.fill(src, "fullrange", 1, dtype="u8")
+    torch.cuda.synchronize()
+    for _ in range(warmup):
+        al.copy(dst, src)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(steps):
+        al.copy(dst, src)
+    ev1.record()
+    torch.cuda.synchronize()
+    ms = ev0.elapsed_time(ev1) / steps
+    ok = bool(torch.equal(src, dst))
+    return {"workload": "copy 1 GiB (alamd_copy)", "bytes_read": n, "bytes_written": n, "kernel_ms": ms,
+            "gbps_kernel": 2 * n / (ms * 1e-3) * 1e-9, "copy_ok": ok}
 
 
 def cpu_baseline():
@@ -124,6 +158,9 @@ def main():
     ap.add_argument("--also", default="c2_bf16_sum",
                     help="comma-separated extra workloads reported under 'also' ('' for none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--raw", action="store_true", help="print only the workload's own measurement record")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only the 1 GiB copy kernel (counter calibration) and print its JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the P logical ranks live in one GPU's HBM); "
@@ -141,10 +178,26 @@ def main():
         print("bench.py: " + al.load().alamd_last_error().decode(), file=sys.stderr)
         sys.exit(1)
 
+    if args.calibrate_copy:
+        print(json.dumps(run_copy_calibration(al, torch, args.steps, args.warmup)))
+        return
     main_res = run_combine_workload(al, torch, args.workload, args.steps, args.warmup)
+    if args.raw:
+        print(json.dumps(main_res))
+        return
+    del torch  # the primary measurement is done; free nothing else here
+    import torch
+    # secondary workloads run in a fresh process each (same command, one workload), so that every
+    # figure is taken with its buffers allocated on an empty device, like the primary one
     also = {}
     for name in [w for w in args.also.split(",") if w and w != args.workload]:
-        also[name] = run_combine_workload(al, torch, name, max(5, args.steps // 2), max(2, args.warmup // 2))
+        torch.cuda.empty_cache()
+        p = subprocess.run([sys.executable, os.path.abspath(__file__), "--workload", name, "--also", "",
+                            "--no-cpu-baseline", "--steps", str(max(5, args.steps // 2)),
+                            "--warmup", str(max(2, args.warmup // 2)), "--raw"],
+                           capture_output=True, text=True, timeout=600)
+        line = [l for l in p.stdout.splitlines() if l.startswith("{")]
+        also[name] = json.loads(line[-1]) if p.returncode == 0 and line else {"error": p.stderr[-300:]}
 
     out = {
         "metric": METRIC, "value": main_res["gbps_wall"], "unit": "GB/s", "n_gpus": 1,
@@ -159,8 +212,10 @@ def main():
         "pct_of_hbm_peak": 100.0 * main_res["gbps_wall"] / HBM_PEAK_GBPS,
         "parity_vs_oracle": main_res.get("parity_vs_oracle"),
         "roofline": {"bound": "hbm", "achieved": main_res["gbps_kernel"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": main_res["gbps_kernel"] / HBM_PEAK_GBPS, "traffic": None,
-                     "kernel": "fold_kernel<float, sum, P=8>", "kernel_ms": main_res["kernel_ms"],
+                     "frac": main_res["gbps_kernel"] / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC.get(args.workload),
+                     "kernel": KERNEL_NAME.get(args.workload, "alamd::fold_vec_kernel"),
+                     "kernel_ms": main_res["kernel_ms"],
                      "algorithmic_bytes": main_res["algorithmic_bytes"]},
         "also": also,
     }
