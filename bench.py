@@ -185,8 +185,6 @@ def main():
     if args.raw:
         print(json.dumps(main_res))
         return
-    del torch  # the primary measurement is done; free nothing else here
-    import torch
     # secondary workloads run in a fresh process each (same command, one workload), so that every
     # figure is taken with its buffers allocated on an empty device, like the primary one
     also = {}

@@ -1,0 +1,625 @@
+/*
+ * Aluminum-shaped C++ front end of the aluminum_amd combine engine.
+ *
+ * Header-only.  It gives the on-device engine the interface a backend policy
+ * class has in the reference, so that
+ *
+ *     Al::Allreduce<Al::HipCombineBackend>(buf, count, Al::ReductionOperator::sum, comm);
+ *
+ * compiles and behaves as `Al::Allreduce<Al::HostTransferBackend>` does
+ * (reference: include/Al.hpp:118-207, 222-421, 550-633, 1866-1883;
+ * include/aluminum/ht_impl.hpp:125-195, 303-343, 866-904, 1113-1138), with the
+ * host round trip (D2H copy, MPI_Iallreduce on the host, H2D copy;
+ * include/aluminum/ht/allreduce.hpp:41-79) replaced by one kernel launch.
+ *
+ * One GPU holds all P logical ranks.  A `World` owns the P communicators; a
+ * collective is launched when the last of the P logical ranks has made its
+ * call (calls may come from one thread in any rank order, or from P threads).
+ * Every call only enqueues work and returns; results are stream-ordered on
+ * the communicator's stream (docs/index.rst:33-40).  Errors are thrown as
+ * Al::al_exception from the calling thread.
+ *
+ * Needs the HIP host API (hip/hip_runtime_api.h) and libaluminum_amd.so.
+ */
+#ifndef ALUMINUM_AMD_AL_HPP
+#define ALUMINUM_AMD_AL_HPP
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <deque>
+#include <exception>
+#include <memory>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "aluminum_amd.h"
+
+namespace Al {
+
+/** Same text layout as the reference's exception (include/aluminum/base.hpp:52-70). */
+class al_exception : public std::exception {
+ public:
+  al_exception(const std::string m, const std::string f, const int l) : msg(m), file(f), line(l) {
+    err = file + ":" + std::to_string(line) + " - " + msg;
+  }
+  const char *what() const noexcept override { return err.c_str(); }
+
+ private:
+  const std::string msg;
+  const std::string file;
+  const int line;
+  std::string err;
+};
+#define AL_AMD_THROW(s) throw ::Al::al_exception((s), __FILE__, __LINE__)
+#define AL_AMD_CHECK(call)                                                   \
+  do {                                                                       \
+    if ((call) != ALAMD_OK) AL_AMD_THROW(std::string(alamd_last_error()));   \
+  } while (0)
+#define AL_AMD_CHECK_HIP(call)                                               \
+  do {                                                                       \
+    hipError_t al_amd_e_ = (call);                                           \
+    if (al_amd_e_ != hipSuccess)                                             \
+      AL_AMD_THROW(std::string("GPU error: ") + hipGetErrorString(al_amd_e_)); \
+  } while (0)
+
+/** Predefined reduction operations (include/aluminum/base.hpp:103-105). */
+enum class ReductionOperator { sum, prod, min, max, lor, land, lxor, bor, band, bxor, avg };
+
+namespace amd {
+
+/** 16-bit float carriers for builds without the HIP half / bfloat16 headers. */
+struct half_bits { uint16_t bits; };
+struct bfloat16_bits { uint16_t bits; };
+
+/** C++ type -> library dtype (the types of mpi::TypeMap, include/aluminum/mpi/utils.hpp:43-67). */
+template <typename T> struct TypeMap;
+#define AL_AMD_TYPEMAP(T, D) \
+  template <> struct TypeMap<T> { static constexpr int value = D; }
+AL_AMD_TYPEMAP(char, (static_cast<char>(-1) < 0 ? ALAMD_I8 : ALAMD_U8));
+AL_AMD_TYPEMAP(signed char, ALAMD_I8);
+AL_AMD_TYPEMAP(unsigned char, ALAMD_U8);
+AL_AMD_TYPEMAP(short, ALAMD_I16);
+AL_AMD_TYPEMAP(unsigned short, ALAMD_U16);
+AL_AMD_TYPEMAP(int, ALAMD_I32);
+AL_AMD_TYPEMAP(unsigned int, ALAMD_U32);
+AL_AMD_TYPEMAP(long, (sizeof(long) == 8 ? ALAMD_I64 : ALAMD_I32));
+AL_AMD_TYPEMAP(unsigned long, (sizeof(long) == 8 ? ALAMD_U64 : ALAMD_U32));
+AL_AMD_TYPEMAP(long long, ALAMD_I64);
+AL_AMD_TYPEMAP(unsigned long long, ALAMD_U64);
+AL_AMD_TYPEMAP(float, ALAMD_F32);
+AL_AMD_TYPEMAP(double, ALAMD_F64);
+AL_AMD_TYPEMAP(half_bits, ALAMD_F16);
+AL_AMD_TYPEMAP(bfloat16_bits, ALAMD_BF16);
+#if defined(__clang__)
+AL_AMD_TYPEMAP(_Float16, ALAMD_F16);
+AL_AMD_TYPEMAP(__bf16, ALAMD_BF16);
+#endif
+#if defined(HIP_INCLUDE_HIP_AMD_DETAIL_HIP_FP16_H)
+AL_AMD_TYPEMAP(__half, ALAMD_F16);
+#endif
+#if defined(_HIP_INCLUDE_HIP_AMD_DETAIL_HIP_BF16_H_)
+AL_AMD_TYPEMAP(__hip_bfloat16, ALAMD_BF16);
+#endif
+#undef AL_AMD_TYPEMAP
+
+/** Combine orders and ring modes a caller can ask for by name. */
+enum class CombineAlgorithm {
+  automatic,      /**< what the reference's MPI backend yields with MPICH on one
+                       host: binomial tree up to 2048 bytes, distance-doubling tree
+                       above (Allreduce / Reduce); distance-halving tree below
+                       512 KiB in total, descending pairwise fold above
+                       (Reduce_scatter) */
+  rank_order,     /**< ((x0 . x1) . x2) ... */
+  tree_doubling,
+  tree_halving,
+  tree_binomial,
+  pairwise,       /**< x_r . x_{r-1} . x_{r-2} ... for the block of rank r */
+  ring,           /**< ring reduce-scatter + allgather, one launch per ring step */
+  ring_fused      /**< the same values from one fused launch */
+};
+
+/** Chunk of the ring pipeline: 4 MiB, a multiple of every element size. */
+inline size_t ring_chunk_bytes(size_t /*elem_size*/) { return static_cast<size_t>(4) << 20; }
+
+class World;
+
+/** A logical rank's communicator: rank, size and a stream
+ *  (shape of internal::MPICommAndStreamWrapper,
+ *  include/aluminum/mpi_comm_and_stream_wrapper.hpp:46-129). */
+class Communicator {
+ public:
+  Communicator(const Communicator &) = delete;
+  Communicator &operator=(const Communicator &) = delete;
+  Communicator(Communicator &&) = default;
+
+  int rank() const { return rank_; }
+  int size() const { return size_; }
+  int local_rank() const { return rank_; }
+  int local_size() const { return size_; }
+  hipStream_t get_stream() const { return stream_; }
+  World &world() const { return *world_; }
+
+ private:
+  friend class World;
+  Communicator(World *w, int r, int p, hipStream_t s) : world_(w), rank_(r), size_(p), stream_(s) {}
+  World *world_;
+  int rank_, size_;
+  hipStream_t stream_;
+  uint64_t next_seq_ = 0;
+  friend struct Poster;
+};
+
+/** Completion handle of a non-blocking operation
+ *  (internal::ht::HostTransferRequest, include/aluminum/ht_impl.hpp:882-888). */
+struct Request {
+  hipEvent_t op_event = nullptr;
+  hipStream_t orig_stream = nullptr;
+  ~Request() {
+    if (op_event) (void)hipEventDestroy(op_event);
+  }
+};
+
+enum class OpKind { allreduce, reduce, reduce_scatter, allgather };
+
+/** What one logical rank contributed to one collective. */
+struct Posting {
+  const void *send = nullptr;
+  void *recv = nullptr;
+  hipStream_t stream = nullptr;
+  std::shared_ptr<Request> req;  // non-blocking: the caller's request, completed at launch
+  bool posted = false;
+};
+
+struct PendingOp {
+  uint64_t seq = 0;
+  OpKind kind = OpKind::allreduce;
+  int dtype = 0;
+  size_t count = 0;
+  ReductionOperator op = ReductionOperator::sum;
+  CombineAlgorithm algo = CombineAlgorithm::automatic;
+  int root = 0;
+  bool nonblocking = false;
+  int nposted = 0;
+  std::vector<Posting> ranks;
+};
+
+/** The P logical ranks that live in one GPU's memory. */
+class World {
+ public:
+  /** P communicators on one stream. */
+  World(int P, hipStream_t stream) : World(std::vector<hipStream_t>(static_cast<size_t>(P > 0 ? P : 0), stream)) {}
+  /** One stream per logical rank. */
+  explicit World(const std::vector<hipStream_t> &streams) {
+    const int P = static_cast<int>(streams.size());
+    if (P < 1 || P > ALAMD_MAX_RANKS) AL_AMD_THROW("Cannot create a world with this many ranks");
+    AL_AMD_CHECK(alamd_init());
+    for (int r = 0; r < P; ++r) comms_.emplace_back(new Communicator(this, r, P, streams[static_cast<size_t>(r)]));
+    // default priority on purpose: the internal stream only has to be a different stream
+    AL_AMD_CHECK_HIP(hipStreamCreateWithFlags(&internal_stream_, hipStreamNonBlocking));
+    AL_AMD_CHECK_HIP(hipEventCreateWithFlags(&sync_event_, hipEventDisableTiming));
+  }
+  ~World() {
+    (void)hipStreamSynchronize(internal_stream_);
+    (void)hipEventDestroy(sync_event_);
+    (void)hipStreamDestroy(internal_stream_);
+  }
+  World(const World &) = delete;
+  World &operator=(const World &) = delete;
+
+  int size() const { return static_cast<int>(comms_.size()); }
+  Communicator &comm(int r) { return *comms_.at(static_cast<size_t>(r)); }
+
+  /** Registers rank's part of its next collective; launches every collective
+   *  that has all P parts, in order. */
+  void post(Communicator &c, OpKind kind, int dtype, const void *send, void *recv, size_t count,
+            ReductionOperator op, CombineAlgorithm algo, int root, std::shared_ptr<Request> *req);
+
+ private:
+  void launch(PendingOp &p);
+  hipStream_t gather_streams(PendingOp &p, hipStream_t target);
+  void release_streams(PendingOp &p, hipStream_t ran_on);
+
+  std::vector<std::unique_ptr<Communicator>> comms_;
+  std::deque<PendingOp> pending_;
+  std::mutex mutex_;
+  hipStream_t internal_stream_ = nullptr;
+  hipEvent_t sync_event_ = nullptr;
+};
+
+struct Poster {
+  static uint64_t take_seq(Communicator &c) { return c.next_seq_++; }
+};
+
+inline void World::post(Communicator &c, OpKind kind, int dtype, const void *send, void *recv, size_t count,
+                        ReductionOperator op, CombineAlgorithm algo, int root, std::shared_ptr<Request> *req) {
+  std::lock_guard<std::mutex> lock(mutex_);
+  const int P = size();
+  const uint64_t seq = Poster::take_seq(c);
+  PendingOp *slot = nullptr;
+  for (auto &p : pending_)
+    if (p.seq == seq) slot = &p;
+  if (!slot) {
+    pending_.emplace_back();
+    slot = &pending_.back();
+    slot->seq = seq;
+    slot->kind = kind;
+    slot->dtype = dtype;
+    slot->count = count;
+    slot->op = op;
+    slot->algo = algo;
+    slot->root = root;
+    slot->nonblocking = req != nullptr;
+    slot->ranks.resize(static_cast<size_t>(P));
+  } else if (slot->kind != kind || slot->dtype != dtype || slot->count != count || slot->op != op ||
+             slot->algo != algo || slot->root != root || slot->nonblocking != (req != nullptr)) {
+    AL_AMD_THROW("Logical ranks disagree on the arguments of a collective");
+  }
+  Posting &me = slot->ranks[static_cast<size_t>(c.rank())];
+  me.send = send;
+  me.recv = recv;
+  me.stream = c.get_stream();
+  if (req) {
+    // handed out now, "not launched yet" until the last logical rank has called
+    *req = std::make_shared<Request>();
+    (*req)->orig_stream = c.get_stream();
+    me.req = *req;
+  }
+  me.posted = true;
+  slot->nposted++;
+  // launch in sequence order only: an operation never overtakes an earlier one
+  while (!pending_.empty() && pending_.front().nposted == P) {
+    PendingOp done = std::move(pending_.front());
+    pending_.pop_front();
+    launch(done);
+  }
+}
+
+/** Makes `target` wait for the prior work of every rank's stream; returns it. */
+inline hipStream_t World::gather_streams(PendingOp &p, hipStream_t target) {
+  for (auto &r : p.ranks) {
+    if (r.stream == target) continue;
+    AL_AMD_CHECK_HIP(hipEventRecord(sync_event_, r.stream));
+    AL_AMD_CHECK_HIP(hipStreamWaitEvent(target, sync_event_, 0));
+  }
+  return target;
+}
+
+/** Makes every rank's stream wait for what ran on `ran_on` (blocking ops), or
+ *  hands out completion events (non-blocking ops). */
+inline void World::release_streams(PendingOp &p, hipStream_t ran_on) {
+  if (p.nonblocking) {
+    for (auto &r : p.ranks) {
+      hipEvent_t ev = nullptr;
+      AL_AMD_CHECK_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+      AL_AMD_CHECK_HIP(hipEventRecord(ev, ran_on));
+      r.req->op_event = ev;
+    }
+    return;
+  }
+  bool recorded = false;
+  for (auto &r : p.ranks) {
+    if (r.stream == ran_on) continue;
+    if (!recorded) {
+      AL_AMD_CHECK_HIP(hipEventRecord(sync_event_, ran_on));
+      recorded = true;
+    }
+    AL_AMD_CHECK_HIP(hipStreamWaitEvent(r.stream, sync_event_, 0));
+  }
+}
+
+inline void World::launch(PendingOp &p) {
+  const int P = size();
+  // blocking operations run on rank 0's stream, non-blocking ones on the internal stream
+  // between the two synchronisations of ht_impl.hpp:866-888
+  hipStream_t target = p.nonblocking ? internal_stream_ : p.ranks[0].stream;
+  gather_streams(p, target);
+  std::vector<const void *> sends(static_cast<size_t>(P));
+  std::vector<void *> recvs(static_cast<size_t>(P));
+  for (int r = 0; r < P; ++r) {
+    sends[static_cast<size_t>(r)] = p.ranks[static_cast<size_t>(r)].send;
+    recvs[static_cast<size_t>(r)] = p.ranks[static_cast<size_t>(r)].recv;
+  }
+  const size_t es = alamd_dtype_size(p.dtype);
+  const int op = static_cast<int>(p.op);
+  int rc = ALAMD_OK;
+  switch (p.kind) {
+  case OpKind::allreduce:
+  case OpKind::reduce: {
+    int order = ALAMD_ORDER_RANK_ASC;
+    bool ring = false;
+    switch (p.algo) {
+    case CombineAlgorithm::automatic:
+      order = p.count * es <= 2048 ? ALAMD_ORDER_TREE_BINOMIAL : ALAMD_ORDER_TREE_DBL;
+      break;
+    case CombineAlgorithm::rank_order: order = ALAMD_ORDER_RANK_ASC; break;
+    case CombineAlgorithm::tree_doubling: order = ALAMD_ORDER_TREE_DBL; break;
+    case CombineAlgorithm::tree_halving: order = ALAMD_ORDER_TREE_HALV; break;
+    case CombineAlgorithm::tree_binomial: order = ALAMD_ORDER_TREE_BINOMIAL; break;
+    case CombineAlgorithm::ring:
+    case CombineAlgorithm::ring_fused: ring = true; break;
+    default: AL_AMD_THROW("Invalid algorithm");
+    }
+    if (p.kind == OpKind::reduce) {
+      if (ring) AL_AMD_THROW("Invalid algorithm");
+      void *out = recvs[static_cast<size_t>(p.root)];
+      rc = alamd_combine(&out, 1, sends.data(), P, p.count, p.dtype, op, order, 0, target);
+    } else if (ring) {
+      // the ring works in place on each rank's receive buffer
+      for (int r = 0; r < P && rc == ALAMD_OK; ++r)
+        if (sends[static_cast<size_t>(r)] != recvs[static_cast<size_t>(r)])
+          rc = alamd_copy(recvs[static_cast<size_t>(r)], sends[static_cast<size_t>(r)], p.count * es, target);
+      if (rc == ALAMD_OK)
+        rc = alamd_ring_allreduce(recvs.data(), P, p.count, p.dtype, op, ring_chunk_bytes(es),
+                                  p.algo == CombineAlgorithm::ring ? ALAMD_RING_STEPWISE : ALAMD_RING_FUSED,
+                                  target);
+    } else {
+      rc = alamd_combine(recvs.data(), P, sends.data(), P, p.count, p.dtype, op, order, 0, target);
+    }
+    break;
+  }
+  case OpKind::reduce_scatter: {
+    int order = ALAMD_ORDER_RANK_ASC;
+    switch (p.algo) {
+    case CombineAlgorithm::automatic:
+      order = p.count * es * static_cast<size_t>(P) < (512u << 10) ? ALAMD_ORDER_TREE_HALV : ALAMD_ORDER_PAIRWISE_DESC;
+      break;
+    case CombineAlgorithm::rank_order: order = ALAMD_ORDER_RANK_ASC; break;
+    case CombineAlgorithm::tree_doubling: order = ALAMD_ORDER_TREE_DBL; break;
+    case CombineAlgorithm::tree_halving: order = ALAMD_ORDER_TREE_HALV; break;
+    case CombineAlgorithm::tree_binomial: order = ALAMD_ORDER_TREE_BINOMIAL; break;
+    case CombineAlgorithm::pairwise: order = ALAMD_ORDER_PAIRWISE_DESC; break;
+    case CombineAlgorithm::ring_fused: order = ALAMD_ORDER_RING; break;
+    default: AL_AMD_THROW("Invalid algorithm");
+    }
+    rc = alamd_reduce_scatter(recvs.data(), sends.data(), P, p.count, p.dtype, op, order, target);
+    break;
+  }
+  case OpKind::allgather:
+    if (p.algo != CombineAlgorithm::automatic) AL_AMD_THROW("Invalid algorithm");
+    rc = alamd_allgather(recvs.data(), sends.data(), P, p.count, p.dtype, target);
+    break;
+  }
+  if (rc != ALAMD_OK) AL_AMD_THROW(std::string(alamd_last_error()));
+  release_streams(p, target);
+}
+
+}  // namespace amd
+
+/** The backend policy class (cf. HostTransferBackend, include/aluminum/ht_impl.hpp:125-146). */
+class HipCombineBackend {
+ public:
+  using comm_type = amd::Communicator;
+  using req_type = std::shared_ptr<amd::Request>;
+  static constexpr std::nullptr_t null_req = nullptr;
+  using allreduce_algo_type = amd::CombineAlgorithm;
+  using reduce_algo_type = amd::CombineAlgorithm;
+  using reduce_scatter_algo_type = amd::CombineAlgorithm;
+  using allgather_algo_type = amd::CombineAlgorithm;
+
+  static std::string Name() { return "HipCombineBackend"; }
+  /** No registration is needed for device memory (ht_impl.hpp:844-853). */
+  template <typename T> static void RegisterMemory(T *, size_t, comm_type &) {}
+  template <typename T> static void UnregisterMemory(T *, comm_type &) {}
+
+  template <typename T>
+  static void Allreduce(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op, comm_type &comm,
+                        allreduce_algo_type algo) {
+    comm.world().post(comm, amd::OpKind::allreduce, amd::TypeMap<T>::value, sendbuf, recvbuf, count, op, algo, 0,
+                      nullptr);
+  }
+  template <typename T>
+  static void Allreduce(T *recvbuf, size_t count, ReductionOperator op, comm_type &comm,
+                        allreduce_algo_type algo) {
+    Allreduce(static_cast<const T *>(recvbuf), recvbuf, count, op, comm, algo);
+  }
+  template <typename T>
+  static void NonblockingAllreduce(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op,
+                                   comm_type &comm, req_type &req, allreduce_algo_type algo) {
+    comm.world().post(comm, amd::OpKind::allreduce, amd::TypeMap<T>::value, sendbuf, recvbuf, count, op, algo, 0,
+                      &req);
+  }
+  template <typename T>
+  static void NonblockingAllreduce(T *recvbuf, size_t count, ReductionOperator op, comm_type &comm,
+                                   req_type &req, allreduce_algo_type algo) {
+    NonblockingAllreduce(static_cast<const T *>(recvbuf), recvbuf, count, op, comm, req, algo);
+  }
+
+  template <typename T>
+  static void Reduce(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op, int root,
+                     comm_type &comm, reduce_algo_type algo) {
+    if (root < 0 || root >= comm.size()) AL_AMD_THROW("Invalid root");
+    comm.world().post(comm, amd::OpKind::reduce, amd::TypeMap<T>::value, sendbuf, recvbuf, count, op, algo, root,
+                      nullptr);
+  }
+  template <typename T>
+  static void Reduce(T *recvbuf, size_t count, ReductionOperator op, int root, comm_type &comm,
+                     reduce_algo_type algo) {
+    Reduce(static_cast<const T *>(recvbuf), recvbuf, count, op, root, comm, algo);
+  }
+
+  /** sendbuf holds size()*count elements, recvbuf receives count
+   *  (include/aluminum/ht/reduce_scatter.hpp:45-74). */
+  template <typename T>
+  static void Reduce_scatter(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op, comm_type &comm,
+                             reduce_scatter_algo_type algo) {
+    comm.world().post(comm, amd::OpKind::reduce_scatter, amd::TypeMap<T>::value, sendbuf, recvbuf, count, op,
+                      algo, 0, nullptr);
+  }
+  template <typename T>
+  static void Reduce_scatter(T *recvbuf, size_t count, ReductionOperator op, comm_type &comm,
+                             reduce_scatter_algo_type algo) {
+    Reduce_scatter(static_cast<const T *>(recvbuf), recvbuf, count, op, comm, algo);
+  }
+  template <typename T>
+  static void NonblockingReduce_scatter(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op,
+                                        comm_type &comm, req_type &req, reduce_scatter_algo_type algo) {
+    comm.world().post(comm, amd::OpKind::reduce_scatter, amd::TypeMap<T>::value, sendbuf, recvbuf, count, op,
+                      algo, 0, &req);
+  }
+
+  /** sendbuf holds count elements, recvbuf receives size()*count; in place the
+   *  caller's slice is already at recvbuf + rank*count
+   *  (include/aluminum/ht/allgather.hpp:48-81). */
+  template <typename T>
+  static void Allgather(const T *sendbuf, T *recvbuf, size_t count, comm_type &comm, allgather_algo_type algo) {
+    comm.world().post(comm, amd::OpKind::allgather, amd::TypeMap<T>::value, sendbuf, recvbuf, count,
+                      ReductionOperator::sum, algo, 0, nullptr);
+  }
+  template <typename T>
+  static void Allgather(T *recvbuf, size_t count, comm_type &comm, allgather_algo_type algo) {
+    Allgather(static_cast<const T *>(recvbuf + static_cast<size_t>(comm.rank()) * count), recvbuf, count, comm,
+              algo);
+  }
+  template <typename T>
+  static void NonblockingAllgather(const T *sendbuf, T *recvbuf, size_t count, comm_type &comm, req_type &req,
+                                   allgather_algo_type algo) {
+    comm.world().post(comm, amd::OpKind::allgather, amd::TypeMap<T>::value, sendbuf, recvbuf, count,
+                      ReductionOperator::sum, algo, 0, &req);
+  }
+};
+
+/* ---- the public API templates (include/Al.hpp) ---------------------------- */
+
+template <typename Backend, typename T>
+void Allreduce(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op,
+               typename Backend::comm_type &comm,
+               typename Backend::allreduce_algo_type algo = Backend::allreduce_algo_type::automatic) {
+  Backend::template Allreduce<T>(sendbuf, recvbuf, count, op, comm, algo);
+}
+template <typename Backend, typename T>
+void Allreduce(T *buffer, size_t count, ReductionOperator op, typename Backend::comm_type &comm,
+               typename Backend::allreduce_algo_type algo = Backend::allreduce_algo_type::automatic) {
+  Backend::template Allreduce<T>(buffer, count, op, comm, algo);
+}
+template <typename Backend, typename T>
+void NonblockingAllreduce(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op,
+                          typename Backend::comm_type &comm, typename Backend::req_type &req,
+                          typename Backend::allreduce_algo_type algo = Backend::allreduce_algo_type::automatic) {
+  Backend::template NonblockingAllreduce<T>(sendbuf, recvbuf, count, op, comm, req, algo);
+}
+template <typename Backend, typename T>
+void NonblockingAllreduce(T *buffer, size_t count, ReductionOperator op, typename Backend::comm_type &comm,
+                          typename Backend::req_type &req,
+                          typename Backend::allreduce_algo_type algo = Backend::allreduce_algo_type::automatic) {
+  Backend::template NonblockingAllreduce<T>(buffer, count, op, comm, req, algo);
+}
+template <typename Backend, typename T>
+void Reduce(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op, int root,
+            typename Backend::comm_type &comm,
+            typename Backend::reduce_algo_type algo = Backend::reduce_algo_type::automatic) {
+  Backend::template Reduce<T>(sendbuf, recvbuf, count, op, root, comm, algo);
+}
+template <typename Backend, typename T>
+void Reduce(T *buffer, size_t count, ReductionOperator op, int root, typename Backend::comm_type &comm,
+            typename Backend::reduce_algo_type algo = Backend::reduce_algo_type::automatic) {
+  Backend::template Reduce<T>(buffer, count, op, root, comm, algo);
+}
+template <typename Backend, typename T>
+void Reduce_scatter(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op,
+                    typename Backend::comm_type &comm,
+                    typename Backend::reduce_scatter_algo_type algo = Backend::reduce_scatter_algo_type::automatic) {
+  Backend::template Reduce_scatter<T>(sendbuf, recvbuf, count, op, comm, algo);
+}
+template <typename Backend, typename T>
+void Reduce_scatter(T *buffer, size_t count, ReductionOperator op, typename Backend::comm_type &comm,
+                    typename Backend::reduce_scatter_algo_type algo = Backend::reduce_scatter_algo_type::automatic) {
+  Backend::template Reduce_scatter<T>(buffer, count, op, comm, algo);
+}
+template <typename Backend, typename T>
+void NonblockingReduce_scatter(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op,
+                               typename Backend::comm_type &comm, typename Backend::req_type &req,
+                               typename Backend::reduce_scatter_algo_type algo =
+                                   Backend::reduce_scatter_algo_type::automatic) {
+  Backend::template NonblockingReduce_scatter<T>(sendbuf, recvbuf, count, op, comm, req, algo);
+}
+template <typename Backend, typename T>
+void Allgather(const T *sendbuf, T *recvbuf, size_t count, typename Backend::comm_type &comm,
+               typename Backend::allgather_algo_type algo = Backend::allgather_algo_type::automatic) {
+  Backend::template Allgather<T>(sendbuf, recvbuf, count, comm, algo);
+}
+template <typename Backend, typename T>
+void Allgather(T *buffer, size_t count, typename Backend::comm_type &comm,
+               typename Backend::allgather_algo_type algo = Backend::allgather_algo_type::automatic) {
+  Backend::template Allgather<T>(buffer, count, comm, algo);
+}
+template <typename Backend, typename T>
+void NonblockingAllgather(const T *sendbuf, T *recvbuf, size_t count, typename Backend::comm_type &comm,
+                          typename Backend::req_type &req,
+                          typename Backend::allgather_algo_type algo = Backend::allgather_algo_type::automatic) {
+  Backend::template NonblockingAllgather<T>(sendbuf, recvbuf, count, comm, req, algo);
+}
+
+/** Host-only completion test; resets the request when complete
+ *  (include/aluminum/ht_impl.hpp:1113-1126). */
+template <typename Backend> bool Test(typename Backend::req_type &req);
+template <> inline bool Test<HipCombineBackend>(HipCombineBackend::req_type &req) {
+  if (req == HipCombineBackend::null_req) return true;
+  if (!req->op_event) return false;  // not launched yet: some logical rank has not made its call
+  const hipError_t e = hipEventQuery(req->op_event);
+  if (e == hipSuccess) {
+    req = HipCombineBackend::null_req;
+    return true;
+  }
+  if (e != hipErrorNotReady) AL_AMD_THROW(std::string("GPU error: ") + hipGetErrorString(e));
+  return false;
+}
+
+/** Makes the communicator's stream wait for the operation; does not block the
+ *  host (include/aluminum/ht_impl.hpp:1128-1138). */
+template <typename Backend> void Wait(typename Backend::req_type &req);
+template <> inline void Wait<HipCombineBackend>(HipCombineBackend::req_type &req) {
+  if (req == HipCombineBackend::null_req) return;
+  if (!req->op_event) AL_AMD_THROW("Wait on an operation that not every logical rank has started");
+  AL_AMD_CHECK_HIP(hipStreamWaitEvent(req->orig_stream, req->op_event, 0));
+  req = HipCombineBackend::null_req;
+}
+
+/* ---- stream flags (include/aluminum/cuda/gpu_wait.hpp, gpu_status_flag.hpp) -- */
+
+namespace amd {
+
+/** Blocks a stream until the host signals (cuda::GPUWait, src/cuda/gpu_wait.cpp:38-74). */
+class GPUWait {
+ public:
+  GPUWait() { AL_AMD_CHECK(alamd_flag_create(&flag_, 0)); }
+  ~GPUWait() { (void)alamd_flag_destroy(flag_); }
+  GPUWait(const GPUWait &) = delete;
+  GPUWait &operator=(const GPUWait &) = delete;
+  /** Enqueue the wait.  max_spins = 0 waits for ever, like the reference. */
+  void wait(hipStream_t stream, uint64_t max_spins = 0) {
+    AL_AMD_CHECK(alamd_stream_wait_flag(stream, flag_, 1, max_spins ? ALAMD_FLAG_KERNEL : ALAMD_FLAG_AUTO, max_spins));
+  }
+  void signal() { AL_AMD_CHECK(alamd_flag_signal(flag_, 1)); }
+  bool timed_out() { return alamd_flag_timed_out(flag_) != 0; }
+
+ private:
+  alamd_flag *flag_ = nullptr;
+};
+
+/** A host-pollable event (cuda::GPUStatusFlag, src/cuda/gpu_status_flag.cpp:38-98):
+ *  created complete; record() stores 0 from the host and has the stream store 1. */
+class GPUStatusFlag {
+ public:
+  GPUStatusFlag() { AL_AMD_CHECK(alamd_flag_create(&flag_, 1)); }
+  ~GPUStatusFlag() { (void)alamd_flag_destroy(flag_); }
+  GPUStatusFlag(const GPUStatusFlag &) = delete;
+  GPUStatusFlag &operator=(const GPUStatusFlag &) = delete;
+  void record(hipStream_t stream) {
+    AL_AMD_CHECK(alamd_flag_signal(flag_, 0));
+    AL_AMD_CHECK(alamd_stream_write_flag(stream, flag_, 1, ALAMD_FLAG_AUTO));
+  }
+  bool query() { return alamd_flag_query(flag_) != 0; }
+
+ private:
+  alamd_flag *flag_ = nullptr;
+};
+
+}  // namespace amd
+
+}  // namespace Al
+
+#endif
