@@ -90,6 +90,108 @@ def run_combine_workload(al, torch, name, steps, warmup, check=True):
     return res
 
 
+def timed(torch, fn, steps, warmup):
+    """Runs fn `warmup` + `steps` times on torch's current stream; returns (wall s/step, kernel ms/step)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        fn()
+    ev1.record()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps, ev0.elapsed_time(ev1) / steps
+
+
+def run_ring_workload(al, torch, mode, steps, warmup):
+    """C3: ring reduce-scatter + allgather over P=8 logical ranks, bf16, 2^27 elements per rank,
+    normal(0,1) seed 2000+rank, 4 MiB chunks, in place."""
+    import numpy as np
+    import oracle
+    dtype, count, chunk = "bf16", 1 << 27, 4 << 20
+    bufs = [torch.empty(count, dtype=torch.int16, device="cuda") for _ in range(P)]
+
+    def refill():
+        for r in range(P):
+            al.fill(bufs[r], "normal", 2000 + r, dtype=dtype)
+
+    refill()
+    al.ring_allreduce(bufs, "sum", chunk_bytes=chunk, mode=mode, dtype=dtype)
+    torch.cuda.synchronize()
+    ok, m = True, 1 << 16
+    for s in (0, 3, 7):  # segment s is the ring-order fold starting at rank s
+        off, ln = al.capi.ring_segment(count, P, s)
+        want = oracle.combine_generated(P, m, dtype, "sum", "ring", s, "normal", 2000, off + ln - m)
+        for r in (0, 5):
+            got = bufs[r][off + ln - m:off + ln].cpu().numpy().view(np.uint16)
+            ok = ok and got.tobytes() == want.tobytes()
+    refill()
+    wall, kms = timed(torch, lambda: al.ring_allreduce(bufs, "sum", chunk_bytes=chunk, mode=mode, dtype=dtype),
+                      steps, warmup)
+    es = 2
+    # stepwise: each of the P-1 reduce-scatter steps reads two segments and writes one per rank, each of the
+    # P-1 allgather steps reads one and writes one; fused: every buffer is read once and written once
+    alg = 5 * (P - 1) * count * es if mode == "stepwise" else 2 * P * count * es
+    return {"workload": "c3_ring_" + mode, "dtype": dtype, "op": "sum", "P": P, "count": count,
+            "chunk_bytes": chunk, "launches_per_step": 2 * (P - 1) if mode == "stepwise" else 1,
+            "algorithmic_bytes": alg, "ms_per_step": wall * 1e3, "kernel_ms": kms,
+            "gbps_wall": alg / wall * 1e-9, "gbps_kernel": alg / (kms * 1e-3) * 1e-9,
+            "parity_vs_oracle": bool(ok)}
+
+
+def run_halo_workload(al, torch, steps, warmup):
+    """C5: fp64 grid, interior 512^3, halo 2 (allocation 516^3, x fastest), uniform[0,1) seed 4000;
+    pack the six faces, loop them back, unpack into the ghost cells."""
+    import numpy as np
+    import oracle
+    n, h = 512, 2
+    dims, side = (n, n, n), n + 2 * h
+    grid = torch.empty(side ** 3, dtype=torch.float64, device="cuda")
+    al.fill(grid, "uniform_01", 4000)
+    bufs = {f: torch.empty(al.halo_face_elems(dims, h, f), dtype=torch.float64, device="cuda") for f in range(6)}
+    al.halo_pack(bufs, grid, dims, h)
+    al.halo_unpack(grid, bufs, dims, h)
+    torch.cuda.synchronize()
+    # parity on the host for the whole grid (1 GiB): oracle pack / unpack of the same generated grid
+    host = oracle.fill(side ** 3, "f64", "uniform_01", 4000)
+    ok = True
+    for f in range(6):
+        want = oracle.halo_pack(host, n, n, n, h, f)
+        ok = ok and bufs[f].cpu().numpy().tobytes() == want.tobytes()
+    for f in range(6):
+        host = oracle.halo_unpack(host, oracle.halo_pack(host, n, n, n, h, f), n, n, n, h, f)
+    ok = ok and grid.cpu().numpy().tobytes() == host.tobytes()
+    face_bytes = bufs[0].numel() * 8
+    res = {"workload": "c5_halo", "dtype": "f64", "grid": [side] * 3, "halo": h, "face_bytes": face_bytes,
+           "parity_vs_oracle": bool(ok)}
+    wall, kms = timed(torch, lambda: al.halo_pack(bufs, grid, dims, h), steps, warmup)
+    res["pack_all_us"], res["pack_all_gbps"] = kms * 1e3, 2 * 6 * face_bytes / (kms * 1e-3) * 1e-9
+    wall2, kms2 = timed(torch, lambda: al.halo_unpack(grid, bufs, dims, h), steps, warmup)
+    res["unpack_all_us"], res["unpack_all_gbps"] = kms2 * 1e3, 2 * 6 * face_bytes / (kms2 * 1e-3) * 1e-9
+    for f, name in enumerate(("-x", "+x", "-y", "+y", "-z", "+z")):
+        _, k1 = timed(torch, lambda: al.halo_pack({f: bufs[f]}, grid, dims, h), steps, warmup)
+        _, k2 = timed(torch, lambda: al.halo_unpack(grid, {f: bufs[f]}, dims, h), steps, warmup)
+        res["face" + name] = {"pack_us": k1 * 1e3, "pack_gbps": 2 * face_bytes / (k1 * 1e-3) * 1e-9,
+                              "unpack_us": k2 * 1e3, "unpack_gbps": 2 * face_bytes / (k2 * 1e-3) * 1e-9}
+    alg = 4 * 6 * face_bytes
+    res.update({"algorithmic_bytes": alg, "ms_per_step": (wall + wall2) * 1e3, "kernel_ms": kms + kms2,
+                "gbps_wall": alg / (wall + wall2) * 1e-9, "gbps_kernel": alg / ((kms + kms2) * 1e-3) * 1e-9})
+    return res
+
+
+def run_flag_workload():
+    exe = os.path.join(ROOT, "tests", "cpp", "bench_flags")
+    p = subprocess.run([exe, "2000"], capture_output=True, text=True, timeout=300)
+    line = [l for l in p.stdout.splitlines() if l.startswith("{")]
+    if p.returncode != 0 or not line:
+        return {"workload": "flags", "error": (p.stdout + p.stderr)[-300:]}
+    res = json.loads(line[-1])
+    res["workload"] = "flags"
+    return res
+
+
 def run_copy_calibration(al, torch, steps, warmup):
     """A plain 1-read + 1-write copy of 1 GiB through alamd_copy: the reference
     point that hardware-counter readings of the combine kernel are scaled by."""
@@ -154,7 +256,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2_f32_sum", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c2_f32_sum",
+                    choices=sorted(WORKLOADS) + ["c3_ring_stepwise", "c3_ring_fused", "c5_halo", "flags"])
     ap.add_argument("--also", default="c2_bf16_sum",
                     help="comma-separated extra workloads reported under 'also' ('' for none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -181,8 +284,15 @@ def main():
     if args.calibrate_copy:
         print(json.dumps(run_copy_calibration(al, torch, args.steps, args.warmup)))
         return
-    main_res = run_combine_workload(al, torch, args.workload, args.steps, args.warmup)
-    if args.raw:
+    if args.workload.startswith("c3_ring_"):
+        main_res = run_ring_workload(al, torch, args.workload[len("c3_ring_"):], args.steps, args.warmup)
+    elif args.workload == "c5_halo":
+        main_res = run_halo_workload(al, torch, args.steps, args.warmup)
+    elif args.workload == "flags":
+        main_res = run_flag_workload()
+    else:
+        main_res = run_combine_workload(al, torch, args.workload, args.steps, args.warmup)
+    if args.raw or args.workload not in WORKLOADS:
         print(json.dumps(main_res))
         return
     # secondary workloads run in a fresh process each (same command, one workload), so that every
