@@ -19,6 +19,13 @@ constexpr int kAuxLoadStream = 2;    // nt
 constexpr int kAuxStoreStream = 17;  // sc0 | sc1
 constexpr unsigned kRsrcFlags = 0x00020000u;
 
+// Workgroups are handed to the eight XCDs round-robin and each XCD then works
+// through its share at its own pace, so over a long launch the XCDs drift
+// apart and the addresses in flight spread over more DRAM pages.  A launch
+// therefore covers at most this many tiles per stream (64 MiB at 16 KiB per
+// tile); longer inputs are cut into consecutive launches on the same stream.
+constexpr size_t kMaxTilesPerLaunch = 4096;
+
 template <int U, int THREADS> struct Tile {
   static constexpr size_t BYTES = (size_t)THREADS * U * 16;
   unsigned vo;

@@ -178,6 +178,7 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   lay.nseg = 1;
   lay.seg.seg_base = count;
   lay.seg.seg_rem = 0;
+  lay.seg.tile0 = 0;
   lay.seg.in_blocked = 0;
   lay.seg.out_mode = OUT_ALL;
   lay.seg.owner_shift = 0;
@@ -217,6 +218,7 @@ int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, si
   Layout lay;
   lay.seg.seg_base = count;
   lay.seg.seg_rem = 0;
+  lay.seg.tile0 = 0;
   lay.seg.in_blocked = 1;
   lay.seg.out_mode = OUT_SEG;
   lay.seg.owner_shift = 0;

@@ -78,7 +78,7 @@ fold_vec_kernel(const FoldParams p) {
   out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
 
   const size_t vec_bytes = (len / N) * 16;
-  const size_t tb = (size_t)blockIdx.x * TL::BYTES;
+  const size_t tb = ((size_t)p.seg.tile0 + blockIdx.x) * TL::BYTES;
   if (tb < vec_bytes) {
     const size_t rem = vec_bytes - tb;
     const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
@@ -142,7 +142,7 @@ fold_vec_kernel(const FoldParams p) {
   }
   // the len % N trailing elements, one per thread of the first workgroup
   const size_t e = (len / N) * N + threadIdx.x;
-  if (blockIdx.x == 0 && e < len) fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
+  if (p.seg.tile0 == 0 && blockIdx.x == 0 && e < len) fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
 }
 
 constexpr int kElemThreads = 256;
@@ -184,19 +184,22 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
                                 std::is_same<T, f16_t>::value || std::is_same<T, bf16_t>::value) &&
                                (OP == ALAMD_MIN || OP == ALAMD_MAX);
     void (*kern)(const FoldParams) = nullptr;
-    dim3 grid, block;
     if (vector) {
       const size_t tile_elems = Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES / sizeof(T);
-      const size_t tiles = (max_len + tile_elems - 1) / tile_elems;
-      if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
-      grid = dim3((unsigned)(tiles ? tiles : 1), nseg, 1);
-      block = dim3(Shape<T, OP>::THREADS, 1, 1);
+      size_t tiles = (max_len + tile_elems - 1) / tile_elems;
+      if (tiles == 0) tiles = 1;
       if (p.P == 8) {
         if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 8> : fold_vec_kernel<T, OP, false, 8>;
         else kern = fold_vec_kernel<T, OP, false, 8>;
       } else {
         if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 0> : fold_vec_kernel<T, OP, false, 0>;
         else kern = fold_vec_kernel<T, OP, false, 0>;
+      }
+      FoldParams q = p;
+      for (size_t t0 = 0; t0 < tiles; t0 += kMaxTilesPerLaunch) {
+        const size_t nt = tiles - t0 < kMaxTilesPerLaunch ? tiles - t0 : kMaxTilesPerLaunch;
+        q.seg.tile0 = t0;
+        hipLaunchKernelGGL(kern, dim3((unsigned)nt, nseg, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
       }
     } else {
       unsigned gx = stream_grid(max_len, (size_t)kElemThreads * 4, 8);
@@ -205,12 +208,10 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
         if (per_seg < 1) per_seg = 1;
         if (gx > per_seg) gx = per_seg;
       }
-      grid = dim3(gx, nseg, 1);
-      block = dim3(kElemThreads, 1, 1);
       if constexpr (FP_MINMAX) kern = roles ? fold_elem_kernel<T, OP, true> : fold_elem_kernel<T, OP, false>;
       else kern = fold_elem_kernel<T, OP, false>;
+      hipLaunchKernelGGL(kern, dim3(gx, nseg, 1), dim3(kElemThreads, 1, 1), 0, stream, p);
     }
-    hipLaunchKernelGGL(kern, grid, block, 0, stream, p);
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;
   });

@@ -70,7 +70,7 @@ tree_vec_kernel(const TreeParams p) {
   const int nvalid = p.nvalid;
 
   const size_t vec_bytes = (len / N) * 16;
-  const size_t tb = (size_t)blockIdx.x * TL::BYTES;
+  const size_t tb = ((size_t)p.seg.tile0 + blockIdx.x) * TL::BYTES;
   if (tb < vec_bytes) {
     const size_t rem = vec_bytes - tb;
     const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
@@ -109,7 +109,7 @@ tree_vec_kernel(const TreeParams p) {
     }
   }
   const size_t e = (len / N) * N + threadIdx.x;
-  if (blockIdx.x == 0 && e < len) tree_elem<T, OP, SLOTS>(p, in_bytes, j0, nj, out_bytes, e);
+  if (p.seg.tile0 == 0 && blockIdx.x == 0 && e < len) tree_elem<T, OP, SLOTS>(p, in_bytes, j0, nj, out_bytes, e);
 }
 
 template <typename T, int OP, int SLOTS>
@@ -131,10 +131,15 @@ int launch_tree_slots(const TreeParams &p, unsigned nseg, size_t max_len, bool v
   if (vector) {
     using S = TreeShape<T, OP, SLOTS>;
     const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
-    const size_t tiles = (max_len + tile_elems - 1) / tile_elems;
-    if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
-    hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS>), dim3((unsigned)(tiles ? tiles : 1), nseg, 1),
-                       dim3(S::THREADS, 1, 1), 0, stream, p);
+    size_t tiles = (max_len + tile_elems - 1) / tile_elems;
+    if (tiles == 0) tiles = 1;
+    TreeParams q = p;
+    for (size_t t0 = 0; t0 < tiles; t0 += kMaxTilesPerLaunch) {
+      const size_t nt = tiles - t0 < kMaxTilesPerLaunch ? tiles - t0 : kMaxTilesPerLaunch;
+      q.seg.tile0 = t0;
+      hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS>), dim3((unsigned)nt, nseg, 1), dim3(S::THREADS, 1, 1), 0,
+                         stream, q);
+    }
   } else {
     unsigned gx = stream_grid(max_len, (size_t)kThreads * 4, 8);
     if (nseg > 1) {

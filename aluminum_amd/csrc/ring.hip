@@ -209,6 +209,7 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   fp.P = P;
   fp.seg.seg_base = count / (size_t)P;
   fp.seg.seg_rem = count % (size_t)P;
+  fp.seg.tile0 = 0;
   fp.seg.in_blocked = 1;
   fp.seg.out_mode = all ? OUT_ALL : OUT_OWNER;
   fp.seg.owner_shift = P - 1;

@@ -37,6 +37,10 @@ WORKLOADS = {
     "i8_sum": ("i8", 1 << 28, "sum", "fullrange", 3000, "rank_asc"),
     "i16_min": ("i16", 1 << 27, "min", "fullrange", 3000, "rank_asc"),
     "f64_sum": ("f64", 1 << 25, "sum", "uniform_pm1", 1000, "rank_asc"),
+    # the primary workload over four rotating buffer sets (9 GiB touched per four launches): nothing a
+    # launch reads or writes was touched by the three launches before it
+    "c2_f32_sum_rotating": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "rank_asc", 4),
+    "c2_bf16_sum_rotating": ("bf16", 1 << 27, "sum", "normal", 2000, "rank_asc", 4),
 }
 P = 8
 
@@ -47,21 +51,27 @@ KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false, 8>
 
 
 def run_combine_workload(al, torch, name, steps, warmup, check=True):
-    dtype, count, op, dist, seed, order = WORKLOADS[name]
+    dtype, count, op, dist, seed, order = WORKLOADS[name][:6]
+    nsets = WORKLOADS[name][6] if len(WORKLOADS[name]) > 6 else 1
     es = al.dtype_size(dtype)
     carrier = al.torch_dtype(dtype)
-    ins = [torch.empty(count, dtype=carrier, device="cuda") for _ in range(P)]
-    out = torch.empty(count, dtype=carrier, device="cuda")
-    for r in range(P):
-        al.fill(ins[r], dist, seed + r, dtype=dtype)
+    sets = []
+    for _ in range(nsets):
+        ins = [torch.empty(count, dtype=carrier, device="cuda") for _ in range(P)]
+        out = torch.empty(count, dtype=carrier, device="cuda")
+        for r in range(P):
+            al.fill(ins[r], dist, seed + r, dtype=dtype)
+        sets.append((ins, out))
     torch.cuda.synchronize()
-    for _ in range(warmup):
+    for i in range(warmup):
+        ins, out = sets[i % nsets]
         al.combine([out], ins, op, order=order, dtype=dtype)
     torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
-    for _ in range(steps):
+    for i in range(steps):
+        ins, out = sets[i % nsets]
         al.combine([out], ins, op, order=order, dtype=dtype)
     ev1.record()
     torch.cuda.synchronize()
@@ -70,6 +80,7 @@ def run_combine_workload(al, torch, name, steps, warmup, check=True):
     alg_bytes = (P + 1) * count * es
     res = {
         "workload": name, "dtype": dtype, "op": op, "order": order, "P": P, "count": count,
+        "buffer_sets": nsets,
         "algorithmic_bytes": alg_bytes, "ms_per_step": wall * 1e3 / steps, "kernel_ms": kernel_ms,
         "gbps_wall": alg_bytes / (wall / steps) * 1e-9, "gbps_kernel": alg_bytes / (kernel_ms * 1e-3) * 1e-9,
     }
@@ -80,12 +91,13 @@ def run_combine_workload(al, torch, name, steps, warmup, check=True):
         m = 1 << 18
         np_dt = oracle.NP_CARRIER[dtype]
         ok = True
-        for lo in (0, count - m):
-            want = oracle.combine_generated(P, m, dtype, op, order, 0, dist, seed, lo)
-            got = out[lo:lo + m].cpu().numpy().view(np_dt)
-            ok = ok and got.tobytes() == want.tobytes()
+        for _, out in sets:
+            for lo in (0, count - m):
+                want = oracle.combine_generated(P, m, dtype, op, order, 0, dist, seed, lo)
+                got = out[lo:lo + m].cpu().numpy().view(np_dt)
+                ok = ok and got.tobytes() == want.tobytes()
         res["parity_vs_oracle"] = bool(ok)
-    del ins, out
+    del sets, ins, out
     torch.cuda.empty_cache()
     return res
 
@@ -258,7 +270,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2_f32_sum",
                     choices=sorted(WORKLOADS) + ["c3_ring_stepwise", "c3_ring_fused", "c5_halo", "flags"])
-    ap.add_argument("--also", default="c2_bf16_sum",
+    ap.add_argument("--also", default="c2_bf16_sum,c2_f32_sum_rotating",
                     help="comma-separated extra workloads reported under 'also' ('' for none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--raw", action="store_true", help="print only the workload's own measurement record")
