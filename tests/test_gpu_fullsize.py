@@ -1,0 +1,142 @@
+"""Parity at the full sizes of the BASELINE configurations.
+
+Inputs are generated on the device by alamd_fill; the oracle regenerates the
+same streams on the host tile by tile (the generator is counter-based), so
+nothing but the result crosses PCIe.  Bit-exact."""
+import numpy as np
+import pytest
+
+import oracle
+from util import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+P = 8
+
+
+def device_inputs(al, torch, dtype, count, dist, seed):
+    carrier = al.torch_dtype(dtype)
+    ins = [torch.empty(count, dtype=carrier, device="cuda") for _ in range(P)]
+    for r in range(P):
+        al.fill(ins[r], dist, seed + r, dtype=dtype)
+    return ins
+
+
+@pytest.mark.parametrize("op,dist,order", [("sum", "uniform_pm1", "rank_asc"), ("prod", "uniform_09_11", "rank_asc"),
+                                           ("sum", "uniform_pm1", "tree_dbl")])
+def test_c2_fp32_full_size(al, op, dist, order):
+    """C2: P=8 fp32 buffers of 2^26 elements, seed 1000+rank."""
+    import torch
+    n = 1 << 26
+    ins = device_inputs(al, torch, "f32", n, dist, 1000)
+    out = torch.empty(n, dtype=torch.float32, device="cuda")
+    al.combine([out], ins, op, order=order)
+    torch.cuda.synchronize()
+    want = oracle.combine_generated(P, n, "f32", op, order, 0, dist, 1000)
+    assert_bits_equal(out.cpu().numpy(), want, "f32", "C2 %s %s" % (op, order))
+
+
+def test_c2_bf16_full_size(al):
+    import torch
+    n = 1 << 27
+    ins = device_inputs(al, torch, "bf16", n, "normal", 2000)
+    out = torch.empty(n, dtype=torch.int16, device="cuda")
+    al.combine([out], ins, "sum", order="rank_asc", dtype="bf16")
+    torch.cuda.synchronize()
+    want = oracle.combine_generated(P, n, "bf16", "sum", "rank_asc", 0, "normal", 2000)
+    assert_bits_equal(out.cpu().numpy().view(np.uint16), want, "bf16", "C2 bf16")
+
+
+@pytest.mark.parametrize("mode", ("stepwise", "fused"))
+def test_c3_ring_full_size(al, mode):
+    """C3: P=8 bf16 buffers of 2^27 elements, seed 2000+rank, 4 MiB chunks."""
+    import torch
+    n = 1 << 27
+    bufs = device_inputs(al, torch, "bf16", n, "normal", 2000)
+    al.ring_allreduce(bufs, "sum", chunk_bytes=4 << 20, mode=mode, dtype="bf16")
+    torch.cuda.synchronize()
+    for r in range(1, P):  # every logical rank ends with the same bytes
+        assert torch.equal(bufs[0], bufs[r]), "rank %d differs from rank 0" % r
+    got = bufs[0].cpu().numpy().view(np.uint16)
+    for s in range(P):  # segment s is the ring-order fold that starts at rank s
+        off, ln = oracle.ring_segment(n, P, s)
+        want = oracle.combine_generated(P, ln, "bf16", "sum", "ring", s, "normal", 2000, off)
+        assert_bits_equal(got[off:off + ln], want, "bf16", "C3 %s segment %d" % (mode, s))
+
+
+@pytest.mark.parametrize("dtype", ("i32", "i64"))
+def test_c4_integer_full_size(al, dtype):
+    """C4: P=8 buffers of 2^28 full-range integers, seed 3000+rank; min / max / band / bor / bxor."""
+    import torch
+    n = 1 << 28
+    ins = device_inputs(al, torch, dtype, n, "fullrange", 3000)
+    out = torch.empty(n, dtype=al.torch_dtype(dtype), device="cuda")
+    for op in ("min", "max", "band", "bor", "bxor"):
+        al.combine([out], ins, op, dtype=dtype)
+        torch.cuda.synchronize()
+        want = oracle.combine_generated(P, n, dtype, op, "rank_asc", 0, "fullrange", 3000)
+        got = out.cpu().numpy()
+        assert got.tobytes() == want.tobytes(), "C4 %s %s" % (dtype, op)
+        del want, got
+
+
+def test_c4_uint8_logical_full_size(al):
+    import torch
+    n = 1 << 28
+    ins = device_inputs(al, torch, "u8", n, "bool01", 3000)
+    out = torch.empty(n, dtype=torch.uint8, device="cuda")
+    for op in ("land", "lor", "lxor"):
+        al.combine([out], ins, op, dtype="u8")
+        torch.cuda.synchronize()
+        want = oracle.combine_generated(P, n, "u8", op, "rank_asc", 0, "bool01", 3000)
+        assert out.cpu().numpy().tobytes() == want.tobytes(), "C4 u8 %s" % op
+    # a checksum of checksums: folding the halves separately gives the halves of the whole fold
+    half = n // 2
+    out2 = torch.empty(n, dtype=torch.uint8, device="cuda")
+    al.combine([out2[:half]], [t[:half] for t in ins], "lxor", dtype="u8", count=half)
+    al.combine([out2[half:]], [t[half:] for t in ins], "lxor", dtype="u8", count=half)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+
+
+def test_c5_halo_full_size(al):
+    """C5: fp64, interior 512^3, halo 2, uniform[0,1) seed 4000; identity loopback."""
+    import torch
+    n, h = 512, 2
+    side = n + 2 * h
+    dims = (n, n, n)
+    grid = torch.empty(side ** 3, dtype=torch.float64, device="cuda")
+    al.fill(grid, "uniform_01", 4000)
+    before = grid.clone()
+    bufs = {f: torch.empty(al.halo_face_elems(dims, h, f), dtype=torch.float64, device="cuda") for f in range(6)}
+    al.halo_pack(bufs, grid, dims, h)
+    al.halo_unpack(grid, bufs, dims, h)
+    torch.cuda.synchronize()
+    host = oracle.fill(side ** 3, "f64", "uniform_01", 4000)
+    assert before.cpu().numpy().tobytes() == host.tobytes()
+    for f in range(6):
+        assert bufs[f].cpu().numpy().tobytes() == oracle.halo_pack(host, n, n, n, h, f).tobytes(), "face %d" % f
+    want = host
+    for f in range(6):
+        want = oracle.halo_unpack(want, oracle.halo_pack(host, n, n, n, h, f), n, n, n, h, f)
+    got = grid.cpu().numpy()
+    assert got.tobytes() == want.tobytes()
+    # the interior is untouched and each ghost slab equals the matching interior slab
+    g3, b3 = got.reshape(side, side, side), host.reshape(side, side, side)
+    assert (g3[h:-h, h:-h, h:-h] == b3[h:-h, h:-h, h:-h]).all()
+    assert (g3[h:-h, h:-h, :h] == b3[h:-h, h:-h, h:2 * h]).all()
+    assert (g3[:h, h:-h, h:-h] == b3[h:2 * h, h:-h, h:-h]).all()
+
+
+def test_multi_launch_boundaries(al):
+    """Counts around the 4096-tile launch cut (64 MiB per stream) and a ragged tail."""
+    import torch
+    tile = 16384 // 4
+    for n in (4096 * tile - 1, 4096 * tile, 4096 * tile + 1, 2 * 4096 * tile + 4099):
+        ins = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(2)]
+        for r in range(2):
+            al.fill(ins[r], "uniform_pm1", 77 + r)
+        out = torch.empty(n, dtype=torch.float32, device="cuda")
+        al.combine([out], ins, "sum")
+        torch.cuda.synchronize()
+        want = oracle.combine_generated(2, n, "f32", "sum", "rank_asc", 0, "uniform_pm1", 77)
+        assert_bits_equal(out.cpu().numpy(), want, "f32", "n=%d" % n)
