@@ -145,6 +145,17 @@ __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
       r[j] = narrow_bf16x2(fp_step<float, OP>(a_lo, b_lo), fp_step<float, OP>(a_hi, b_hi));
     }
     return r;
+  } else if constexpr (sizeof(T) == 1 && (OP == ALAMD_LOR || OP == ALAMD_LAND || OP == ALAMD_LXOR)) {
+    // four bytes at a time: 0x01 in every byte that is nonzero, then the bitwise op
+    u32x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t a = in[j], b = inout[j];
+      const uint32_t na = ((((a & 0x7f7f7f7fu) + 0x7f7f7f7fu) | a) & 0x80808080u) >> 7;
+      const uint32_t nb = ((((b & 0x7f7f7f7fu) + 0x7f7f7f7fu) | b) & 0x80808080u) >> 7;
+      r[j] = OP == ALAMD_LOR ? (nb | na) : OP == ALAMD_LAND ? (nb & na) : (nb ^ na);
+    }
+    return r;
   } else {
     constexpr int N = 16 / sizeof(T);
     union U { u32x4 v; T e[N]; __device__ U() {} } a, b;
