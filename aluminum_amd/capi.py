@@ -61,6 +61,8 @@ def load():
     L.alamd_combine.argtypes = [pvp, i, pvp, i, sz, i, i, i, i, vp]
     L.alamd_reduce_scatter.argtypes = [pvp, pvp, i, sz, i, i, i, vp]
     L.alamd_allgather.argtypes = [pvp, pvp, i, sz, i, vp]
+    L.alamd_reduce_scatterv.argtypes = [pvp, pvp, i, C.POINTER(sz), i, i, i, vp]
+    L.alamd_allgatherv.argtypes = [pvp, pvp, i, C.POINTER(sz), C.POINTER(sz), i, vp]
     L.alamd_ring_allreduce.argtypes = [pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_reduce_scatter.argtypes = [pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_allgather.argtypes = [pvp, i, sz, i, sz, vp]
@@ -174,6 +176,20 @@ def allgather(recvs, sends, dtype=None, count=None, stream=None):
     count = sends[0].numel() if count is None else count
     _check(load().alamd_allgather(_table(recvs), _table(sends), len(sends), count, _dt(dtype),
                                   _stream(stream)))
+
+
+def reduce_scatterv(recvs, sends, counts, op, order="rank_asc", dtype=None, stream=None):
+    dtype = dtype or _infer_dtype(sends[0])
+    P = len(sends)
+    _check(load().alamd_reduce_scatterv(_table(recvs), _table(sends), P, (C.c_size_t * P)(*counts), _dt(dtype),
+                                        _op(op), _order(order), _stream(stream)))
+
+
+def allgatherv(recvs, sends, counts, displs, dtype=None, stream=None):
+    dtype = dtype or _infer_dtype(recvs[0])
+    P = len(recvs)
+    _check(load().alamd_allgatherv(_table(recvs), _table(sends), P, (C.c_size_t * P)(*counts),
+                                   (C.c_size_t * P)(*displs), _dt(dtype), _stream(stream)))
 
 
 def ring_allreduce(bufs, op, chunk_bytes=4 << 20, mode="stepwise", dtype=None, count=None,

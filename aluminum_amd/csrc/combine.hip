@@ -128,6 +128,40 @@ __global__ void __launch_bounds__(256) gather_kernel_bytes(FoldParams p, size_t 
   }
 }
 
+// One source block copied to up to P destinations (allgatherv).
+__global__ void __launch_bounds__(kGatherThreads) bcast_kernel_vec(const char *src, FoldParams p, size_t vec_bytes,
+                                                                   size_t tail_bytes) {
+  using TL = Tile<kGatherU, kGatherThreads>;
+  const TL tl;
+  const size_t tb = (size_t)blockIdx.x * TL::BYTES;
+  if (tb < vec_bytes) {
+    const int nrec = vec_bytes - tb > TL::BYTES ? (int)TL::BYTES : (int)(vec_bytes - tb);
+    const auto rs = TL::rsrc(src + tb, nrec);
+    u32x4 v[kGatherU];
+#pragma unroll
+    for (int u = 0; u < kGatherU; ++u) v[u] = tl.load(rs, u);
+    for (int r = 0; r < p.P; ++r) {
+      if (p.out[r] == src) continue;
+      const auto rd = TL::rsrc(p.out[r] + tb, nrec);
+#pragma unroll
+      for (int u = 0; u < kGatherU; ++u) tl.store(rd, u, v[u]);
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail_bytes) {
+    const char c = src[vec_bytes + threadIdx.x];
+    for (int r = 0; r < p.P; ++r)
+      if (p.out[r] != src) p.out[r][vec_bytes + threadIdx.x] = c;
+  }
+}
+
+__global__ void __launch_bounds__(256) bcast_kernel_bytes(const char *src, FoldParams p, size_t bytes) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < bytes; i += (size_t)gridDim.x * 256) {
+    const char c = src[i];
+    for (int r = 0; r < p.P; ++r)
+      if (p.out[r] != src) p.out[r][i] = c;
+  }
+}
+
 int check_common(int P, size_t count, int dtype) {
   if (P < 1 || P > ALAMD_MAX_RANKS)
     return set_error(ALAMD_ERR_INVALID_ARG, "number of ranks %d outside [1, %d]", P, ALAMD_MAX_RANKS);
@@ -287,6 +321,139 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
     hipLaunchKernelGGL(gather_kernel_bytes, dim3(gx, P, 1), dim3(256, 1, 1), 0, st, fp, blk);
   }
   ALAMD_HIP(hipGetLastError());
+  return ALAMD_OK;
+}
+
+int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, const size_t *counts, int dtype,
+                          int op, int order, void *stream) {
+  int rc = check_common(P, 0, dtype);
+  if (rc) return rc;
+  if ((rc = check_type_op(dtype, op))) return rc;
+  if (!order_valid(order)) return set_error(ALAMD_ERR_INVALID_ALGO, "Invalid algorithm");
+  if (!recvs || !sends || !counts) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
+  const size_t es = alamd_dtype_size(dtype);
+  size_t displ[ALAMD_MAX_RANKS + 1];
+  displ[0] = 0;
+  for (int b = 0; b < P; ++b) {
+    if (counts[b] > (size_t)1 << 48) return set_error(ALAMD_ERR_INVALID_ARG, "count too large");
+    displ[b + 1] = displ[b] + counts[b];
+  }
+  const size_t total = displ[P] * es;
+  if (total == 0) return ALAMD_OK;
+  for (int r = 0; r < P; ++r)
+    if (!sends[r]) return set_error(ALAMD_ERR_INVALID_ARG, "send buffer %d is null", r);
+  for (int b = 0; b < P; ++b) {
+    if (counts[b] == 0) continue;
+    if (!recvs[b]) return set_error(ALAMD_ERR_INVALID_ARG, "receive buffer %d is null", b);
+    for (int r = 0; r < P; ++r) {
+      if (b == r && recvs[b] == sends[r]) continue;  // in place
+      if (ranges_overlap(recvs[b], counts[b] * es, sends[r], total))
+        return set_error(ALAMD_ERR_OVERLAP, "receive buffer %d overlaps send buffer %d", b, r);
+    }
+    for (int k = 0; k < b; ++k)
+      if (counts[k] && ranges_overlap(recvs[b], counts[b] * es, recvs[k], counts[k] * es))
+        return set_error(ALAMD_ERR_OVERLAP, "receive buffers %d and %d overlap", k, b);
+  }
+  // One fold per block, in ascending block order: in place, block b's result
+  // overwrites the start of rank b's buffer, which only blocks <= b read.
+  for (int b = 0; b < P; ++b) {
+    if (counts[b] == 0) continue;
+    const bool inplace = recvs[b] == sends[b];
+    // In place, block b reads its own rank's elements displ[b] + i while writing
+    // element i of the same buffer: go through the block in runs no longer than
+    // displ[b], each launched after the previous one, so no run reads what an
+    // unfinished run writes.
+    size_t run = counts[b];
+    if (inplace && displ[b] != 0 && displ[b] < counts[b]) {
+      run = displ[b];
+      if ((counts[b] + run - 1) / run > 4096)
+        return set_error(ALAMD_ERR_OVERLAP,
+                         "in-place reduce_scatterv: block %d of %zu elements starts only %zu elements into its own "
+                         "buffer; use separate receive buffers", b, counts[b], displ[b]);
+    }
+    for (size_t done = 0; done < counts[b]; done += run) {
+      const size_t n = counts[b] - done < run ? counts[b] - done : run;
+      const void *ins[ALAMD_MAX_RANKS];
+      void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
+      bool vector = true;
+      for (int r = 0; r < P; ++r) {
+        ins[r] = static_cast<const char *>(sends[r]) + (displ[b] + done) * es;
+        vector = vector && aligned16(ins[r]);
+      }
+      out_tab[0] = static_cast<char *>(recvs[b]) + done * es;
+      vector = vector && aligned16(out_tab[0]);
+      Layout lay;
+      lay.nseg = 1;
+      lay.seg.seg_base = n;
+      lay.seg.seg_rem = 0;
+      lay.seg.tile0 = 0;
+      lay.seg.in_blocked = 0;
+      lay.seg.out_mode = OUT_ALL;
+      lay.seg.owner_shift = 0;
+      lay.seg.nout = 1;
+      lay.max_len = n;
+      lay.start0 = order_has_start(order) ? b : 0;
+      lay.start_stride = 0;
+      if ((rc = launch_order(out_tab, ins, P, lay, dtype, op, order, vector, as_stream(stream)))) return rc;
+    }
+  }
+  return ALAMD_OK;
+}
+
+int alamd_allgatherv(void *const *recvs, const void *const *sends, int P, const size_t *counts,
+                     const size_t *displs, int dtype, void *stream) {
+  int rc = check_common(P, 0, dtype);
+  if (rc) return rc;
+  if (!recvs || !sends || !counts || !displs) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
+  const size_t es = alamd_dtype_size(dtype);
+  size_t extent = 0;  // elements a receive buffer must hold
+  for (int q = 0; q < P; ++q) {
+    if (counts[q] > (size_t)1 << 48 || displs[q] > (size_t)1 << 48)
+      return set_error(ALAMD_ERR_INVALID_ARG, "count or displacement too large");
+    if (counts[q] && displs[q] + counts[q] > extent) extent = displs[q] + counts[q];
+    for (int k = 0; k < q; ++k)
+      if (counts[q] && counts[k] && displs[q] < displs[k] + counts[k] && displs[k] < displs[q] + counts[q])
+        return set_error(ALAMD_ERR_OVERLAP, "slices %d and %d overlap in the receive buffer", k, q);
+  }
+  if (extent == 0) return ALAMD_OK;
+  for (int r = 0; r < P; ++r) {
+    if (!recvs[r]) return set_error(ALAMD_ERR_INVALID_ARG, "receive buffer %d is null", r);
+    for (int q = 0; q < P; ++q) {
+      if (counts[q] == 0) continue;
+      if (!sends[q]) return set_error(ALAMD_ERR_INVALID_ARG, "send buffer %d is null", q);
+      const char *slot = static_cast<const char *>(recvs[r]) + displs[q] * es;
+      if (r == q && sends[q] == slot) continue;  // in place
+      if (ranges_overlap(recvs[r], extent * es, sends[q], counts[q] * es))
+        return set_error(ALAMD_ERR_OVERLAP, "receive buffer %d overlaps send buffer %d", r, q);
+    }
+    for (int k = 0; k < r; ++k)
+      if (ranges_overlap(recvs[r], extent * es, recvs[k], extent * es))
+        return set_error(ALAMD_ERR_OVERLAP, "receive buffers %d and %d overlap", k, r);
+  }
+  hipStream_t st = as_stream(stream);
+  for (int q = 0; q < P; ++q) {
+    if (counts[q] == 0) continue;
+    const size_t bytes = counts[q] * es;
+    const char *src = static_cast<const char *>(sends[q]);
+    FoldParams fp;
+    bool vector = aligned16(src);
+    for (int r = 0; r < ALAMD_MAX_RANKS; ++r) { fp.in[r] = nullptr; fp.out[r] = nullptr; }
+    for (int r = 0; r < P; ++r) {
+      fp.out[r] = static_cast<char *>(recvs[r]) + displs[q] * es;
+      vector = vector && aligned16(fp.out[r]);
+    }
+    fp.P = P;
+    if (vector) {
+      const size_t vec_bytes = bytes & ~(size_t)15, tile = Tile<kGatherU, kGatherThreads>::BYTES;
+      const size_t tiles = (vec_bytes + tile - 1) / tile;
+      if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
+      hipLaunchKernelGGL(bcast_kernel_vec, dim3((unsigned)(tiles ? tiles : 1)), dim3(kGatherThreads), 0, st, src, fp,
+                         vec_bytes, bytes - vec_bytes);
+    } else {
+      hipLaunchKernelGGL(bcast_kernel_bytes, dim3(stream_grid(bytes, 256 * 16, 8)), dim3(256), 0, st, src, fp, bytes);
+    }
+    ALAMD_HIP(hipGetLastError());
+  }
   return ALAMD_OK;
 }
 

@@ -7,7 +7,7 @@
  * pointers.  Every call that takes a stream only enqueues work on it and
  * returns; buffers are caller-owned and must stay valid until the stream has
  * passed the call (reference contract: docs/comm.rst:18, docs/index.rst:33-40).
- * Calls return ALAMD_OK or a negative-free small error code; the message of
+ * Calls return ALAMD_OK or a small positive status code; the message of
  * the last error on the calling thread is alamd_last_error().  The library is
  * thread-compatible: concurrent calls are fine as long as they do not share a
  * stream or output buffers.
@@ -144,6 +144,23 @@ int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P,
  * (include/aluminum/ht/allgather.hpp:48-81; docs/comm.rst:152). */
 int alamd_allgather(void *const *recvs, const void *const *sends, int P,
                     size_t count, int dtype, void *stream);
+
+/* Reduce_scatterv: sends[r] holds sum(counts) elements; recvs[b] receives
+ * counts[b] elements, the fold of elements [displ_b, displ_b + counts[b]) of
+ * every sends[r], displ_b = counts[0] + ... + counts[b-1], with start = b for
+ * the orders that have one.  In-place form (recvs[b] == sends[b]) puts the
+ * result at the start of the buffer.  Replaces MPI_Ireduce_scatter on the
+ * host copy (include/aluminum/ht/reduce_scatterv.hpp:40-87). */
+int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P,
+                          const size_t *counts, int dtype, int op, int order,
+                          void *stream);
+
+/* Allgatherv: recvs[r][displs[q] + i] = sends[q][i], i < counts[q].
+ * In-place form: sends[q] == recvs[q] + displs[q] elements
+ * (include/aluminum/ht/allgatherv.hpp:38-100). */
+int alamd_allgatherv(void *const *recvs, const void *const *sends, int P,
+                     const size_t *counts, const size_t *displs, int dtype,
+                     void *stream);
 
 /* ---- ring reduce-scatter + allgather over P logical ranks ------------- */
 

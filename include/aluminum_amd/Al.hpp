@@ -163,7 +163,7 @@ struct Request {
   }
 };
 
-enum class OpKind { allreduce, reduce, reduce_scatter, allgather };
+enum class OpKind { allreduce, reduce, reduce_scatter, allgather, reduce_scatterv, allgatherv };
 
 /** What one logical rank contributed to one collective. */
 struct Posting {
@@ -184,6 +184,7 @@ struct PendingOp {
   int root = 0;
   bool nonblocking = false;
   int nposted = 0;
+  std::vector<size_t> counts, displs;  // the *v collectives
   std::vector<Posting> ranks;
 };
 
@@ -216,7 +217,8 @@ class World {
   /** Registers rank's part of its next collective; launches every collective
    *  that has all P parts, in order. */
   void post(Communicator &c, OpKind kind, int dtype, const void *send, void *recv, size_t count,
-            ReductionOperator op, CombineAlgorithm algo, int root, std::shared_ptr<Request> *req);
+            ReductionOperator op, CombineAlgorithm algo, int root, std::shared_ptr<Request> *req,
+            const std::vector<size_t> *counts = nullptr, const std::vector<size_t> *displs = nullptr);
 
  private:
   void launch(PendingOp &p);
@@ -235,9 +237,14 @@ struct Poster {
 };
 
 inline void World::post(Communicator &c, OpKind kind, int dtype, const void *send, void *recv, size_t count,
-                        ReductionOperator op, CombineAlgorithm algo, int root, std::shared_ptr<Request> *req) {
+                        ReductionOperator op, CombineAlgorithm algo, int root, std::shared_ptr<Request> *req,
+                        const std::vector<size_t> *counts, const std::vector<size_t> *displs) {
   std::lock_guard<std::mutex> lock(mutex_);
   const int P = size();
+  static const std::vector<size_t> none;
+  const std::vector<size_t> &cv = counts ? *counts : none, &dv = displs ? *displs : none;
+  if ((counts && cv.size() != static_cast<size_t>(P)) || (displs && dv.size() != static_cast<size_t>(P)))
+    AL_AMD_THROW("Vector of counts or displacements is not communicator-sized");
   const uint64_t seq = Poster::take_seq(c);
   PendingOp *slot = nullptr;
   for (auto &p : pending_)
@@ -253,9 +260,12 @@ inline void World::post(Communicator &c, OpKind kind, int dtype, const void *sen
     slot->algo = algo;
     slot->root = root;
     slot->nonblocking = req != nullptr;
+    slot->counts = cv;
+    slot->displs = dv;
     slot->ranks.resize(static_cast<size_t>(P));
   } else if (slot->kind != kind || slot->dtype != dtype || slot->count != count || slot->op != op ||
-             slot->algo != algo || slot->root != root || slot->nonblocking != (req != nullptr)) {
+             slot->algo != algo || slot->root != root || slot->nonblocking != (req != nullptr) ||
+             slot->counts != cv || slot->displs != dv) {
     AL_AMD_THROW("Logical ranks disagree on the arguments of a collective");
   }
   Posting &me = slot->ranks[static_cast<size_t>(c.rank())];
@@ -382,6 +392,28 @@ inline void World::launch(PendingOp &p) {
     if (p.algo != CombineAlgorithm::automatic) AL_AMD_THROW("Invalid algorithm");
     rc = alamd_allgather(recvs.data(), sends.data(), P, p.count, p.dtype, target);
     break;
+  case OpKind::reduce_scatterv: {
+    size_t total = 0;
+    for (size_t c : p.counts) total += c;
+    int order = ALAMD_ORDER_RANK_ASC;
+    switch (p.algo) {
+    case CombineAlgorithm::automatic:
+      order = total * es < (512u << 10) ? ALAMD_ORDER_TREE_HALV : ALAMD_ORDER_PAIRWISE_DESC;
+      break;
+    case CombineAlgorithm::rank_order: order = ALAMD_ORDER_RANK_ASC; break;
+    case CombineAlgorithm::tree_doubling: order = ALAMD_ORDER_TREE_DBL; break;
+    case CombineAlgorithm::tree_halving: order = ALAMD_ORDER_TREE_HALV; break;
+    case CombineAlgorithm::tree_binomial: order = ALAMD_ORDER_TREE_BINOMIAL; break;
+    case CombineAlgorithm::pairwise: order = ALAMD_ORDER_PAIRWISE_DESC; break;
+    default: AL_AMD_THROW("Invalid algorithm");
+    }
+    rc = alamd_reduce_scatterv(recvs.data(), sends.data(), P, p.counts.data(), p.dtype, op, order, target);
+    break;
+  }
+  case OpKind::allgatherv:
+    if (p.algo != CombineAlgorithm::automatic) AL_AMD_THROW("Invalid algorithm");
+    rc = alamd_allgatherv(recvs.data(), sends.data(), P, p.counts.data(), p.displs.data(), p.dtype, target);
+    break;
   }
   if (rc != ALAMD_OK) AL_AMD_THROW(std::string(alamd_last_error()));
   release_streams(p, target);
@@ -399,6 +431,8 @@ class HipCombineBackend {
   using reduce_algo_type = amd::CombineAlgorithm;
   using reduce_scatter_algo_type = amd::CombineAlgorithm;
   using allgather_algo_type = amd::CombineAlgorithm;
+  using reduce_scatterv_algo_type = amd::CombineAlgorithm;
+  using allgatherv_algo_type = amd::CombineAlgorithm;
 
   static std::string Name() { return "HipCombineBackend"; }
   /** No registration is needed for device memory (ht_impl.hpp:844-853). */
@@ -459,6 +493,37 @@ class HipCombineBackend {
                                         comm_type &comm, req_type &req, reduce_scatter_algo_type algo) {
     comm.world().post(comm, amd::OpKind::reduce_scatter, amd::TypeMap<T>::value, sendbuf, recvbuf, count, op,
                       algo, 0, &req);
+  }
+
+  /** sendbuf holds sum(counts) elements, recvbuf receives counts[rank]
+   *  (include/aluminum/ht/reduce_scatterv.hpp:40-87). */
+  template <typename T>
+  static void Reduce_scatterv(const T *sendbuf, T *recvbuf, std::vector<size_t> counts, ReductionOperator op,
+                              comm_type &comm, reduce_scatterv_algo_type algo) {
+    comm.world().post(comm, amd::OpKind::reduce_scatterv, amd::TypeMap<T>::value, sendbuf, recvbuf, 0, op, algo, 0,
+                      nullptr, &counts);
+  }
+  template <typename T>
+  static void Reduce_scatterv(T *recvbuf, std::vector<size_t> counts, ReductionOperator op, comm_type &comm,
+                              reduce_scatterv_algo_type algo) {
+    Reduce_scatterv(static_cast<const T *>(recvbuf), recvbuf, std::move(counts), op, comm, algo);
+  }
+
+  /** sendbuf holds counts[rank] elements; recvbuf receives every rank's slice at displs[rank]
+   *  (include/aluminum/ht/allgatherv.hpp:38-100). */
+  template <typename T>
+  static void Allgatherv(const T *sendbuf, T *recvbuf, std::vector<size_t> counts, std::vector<size_t> displs,
+                         comm_type &comm, allgatherv_algo_type algo) {
+    comm.world().post(comm, amd::OpKind::allgatherv, amd::TypeMap<T>::value, sendbuf, recvbuf, 0,
+                      ReductionOperator::sum, algo, 0, nullptr, &counts, &displs);
+  }
+  template <typename T>
+  static void Allgatherv(T *recvbuf, std::vector<size_t> counts, std::vector<size_t> displs, comm_type &comm,
+                         allgatherv_algo_type algo) {
+    if (displs.size() != static_cast<size_t>(comm.size()))
+      AL_AMD_THROW("Vector of counts or displacements is not communicator-sized");
+    const T *mine = recvbuf + displs[static_cast<size_t>(comm.rank())];
+    Allgatherv(mine, recvbuf, std::move(counts), std::move(displs), comm, algo);
   }
 
   /** sendbuf holds count elements, recvbuf receives size()*count; in place the
@@ -551,6 +616,33 @@ void NonblockingAllgather(const T *sendbuf, T *recvbuf, size_t count, typename B
                           typename Backend::req_type &req,
                           typename Backend::allgather_algo_type algo = Backend::allgather_algo_type::automatic) {
   Backend::template NonblockingAllgather<T>(sendbuf, recvbuf, count, comm, req, algo);
+}
+
+template <typename Backend, typename T>
+void Reduce_scatterv(const T *sendbuf, T *recvbuf, std::vector<size_t> counts, ReductionOperator op,
+                     typename Backend::comm_type &comm,
+                     typename Backend::reduce_scatterv_algo_type algo =
+                         Backend::reduce_scatterv_algo_type::automatic) {
+  Backend::template Reduce_scatterv<T>(sendbuf, recvbuf, std::move(counts), op, comm, algo);
+}
+template <typename Backend, typename T>
+void Reduce_scatterv(T *buffer, std::vector<size_t> counts, ReductionOperator op,
+                     typename Backend::comm_type &comm,
+                     typename Backend::reduce_scatterv_algo_type algo =
+                         Backend::reduce_scatterv_algo_type::automatic) {
+  Backend::template Reduce_scatterv<T>(buffer, std::move(counts), op, comm, algo);
+}
+template <typename Backend, typename T>
+void Allgatherv(const T *sendbuf, T *recvbuf, std::vector<size_t> counts, std::vector<size_t> displs,
+                typename Backend::comm_type &comm,
+                typename Backend::allgatherv_algo_type algo = Backend::allgatherv_algo_type::automatic) {
+  Backend::template Allgatherv<T>(sendbuf, recvbuf, std::move(counts), std::move(displs), comm, algo);
+}
+template <typename Backend, typename T>
+void Allgatherv(T *buffer, std::vector<size_t> counts, std::vector<size_t> displs,
+                typename Backend::comm_type &comm,
+                typename Backend::allgatherv_algo_type algo = Backend::allgatherv_algo_type::automatic) {
+  Backend::template Allgatherv<T>(buffer, std::move(counts), std::move(displs), comm, algo);
 }
 
 /** Host-only completion test; resets the request when complete

@@ -64,6 +64,8 @@ def lib():
         L.alo_combine_generated.argtypes = [vp, i, sz, i, i, i, i, i, u64, u64]
         L.alo_reduce_scatter.argtypes = [C.POINTER(vp), C.POINTER(vp), i, sz, i, i, i]
         L.alo_allgather.argtypes = [C.POINTER(vp), C.POINTER(vp), i, sz, i]
+        L.alo_reduce_scatterv.argtypes = [C.POINTER(vp), C.POINTER(vp), i, C.POINTER(sz), i, i, i]
+        L.alo_allgatherv.argtypes = [C.POINTER(vp), C.POINTER(vp), i, C.POINTER(sz), C.POINTER(sz), i]
         L.alo_ring_segment.restype = None
         L.alo_ring_segment.argtypes = [sz, i, i, C.POINTER(sz), C.POINTER(sz)]
         L.alo_ring_allreduce.argtypes = [C.POINTER(vp), i, sz, i, i, sz]
@@ -214,6 +216,30 @@ def allgather(sends, dtype):
     count = sends[0].size
     recvs = [np.empty(count * P, dtype=sends[0].dtype) for _ in range(P)]
     rc = lib().alo_allgather(_ptr_array(recvs), _ptr_array(sends), P, count, _dt(dtype))
+    if rc:
+        raise ValueError("oracle error %d" % rc)
+    return recvs
+
+
+def reduce_scatterv(sends, counts, dtype, op, order):
+    P = len(sends)
+    sends = [np.ascontiguousarray(a) for a in sends]
+    recvs = [np.empty(counts[b], dtype=sends[0].dtype) for b in range(P)]
+    rc = lib().alo_reduce_scatterv(_ptr_array(recvs), _ptr_array(sends), P, (C.c_size_t * P)(*counts),
+                                   _dt(dtype), _op(op), _order(order))
+    if rc:
+        raise ValueError("oracle error %d" % rc)
+    return recvs
+
+
+def allgatherv(sends, counts, displs, dtype, fill_value=0):
+    """Returns the P receive buffers (positions no slice covers hold `fill_value`)."""
+    P = len(sends)
+    sends = [np.ascontiguousarray(a) for a in sends]
+    extent = max([d + c for c, d in zip(counts, displs) if c] + [0])
+    recvs = [np.full(extent, fill_value, dtype=sends[0].dtype) for _ in range(P)]
+    rc = lib().alo_allgatherv(_ptr_array(recvs), _ptr_array(sends), P, (C.c_size_t * P)(*counts),
+                              (C.c_size_t * P)(*displs), _dt(dtype))
     if rc:
         raise ValueError("oracle error %d" % rc)
     return recvs

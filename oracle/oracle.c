@@ -510,6 +510,35 @@ int alo_allgather(void *const *recv, const void *const *send, int P,
   return 0;
 }
 
+int alo_reduce_scatterv(void *const *recv, const void *const *send, int P,
+                        const size_t *counts, int dtype, int op, int order) {
+  const size_t es = alo_dtype_size(dtype);
+  int rc = alo_check_op(dtype, op);
+  if (rc) return rc;
+  const void **blk = (const void **)malloc(sizeof(void *) * (size_t)P);
+  if (!blk) return 3;
+  size_t displ = 0;
+  for (int b = 0; b < P && rc == 0; b++) {
+    for (int r = 0; r < P; r++) blk[r] = (const char *)send[r] + displ * es;
+    if (counts[b]) rc = alo_combine(recv[b], blk, P, counts[b], dtype, op, order, b);
+    displ += counts[b];
+  }
+  free(blk);
+  return rc;
+}
+
+int alo_allgatherv(void *const *recv, const void *const *send, int P,
+                   const size_t *counts, const size_t *displs, int dtype) {
+  const size_t es = alo_dtype_size(dtype);
+  if (es == 0) return 2;
+  for (int r = 0; r < P; r++)
+    for (int q = 0; q < P; q++) {
+      char *dst = (char *)recv[r] + displs[q] * es;
+      if (counts[q] && dst != (const char *)send[q]) memmove(dst, send[q], counts[q] * es);
+    }
+  return 0;
+}
+
 /* ------------------------------------------------------------------------ */
 /* Ring reduce-scatter + allgather, moved literally chunk by chunk           */
 /* ------------------------------------------------------------------------ */

@@ -141,6 +141,18 @@ int alo_reduce_scatter(void *const *recv, const void *const *send, int P,
 int alo_allgather(void *const *recv, const void *const *send, int P,
                   size_t count, int dtype);
 
+/* MPI_Reduce_scatter with per-rank counts: send[r] holds sum(counts)
+ * elements; recv[b] receives counts[b] elements, the fold of elements
+ * [displ_b, displ_b + counts[b]) with start = b
+ * (layout: include/aluminum/ht/reduce_scatterv.hpp:40-87). */
+int alo_reduce_scatterv(void *const *recv, const void *const *send, int P,
+                        const size_t *counts, int dtype, int op, int order);
+
+/* MPI_Allgatherv: recv[r][displs[q] + i] = send[q][i], i < counts[q]
+ * (layout: include/aluminum/ht/allgatherv.hpp:38-100). */
+int alo_allgatherv(void *const *recv, const void *const *send, int P,
+                   const size_t *counts, const size_t *displs, int dtype);
+
 /* Segment s of an n-element buffer split over P ranks. */
 void alo_ring_segment(size_t n, int P, int s, size_t *offset, size_t *len);
 

@@ -189,6 +189,67 @@ template <typename T> void test_allgather(int P, size_t count, bool inplace, hip
     EXPECT(same_bits(recv[r]->down(), want), "allgather P=%d count=%zu inplace=%d rank %d", P, count, inplace, r);
 }
 
+template <typename T> void test_v_variants(int P, bool inplace, hipStream_t stream) {
+  const int dt = Al::amd::TypeMap<T>::value;
+  std::vector<size_t> counts, displs_ag;
+  size_t total = 0;
+  for (int b = 0; b < P; ++b) { counts.push_back(b == 1 ? 0 : 5 + 37 * (size_t)((b * 3) % 5)); total += counts.back(); }
+  // reduce_scatterv
+  {
+    std::vector<std::vector<T>> in;
+    std::vector<std::unique_ptr<DevBuf<T>>> send, recv;
+    for (int r = 0; r < P; ++r) {
+      in.push_back(gen<T>(total, ALO_DIST_UNIFORM_PM1, 300u + (unsigned)r));
+      send.emplace_back(new DevBuf<T>(total));
+      recv.emplace_back(new DevBuf<T>(counts[r]));
+      send[r]->up(in[r]);
+    }
+    Al::amd::World world(P, stream);
+    for (int r = 0; r < P; ++r) {
+      if (inplace) Al::Reduce_scatterv<Backend>(send[r]->p, counts, Op::sum, world.comm(r));
+      else Al::Reduce_scatterv<Backend>(static_cast<const T *>(send[r]->p), recv[r]->p, counts, Op::sum, world.comm(r));
+    }
+    HIPCHK(hipStreamSynchronize(stream));
+    std::vector<std::vector<T>> want;
+    std::vector<const void *> sp;
+    std::vector<void *> rp;
+    for (int r = 0; r < P; ++r) { want.emplace_back(counts[r] ? counts[r] : 1); sp.push_back(in[r].data()); }
+    for (int r = 0; r < P; ++r) rp.push_back(want[r].data());
+    alo_reduce_scatterv(rp.data(), sp.data(), P, counts.data(), dt, ALO_SUM, ALO_ORDER_TREE_HALV);
+    for (int r = 0; r < P; ++r) {
+      auto got = inplace ? send[r]->down() : recv[r]->down();
+      got.resize(counts[r]);
+      want[r].resize(counts[r]);
+      EXPECT(same_bits(got, want[r]), "reduce_scatterv P=%d inplace=%d rank %d", P, inplace, r);
+    }
+  }
+  // allgatherv: slices placed back to front
+  {
+    size_t at = total;
+    for (int q = 0; q < P; ++q) { at -= counts[q]; displs_ag.push_back(at); }
+    std::vector<std::vector<T>> in;
+    std::vector<std::unique_ptr<DevBuf<T>>> send, recv;
+    std::vector<T> want(total);
+    for (int r = 0; r < P; ++r) {
+      in.push_back(gen<T>(counts[r], ALO_DIST_UNIFORM_PM1, 400u + (unsigned)r));
+      std::copy(in[r].begin(), in[r].end(), want.begin() + (long)displs_ag[r]);
+      send.emplace_back(new DevBuf<T>(counts[r]));
+      recv.emplace_back(new DevBuf<T>(total));
+      send[r]->up(in[r]);
+      if (inplace && counts[r])
+        HIPCHK(hipMemcpy(recv[r]->p + displs_ag[r], in[r].data(), counts[r] * sizeof(T), hipMemcpyHostToDevice));
+    }
+    Al::amd::World world(P, stream);
+    for (int r = 0; r < P; ++r) {
+      if (inplace) Al::Allgatherv<Backend>(recv[r]->p, counts, displs_ag, world.comm(r));
+      else Al::Allgatherv<Backend>(static_cast<const T *>(send[r]->p), recv[r]->p, counts, displs_ag, world.comm(r));
+    }
+    HIPCHK(hipStreamSynchronize(stream));
+    for (int r = 0; r < P; ++r)
+      EXPECT(same_bits(recv[r]->down(), want), "allgatherv P=%d inplace=%d rank %d", P, inplace, r);
+  }
+}
+
 static void test_errors(hipStream_t stream) {
   DevBuf<float> a(64), b(64);
   Al::amd::World world(2, stream);
@@ -314,6 +375,11 @@ int main() {
         test_allgather<float>(P, count, inplace, stream);
         test_allgather<unsigned char>(P, count, inplace, stream);
       }
+  for (int P : {1, 2, 5, 8})
+    for (bool inplace : {false, true}) {
+      test_v_variants<float>(P, inplace, stream);
+      test_v_variants<double>(P, inplace, stream);
+    }
   test_errors(stream);
   test_threads_and_streams();
   test_flags(stream);

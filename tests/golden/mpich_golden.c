@@ -155,6 +155,28 @@ static void case_reduce_scatter(int dt, int op, size_t count, int dist, int full
   free(in); free(out);
 }
 
+/* MPI_Reduce_scatter with uneven counts: rank b receives 3 + 2*((b*5) % 4) elements, rank 1 none. */
+static void case_reduce_scatterv(int dt, int op, int dist, const char *note) {
+  const unsigned long long seed = 1000;
+  size_t es = alo_dtype_size(dt), n = 0;
+  int *counts = (int *)malloc(sizeof(int) * (size_t)P_);
+  for (int b = 0; b < P_; b++) { counts[b] = b == 1 ? 0 : 3 + 2 * ((b * 5) % 4); n += (size_t)counts[b]; }
+  void *in = malloc(n * es), *out = malloc(16 * es);
+  memset(out, 0, 16 * es);
+  alo_fill(in, n, dt, dist, seed + (unsigned long long)rank_, 0);
+  MPI_Reduce_scatter(in, out, counts, mpi_type(dt), mpi_op(op), MPI_COMM_WORLD);
+  head("reduce_scatterv", dt, op, n, dist, seed, note);
+  if (rank_ == 0) {
+    printf(", \"counts\": [");
+    for (int b = 0; b < P_; b++) printf("%s%d", b ? ", " : "", counts[b]);
+    printf("]");
+  }
+  emit_list("in", in, n * es);
+  emit_list("out", out, 16 * es); /* first counts[rank] elements are significant */
+  tail();
+  free(in); free(out); free(counts);
+}
+
 int main(int argc, char **argv) {
   MPI_Init(&argc, &argv);
   MPI_Comm_rank(MPI_COMM_WORLD, &rank_);
@@ -186,6 +208,7 @@ int main(int argc, char **argv) {
         case_allreduce(fdt[d], op, 48, ALO_DIST_UNIFORM_PM1, 1, "specials");
     }
     case_reduce_scatter(fdt[d], ALO_SUM, 8, ALO_DIST_UNIFORM_PM1, 1, "short message");
+    case_reduce_scatterv(fdt[d], ALO_SUM, ALO_DIST_UNIFORM_PM1, "uneven counts");
     if (big) /* >= 512 KiB in total selects the pairwise exchange */
       case_reduce_scatter(fdt[d], ALO_SUM, (size_t)(1u << 20) / (size_t)P_ / alo_dtype_size(fdt[d]) + 64,
                           ALO_DIST_UNIFORM_PM1, 0, "long message");

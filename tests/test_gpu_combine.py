@@ -171,6 +171,63 @@ def test_allgather(al, dtype):
                 assert_bits_equal(to_host(bufs[r], sends[0].dtype), want[r], dtype, "in-place allgather")
 
 
+@pytest.mark.parametrize("dtype", ("f32", "bf16", "i16", "f64"))
+@pytest.mark.parametrize("order", ("rank_asc", "tree_halv", "pairwise_desc"))
+def test_reduce_scatterv(al, dtype, order):
+    import torch
+    for P, counts in ((1, [9]), (3, [5, 0, 12]), (4, [1, 100, 3, 64]), (8, [4096, 8, 0, 1000, 8192, 1, 33, 4100])):
+        total = sum(counts)
+        sends = make_inputs(P, total, dtype, "sum")
+        want = oracle.reduce_scatterv(sends, counts, dtype, "sum", order)
+        d_sends = [to_dev(a) for a in sends]
+        recvs = [dev_empty(max(c, 1), sends[0].dtype) for c in counts]
+        al.reduce_scatterv(recvs, d_sends, counts, "sum", order=order, dtype=dtype)
+        torch.cuda.synchronize()
+        for b in range(P):
+            assert_bits_equal(to_host(recvs[b], sends[0].dtype)[:counts[b]], want[b], dtype,
+                              "reduce_scatterv %s P=%d rank %d" % (order, P, b))
+        # in place: the result replaces the start of each send buffer, also where a rank's own
+        # block starts inside the region its result overwrites (counts [1, 100, ...])
+        al.reduce_scatterv(d_sends, d_sends, counts, "sum", order=order, dtype=dtype)
+        torch.cuda.synchronize()
+        for b in range(P):
+            assert_bits_equal(to_host(d_sends[b], sends[0].dtype)[:counts[b]], want[b], dtype,
+                              "in-place reduce_scatterv %s P=%d rank %d" % (order, P, b))
+
+
+@pytest.mark.parametrize("dtype", ("u8", "i16", "f32", "f64"))
+def test_allgatherv(al, dtype):
+    import torch
+    np_dt = oracle.NP_CARRIER[dtype]
+    for P, counts, displs in ((1, [5], [2]), (3, [4, 0, 9], [9, 0, 0]), (4, [1000, 3, 64, 4099], [8, 5400, 1100, 1200]),
+                              (8, [16] * 8, [16 * (7 - q) for q in range(8)])):
+        sends = [oracle.fill(max(c, 1), dtype, "fullrange" if dtype in ("u8", "i16") else "uniform_pm1", 9 + q)[:c]
+                 for q, c in enumerate(counts)]
+        want = oracle.allgatherv(sends, counts, displs, dtype, fill_value=0)
+        extent = want[0].size
+        d_sends = [to_dev(a) if a.size else dev_empty(1, np_dt) for a in sends]
+        recvs = [to_dev(np.zeros(extent, np_dt)) for _ in range(P)]
+        al.allgatherv(recvs, d_sends, counts, displs, dtype=dtype)
+        torch.cuda.synchronize()
+        for r in range(P):
+            assert_bits_equal(to_host(recvs[r], np_dt), want[r], dtype, "allgatherv P=%d rank %d" % (P, r))
+        # in place: each rank's slice already sits at its displacement
+        bufs = [to_dev(np.zeros(extent, np_dt)) for _ in range(P)]
+        views = []
+        for q in range(P):
+            v = bufs[q][displs[q]:displs[q] + counts[q]]
+            if counts[q]:
+                v.copy_(d_sends[q][:counts[q]])
+            views.append(v if counts[q] else d_sends[q])
+        al.allgatherv(bufs, views, counts, displs, dtype=dtype)
+        torch.cuda.synchronize()
+        for r in range(P):
+            assert_bits_equal(to_host(bufs[r], np_dt), want[r], dtype, "in-place allgatherv P=%d rank %d" % (P, r))
+    with pytest.raises(al.AlError) as e:  # slices 0 and 1 collide in the receive buffer
+        al.allgatherv(recvs, d_sends, counts, [0, 8] + [100 + 16 * q for q in range(6)], dtype=dtype)
+    assert e.value.code == 5
+
+
 def test_errors(al):
     import torch
     a = [to_dev(np.zeros(16, np.float32)) for _ in range(2)]

@@ -89,6 +89,23 @@ def test_reduce_scatter_vectors(path):
     assert seen >= 4
 
 
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-8] for p in GOLDEN])
+def test_reduce_scatterv_vectors(path):
+    """MPI_Reduce_scatter with uneven counts (one of them zero): distance-halving tree."""
+    doc = load(path)
+    P = doc["P"]
+    cases = [c for c in doc["cases"] if c["coll"] == "reduce_scatterv"]
+    assert len(cases) == 2
+    for c in cases:
+        dt, counts = c["dtype"], c["counts"]
+        ins = [arr(h, dt) for h in c["in"]]
+        outs = [arr(h, dt) for h in c["out"]]
+        assert ins[0].size == sum(counts)
+        got = oracle.reduce_scatterv(ins, counts, dt, c["op"], "tree_halv")
+        for b in range(P):
+            assert_bits_equal(got[b], outs[b][:counts[b]], dt, "reduce_scatterv P=%d rank %d" % (P, b))
+
+
 def test_orders_are_distinguishable():
     """The vectors really separate the orders: a wrong order fails them."""
     doc = load([p for p in GOLDEN if p.endswith("P8.json.gz")][0])

@@ -267,6 +267,26 @@ def test_reduce_scatter_and_allgather_layout():
         assert (ag[r] == np.concatenate([s[:count] for s in sends])).all()
 
 
+def test_v_variants_layout():
+    P = 4
+    counts = [3, 0, 5, 2]
+    total = sum(counts)
+    sends = [np.arange(total, dtype=np.int64) * (r + 1) for r in range(P)]
+    rs = oracle.reduce_scatterv(sends, counts, "i64", "sum", "rank_asc")
+    displ = np.concatenate([[0], np.cumsum(counts)])
+    for b in range(P):
+        want = sum(s[displ[b]:displ[b + 1]] for s in sends)
+        assert rs[b].size == counts[b] and (rs[b] == want).all()
+    displs = [7, 0, 1, 12]  # arbitrary order, with gaps
+    pieces = [np.full(counts[q], q + 1, dtype=np.int16) for q in range(P)]
+    ag = oracle.allgatherv(pieces, counts, displs, "i16", fill_value=-1)
+    want = np.full(14, -1, dtype=np.int16)
+    for q in range(P):
+        want[displs[q]:displs[q] + counts[q]] = q + 1
+    for r in range(P):
+        assert (ag[r] == want).all()
+
+
 # ---- ring ---------------------------------------------------------------------
 
 @pytest.mark.parametrize("P", (1, 2, 3, 4, 8))
