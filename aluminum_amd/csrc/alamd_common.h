@@ -167,16 +167,8 @@ __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
   }
 }
 
-// ---- streaming loads and stores ---------------------------------------------
-// Every byte on this path is touched once, so loads and stores are marked
-// non-temporal to keep them from displacing each other in L2 / MALL.
+// ---- element access (any alignment) --------------------------------------
 
-__device__ __forceinline__ u32x4 ld_stream(const void *p) {
-  return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
-}
-__device__ __forceinline__ void st_stream(void *p, u32x4 v) {
-  __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
-}
 template <typename T> __device__ __forceinline__ T ld_elem(const void *p) {
   return *reinterpret_cast<const T *>(p);
 }
@@ -190,30 +182,5 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 // items per workgroup pass: enough workgroups to cover the work, capped at
 // `waves` workgroups per compute unit.
 unsigned stream_grid(size_t work_items, size_t per_block, int waves);
-
-}  // namespace alamd
-
-// ---- lanes: what one thread handles per access ------------------------------
-namespace alamd {
-
-// VECTOR = true: a 128-bit vector of 16/sizeof(T) elements (needs 16-byte
-// aligned addresses); VECTOR = false: one element.
-template <typename T, bool VECTOR> struct Lane;
-
-template <typename T> struct Lane<T, true> {
-  using V = u32x4;
-  static constexpr int N = 16 / sizeof(T);
-  static __device__ __forceinline__ V ld(const char *base, size_t i) { return ld_stream(base + i * 16); }
-  static __device__ __forceinline__ void st(char *base, size_t i, V v) { st_stream(base + i * 16, v); }
-  template <int OP> static __device__ __forceinline__ V step(V in, V inout) { return step_vec<T, OP>(in, inout); }
-};
-
-template <typename T> struct Lane<T, false> {
-  using V = T;
-  static constexpr int N = 1;
-  static __device__ __forceinline__ V ld(const char *base, size_t i) { return ld_elem<T>(base + i * sizeof(T)); }
-  static __device__ __forceinline__ void st(char *base, size_t i, V v) { st_elem<T>(base + i * sizeof(T), v); }
-  template <int OP> static __device__ __forceinline__ V step(V in, V inout) { return Step<T, OP>::apply(in, inout); }
-};
 
 }  // namespace alamd

@@ -165,14 +165,6 @@ __global__ void __launch_bounds__(kElemThreads) fold_elem_kernel(const FoldParam
 
 }  // namespace
 
-unsigned stream_grid(size_t work_items, size_t per_block, int waves) {
-  const int cus = device_cus();
-  size_t need = (work_items + per_block - 1) / per_block;
-  size_t cap = (size_t)(cus > 0 ? cus : 256) * (size_t)(waves > 0 ? waves : 1);
-  if (need < 1) need = 1;
-  return (unsigned)(need < cap ? need : cap);
-}
-
 int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op,
                 bool acc_is_in, bool vector, hipStream_t stream) {
   // operand roles only matter where a tie or a NaN can pick a side

@@ -2,6 +2,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <mutex>
+#include <string>
 
 #include "alamd_common.h"
 
@@ -45,6 +46,14 @@ int device_cus() {
     g_dev_known[dev] = true;
   }
   return g_dev_cus[dev];
+}
+
+unsigned stream_grid(size_t work_items, size_t per_block, int waves) {
+  const int cus = device_cus();
+  size_t need = (work_items + per_block - 1) / per_block;
+  size_t cap = (size_t)(cus > 0 ? cus : 256) * (size_t)(waves > 0 ? waves : 1);
+  if (need < 1) need = 1;
+  return (unsigned)(need < cap ? need : cap);
 }
 
 int check_type_op(int dtype, int op) {

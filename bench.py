@@ -46,7 +46,7 @@ P = 8
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
 # the same counter's reading for the 1 GiB copy kernel (profiles/fold_vec_kernel_f32_sum_P8_c2.md).
-MEASURED_TRAFFIC = {"c2_f32_sum": 2415955967}
+MEASURED_TRAFFIC = {"c2_f32_sum": 2416198138}
 KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false, 8>"}
 
 
@@ -80,7 +80,7 @@ def run_combine_workload(al, torch, name, steps, warmup, check=True):
     alg_bytes = (P + 1) * count * es
     res = {
         "workload": name, "dtype": dtype, "op": op, "order": order, "P": P, "count": count,
-        "buffer_sets": nsets,
+        "buffer_sets": nsets, "launches_per_step": -(-(count * es) // (4096 * 16384)),
         "algorithmic_bytes": alg_bytes, "ms_per_step": wall * 1e3 / steps, "kernel_ms": kernel_ms,
         "gbps_wall": alg_bytes / (wall / steps) * 1e-9, "gbps_kernel": alg_bytes / (kernel_ms * 1e-3) * 1e-9,
     }
@@ -336,6 +336,10 @@ def main():
                      "traffic": MEASURED_TRAFFIC.get(args.workload),
                      "kernel": KERNEL_NAME.get(args.workload, "alamd::fold_vec_kernel"),
                      "kernel_ms": main_res["kernel_ms"],
+                     # one call is cut into launches of at most 4096 tiles of 16 KiB per stream
+                     "launches_per_step": main_res["launches_per_step"],
+                     "launch_avg_us": main_res["kernel_ms"] * 1e3 / main_res["launches_per_step"],
+                     "algorithmic_bytes_per_launch": main_res["algorithmic_bytes"] // main_res["launches_per_step"],
                      "algorithmic_bytes": main_res["algorithmic_bytes"]},
         "also": also,
     }
