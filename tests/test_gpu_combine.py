@@ -247,3 +247,27 @@ def test_errors(al):
     # zero-length is a no-op
     al.combine(out, a, "sum", count=0)
     torch.cuda.synchronize()
+
+
+def test_combine_in_a_hip_graph(al):
+    """The library only launches kernels, so a call can be captured into a HIP
+    graph; every replay must give the eager result (fresh inputs each time)."""
+    import torch
+    P, n = 8, 300007
+    ins = [to_dev(a) for a in make_inputs(P, n, "f32", "sum")]
+    out = dev_empty(n, np.float32)
+    al.combine([out], ins, "sum", order="tree_dbl")  # eager warm-up outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        al.combine([out], ins, "sum", order="tree_dbl")
+    for rep in range(3):
+        fresh = make_inputs(P, n, "f32", "sum", seed=500 + 10 * rep)
+        for t, a in zip(ins, fresh):
+            t.copy_(torch.from_numpy(a))       # eager work between the replays
+        out.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        want = oracle.combine(fresh, "f32", "sum", "tree_dbl")
+        assert_bits_equal(to_host(out, np.float32), want, "f32", "graph replay %d" % rep)
