@@ -36,3 +36,24 @@ def test_front_end_parity_program():
     print(p.stderr[-2000:])
     assert p.returncode == 0, p.stdout[-3000:]
     assert "PASSED" in p.stdout
+
+
+@pytest.mark.gpu
+def test_benchmark_sweep_rows():
+    """bench_ops prints the reference's per-trial rows (benchmark/benchmark_utils.hpp:151-184)."""
+    exe = os.path.join(ROOT, "tests", "cpp", "bench_ops")
+    assert os.path.exists(exe), "tests/cpp/bench_ops is not built (make -C tests/cpp)"
+    p = subprocess.run([exe, "--op", "allreduce", "--datatype", "float", "--ranks", "4", "--max-size", "4096",
+                        "--num-iters", "3", "--num-warmup", "1", "--nonblocking"], capture_output=True, text=True,
+                       timeout=120)
+    assert p.returncode == 0, p.stderr
+    lines = p.stdout.strip().splitlines()
+    assert lines[0] == "Backend Type Operation Algo NonBlocking InPlace Root CommSize Size CommRank Time"
+    rows = [l.split() for l in lines[1:]]
+    assert len(rows) == 13 * 4 * 3  # sizes 1..4096, 4 ranks, 3 timed trials
+    for r in rows:
+        assert r[0] == "HipCombineBackend" and r[2] == "allreduce" and r[4] == "1" and r[7] == "4"
+        assert 0 < float(r[10]) < 1.0
+    bad = subprocess.run([exe, "--op", "allreduce", "--reduction-op", "avg", "--max-size", "4"], capture_output=True,
+                         text=True, timeout=60)
+    assert bad.returncode == 1 and "Reduction operator not supported" in bad.stderr

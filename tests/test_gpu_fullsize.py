@@ -1,4 +1,5 @@
-"""Parity at the full sizes of the BASELINE configurations.
+"""Parity at the full sizes of the benchmark configurations (P = 8; 2^26 fp32, 2^27 bf16,
+2^28 integers, a 516^3 fp64 grid).
 
 Inputs are generated on the device by alamd_fill; the oracle regenerates the
 same streams on the host tile by tile (the generator is counter-based), so
