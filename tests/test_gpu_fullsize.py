@@ -141,3 +141,24 @@ def test_multi_launch_boundaries(al):
         torch.cuda.synchronize()
         want = oracle.combine_generated(2, n, "f32", "sum", "rank_asc", 0, "uniform_pm1", 77)
         assert_bits_equal(out.cpu().numpy(), want, "f32", "n=%d" % n)
+
+
+def test_buffers_beyond_4_gib(al):
+    """Byte offsets past 2^32: two buffers of 4 GiB + 8 MiB + 4099 bytes, bitwise xor, checked in slices."""
+    import torch
+    n = (1 << 32) + (1 << 23) + 4099
+    ins = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    for r in range(2):
+        al.fill(ins[r], "fullrange", 900 + r, dtype="u8")
+    out = torch.empty(n, dtype=torch.uint8, device="cuda")
+    al.combine([out], ins, "bxor", dtype="u8")
+    torch.cuda.synchronize()
+    m = 1 << 22
+    for lo in (0, (1 << 31) - m // 2, (1 << 32) - m // 2, n - m):
+        want = oracle.combine_generated(2, m, "u8", "bxor", "rank_asc", 0, "fullrange", 900, lo)
+        assert out[lo:lo + m].cpu().numpy().tobytes() == want.tobytes(), "slice at %d" % lo
+    # a whole-buffer property: folding the result with one input again gives back the other input
+    back = torch.empty(n, dtype=torch.uint8, device="cuda")
+    al.combine([back], [out, ins[1]], "bxor", dtype="u8")
+    torch.cuda.synchronize()
+    assert torch.equal(back, ins[0])
