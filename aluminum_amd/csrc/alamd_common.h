@@ -145,6 +145,23 @@ __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
       r[j] = narrow_bf16x2(fp_step<float, OP>(a_lo, b_lo), fp_step<float, OP>(a_hi, b_hi));
     }
     return r;
+  } else if constexpr (sizeof(T) == 1 && (OP == ALAMD_MIN || OP == ALAMD_MAX)) {
+    // bytes compared as packed 16-bit pairs: even and odd bytes of a dword are
+    // zero-extended into two 2 x u16 registers; signed bytes are first biased
+    // by 0x80 so that unsigned order equals signed order
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+    constexpr uint32_t bias = std::is_signed<T>::value ? 0x80808080u : 0u;
+    u32x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t a = in[j] ^ bias, b = inout[j] ^ bias;
+      const u16x2 ae = __builtin_bit_cast(u16x2, a & 0x00ff00ffu), ao = __builtin_bit_cast(u16x2, (a >> 8) & 0x00ff00ffu);
+      const u16x2 be = __builtin_bit_cast(u16x2, b & 0x00ff00ffu), bo = __builtin_bit_cast(u16x2, (b >> 8) & 0x00ff00ffu);
+      const u16x2 re = OP == ALAMD_MIN ? __builtin_elementwise_min(be, ae) : __builtin_elementwise_max(be, ae);
+      const u16x2 ro = OP == ALAMD_MIN ? __builtin_elementwise_min(bo, ao) : __builtin_elementwise_max(bo, ao);
+      r[j] = (__builtin_bit_cast(uint32_t, re) | (__builtin_bit_cast(uint32_t, ro) << 8)) ^ bias;
+    }
+    return r;
   } else if constexpr (sizeof(T) == 1 && (OP == ALAMD_LOR || OP == ALAMD_LAND || OP == ALAMD_LXOR)) {
     // four bytes at a time: 0x01 in every byte that is nonzero, then the bitwise op
     u32x4 r;

@@ -52,7 +52,7 @@ __device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, siz
 // operations per byte, so they keep fewer loads in flight per lane and more
 // waves resident to overlap arithmetic with memory.
 template <typename T, int OP> struct Shape {
-  static constexpr bool heavy = sizeof(T) == 1 && OP <= ALAMD_MAX;
+  static constexpr bool heavy = sizeof(T) == 1 && OP <= ALAMD_PROD;
   static constexpr int U = heavy ? 4 : 8;
   static constexpr int THREADS = heavy ? 256 : 128;
 };
