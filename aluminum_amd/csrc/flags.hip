@@ -3,6 +3,7 @@
 // These are what a progress thread and a stream synchronise through
 // (reference: src/cuda/gpu_wait.cpp, src/cuda/gpu_status_flag.cpp,
 // src/cuda/helper_kernels.cu, include/aluminum/cuda/sync_memory.hpp).
+#include <mutex>
 #include <new>
 
 #include "alamd_common.h"
@@ -12,6 +13,7 @@ struct alamd_flag {
   char *block;
   int32_t *word;       // host address == device address (pinned, mapped)
   int32_t *timed_out;
+  alamd_flag *next_free;
 };
 
 namespace alamd {
@@ -36,6 +38,43 @@ __global__ void __launch_bounds__(64) wait_flag_kernel(const int32_t *word, int3
 
 __global__ void __launch_bounds__(64) write_flag_kernel(int32_t *word, int32_t value) {
   if (threadIdx.x == 0) __hip_atomic_store(word, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// Flags come from a pool of pinned slabs: pinning host memory costs far more
+// than a collective, and a host-transfer style operation uses three flags
+// (reference: sync_pool with 1024 preallocated words,
+// include/aluminum/cuda/sync_memory.hpp:46-63, src/cuda/cuda.cpp:70-74).
+// Slabs stay pinned until the process ends.
+constexpr size_t kFlagBytes = 256, kFlagsPerSlab = 128;
+std::mutex g_pool_mutex;
+alamd_flag *g_free_list = nullptr;
+
+int pool_get(alamd_flag **out) {
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  if (!g_free_list) {
+    void *slab = nullptr;
+    // Pinned memory must be allocated, not registered after the fact.
+    ALAMD_HIP(hipHostMalloc(&slab, kFlagBytes * kFlagsPerSlab, hipHostMallocMapped | hipHostMallocCoherent));
+    alamd_flag *nodes = new (std::nothrow) alamd_flag[kFlagsPerSlab];
+    if (!nodes) { (void)hipHostFree(slab); return set_error(ALAMD_ERR_INVALID_ARG, "out of host memory"); }
+    for (size_t k = 0; k < kFlagsPerSlab; ++k) {
+      nodes[k].block = static_cast<char *>(slab) + k * kFlagBytes;
+      nodes[k].word = reinterpret_cast<int32_t *>(nodes[k].block);
+      nodes[k].timed_out = reinterpret_cast<int32_t *>(nodes[k].block + 128);
+      nodes[k].next_free = g_free_list;
+      g_free_list = &nodes[k];
+    }
+  }
+  *out = g_free_list;
+  g_free_list = g_free_list->next_free;
+  (*out)->next_free = nullptr;
+  return ALAMD_OK;
+}
+
+void pool_put(alamd_flag *f) {
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  f->next_free = g_free_list;
+  g_free_list = f;
 }
 
 int memops_supported() {
@@ -71,25 +110,18 @@ int alamd_stream_memops_supported(void) { return memops_supported(); }
 
 int alamd_flag_create(alamd_flag **flag, int32_t initial) {
   if (!flag) return set_error(ALAMD_ERR_INVALID_ARG, "null flag pointer");
-  void *block = nullptr;
-  // Pinned memory must be allocated, not registered after the fact.
-  ALAMD_HIP(hipHostMalloc(&block, 256, hipHostMallocMapped | hipHostMallocCoherent));
-  alamd_flag *f = new (std::nothrow) alamd_flag;
-  if (!f) { (void)hipHostFree(block); return set_error(ALAMD_ERR_INVALID_ARG, "out of host memory"); }
-  f->block = static_cast<char *>(block);
-  f->word = reinterpret_cast<int32_t *>(f->block);
-  f->timed_out = reinterpret_cast<int32_t *>(f->block + 128);
+  alamd_flag *f = nullptr;
+  int rc = pool_get(&f);
+  if (rc) return rc;
   __atomic_store_n(f->word, initial, __ATOMIC_SEQ_CST);
   __atomic_store_n(f->timed_out, 0, __ATOMIC_SEQ_CST);
   *flag = f;
   return ALAMD_OK;
 }
 
+/* The caller must not destroy a flag that a stream may still wait on or write to. */
 int alamd_flag_destroy(alamd_flag *flag) {
-  if (!flag) return ALAMD_OK;
-  hipError_t e = hipHostFree(flag->block);
-  delete flag;
-  if (e != hipSuccess) return set_error(ALAMD_ERR_HIP, "hipHostFree failed: %s", hipGetErrorString(e));
+  if (flag) pool_put(flag);
   return ALAMD_OK;
 }
 

@@ -215,7 +215,9 @@ size_t alamd_halo_face_elems(const size_t dims[3], size_t halo, int face);
 /* ---- stream flags ------------------------------------------------------ */
 
 /* One int32 synchronisation word in pinned, device-mapped host memory on its
- * own 128-byte line (include/aluminum/cuda/sync_memory.hpp:46-60). */
+ * own 128-byte line, taken from a pool of pinned slabs that live until the
+ * process ends (include/aluminum/cuda/sync_memory.hpp:46-63).  Destroy a flag
+ * only when no stream can still wait on it or write to it. */
 typedef struct alamd_flag alamd_flag;
 
 typedef enum {

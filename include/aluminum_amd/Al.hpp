@@ -474,6 +474,18 @@ class HipCombineBackend {
                      reduce_algo_type algo) {
     Reduce(static_cast<const T *>(recvbuf), recvbuf, count, op, root, comm, algo);
   }
+  template <typename T>
+  static void NonblockingReduce(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op, int root,
+                                comm_type &comm, req_type &req, reduce_algo_type algo) {
+    if (root < 0 || root >= comm.size()) AL_AMD_THROW("Invalid root");
+    comm.world().post(comm, amd::OpKind::reduce, amd::TypeMap<T>::value, sendbuf, recvbuf, count, op, algo, root,
+                      &req);
+  }
+  template <typename T>
+  static void NonblockingReduce(T *recvbuf, size_t count, ReductionOperator op, int root, comm_type &comm,
+                                req_type &req, reduce_algo_type algo) {
+    NonblockingReduce(static_cast<const T *>(recvbuf), recvbuf, count, op, root, comm, req, algo);
+  }
 
   /** sendbuf holds size()*count elements, recvbuf receives count
    *  (include/aluminum/ht/reduce_scatter.hpp:45-74). */
@@ -582,6 +594,18 @@ template <typename Backend, typename T>
 void Reduce(T *buffer, size_t count, ReductionOperator op, int root, typename Backend::comm_type &comm,
             typename Backend::reduce_algo_type algo = Backend::reduce_algo_type::automatic) {
   Backend::template Reduce<T>(buffer, count, op, root, comm, algo);
+}
+template <typename Backend, typename T>
+void NonblockingReduce(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op, int root,
+                       typename Backend::comm_type &comm, typename Backend::req_type &req,
+                       typename Backend::reduce_algo_type algo = Backend::reduce_algo_type::automatic) {
+  Backend::template NonblockingReduce<T>(sendbuf, recvbuf, count, op, root, comm, req, algo);
+}
+template <typename Backend, typename T>
+void NonblockingReduce(T *buffer, size_t count, ReductionOperator op, int root,
+                       typename Backend::comm_type &comm, typename Backend::req_type &req,
+                       typename Backend::reduce_algo_type algo = Backend::reduce_algo_type::automatic) {
+  Backend::template NonblockingReduce<T>(buffer, count, op, root, comm, req, algo);
 }
 template <typename Backend, typename T>
 void Reduce_scatter(const T *sendbuf, T *recvbuf, size_t count, ReductionOperator op,

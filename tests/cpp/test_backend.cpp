@@ -125,8 +125,13 @@ template <typename T> void test_reduce(int P, size_t n, Op op, int root, hipStre
     recv[r]->up(marker);
   }
   Al::amd::World world(P, stream);
-  for (int r = P - 1; r >= 0; --r)  // any calling order
-    Al::Reduce<Backend>(static_cast<const T *>(send[r]->p), recv[r]->p, n, op, root, world.comm(r));
+  std::vector<Backend::req_type> reqs(P);
+  const bool nb = (n % 2) == 0;  // even sizes go through the non-blocking form
+  for (int r = P - 1; r >= 0; --r) {  // any calling order
+    if (nb) Al::NonblockingReduce<Backend>(static_cast<const T *>(send[r]->p), recv[r]->p, n, op, root, world.comm(r), reqs[r]);
+    else Al::Reduce<Backend>(static_cast<const T *>(send[r]->p), recv[r]->p, n, op, root, world.comm(r));
+  }
+  for (int r = 0; r < P; ++r) Al::Wait<Backend>(reqs[r]);
   HIPCHK(hipStreamSynchronize(stream));
   std::vector<T> want(n);
   std::vector<const void *> ptrs;

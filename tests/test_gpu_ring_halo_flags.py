@@ -276,3 +276,20 @@ def test_flag_signal_from_another_thread(al):
         assert float(x[3]) == 2.0 and not go.timed_out()
         started.destroy()
         go.destroy()
+
+
+def test_flag_pool_reuse(al):
+    """Flags come from pooled pinned slabs: many create / destroy cycles are cheap and each flag
+    starts with the value asked for, whatever its previous owner left."""
+    t0 = time.time()
+    flags = [al.Flag(k & 1) for k in range(300)]  # more than one slab
+    for k, f in enumerate(flags):
+        assert f.query() == (k & 1)
+        f.signal(1234)
+    for f in flags:
+        f.destroy()
+    for _ in range(2000):
+        f = al.Flag(7)
+        assert f.query() == 7 and not f.timed_out()
+        f.destroy()
+    assert time.time() - t0 < 20
