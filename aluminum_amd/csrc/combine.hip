@@ -309,7 +309,19 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
   }
   fp.P = P;
   hipStream_t st = as_stream(stream);
-  if (vector) {
+  if (vector && blk >= ((size_t)1 << 20)) {
+    // large slices: one launch per source keeps the writes of a launch within P
+    // destination regions (measured a few per cent faster than one grid over all sources)
+    const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
+    const size_t tiles = (blk + tile - 1) / tile;
+    if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
+    for (int q = 0; q < P; ++q) {
+      FoldParams fq = fp;
+      for (int r = 0; r < P; ++r) fq.out[r] = fp.out[r] + (size_t)q * blk;
+      hipLaunchKernelGGL(bcast_kernel_vec, dim3((unsigned)tiles), dim3(kGatherThreads), 0, st, fp.in[q], fq, blk,
+                         (size_t)0);
+    }
+  } else if (vector) {
     const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
     const size_t tiles = (blk + tile - 1) / tile;
     if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");

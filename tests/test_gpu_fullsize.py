@@ -162,3 +162,32 @@ def test_buffers_beyond_4_gib(al):
     al.combine([back], [out, ins[1]], "bxor", dtype="u8")
     torch.cuda.synchronize()
     assert torch.equal(back, ins[0])
+
+
+def test_allgather_large_slices(al):
+    """Slices above 1 MiB take the one-launch-per-source path; also in place."""
+    import torch
+    P = 5
+    for count in (700001, 700004):  # 2.8 MB fp32 slices: byte path, then 16-byte aligned vector path
+        sends = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+        for r in range(P):
+            al.fill(sends[r], "uniform_pm1", 60 + r)
+        recvs = [torch.zeros(P * count, dtype=torch.float32, device="cuda") for _ in range(P)]
+        al.allgather(recvs, sends, count=count)
+        torch.cuda.synchronize()
+        want = torch.cat(sends)
+        for r in range(P):
+            assert torch.equal(recvs[r], want), "rank %d" % r
+        host = np.concatenate([oracle.fill(count, "f32", "uniform_pm1", 60 + r) for r in range(P)])
+        assert recvs[0].cpu().numpy().tobytes() == host.tobytes()
+    # a 16-byte-aligned in-place form: slices of 700004 elements
+    count = 700004
+    bufs = [torch.zeros(P * count, dtype=torch.float32, device="cuda") for _ in range(P)]
+    views = [bufs[r][r * count:(r + 1) * count] for r in range(P)]
+    for r in range(P):
+        al.fill(views[r], "uniform_pm1", 80 + r, count=count)
+    want = torch.cat([v.clone() for v in views])
+    al.allgather(bufs, views, count=count)
+    torch.cuda.synchronize()
+    for r in range(P):
+        assert torch.equal(bufs[r], want), "in place, rank %d" % r
