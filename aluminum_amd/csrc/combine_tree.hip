@@ -52,7 +52,9 @@ __device__ __forceinline__ void tree_out_select(const TreeParams &p, unsigned se
   else { j0 = ((int)seg + p.seg.owner_shift) % p.P; nj = 1; out_bytes = off_bytes; }
 }
 
-template <typename T, int OP, int SLOTS>
+// FULL: every slot occupied and none pre-folded (P a power of two): straight-line
+// code, no uniform branches between the loads and their uses.
+template <typename T, int OP, int SLOTS, bool FULL>
 __global__ void __launch_bounds__((TreeShape<T, OP, SLOTS>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
 tree_vec_kernel(const TreeParams p) {
   constexpr int U = TreeShape<T, OP, SLOTS>::U, THREADS = TreeShape<T, OP, SLOTS>::THREADS;
@@ -67,7 +69,7 @@ tree_vec_kernel(const TreeParams p) {
   int j0, nj;
   size_t out_bytes;
   tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
-  const int nvalid = p.nvalid;
+  const int nvalid = FULL ? SLOTS : p.nvalid;
 
   const size_t vec_bytes = (len / N) * 16;
   const size_t tb = ((size_t)p.seg.tile0 + blockIdx.x) * TL::BYTES;
@@ -86,7 +88,7 @@ tree_vec_kernel(const TreeParams p) {
     // pre-folded slots: the odd rank keeps step(in = even rank, inout = odd rank)
 #pragma unroll
     for (int j = 0; j < SLOTS; ++j) {
-      if (j < nvalid && p.b[j] != nullptr) {
+      if (!FULL && j < nvalid && p.b[j] != nullptr) {
         const auto r = TL::rsrc(p.b[j] + in_bytes + tb, nrec);
 #pragma unroll
         for (int u = 0; u < U; ++u) v[j][u] = step_vec<T, OP>(v[j][u], tl.load(r, u));
@@ -134,11 +136,13 @@ int launch_tree_slots(const TreeParams &p, unsigned nseg, size_t max_len, bool v
     size_t tiles = (max_len + tile_elems - 1) / tile_elems;
     if (tiles == 0) tiles = 1;
     TreeParams q = p;
+    bool full = p.nvalid == SLOTS;
+    for (int j = 0; j < SLOTS; ++j) full = full && p.b[j] == nullptr;
+    void (*kern)(const TreeParams) = full ? tree_vec_kernel<T, OP, SLOTS, true> : tree_vec_kernel<T, OP, SLOTS, false>;
     for (size_t t0 = 0; t0 < tiles; t0 += kMaxTilesPerLaunch) {
       const size_t nt = tiles - t0 < kMaxTilesPerLaunch ? tiles - t0 : kMaxTilesPerLaunch;
       q.seg.tile0 = t0;
-      hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS>), dim3((unsigned)nt, nseg, 1), dim3(S::THREADS, 1, 1), 0,
-                         stream, q);
+      hipLaunchKernelGGL(kern, dim3((unsigned)nt, nseg, 1), dim3(S::THREADS, 1, 1), 0, stream, q);
     }
   } else {
     unsigned gx = stream_grid(max_len, (size_t)kThreads * 4, 8);
