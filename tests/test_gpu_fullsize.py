@@ -191,3 +191,31 @@ def test_allgather_large_slices(al):
     torch.cuda.synchronize()
     for r in range(P):
         assert torch.equal(bufs[r], want), "in place, rank %d" % r
+
+
+@pytest.mark.parametrize("op", ("sum", "prod", "min", "max"))
+@pytest.mark.parametrize("dtype", ("bf16", "f16"))
+def test_every_pair_of_16bit_patterns(al, dtype, op):
+    """One combine step over all 2^32 (inout, in) pairs of 16-bit patterns: NaNs, infinities,
+    subnormals, signed zeros, ties and every rounding case, against the oracle's
+    widen / one fp32 operation / narrow (src/mpi_impl.cpp:61-145)."""
+    import torch
+    rows = 1 << 10
+    n = rows << 16
+    allbits = np.arange(1 << 16, dtype=np.uint32).astype(np.uint16)
+    b_host = np.tile(allbits, rows)
+    b_dev = torch.from_numpy(b_host.view(np.int16)).cuda()
+    a_dev = torch.empty(n, dtype=torch.int16, device="cuda")
+    out = torch.empty(n, dtype=torch.int16, device="cuda")
+    idx = torch.arange(n, dtype=torch.int32, device="cuda") >> 16
+    nan_above = 0x7f80 if dtype == "bf16" else 0x7c00
+    for base in range(0, 1 << 16, rows):
+        a_host = np.repeat(allbits[base:base + rows], 1 << 16)
+        v = idx + base
+        a_dev.copy_(torch.where(v >= (1 << 15), v - (1 << 16), v).to(torch.int16))
+        al.combine([out], [a_dev, b_dev], op, order="rank_asc", dtype=dtype)
+        want = torch.from_numpy(oracle.step(a_host, b_host, dtype, op).view(np.int16)).cuda()
+        both_nan = ((out & 0x7fff) > nan_above) & ((want & 0x7fff) > nan_above)
+        if not bool(((out == want) | both_nan).all()):
+            assert_bits_equal(out.cpu().numpy().view(np.uint16), want.cpu().numpy().view(np.uint16), dtype,
+                              "%s %s, inout patterns from %#x" % (dtype, op, base))
