@@ -219,3 +219,49 @@ def test_every_pair_of_16bit_patterns(al, dtype, op):
         if not bool(((out == want) | both_nan).all()):
             assert_bits_equal(out.cpu().numpy().view(np.uint16), want.cpu().numpy().view(np.uint16), dtype,
                               "%s %s, inout patterns from %#x" % (dtype, op, base))
+
+
+@pytest.mark.parametrize("dtype,op", [("u16", o) for o in ("sum", "prod", "min", "max", "lor", "land", "lxor", "bor",
+                                                            "band", "bxor")] + [("i16", "min"), ("i16", "max"),
+                                                                                ("i16", "prod")])
+def test_every_pair_of_16bit_integers(al, dtype, op):
+    """All 2^32 operand pairs; sum, prod and the bit/logical operators do not depend on the
+    sign, so the signed type adds only min, max (and prod once more, for the wrap)."""
+    import torch
+    rows = 1 << 10
+    n = rows << 16
+    allbits = np.arange(1 << 16, dtype=np.uint32).astype(np.uint16)
+    npdt = oracle.NP_CARRIER[dtype]
+    b_host = np.tile(allbits, rows).view(npdt)
+    b_dev = torch.from_numpy(b_host.view(np.int16)).cuda()
+    a_dev = torch.empty(n, dtype=torch.int16, device="cuda")
+    out = torch.empty(n, dtype=torch.int16, device="cuda")
+    idx = torch.arange(n, dtype=torch.int32, device="cuda") >> 16
+    for base in range(0, 1 << 16, rows):
+        a_host = np.repeat(allbits[base:base + rows], 1 << 16).view(npdt)
+        v = idx + base
+        a_dev.copy_(torch.where(v >= (1 << 15), v - (1 << 16), v).to(torch.int16))
+        al.combine([out], [a_dev, b_dev], op, order="rank_asc", dtype=dtype)
+        want = torch.from_numpy(oracle.step(a_host, b_host, dtype, op).view(np.int16)).cuda()
+        if not bool((out == want).all()):
+            assert_bits_equal(out.cpu().numpy().view(npdt), want.cpu().numpy().view(npdt), dtype,
+                              "%s %s, first operands from %#x" % (dtype, op, base))
+
+
+@pytest.mark.parametrize("dtype", ("u8", "i8"))
+def test_every_pair_of_bytes_in_every_lane(al, dtype):
+    """All 65536 byte pairs under all ten operators, each pair visiting all 16 byte
+    positions of a 128-bit vector, plus a ragged tail for the element path."""
+    import torch
+    npdt = oracle.NP_CARRIER[dtype]
+    n = 65536 * 16 + 11
+    j = np.arange(n, dtype=np.int64)
+    j = j + j // 65536
+    a = (j % 256).astype(np.uint8).view(npdt)
+    b = ((j // 256) % 256).astype(np.uint8).view(npdt)
+    a_dev, b_dev = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    out = torch.empty(n, dtype=a_dev.dtype, device="cuda")
+    for op in ("sum", "prod", "min", "max", "lor", "land", "lxor", "bor", "band", "bxor"):
+        al.combine([out], [a_dev, b_dev], op, order="rank_asc", dtype=dtype)
+        torch.cuda.synchronize()
+        assert_bits_equal(out.cpu().numpy().view(npdt), oracle.step(a, b, dtype, op), dtype, "%s %s" % (dtype, op))
