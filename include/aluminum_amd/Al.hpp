@@ -506,6 +506,11 @@ class HipCombineBackend {
     comm.world().post(comm, amd::OpKind::reduce_scatter, amd::TypeMap<T>::value, sendbuf, recvbuf, count, op,
                       algo, 0, &req);
   }
+  template <typename T>
+  static void NonblockingReduce_scatter(T *recvbuf, size_t count, ReductionOperator op, comm_type &comm,
+                                        req_type &req, reduce_scatter_algo_type algo) {
+    NonblockingReduce_scatter(static_cast<const T *>(recvbuf), recvbuf, count, op, comm, req, algo);
+  }
 
   /** sendbuf holds sum(counts) elements, recvbuf receives counts[rank]
    *  (include/aluminum/ht/reduce_scatterv.hpp:40-87). */
@@ -519,6 +524,18 @@ class HipCombineBackend {
   static void Reduce_scatterv(T *recvbuf, std::vector<size_t> counts, ReductionOperator op, comm_type &comm,
                               reduce_scatterv_algo_type algo) {
     Reduce_scatterv(static_cast<const T *>(recvbuf), recvbuf, std::move(counts), op, comm, algo);
+  }
+  template <typename T>
+  static void NonblockingReduce_scatterv(const T *sendbuf, T *recvbuf, std::vector<size_t> counts,
+                                         ReductionOperator op, comm_type &comm, req_type &req,
+                                         reduce_scatterv_algo_type algo) {
+    comm.world().post(comm, amd::OpKind::reduce_scatterv, amd::TypeMap<T>::value, sendbuf, recvbuf, 0, op, algo, 0,
+                      &req, &counts);
+  }
+  template <typename T>
+  static void NonblockingReduce_scatterv(T *recvbuf, std::vector<size_t> counts, ReductionOperator op,
+                                         comm_type &comm, req_type &req, reduce_scatterv_algo_type algo) {
+    NonblockingReduce_scatterv(static_cast<const T *>(recvbuf), recvbuf, std::move(counts), op, comm, req, algo);
   }
 
   /** sendbuf holds counts[rank] elements; recvbuf receives every rank's slice at displs[rank]
@@ -536,6 +553,21 @@ class HipCombineBackend {
       AL_AMD_THROW("Vector of counts or displacements is not communicator-sized");
     const T *mine = recvbuf + displs[static_cast<size_t>(comm.rank())];
     Allgatherv(mine, recvbuf, std::move(counts), std::move(displs), comm, algo);
+  }
+  template <typename T>
+  static void NonblockingAllgatherv(const T *sendbuf, T *recvbuf, std::vector<size_t> counts,
+                                    std::vector<size_t> displs, comm_type &comm, req_type &req,
+                                    allgatherv_algo_type algo) {
+    comm.world().post(comm, amd::OpKind::allgatherv, amd::TypeMap<T>::value, sendbuf, recvbuf, 0,
+                      ReductionOperator::sum, algo, 0, &req, &counts, &displs);
+  }
+  template <typename T>
+  static void NonblockingAllgatherv(T *recvbuf, std::vector<size_t> counts, std::vector<size_t> displs,
+                                    comm_type &comm, req_type &req, allgatherv_algo_type algo) {
+    if (displs.size() != static_cast<size_t>(comm.size()))
+      AL_AMD_THROW("Vector of counts or displacements is not communicator-sized");
+    const T *mine = recvbuf + displs[static_cast<size_t>(comm.rank())];
+    NonblockingAllgatherv(mine, recvbuf, std::move(counts), std::move(displs), comm, req, algo);
   }
 
   /** sendbuf holds count elements, recvbuf receives size()*count; in place the
@@ -556,6 +588,12 @@ class HipCombineBackend {
                                    allgather_algo_type algo) {
     comm.world().post(comm, amd::OpKind::allgather, amd::TypeMap<T>::value, sendbuf, recvbuf, count,
                       ReductionOperator::sum, algo, 0, &req);
+  }
+  template <typename T>
+  static void NonblockingAllgather(T *recvbuf, size_t count, comm_type &comm, req_type &req,
+                                   allgather_algo_type algo) {
+    NonblockingAllgather(static_cast<const T *>(recvbuf + static_cast<size_t>(comm.rank()) * count), recvbuf, count,
+                         comm, req, algo);
   }
 };
 
@@ -626,6 +664,13 @@ void NonblockingReduce_scatter(const T *sendbuf, T *recvbuf, size_t count, Reduc
   Backend::template NonblockingReduce_scatter<T>(sendbuf, recvbuf, count, op, comm, req, algo);
 }
 template <typename Backend, typename T>
+void NonblockingReduce_scatter(T *buffer, size_t count, ReductionOperator op, typename Backend::comm_type &comm,
+                               typename Backend::req_type &req,
+                               typename Backend::reduce_scatter_algo_type algo =
+                                   Backend::reduce_scatter_algo_type::automatic) {
+  Backend::template NonblockingReduce_scatter<T>(buffer, count, op, comm, req, algo);
+}
+template <typename Backend, typename T>
 void Allgather(const T *sendbuf, T *recvbuf, size_t count, typename Backend::comm_type &comm,
                typename Backend::allgather_algo_type algo = Backend::allgather_algo_type::automatic) {
   Backend::template Allgather<T>(sendbuf, recvbuf, count, comm, algo);
@@ -640,6 +685,12 @@ void NonblockingAllgather(const T *sendbuf, T *recvbuf, size_t count, typename B
                           typename Backend::req_type &req,
                           typename Backend::allgather_algo_type algo = Backend::allgather_algo_type::automatic) {
   Backend::template NonblockingAllgather<T>(sendbuf, recvbuf, count, comm, req, algo);
+}
+template <typename Backend, typename T>
+void NonblockingAllgather(T *buffer, size_t count, typename Backend::comm_type &comm,
+                          typename Backend::req_type &req,
+                          typename Backend::allgather_algo_type algo = Backend::allgather_algo_type::automatic) {
+  Backend::template NonblockingAllgather<T>(buffer, count, comm, req, algo);
 }
 
 template <typename Backend, typename T>
@@ -657,6 +708,20 @@ void Reduce_scatterv(T *buffer, std::vector<size_t> counts, ReductionOperator op
   Backend::template Reduce_scatterv<T>(buffer, std::move(counts), op, comm, algo);
 }
 template <typename Backend, typename T>
+void NonblockingReduce_scatterv(const T *sendbuf, T *recvbuf, std::vector<size_t> counts, ReductionOperator op,
+                                typename Backend::comm_type &comm, typename Backend::req_type &req,
+                                typename Backend::reduce_scatterv_algo_type algo =
+                                    Backend::reduce_scatterv_algo_type::automatic) {
+  Backend::template NonblockingReduce_scatterv<T>(sendbuf, recvbuf, std::move(counts), op, comm, req, algo);
+}
+template <typename Backend, typename T>
+void NonblockingReduce_scatterv(T *buffer, std::vector<size_t> counts, ReductionOperator op,
+                                typename Backend::comm_type &comm, typename Backend::req_type &req,
+                                typename Backend::reduce_scatterv_algo_type algo =
+                                    Backend::reduce_scatterv_algo_type::automatic) {
+  Backend::template NonblockingReduce_scatterv<T>(buffer, std::move(counts), op, comm, req, algo);
+}
+template <typename Backend, typename T>
 void Allgatherv(const T *sendbuf, T *recvbuf, std::vector<size_t> counts, std::vector<size_t> displs,
                 typename Backend::comm_type &comm,
                 typename Backend::allgatherv_algo_type algo = Backend::allgatherv_algo_type::automatic) {
@@ -667,6 +732,18 @@ void Allgatherv(T *buffer, std::vector<size_t> counts, std::vector<size_t> displ
                 typename Backend::comm_type &comm,
                 typename Backend::allgatherv_algo_type algo = Backend::allgatherv_algo_type::automatic) {
   Backend::template Allgatherv<T>(buffer, std::move(counts), std::move(displs), comm, algo);
+}
+template <typename Backend, typename T>
+void NonblockingAllgatherv(const T *sendbuf, T *recvbuf, std::vector<size_t> counts, std::vector<size_t> displs,
+                           typename Backend::comm_type &comm, typename Backend::req_type &req,
+                           typename Backend::allgatherv_algo_type algo = Backend::allgatherv_algo_type::automatic) {
+  Backend::template NonblockingAllgatherv<T>(sendbuf, recvbuf, std::move(counts), std::move(displs), comm, req, algo);
+}
+template <typename Backend, typename T>
+void NonblockingAllgatherv(T *buffer, std::vector<size_t> counts, std::vector<size_t> displs,
+                           typename Backend::comm_type &comm, typename Backend::req_type &req,
+                           typename Backend::allgatherv_algo_type algo = Backend::allgatherv_algo_type::automatic) {
+  Backend::template NonblockingAllgatherv<T>(buffer, std::move(counts), std::move(displs), comm, req, algo);
 }
 
 /** Host-only completion test; resets the request when complete

@@ -57,3 +57,45 @@ def test_benchmark_sweep_rows():
     bad = subprocess.run([exe, "--op", "allreduce", "--reduction-op", "avg", "--max-size", "4"], capture_output=True,
                          text=True, timeout=60)
     assert bad.returncode == 1 and "Reduction operator not supported" in bad.stderr
+
+
+OPS_EXE = os.path.join(ROOT, "tests", "cpp", "test_ops")
+
+# (arguments) in the manner of the reference's sweep (test/run_tests.py): collective x datatype x
+# in place x non-blocking over power-of-two and odd sizes
+OPS_SWEEPS = [
+    "--op allreduce --datatype float --odd-sizes --max-size 262144 --ranks 4",
+    "--op allreduce --datatype bfloat16 --inplace --nonblocking --odd-sizes --max-size 65536 --ranks 8",
+    "--op allreduce --datatype half --reduction-op max --algorithm rank_order --odd-sizes --max-size 65536 --ranks 3",
+    "--op allreduce --datatype uchar --reduction-op lxor --inplace --odd-sizes --max-size 65536 --ranks 5",
+    "--op allreduce --datatype longlong --reduction-op band --nonblocking --max-size 65536 --ranks 8",
+    "--op allreduce --datatype double --reduction-op prod --algorithm ring --min-size 0 --max-size 32768 --ranks 8",
+    "--op reduce --datatype float --root 2 --inplace --odd-sizes --max-size 65536 --ranks 4",
+    "--op reduce --datatype int --reduction-op min --root 0 --nonblocking --max-size 65536 --ranks 7",
+    "--op reduce_scatter --datatype float --inplace --nonblocking --odd-sizes --max-size 65536 --ranks 8",
+    "--op reduce_scatter --datatype ushort --reduction-op bor --algorithm pairwise --max-size 16384 --ranks 5",
+    "--op allgather --datatype short --inplace --nonblocking --odd-sizes --max-size 65536 --ranks 8",
+    "--op reduce_scatterv --datatype double --nonblocking --odd-sizes --max-size 16384 --ranks 5",
+    "--op allgatherv --datatype char --inplace --nonblocking --odd-sizes --max-size 16384 --ranks 8",
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("args", OPS_SWEEPS)
+def test_ops_sweep(args):
+    assert os.path.exists(OPS_EXE), "tests/cpp/test_ops is not built (make -C tests/cpp)"
+    p = subprocess.run([OPS_EXE] + args.split(), capture_output=True, text=True, timeout=280)
+    print(p.stdout[-3000:])
+    print(p.stderr[-2000:])
+    assert p.returncode == 0, p.stdout[-3000:]
+    assert "PASSED" in p.stdout
+
+
+def test_ops_rejects_bad_arguments():
+    """Argument errors are reported before any GPU call."""
+    if not os.path.exists(OPS_EXE):
+        pytest.skip("tests/cpp/test_ops is not built")
+    for args in ("--op alltoall", "--op allreduce --backend nccl", "--op allreduce --reduction-op median",
+                 "--op allreduce --ranks 4 --root 9", "--op allreduce --bogus"):
+        p = subprocess.run([OPS_EXE] + args.split(), capture_output=True, text=True, timeout=60)
+        assert p.returncode == 2, (args, p.stdout, p.stderr)
