@@ -153,14 +153,61 @@ class Communicator {
   friend struct Poster;
 };
 
-/** Completion handle of a non-blocking operation
- *  (internal::ht::HostTransferRequest, include/aluminum/ht_impl.hpp:882-888). */
-struct Request {
-  hipEvent_t op_event = nullptr;
-  hipStream_t orig_stream = nullptr;
-  ~Request() {
-    if (op_event) (void)hipEventDestroy(op_event);
+/** Timing-less events, reused: creating one costs more than recording it. */
+class EventPool {
+ public:
+  ~EventPool() {
+    for (hipEvent_t e : free_) (void)hipEventDestroy(e);
   }
+  hipEvent_t take() {
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      if (!free_.empty()) {
+        hipEvent_t e = free_.back();
+        free_.pop_back();
+        return e;
+      }
+    }
+    hipEvent_t e = nullptr;
+    AL_AMD_CHECK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    return e;
+  }
+  void give(hipEvent_t e) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    free_.push_back(e);
+  }
+
+ private:
+  std::mutex mutex_;
+  std::vector<hipEvent_t> free_;
+};
+
+/** Completion of one launched non-blocking operation: one event, shared by
+ *  the requests of all P logical ranks. */
+struct OpCompletion {
+  std::shared_ptr<EventPool> pool;
+  hipEvent_t event = nullptr;
+  std::mutex mutex;
+  std::vector<hipStream_t> waited;  // streams already made to wait for this operation
+  ~OpCompletion() {
+    if (event) pool->give(event);
+  }
+  /** True the first time `s` asks: later waits of the same stream add nothing. */
+  bool first_wait(hipStream_t s) {
+    std::lock_guard<std::mutex> lock(mutex);
+    for (hipStream_t w : waited)
+      if (w == s) return false;
+    waited.push_back(s);
+    return true;
+  }
+};
+
+/** Completion handle of a non-blocking operation
+ *  (internal::ht::HostTransferRequest, include/aluminum/ht_impl.hpp:882-888).
+ *  `done` is empty until the last logical rank has made its call. */
+struct Request {
+  std::shared_ptr<OpCompletion> done;
+  hipStream_t orig_stream = nullptr;
 };
 
 enum class OpKind { allreduce, reduce, reduce_scatter, allgather, reduce_scatterv, allgatherv };
@@ -202,6 +249,7 @@ class World {
     // default priority on purpose: the internal stream only has to be a different stream
     AL_AMD_CHECK_HIP(hipStreamCreateWithFlags(&internal_stream_, hipStreamNonBlocking));
     AL_AMD_CHECK_HIP(hipEventCreateWithFlags(&sync_event_, hipEventDisableTiming));
+    events_ = std::make_shared<EventPool>();
   }
   ~World() {
     (void)hipStreamSynchronize(internal_stream_);
@@ -230,6 +278,7 @@ class World {
   std::mutex mutex_;
   hipStream_t internal_stream_ = nullptr;
   hipEvent_t sync_event_ = nullptr;
+  std::shared_ptr<EventPool> events_;
 };
 
 struct Poster {
@@ -290,9 +339,12 @@ inline void World::post(Communicator &c, OpKind kind, int dtype, const void *sen
 
 /** Makes `target` wait for the prior work of every rank's stream; returns it. */
 inline hipStream_t World::gather_streams(PendingOp &p, hipStream_t target) {
-  for (auto &r : p.ranks) {
-    if (r.stream == target) continue;
-    AL_AMD_CHECK_HIP(hipEventRecord(sync_event_, r.stream));
+  for (size_t i = 0; i < p.ranks.size(); ++i) {
+    const hipStream_t s = p.ranks[i].stream;
+    bool seen = s == target;
+    for (size_t k = 0; k < i && !seen; ++k) seen = p.ranks[k].stream == s;
+    if (seen) continue;  // logical ranks often share a stream: one dependency per distinct stream
+    AL_AMD_CHECK_HIP(hipEventRecord(sync_event_, s));
     AL_AMD_CHECK_HIP(hipStreamWaitEvent(target, sync_event_, 0));
   }
   return target;
@@ -302,22 +354,24 @@ inline hipStream_t World::gather_streams(PendingOp &p, hipStream_t target) {
  *  hands out completion events (non-blocking ops). */
 inline void World::release_streams(PendingOp &p, hipStream_t ran_on) {
   if (p.nonblocking) {
-    for (auto &r : p.ranks) {
-      hipEvent_t ev = nullptr;
-      AL_AMD_CHECK_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
-      AL_AMD_CHECK_HIP(hipEventRecord(ev, ran_on));
-      r.req->op_event = ev;
-    }
+    auto done = std::make_shared<OpCompletion>();
+    done->pool = events_;
+    done->event = events_->take();
+    AL_AMD_CHECK_HIP(hipEventRecord(done->event, ran_on));
+    for (auto &r : p.ranks) r.req->done = done;
     return;
   }
   bool recorded = false;
-  for (auto &r : p.ranks) {
-    if (r.stream == ran_on) continue;
+  for (size_t i = 0; i < p.ranks.size(); ++i) {
+    const hipStream_t s = p.ranks[i].stream;
+    bool seen = s == ran_on;
+    for (size_t k = 0; k < i && !seen; ++k) seen = p.ranks[k].stream == s;
+    if (seen) continue;
     if (!recorded) {
       AL_AMD_CHECK_HIP(hipEventRecord(sync_event_, ran_on));
       recorded = true;
     }
-    AL_AMD_CHECK_HIP(hipStreamWaitEvent(r.stream, sync_event_, 0));
+    AL_AMD_CHECK_HIP(hipStreamWaitEvent(s, sync_event_, 0));
   }
 }
 
@@ -751,8 +805,8 @@ void NonblockingAllgatherv(T *buffer, std::vector<size_t> counts, std::vector<si
 template <typename Backend> bool Test(typename Backend::req_type &req);
 template <> inline bool Test<HipCombineBackend>(HipCombineBackend::req_type &req) {
   if (req == HipCombineBackend::null_req) return true;
-  if (!req->op_event) return false;  // not launched yet: some logical rank has not made its call
-  const hipError_t e = hipEventQuery(req->op_event);
+  if (!req->done) return false;  // not launched yet: some logical rank has not made its call
+  const hipError_t e = hipEventQuery(req->done->event);
   if (e == hipSuccess) {
     req = HipCombineBackend::null_req;
     return true;
@@ -766,8 +820,9 @@ template <> inline bool Test<HipCombineBackend>(HipCombineBackend::req_type &req
 template <typename Backend> void Wait(typename Backend::req_type &req);
 template <> inline void Wait<HipCombineBackend>(HipCombineBackend::req_type &req) {
   if (req == HipCombineBackend::null_req) return;
-  if (!req->op_event) AL_AMD_THROW("Wait on an operation that not every logical rank has started");
-  AL_AMD_CHECK_HIP(hipStreamWaitEvent(req->orig_stream, req->op_event, 0));
+  if (!req->done) AL_AMD_THROW("Wait on an operation that not every logical rank has started");
+  if (req->done->first_wait(req->orig_stream))
+    AL_AMD_CHECK_HIP(hipStreamWaitEvent(req->orig_stream, req->done->event, 0));
   req = HipCombineBackend::null_req;
 }
 

@@ -70,13 +70,16 @@ template <typename T> int run(const Options &o, Al::ReductionOperator rop, Algo 
           if (o.nonblocking) { if (o.inplace) Al::NonblockingAllreduce<Backend>(buf, size, rop, comm, reqs[r], algo); else Al::NonblockingAllreduce<Backend>(send, recv, size, rop, comm, reqs[r], algo); }
           else { if (o.inplace) Al::Allreduce<Backend>(buf, size, rop, comm, algo); else Al::Allreduce<Backend>(send, recv, size, rop, comm, algo); }
         } else if (o.op == "reduce") {
-          if (o.inplace) Al::Reduce<Backend>(buf, size, rop, o.root, comm, algo); else Al::Reduce<Backend>(send, recv, size, rop, o.root, comm, algo);
+          if (o.nonblocking) { if (o.inplace) Al::NonblockingReduce<Backend>(buf, size, rop, o.root, comm, reqs[r], algo); else Al::NonblockingReduce<Backend>(send, recv, size, rop, o.root, comm, reqs[r], algo); }
+          else { if (o.inplace) Al::Reduce<Backend>(buf, size, rop, o.root, comm, algo); else Al::Reduce<Backend>(send, recv, size, rop, o.root, comm, algo); }
         } else if (o.op == "reduce_scatter") {
-          if (o.nonblocking && !o.inplace) Al::NonblockingReduce_scatter<Backend>(send, recv, size, rop, comm, reqs[r], algo);
+          if (o.nonblocking && o.inplace) Al::NonblockingReduce_scatter<Backend>(buf, size, rop, comm, reqs[r], algo);
+          else if (o.nonblocking) Al::NonblockingReduce_scatter<Backend>(send, recv, size, rop, comm, reqs[r], algo);
           else if (o.inplace) Al::Reduce_scatter<Backend>(buf, size, rop, comm, algo);
           else Al::Reduce_scatter<Backend>(send, recv, size, rop, comm, algo);
         } else {
-          if (o.nonblocking && !o.inplace) Al::NonblockingAllgather<Backend>(send, recv, size, comm, reqs[r], algo);
+          if (o.nonblocking && o.inplace) Al::NonblockingAllgather<Backend>(recv, size, comm, reqs[r], algo);
+          else if (o.nonblocking) Al::NonblockingAllgather<Backend>(send, recv, size, comm, reqs[r], algo);
           else if (o.inplace) Al::Allgather<Backend>(recv, size, comm, algo);
           else Al::Allgather<Backend>(send, recv, size, comm, algo);
         }
