@@ -17,6 +17,11 @@ namespace alamd {
 
 constexpr int kAuxLoadStream = 2;    // nt
 constexpr int kAuxStoreStream = 17;  // sc0 | sc1
+// Write-dominated kernels (one source to several destinations): the source is
+// read again for every destination, so its loads stay cacheable; the stores
+// are non-temporal and written through.
+constexpr int kAuxLoadCached = 0;
+constexpr int kAuxStoreNt = 19;      // sc0 | sc1 | nt
 constexpr unsigned kRsrcFlags = 0x00020000u;
 
 // Workgroups are handed to the eight XCDs round-robin and each XCD then works
@@ -42,6 +47,12 @@ template <int U, int THREADS> struct Tile {
   }
   __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t r, int u, u32x4 v) const {
     __builtin_amdgcn_raw_buffer_store_b128(v, r, vo + (unsigned)u * 1024u, 0, kAuxStoreStream);
+  }
+  __device__ __forceinline__ u32x4 load_cached(__amdgpu_buffer_rsrc_t r, int u) const {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, vo + (unsigned)u * 1024u, 0, kAuxLoadCached);
+  }
+  __device__ __forceinline__ void store_nt(__amdgpu_buffer_rsrc_t r, int u, u32x4 v) const {
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, vo + (unsigned)u * 1024u, 0, kAuxStoreNt);
   }
 };
 

@@ -162,6 +162,39 @@ __global__ void __launch_bounds__(256) bcast_kernel_bytes(const char *src, FoldP
   }
 }
 
+// One source region to p.P destinations, one workgroup per (destination, tile).
+// Block ids run chunk by chunk (tpc tiles, 8 MiB); inside a chunk all tiles of
+// destination 0 come first, then destination 1, ...: at any time the device
+// writes one contiguous stream per chunk instead of P interleaved ones, and
+// re-reads the chunk of the source from cache.  Measured for 1 read + 8 writes
+// of 32 MiB: 88 % of the HBM peak, against 67 % when every workgroup writes
+// its tile to all destinations (69 % for those writes alone).
+constexpr unsigned kSpreadChunkTiles = 512;
+__global__ void __launch_bounds__(kGatherThreads) spread_kernel_vec(const char *src, FoldParams p, size_t vec_bytes,
+                                                                    size_t tail_bytes, unsigned tpc, unsigned tiles) {
+  using TL = Tile<kGatherU, kGatherThreads>;
+  const TL tl;
+  const unsigned ndest = (unsigned)p.P;
+  const unsigned per_chunk = tpc * ndest;
+  const unsigned chunk = blockIdx.x / per_chunk, rem = blockIdx.x % per_chunk;
+  const unsigned dest = rem / tpc, tile = chunk * tpc + rem % tpc;
+  if (tile < tiles) {
+    const size_t tb = (size_t)tile * TL::BYTES;
+    const int nrec = vec_bytes - tb > TL::BYTES ? (int)TL::BYTES : (int)(vec_bytes - tb);
+    const auto rs = TL::rsrc(src + tb, nrec);
+    const auto rd = TL::rsrc(p.out[dest] + tb, nrec);
+    u32x4 v[kGatherU];
+#pragma unroll
+    for (int u = 0; u < kGatherU; ++u) v[u] = tl.load_cached(rs, u);
+#pragma unroll
+    for (int u = 0; u < kGatherU; ++u) tl.store_nt(rd, u, v[u]);
+  }
+  if (blockIdx.x == 0 && threadIdx.x < tail_bytes) {
+    const char c = src[vec_bytes + threadIdx.x];
+    for (unsigned r = 0; r < ndest; ++r) p.out[r][vec_bytes + threadIdx.x] = c;
+  }
+}
+
 int check_common(int P, size_t count, int dtype) {
   if (P < 1 || P > ALAMD_MAX_RANKS)
     return set_error(ALAMD_ERR_INVALID_ARG, "number of ranks %d outside [1, %d]", P, ALAMD_MAX_RANKS);
@@ -171,6 +204,27 @@ int check_common(int P, size_t count, int dtype) {
 }
 
 }  // namespace
+
+int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, hipStream_t stream) {
+  if (ndest <= 0 || bytes == 0) return ALAMD_OK;
+  FoldParams fp;
+  for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
+    fp.in[r] = nullptr;
+    fp.out[r] = r < ndest ? dests[r] : nullptr;
+  }
+  fp.P = ndest;
+  const size_t vec_bytes = bytes & ~(size_t)15, tile = Tile<kGatherU, kGatherThreads>::BYTES;
+  size_t tiles = (vec_bytes + tile - 1) / tile;
+  if (tiles == 0) tiles = 1;
+  const size_t tpc = tiles < kSpreadChunkTiles ? tiles : kSpreadChunkTiles;
+  const size_t chunks = (tiles + tpc - 1) / tpc;
+  const size_t blocks = chunks * tpc * (size_t)ndest;
+  if (blocks > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
+  hipLaunchKernelGGL(spread_kernel_vec, dim3((unsigned)blocks), dim3(kGatherThreads), 0, stream, src, fp, vec_bytes,
+                     bytes - vec_bytes, (unsigned)tpc, (unsigned)tiles);
+  ALAMD_HIP(hipGetLastError());
+  return ALAMD_OK;
+}
 
 }  // namespace alamd
 
@@ -220,7 +274,31 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   lay.max_len = count;
   lay.start0 = start;
   lay.start_stride = 0;
-  return launch_order(out_tab, ins, P, lay, dtype, op, order, vector, as_stream(stream));
+  if (nout == 1 || !vector || bytes < kSpreadMinBytes)
+    return launch_order(out_tab, ins, P, lay, dtype, op, order, vector, as_stream(stream));
+  // Several outputs of a large result: a workgroup that wrote its tile to every
+  // output would interleave nout write streams (measured 69 % of peak).  Instead
+  // the result goes to outs[0] and is then spread, 64 MiB at a time so that the
+  // spread reads what the fold has just written while it is still in cache.
+  // In place (outs[j] == ins[j]) this is safe: a piece of an input is
+  // overwritten only after the fold of that piece has been launched before it
+  // on the same stream.
+  const size_t piece = kMaxTilesPerLaunch * (size_t)16384 / es;  // elements; a multiple of every tile size
+  lay.seg.nout = 1;
+  const void *in_tab[ALAMD_MAX_RANKS];
+  for (size_t e0 = 0; e0 < count; e0 += piece) {
+    const size_t len = count - e0 < piece ? count - e0 : piece;
+    for (int r = 0; r < P; ++r) in_tab[r] = static_cast<const char *>(ins[r]) + e0 * es;
+    void *first[ALAMD_MAX_RANKS] = {nullptr};
+    first[0] = static_cast<char *>(outs[0]) + e0 * es;
+    lay.seg.seg_base = len;
+    lay.max_len = len;
+    if ((rc = launch_order(first, in_tab, P, lay, dtype, op, order, vector, as_stream(stream)))) return rc;
+    char *dests[ALAMD_MAX_RANKS];
+    for (int j = 1; j < nout; ++j) dests[j - 1] = static_cast<char *>(outs[j]) + e0 * es;
+    if ((rc = launch_spread(static_cast<char *>(first[0]), dests, nout - 1, len * es, as_stream(stream)))) return rc;
+  }
+  return ALAMD_OK;
 }
 
 int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, size_t count, int dtype,
@@ -309,18 +387,18 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
   }
   fp.P = P;
   hipStream_t st = as_stream(stream);
-  if (vector && blk >= ((size_t)1 << 20)) {
-    // large slices: one launch per source keeps the writes of a launch within P
-    // destination regions (measured a few per cent faster than one grid over all sources)
-    const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
-    const size_t tiles = (blk + tile - 1) / tile;
-    if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
+  if (vector && blk >= kSpreadMinBytes) {
+    // large slices: one launch per source, one destination stream at a time
     for (int q = 0; q < P; ++q) {
-      FoldParams fq = fp;
-      for (int r = 0; r < P; ++r) fq.out[r] = fp.out[r] + (size_t)q * blk;
-      hipLaunchKernelGGL(bcast_kernel_vec, dim3((unsigned)tiles), dim3(kGatherThreads), 0, st, fp.in[q], fq, blk,
-                         (size_t)0);
+      char *dests[ALAMD_MAX_RANKS];
+      int nd = 0;
+      for (int r = 0; r < P; ++r) {
+        char *slot = fp.out[r] + (size_t)q * blk;
+        if (slot != fp.in[q]) dests[nd++] = slot;  // in place: rank q's own slice is already there
+      }
+      if ((rc = launch_spread(fp.in[q], dests, nd, blk, st))) return rc;
     }
+    return ALAMD_OK;
   } else if (vector) {
     const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
     const size_t tiles = (blk + tile - 1) / tile;
@@ -455,7 +533,13 @@ int alamd_allgatherv(void *const *recvs, const void *const *sends, int P, const 
       vector = vector && aligned16(fp.out[r]);
     }
     fp.P = P;
-    if (vector) {
+    if (vector && bytes >= kSpreadMinBytes) {
+      char *dests[ALAMD_MAX_RANKS];
+      int nd = 0;
+      for (int r = 0; r < P; ++r)
+        if (fp.out[r] != src) dests[nd++] = fp.out[r];
+      if ((rc = launch_spread(src, dests, nd, bytes, st))) return rc;
+    } else if (vector) {
       const size_t vec_bytes = bytes & ~(size_t)15, tile = Tile<kGatherU, kGatherThreads>::BYTES;
       const size_t tiles = (vec_bytes + tile - 1) / tile;
       if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");

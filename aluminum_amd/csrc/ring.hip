@@ -219,7 +219,35 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   fp.dir = 1;
   const size_t max_len = fp.seg.seg_base + (fp.seg.seg_rem ? 1 : 0);
   if (max_len == 0) return ALAMD_OK;
-  return launch_fold(fp, (unsigned)P, max_len, dtype, op, true, vector, stream);
+  const size_t es = alamd_dtype_size(dtype);
+  if (!all || !vector || fp.seg.seg_base * es < kSpreadMinBytes)
+    return launch_fold(fp, (unsigned)P, max_len, dtype, op, true, vector, stream);
+  // Large allreduce: segment by segment, fold into the owner's buffer (what the
+  // reduce-scatter leaves there), then spread the segment from the owner to the
+  // other ranks while it is still in cache.  Writing each result tile to all P
+  // buffers from one workgroup interleaves P write streams and is slower.
+  // `vector` implies count % P == 0, so every segment has seg_base elements.
+  const size_t seg_bytes = fp.seg.seg_base * es;
+  FoldParams fs = fp;
+  fs.seg.seg_rem = 0;
+  fs.seg.in_blocked = 0;
+  fs.seg.out_mode = OUT_ALL;
+  fs.seg.nout = 1;
+  fs.start_stride = 0;
+  for (int s = 0; s < P; ++s) {
+    const int owner = (s + P - 1) % P;
+    for (int r = 0; r < P; ++r) fs.in[r] = static_cast<const char *>(bufs[r]) + (size_t)s * seg_bytes;
+    fs.out[0] = static_cast<char *>(bufs[owner]) + (size_t)s * seg_bytes;
+    fs.start0 = s;
+    int rc = launch_fold(fs, 1, fp.seg.seg_base, dtype, op, true, vector, stream);
+    if (rc) return rc;
+    char *dests[ALAMD_MAX_RANKS];
+    int nd = 0;
+    for (int r = 0; r < P; ++r)
+      if (r != owner) dests[nd++] = static_cast<char *>(bufs[r]) + (size_t)s * seg_bytes;
+    if ((rc = launch_spread(fs.out[0], dests, nd, seg_bytes, stream))) return rc;
+  }
+  return ALAMD_OK;
 }
 
 }  // namespace

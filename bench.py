@@ -46,7 +46,7 @@ P = 8
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
 # the same counter's reading for the 1 GiB copy kernel (profiles/fold_vec_kernel_f32_sum_P8_c2.md).
-MEASURED_TRAFFIC = {"c2_f32_sum": 2416197755}
+MEASURED_TRAFFIC = {"c2_f32_sum": 2416198395}
 KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false, 8>"}
 
 
@@ -147,7 +147,7 @@ def run_ring_workload(al, torch, mode, steps, warmup):
     # P-1 allgather steps reads one and writes one; fused: every buffer is read once and written once
     alg = 5 * (P - 1) * count * es if mode == "stepwise" else 2 * P * count * es
     return {"workload": "c3_ring_" + mode, "dtype": dtype, "op": "sum", "P": P, "count": count,
-            "chunk_bytes": chunk, "launches_per_step": 2 * (P - 1) if mode == "stepwise" else 1,
+            "chunk_bytes": chunk, "launches_per_step": 2 * (P - 1) if mode == "stepwise" else 2 * P,
             "algorithmic_bytes": alg, "ms_per_step": wall * 1e3, "kernel_ms": kms,
             "gbps_wall": alg / wall * 1e-9, "gbps_kernel": alg / (kms * 1e-3) * 1e-9,
             "parity_vs_oracle": bool(ok)}

@@ -193,6 +193,68 @@ def test_allgather_large_slices(al):
         assert torch.equal(bufs[r], want), "in place, rank %d" % r
 
 
+@pytest.mark.parametrize("order", ("rank_asc", "tree_dbl"))
+@pytest.mark.parametrize("inplace", (False, True))
+def test_large_combine_to_several_outputs(al, order, inplace):
+    """Above 1 MiB a result for several outputs is folded into the first and then spread,
+    64 MiB at a time: counts around that piece size, three ranks, separate and in-place outputs."""
+    import torch
+    P = 3
+    piece = (64 << 20) // 4
+    for n in (300000, piece - 4, piece + 4, piece + (1 << 20) + 12):
+        ins = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(P)]
+        for r in range(P):
+            al.fill(ins[r], "uniform_pm1", 500 + r)
+        outs = ins if inplace else [torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(P)]
+        al.combine(outs, ins, "sum", order=order)
+        torch.cuda.synchronize()
+        want = oracle.combine_generated(P, n, "f32", "sum", order, 0, "uniform_pm1", 500)
+        for j in range(P):
+            assert_bits_equal(outs[j].cpu().numpy(), want, "f32", "n=%d output %d" % (n, j))
+
+
+def test_allgatherv_large_slices_with_tails(al):
+    """Slices above 1 MiB whose byte counts are not multiples of 16, placed back to front."""
+    import torch
+    P = 4
+    counts = [300001, 0, 262147, 500003]
+    # slots 16-byte aligned, with gaps, laid out from the last rank to the first
+    displs, at = [0] * P, 4
+    for q in reversed(range(P)):
+        displs[q] = at
+        at += (counts[q] + 3) // 4 * 4 + 8
+    extent = max(d + c for d, c in zip(displs, counts))
+    sends = [torch.empty(max(c, 1), dtype=torch.float32, device="cuda") for c in counts]
+    for r in range(P):
+        al.fill(sends[r], "uniform_pm1", 700 + r)
+    recvs = [torch.full((extent,), -3.0, dtype=torch.float32, device="cuda") for _ in range(P)]
+    al.allgatherv(recvs, sends, counts, displs)
+    torch.cuda.synchronize()
+    want = np.full(extent, -3.0, dtype=np.float32)
+    for q in range(P):
+        want[displs[q]:displs[q] + counts[q]] = oracle.fill(max(counts[q], 1), "f32", "uniform_pm1", 700 + q)[:counts[q]]
+    for r in range(P):
+        assert recvs[r].cpu().numpy().tobytes() == want.tobytes(), "rank %d" % r
+
+
+@pytest.mark.parametrize("P,count", [(3, 3 * 300000), (8, 8 * 262144 + 8 * 4)])
+def test_fused_ring_large_segments(al, P, count):
+    """Segments above 1 MiB: fold into the owner, then spread; same bits as the stepwise ring."""
+    import torch
+    bufs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+    for r in range(P):
+        al.fill(bufs[r], "uniform_pm1", 800 + r)
+    step = [b.clone() for b in bufs]
+    al.ring_allreduce(bufs, "sum", mode="fused")
+    al.ring_allreduce(step, "sum", mode="stepwise")
+    torch.cuda.synchronize()
+    host = [oracle.fill(count, "f32", "uniform_pm1", 800 + r) for r in range(P)]
+    want = oracle.ring_allreduce(host, "f32", "sum", (4 << 20) // 4)[0]
+    for r in range(P):
+        assert_bits_equal(bufs[r].cpu().numpy(), want, "f32", "fused rank %d" % r)
+        assert torch.equal(step[r], bufs[r])
+
+
 @pytest.mark.parametrize("op", ("sum", "prod", "min", "max"))
 @pytest.mark.parametrize("dtype", ("bf16", "f16"))
 def test_every_pair_of_16bit_patterns(al, dtype, op):
