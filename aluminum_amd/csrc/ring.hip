@@ -4,7 +4,8 @@
 // (blockIdx.y) folds the segment it "receives" from rank r-1 into its own
 // copy; in allgather step t it copies the segment.  A segment is worked
 // through chunk by chunk: a chunk is owned by a fixed group of workgroups.
-// FUSED: the fold kernels walk each segment once in ring order.
+// FUSED: the fold kernels walk each segment once in ring order; an allreduce
+// then spreads every folded segment from its owner to the other ranks.
 #include "alamd_dispatch.h"
 #include "alamd_tile.h"
 

@@ -167,8 +167,8 @@ int alamd_allgatherv(void *const *recvs, const void *const *sends, int P,
 typedef enum {
   /* one launch per ring step; every byte a real ring moves is moved */
   ALAMD_RING_STEPWISE = 0,
-  /* one launch; each segment is folded in registers in ring order and
-   * written once to every rank (same bits, fewer bytes) */
+  /* each segment is folded in registers in ring order, written once and
+   * (allreduce) copied once to every other rank: same bits, fewer bytes */
   ALAMD_RING_FUSED = 1
 } alamd_ring_mode;
 

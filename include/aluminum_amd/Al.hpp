@@ -119,7 +119,7 @@ enum class CombineAlgorithm {
   tree_binomial,
   pairwise,       /**< x_r . x_{r-1} . x_{r-2} ... for the block of rank r */
   ring,           /**< ring reduce-scatter + allgather, one launch per ring step */
-  ring_fused      /**< the same values from one fused launch */
+  ring_fused      /**< the same values with every segment folded in one pass */
 };
 
 /** Chunk of the ring pipeline: 4 MiB, a multiple of every element size. */
