@@ -34,6 +34,7 @@
 #include <mutex>
 #include <sstream>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "aluminum_amd.h"
@@ -68,6 +69,23 @@ class al_exception : public std::exception {
 
 /** Predefined reduction operations (include/aluminum/base.hpp:103-105). */
 enum class ReductionOperator { sum, prod, min, max, lor, land, lxor, bor, band, bxor, avg };
+
+namespace amd {
+inline bool &initialized_flag() {
+  static bool flag = false;
+  return flag;
+}
+}  // namespace amd
+
+/** Start-up as in the reference (include/Al.hpp:73-104); there is no MPI to
+ *  initialise, so the arguments are unused.  Checks that the current device is a
+ *  gfx950.  May be called more than once. */
+inline void Initialize(int & /*argc*/, char **& /*argv*/) {
+  AL_AMD_CHECK(alamd_init());
+  amd::initialized_flag() = true;
+}
+inline void Finalize() { amd::initialized_flag() = false; }
+inline bool Initialized() { return amd::initialized_flag(); }
 
 namespace amd {
 
@@ -649,6 +667,45 @@ class HipCombineBackend {
     NonblockingAllgather(static_cast<const T *>(recvbuf + static_cast<size_t>(comm.rank()) * count), recvbuf, count,
                          comm, req, algo);
   }
+};
+
+/* ---- compile-time traits (include/aluminum/traits/traits_base.hpp:43-62, 86-92, 155-184;
+ *      the host-transfer backend's answers: traits/ht_traits.hpp:41-105) ------ */
+
+enum class AlOperation {
+  allgather, allgatherv, allreduce, alltoall, alltoallv, barrier, bcast, gather, gatherv, reduce,
+  reduce_scatter, reduce_scatterv, scatter, scatterv, send, recv, sendrecv, multisendrecv
+};
+
+template <typename Backend> constexpr char AlBackendName[] = "unknown";
+template <> inline constexpr char AlBackendName<HipCombineBackend>[] = "hip";
+
+namespace amd {
+/** The collectives this engine implements: the ones that combine or lay out rank contributions. */
+constexpr bool implements(AlOperation op) {
+  return op == AlOperation::allreduce || op == AlOperation::reduce || op == AlOperation::reduce_scatter ||
+         op == AlOperation::reduce_scatterv || op == AlOperation::allgather || op == AlOperation::allgatherv;
+}
+template <typename T, typename = void> struct HasTypeMap : std::false_type {};
+template <typename T> struct HasTypeMap<T, decltype(void(TypeMap<T>::value))> : std::true_type {};
+}  // namespace amd
+
+template <AlOperation Op, typename Backend> struct IsOpSupported : std::false_type {};
+template <AlOperation Op>
+struct IsOpSupported<Op, HipCombineBackend> : std::integral_constant<bool, amd::implements(Op)> {};
+
+template <typename Backend, typename T> struct IsTypeSupported : std::false_type {};
+template <typename T> struct IsTypeSupported<HipCombineBackend, T> : amd::HasTypeMap<T> {};
+
+/** Every operator but avg, like the MPI and host-transfer backends (mpi/utils.hpp:192-194). */
+template <typename Backend, ReductionOperator op> struct IsReductionOpSupported : std::false_type {};
+template <ReductionOperator op>
+struct IsReductionOpSupported<HipCombineBackend, op> : std::integral_constant<bool, op != ReductionOperator::avg> {};
+
+template <AlOperation Op, typename Backend, typename = void> struct OpAlgoType {};
+template <AlOperation Op>
+struct OpAlgoType<Op, HipCombineBackend, typename std::enable_if<amd::implements(Op)>::type> {
+  using type = amd::CombineAlgorithm;
 };
 
 /* ---- the public API templates (include/Al.hpp) ---------------------------- */

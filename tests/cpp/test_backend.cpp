@@ -7,6 +7,17 @@
 // Runs on one GPU; every logical rank of the World lives in its memory.
 #include "parity_harness.hpp"
 
+// compile-time traits of the backend
+static_assert(Al::IsOpSupported<Al::AlOperation::allreduce, Backend>::value, "allreduce");
+static_assert(Al::IsOpSupported<Al::AlOperation::reduce_scatterv, Backend>::value, "reduce_scatterv");
+static_assert(!Al::IsOpSupported<Al::AlOperation::alltoall, Backend>::value, "alltoall is not on the path");
+static_assert(Al::IsTypeSupported<Backend, float>::value && Al::IsTypeSupported<Backend, unsigned long long>::value &&
+                  Al::IsTypeSupported<Backend, Al::amd::bfloat16_bits>::value, "types");
+static_assert(!Al::IsTypeSupported<Backend, long double>::value, "long double has no device type");
+static_assert(Al::IsReductionOpSupported<Backend, Op::bxor>::value && !Al::IsReductionOpSupported<Backend, Op::avg>::value,
+              "operators");
+static_assert(std::is_same<Al::OpAlgoType<Al::AlOperation::allgather, Backend>::type, Algo>::value, "algo type");
+
 static void test_errors(hipStream_t stream) {
   DevBuf<float> a(64), b(64);
   Al::amd::World world(2, stream);
@@ -33,6 +44,7 @@ static void test_errors(hipStream_t stream) {
   try { Al::amd::World w4(0, stream); } catch (const Al::al_exception &) { threw = true; }
   EXPECT(threw, "empty world must throw");
   EXPECT(Backend::Name() == "HipCombineBackend", "backend name");
+  EXPECT(std::string(Al::AlBackendName<Backend>) == "hip", "backend short name");
   Backend::req_type none = Backend::null_req;
   EXPECT(Al::Test<Backend>(none), "null request tests complete");
   Al::Wait<Backend>(none);
@@ -96,6 +108,11 @@ int main() {
   int ndev = 0;
   if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) { std::printf("no GPU\n"); return 2; }
   HIPCHK(hipSetDevice(0));
+  int argc = 0;
+  char **argv = nullptr;
+  EXPECT(!Al::Initialized(), "not initialised before Initialize");
+  Al::Initialize(argc, argv);
+  EXPECT(Al::Initialized(), "initialised after Initialize");
   hipStream_t stream;
   HIPCHK(hipStreamCreate(&stream));
   alo_set_num_threads(4);
@@ -142,6 +159,8 @@ int main() {
   test_flags(stream);
 
   HIPCHK(hipStreamDestroy(stream));
+  Al::Finalize();
+  EXPECT(!Al::Initialized(), "not initialised after Finalize");
   std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks, g_fail);
   return g_fail ? 1 : 0;
 }
