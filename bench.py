@@ -153,6 +153,54 @@ def run_ring_workload(al, torch, mode, steps, warmup):
             "parity_vs_oracle": bool(ok)}
 
 
+def run_layout_workload(al, torch, name, steps, warmup):
+    """The two write-heavy layouts at the C2 shape (P = 8 fp32 ranks, seed 1000+rank):
+    c2_f32_allreduce - the combine delivered to all eight ranks' receive buffers (8 reads + 8 writes of
+    2^26 elements, order tree_dbl: what Al::Allreduce yields above 2 KiB);
+    c2_f32_allgather - eight slices of 2^23 elements gathered into eight receive buffers of 2^26
+    (each slice read once, written eight times)."""
+    import numpy as np
+    import oracle
+    m = 1 << 18
+    if name == "c2_f32_allreduce":
+        count = 1 << 26
+        ins = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+        outs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+        for r in range(P):
+            al.fill(ins[r], "uniform_pm1", 1000 + r)
+        fn = lambda: al.combine(outs, ins, "sum", order="tree_dbl")
+        alg = 2 * P * count * 4
+        launches = 2 * (count * 4 // (64 << 20))
+        fn()
+        torch.cuda.synchronize()
+        ok = True
+        for j in (0, P - 1):
+            for lo in (0, count - m):
+                want = oracle.combine_generated(P, m, "f32", "sum", "tree_dbl", 0, "uniform_pm1", 1000, lo)
+                ok = ok and outs[j][lo:lo + m].cpu().numpy().tobytes() == want.tobytes()
+    else:
+        count = 1 << 23
+        sends = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+        recvs = [torch.empty(P * count, dtype=torch.float32, device="cuda") for _ in range(P)]
+        for r in range(P):
+            al.fill(sends[r], "uniform_pm1", 1000 + r)
+        fn = lambda: al.allgather(recvs, sends, count=count)
+        alg = (P + P * P) * count * 4
+        launches = P
+        fn()
+        torch.cuda.synchronize()
+        ok = True
+        for j in (0, P - 1):
+            for q in (0, P - 1):
+                want = oracle.fill(m, "f32", "uniform_pm1", 1000 + q, count - m)
+                got = recvs[j][(q + 1) * count - m:(q + 1) * count].cpu().numpy()
+                ok = ok and got.tobytes() == want.tobytes()
+    wall, kms = timed(torch, fn, steps, warmup)
+    return {"workload": name, "dtype": "f32", "op": "sum", "P": P, "count": count, "launches_per_step": launches,
+            "algorithmic_bytes": alg, "ms_per_step": wall * 1e3, "kernel_ms": kms,
+            "gbps_wall": alg / wall * 1e-9, "gbps_kernel": alg / (kms * 1e-3) * 1e-9, "parity_vs_oracle": bool(ok)}
+
+
 def run_halo_workload(al, torch, steps, warmup):
     """C5: fp64 grid, interior 512^3, halo 2 (allocation 516^3, x fastest), uniform[0,1) seed 4000;
     pack the six faces, loop them back, unpack into the ghost cells."""
@@ -288,8 +336,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2_f32_sum",
-                    choices=sorted(WORKLOADS) + ["c3_ring_stepwise", "c3_ring_fused", "c5_halo", "flags"])
-    ap.add_argument("--also", default="c2_bf16_sum,c2_f32_sum_rotating",
+                    choices=sorted(WORKLOADS) + ["c3_ring_stepwise", "c3_ring_fused", "c5_halo", "flags",
+                                               "c2_f32_allreduce", "c2_f32_allgather"])
+    ap.add_argument("--also", default="c2_bf16_sum,c2_f32_sum_rotating,c2_f32_allreduce,c2_f32_allgather,c3_ring_fused",
                     help="comma-separated extra workloads reported under 'also' ('' for none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--raw", action="store_true", help="print only the workload's own measurement record")
@@ -321,6 +370,8 @@ def main():
         main_res = run_halo_workload(al, torch, args.steps, args.warmup)
     elif args.workload == "flags":
         main_res = run_flag_workload()
+    elif args.workload in ("c2_f32_allreduce", "c2_f32_allgather"):
+        main_res = run_layout_workload(al, torch, args.workload, args.steps, args.warmup)
     else:
         main_res = run_combine_workload(al, torch, args.workload, args.steps, args.warmup)
     if args.raw or args.workload not in WORKLOADS:
