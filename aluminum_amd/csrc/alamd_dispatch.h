@@ -106,8 +106,8 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
 int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, int dtype,
                 int op, bool vector, hipStream_t stream);
 
-// Copies [src, src + bytes) to each of dests[0..ndest) (16-byte aligned, none
-// overlapping the source); used where one result goes to several buffers.
+// Copies [src, src + bytes) to each of dests[0..ndest) (none overlapping the
+// source, any alignment); used where one result goes to several buffers.
 constexpr size_t kSpreadMinBytes = (size_t)1 << 20;  // below this the all-in-one kernels are used
 int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, hipStream_t stream);
 

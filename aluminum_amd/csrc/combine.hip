@@ -154,14 +154,6 @@ __global__ void __launch_bounds__(kGatherThreads) bcast_kernel_vec(const char *s
   }
 }
 
-__global__ void __launch_bounds__(256) bcast_kernel_bytes(const char *src, FoldParams p, size_t bytes) {
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < bytes; i += (size_t)gridDim.x * 256) {
-    const char c = src[i];
-    for (int r = 0; r < p.P; ++r)
-      if (p.out[r] != src) p.out[r][i] = c;
-  }
-}
-
 // One source region to p.P destinations, one workgroup per (destination, tile).
 // Block ids run chunk by chunk (tpc tiles, 8 MiB); inside a chunk all tiles of
 // destination 0 come first, then destination 1, ...: at any time the device
@@ -248,12 +240,12 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   bool vector = true;
   for (int r = 0; r < P; ++r) {
     if (!ins[r]) return set_error(ALAMD_ERR_INVALID_ARG, "input %d is null", r);
-    vector = vector && aligned16(ins[r]);
+    vector = vector && aligned_to(ins[r], es);
   }
   void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
   for (int j = 0; j < nout; ++j) {
     if (!outs[j]) return set_error(ALAMD_ERR_INVALID_ARG, "output %d is null", j);
-    vector = vector && aligned16(outs[j]);
+    vector = vector && aligned_to(outs[j], es);
     for (int r = 0; r < P; ++r)
       if (outs[j] != ins[r] && ranges_overlap(outs[j], bytes, ins[r], bytes))
         return set_error(ALAMD_ERR_OVERLAP, "output %d partially overlaps input %d", j, r);
@@ -310,11 +302,11 @@ int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, si
   if (!recvs || !sends) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
   if (count == 0) return ALAMD_OK;
   const size_t es = alamd_dtype_size(dtype), blk = count * es, total = blk * (size_t)P;
-  bool vector = (blk % 16) == 0, inplace = false;
+  bool vector = true, inplace = false;
   void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
   for (int r = 0; r < P; ++r) {
     if (!sends[r] || !recvs[r]) return set_error(ALAMD_ERR_INVALID_ARG, "buffer %d is null", r);
-    vector = vector && aligned16(sends[r]) && aligned16(recvs[r]);
+    vector = vector && aligned_to(sends[r], es) && aligned_to(recvs[r], es);
     out_tab[r] = recvs[r];
   }
   for (int b = 0; b < P; ++b) {
@@ -366,13 +358,11 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
   if (count == 0) return ALAMD_OK;
   const size_t es = alamd_dtype_size(dtype), blk = count * es;
   FoldParams fp;
-  bool vector = (blk % 16) == 0;
   for (int r = 0; r < ALAMD_MAX_RANKS; ++r) { fp.in[r] = nullptr; fp.out[r] = nullptr; }
   for (int r = 0; r < P; ++r) {
     if (!sends[r] || !recvs[r]) return set_error(ALAMD_ERR_INVALID_ARG, "buffer %d is null", r);
     fp.in[r] = static_cast<const char *>(sends[r]);
     fp.out[r] = static_cast<char *>(recvs[r]);
-    vector = vector && aligned16(sends[r]) && aligned16(recvs[r]);
   }
   for (int r = 0; r < P; ++r) {
     for (int q = 0; q < P; ++q) {
@@ -387,7 +377,7 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
   }
   fp.P = P;
   hipStream_t st = as_stream(stream);
-  if (vector && blk >= kSpreadMinBytes) {
+  if (blk >= kSpreadMinBytes) {
     // large slices: one launch per source, one destination stream at a time
     for (int q = 0; q < P; ++q) {
       char *dests[ALAMD_MAX_RANKS];
@@ -399,7 +389,7 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
       if ((rc = launch_spread(fp.in[q], dests, nd, blk, st))) return rc;
     }
     return ALAMD_OK;
-  } else if (vector) {
+  } else if (blk % 16 == 0) {
     const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
     const size_t tiles = (blk + tile - 1) / tile;
     if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
@@ -468,10 +458,10 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, c
       bool vector = true;
       for (int r = 0; r < P; ++r) {
         ins[r] = static_cast<const char *>(sends[r]) + (displ[b] + done) * es;
-        vector = vector && aligned16(ins[r]);
+        vector = vector && aligned_to(ins[r], es);
       }
       out_tab[0] = static_cast<char *>(recvs[b]) + done * es;
-      vector = vector && aligned16(out_tab[0]);
+      vector = vector && aligned_to(out_tab[0], es);
       Layout lay;
       lay.nseg = 1;
       lay.seg.seg_base = n;
@@ -526,27 +516,20 @@ int alamd_allgatherv(void *const *recvs, const void *const *sends, int P, const 
     const size_t bytes = counts[q] * es;
     const char *src = static_cast<const char *>(sends[q]);
     FoldParams fp;
-    bool vector = aligned16(src);
     for (int r = 0; r < ALAMD_MAX_RANKS; ++r) { fp.in[r] = nullptr; fp.out[r] = nullptr; }
-    for (int r = 0; r < P; ++r) {
-      fp.out[r] = static_cast<char *>(recvs[r]) + displs[q] * es;
-      vector = vector && aligned16(fp.out[r]);
-    }
+    for (int r = 0; r < P; ++r) fp.out[r] = static_cast<char *>(recvs[r]) + displs[q] * es;
     fp.P = P;
-    if (vector && bytes >= kSpreadMinBytes) {
+    if (bytes >= kSpreadMinBytes) {
       char *dests[ALAMD_MAX_RANKS];
       int nd = 0;
       for (int r = 0; r < P; ++r)
         if (fp.out[r] != src) dests[nd++] = fp.out[r];
       if ((rc = launch_spread(src, dests, nd, bytes, st))) return rc;
-    } else if (vector) {
+    } else {
       const size_t vec_bytes = bytes & ~(size_t)15, tile = Tile<kGatherU, kGatherThreads>::BYTES;
       const size_t tiles = (vec_bytes + tile - 1) / tile;
-      if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
       hipLaunchKernelGGL(bcast_kernel_vec, dim3((unsigned)(tiles ? tiles : 1)), dim3(kGatherThreads), 0, st, src, fp,
                          vec_bytes, bytes - vec_bytes);
-    } else {
-      hipLaunchKernelGGL(bcast_kernel_bytes, dim3(stream_grid(bytes, 256 * 16, 8)), dim3(256), 0, st, src, fp, bytes);
     }
     ALAMD_HIP(hipGetLastError());
   }

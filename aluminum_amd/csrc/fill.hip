@@ -94,9 +94,12 @@ __global__ void __launch_bounds__(256) widen_kernel(float *dst, const uint16_t *
 }
 
 constexpr int kCopyU = 8, kCopyThreads = 128;
-__global__ void __launch_bounds__(kCopyThreads) copy_kernel_vec(char *dst, const char *src, size_t vec_bytes) {
+// vec_bytes (a multiple of 16) in tiles, then the tail_bytes < 16 that follow; any alignment.
+__global__ void __launch_bounds__(kCopyThreads) copy_kernel_vec(char *dst, const char *src, size_t vec_bytes,
+                                                                size_t tail_bytes) {
   using TL = Tile<kCopyU, kCopyThreads>;
   const TL tl;
+  if (blockIdx.x == 0 && threadIdx.x < tail_bytes) dst[vec_bytes + threadIdx.x] = src[vec_bytes + threadIdx.x];
   const size_t tb = (size_t)blockIdx.x * TL::BYTES;
   if (tb >= vec_bytes) return;
   const int nrec = vec_bytes - tb > TL::BYTES ? (int)TL::BYTES : (int)(vec_bytes - tb);
@@ -107,10 +110,6 @@ __global__ void __launch_bounds__(kCopyThreads) copy_kernel_vec(char *dst, const
   for (int u = 0; u < kCopyU; ++u) v[u] = tl.load(rs, u);
 #pragma unroll
   for (int u = 0; u < kCopyU; ++u) tl.store(rd, u, v[u]);
-}
-
-__global__ void __launch_bounds__(256) copy_kernel_bytes(char *dst, const char *src, size_t n) {
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = src[i];
 }
 
 }  // namespace
@@ -168,16 +167,12 @@ int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void
 int alamd_copy(void *dst, const void *src, size_t bytes, void *stream) {
   if (bytes == 0) return ALAMD_OK;
   if (!dst || !src) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer");
-  if (aligned16(dst) && aligned16(src) && bytes % 16 == 0) {
-    const size_t tile = Tile<kCopyU, kCopyThreads>::BYTES;
-    const size_t tiles = (bytes + tile - 1) / tile;
-    if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "copy too large for one launch");
-    hipLaunchKernelGGL(copy_kernel_vec, dim3((unsigned)tiles), dim3(kCopyThreads), 0, as_stream(stream), (char *)dst,
-                       (const char *)src, bytes);
-  } else {
-    const unsigned grid = stream_grid(bytes, 256 * 16, 8);
-    hipLaunchKernelGGL(copy_kernel_bytes, dim3(grid), dim3(256), 0, as_stream(stream), (char *)dst, (const char *)src, bytes);
-  }
+  const size_t vec_bytes = bytes & ~(size_t)15, tile = Tile<kCopyU, kCopyThreads>::BYTES;
+  size_t tiles = (vec_bytes + tile - 1) / tile;
+  if (tiles == 0) tiles = 1;
+  if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "copy too large for one launch");
+  hipLaunchKernelGGL(copy_kernel_vec, dim3((unsigned)tiles), dim3(kCopyThreads), 0, as_stream(stream), (char *)dst,
+                     (const char *)src, vec_bytes, bytes - vec_bytes);
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
 }

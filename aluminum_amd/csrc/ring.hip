@@ -89,7 +89,19 @@ ring_step_vec_kernel(const RingParams p) {
   ring_seg(p, seg, off, len);
   char *local = p.buf[r] + off * sizeof(T);
   const char *recv = p.buf[from] + off * sizeof(T);
-  const size_t seg_bytes = len * sizeof(T);  // a multiple of 16 on this path
+  constexpr size_t N = 16 / sizeof(T);
+  // the len % N elements after the last whole vector, one per thread of the segment's first workgroup
+  if (blockIdx.x == 0 && threadIdx.x < len % N) {
+    const size_t e = (len / N) * N + threadIdx.x;
+    const T a = ld_elem<T>(recv + e * sizeof(T));
+    if constexpr (OP >= 0) {
+      const T b = ld_elem<T>(local + e * sizeof(T));
+      st_elem<T>(local + e * sizeof(T), Step<T, (OP >= 0 ? OP : 0)>::apply(a, b));
+    } else {
+      st_elem<T>(local + e * sizeof(T), a);
+    }
+  }
+  const size_t seg_bytes = (len / N) * 16;  // whole vectors
   const size_t chunk_bytes = (size_t)p.chunk_accesses * 16;
   const size_t c = blockIdx.x / p.tiles_per_chunk, ti = blockIdx.x % p.tiles_per_chunk;
   const size_t c0 = c * chunk_bytes;
@@ -130,12 +142,12 @@ int make_plan(RingPlan &pl, void *const *bufs, int P, size_t count, int dtype, s
   if (chunk_bytes == 0 || chunk_bytes % pl.es != 0)
     return set_error(ALAMD_ERR_INVALID_ARG, "chunk size %zu is not a positive multiple of the element size", chunk_bytes);
   const size_t bytes = count * pl.es;
-  pl.vector = (count % (size_t)P == 0) && ((count / (size_t)P) * pl.es) % 16 == 0;
+  pl.vector = true;  // any element-aligned buffers; ragged segments end in an element-wise tail
   for (int r = 0; r < ALAMD_MAX_RANKS; ++r) pl.rp.buf[r] = nullptr;
   for (int r = 0; r < P; ++r) {
     if (!bufs[r] && count) return set_error(ALAMD_ERR_INVALID_ARG, "buffer %d is null", r);
     pl.rp.buf[r] = static_cast<char *>(bufs[r]);
-    pl.vector = pl.vector && aligned16(bufs[r]);
+    pl.vector = pl.vector && aligned_to(bufs[r], pl.es);
     for (int k = 0; k < r; ++k) {
       const uintptr_t x = reinterpret_cast<uintptr_t>(bufs[r]), y = reinterpret_cast<uintptr_t>(bufs[k]);
       if (count && x < y + bytes && y < x + bytes)
@@ -227,8 +239,6 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   // reduce-scatter leaves there), then spread the segment from the owner to the
   // other ranks while it is still in cache.  Writing each result tile to all P
   // buffers from one workgroup interleaves P write streams and is slower.
-  // `vector` implies count % P == 0, so every segment has seg_base elements.
-  const size_t seg_bytes = fp.seg.seg_base * es;
   FoldParams fs = fp;
   fs.seg.seg_rem = 0;
   fs.seg.in_blocked = 0;
@@ -236,17 +246,21 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   fs.seg.nout = 1;
   fs.start_stride = 0;
   for (int s = 0; s < P; ++s) {
+    const size_t sg = (size_t)s, rem = (size_t)fp.seg.seg_rem;
+    const size_t off = (sg * fp.seg.seg_base + (sg < rem ? sg : rem)) * es;
+    const size_t len = fp.seg.seg_base + (sg < rem ? 1 : 0);
     const int owner = (s + P - 1) % P;
-    for (int r = 0; r < P; ++r) fs.in[r] = static_cast<const char *>(bufs[r]) + (size_t)s * seg_bytes;
-    fs.out[0] = static_cast<char *>(bufs[owner]) + (size_t)s * seg_bytes;
+    for (int r = 0; r < P; ++r) fs.in[r] = static_cast<const char *>(bufs[r]) + off;
+    fs.out[0] = static_cast<char *>(bufs[owner]) + off;
     fs.start0 = s;
-    int rc = launch_fold(fs, 1, fp.seg.seg_base, dtype, op, true, vector, stream);
+    fs.seg.seg_base = len;
+    int rc = launch_fold(fs, 1, len, dtype, op, true, vector, stream);
     if (rc) return rc;
     char *dests[ALAMD_MAX_RANKS];
     int nd = 0;
     for (int r = 0; r < P; ++r)
-      if (r != owner) dests[nd++] = static_cast<char *>(bufs[r]) + (size_t)s * seg_bytes;
-    if ((rc = launch_spread(fs.out[0], dests, nd, seg_bytes, stream))) return rc;
+      if (r != owner) dests[nd++] = static_cast<char *>(bufs[r]) + off;
+    if ((rc = launch_spread(fs.out[0], dests, nd, len * es, stream))) return rc;
   }
   return ALAMD_OK;
 }

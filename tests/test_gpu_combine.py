@@ -94,6 +94,49 @@ def test_combine_unaligned_pointers(al):
     assert_bits_equal(to_host(out, np.float32)[1:], want, "f32", "unaligned")
 
 
+def _offset_view(a, off):
+    """Device copy of `a` that starts `off` elements into its allocation."""
+    pad = np.zeros(off, a.dtype)
+    return to_dev(np.concatenate([pad, a]))[off:]
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_vector_path_at_any_element_alignment(al, dtype):
+    """Buffers that are only element-aligned (each input and the output at its own offset) go through the
+    128-bit kernels: several tiles plus a ragged tail, fold and tree orders, two outputs."""
+    import torch
+    P, n = 5, 3 * 4096 + 37
+    op = "sum"
+    ins = make_inputs(P, n, dtype, op)
+    views = [_offset_view(a, 1 + (r % 3)) for r, a in enumerate(ins)]
+    for order in ("rank_asc", "tree_dbl"):
+        want = oracle.combine(ins, dtype, op, order)
+        outs = [dev_empty(n + 3, ins[0].dtype)[3:], dev_empty(n + 2, ins[0].dtype)[2:]]
+        al.combine(outs, views, op, order=order, dtype=dtype, count=n)
+        torch.cuda.synchronize()
+        for o in outs:
+            assert_bits_equal(to_host(o, ins[0].dtype), want, dtype, "%s %s" % (dtype, order))
+
+
+@pytest.mark.parametrize("dtype", ("u8", "bf16", "f32", "f64"))
+@pytest.mark.parametrize("inplace", (False, True))
+def test_reduce_scatter_odd_block_sizes(al, dtype, inplace):
+    """Block sizes that put every block but the first off a 16-byte boundary."""
+    import torch
+    P = 4
+    for count in (1, 7, 4099, 70001):
+        op, order = "sum", "pairwise_desc"
+        sends = make_inputs(P, P * count, dtype, op, seed=40)
+        want = oracle.reduce_scatter(sends, dtype, op, order)
+        d_sends = [to_dev(a) for a in sends]
+        d_recvs = d_sends if inplace else [dev_empty(count, sends[0].dtype) for _ in range(P)]
+        al.reduce_scatter(d_recvs, d_sends, op, order=order, dtype=dtype, count=count)
+        torch.cuda.synchronize()
+        for r in range(P):
+            assert_bits_equal(to_host(d_recvs[r], sends[0].dtype)[:count], want[r], dtype,
+                              "%s count=%d rank %d" % (dtype, count, r))
+
+
 @pytest.mark.parametrize("dtype", ("f32", "f64", "bf16", "f16"))
 def test_combine_special_values(al, dtype):
     # NaN, infinities, signed zeros, denormals and ties on every side

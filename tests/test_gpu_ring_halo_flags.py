@@ -69,6 +69,23 @@ def test_ring_reduce_scatter_then_allgather(al, dtype, op):
                           "fused reduce-scatter rank %d" % r)
 
 
+@pytest.mark.parametrize("dtype,op", [("bf16", "sum"), ("f32", "max"), ("u8", "bxor"), ("f64", "prod")])
+@pytest.mark.parametrize("mode", ("stepwise", "fused"))
+def test_ring_ragged_segments_and_offsets(al, dtype, op, mode):
+    """Counts that are not multiples of P (segments differ by one element and start off 16-byte
+    boundaries), buffers that are only element-aligned, several tiles per segment."""
+    import torch
+    for P, n in ((3, 3 * 20000 + 2), (8, 8 * 5000 + 5), (5, 4)):
+        host = ring_inputs(P, n, dtype, op)
+        want = oracle.ring_allreduce(host, dtype, op, 4096)
+        pads = [np.zeros(1 + r % 2, host[0].dtype) for r in range(P)]
+        bufs = [to_dev(np.concatenate([pads[r], host[r]]))[pads[r].size:] for r in range(P)]
+        al.ring_allreduce(bufs, op, chunk_bytes=4096 * host[0].itemsize, mode=mode, dtype=dtype, count=n)
+        torch.cuda.synchronize()
+        for r in range(P):
+            assert_bits_equal(to_host(bufs[r], host[0].dtype), want[r], dtype, "%s P=%d rank %d" % (mode, P, r))
+
+
 def test_ring_errors(al):
     bufs = [to_dev(np.zeros(64, np.float32)) for _ in range(4)]
     with pytest.raises(al.AlError):
@@ -176,6 +193,17 @@ def test_copy(al):
         torch.cuda.synchronize()
         if n:
             assert to_host(dst, np.uint8).tobytes() == a.tobytes()
+    # any byte alignment on either side; the bytes around the destination stay untouched
+    n = 100003
+    a = np.random.default_rng(7).integers(0, 255, n + 8).astype(np.uint8)
+    src = to_dev(a)
+    for so, do in ((1, 0), (0, 3), (5, 2)):
+        dst = to_dev(np.full(n + 16, 0xEE, np.uint8))
+        al.copy(dst[do:], src[so:], nbytes=n)
+        torch.cuda.synchronize()
+        got = to_host(dst, np.uint8)
+        assert got[do:do + n].tobytes() == a[so:so + n].tobytes()
+        assert (got[:do] == 0xEE).all() and (got[do + n:] == 0xEE).all()
 
 
 # ---- stream flags ------------------------------------------------------------
