@@ -70,7 +70,7 @@ template <typename F> int dispatch_any(int dtype, int op, F &&f) {
 struct SegParams {
   unsigned long long seg_base;
   unsigned long long seg_rem;
-  unsigned long long tile0;  // vector path: index of the first tile of this launch
+  unsigned long long tile0;  // index of the first tile of this launch
   int in_blocked;   // 1: inputs are read at the segment's offset, 0: at 0
   int out_mode;     // OUT_ALL / OUT_SEG / OUT_OWNER
   int owner_shift;  // OUT_OWNER: output index is (segment + owner_shift) mod P
@@ -101,10 +101,10 @@ struct TreeParams {
   int nvalid;   // occupied slots
 };
 
-int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op,
-                bool acc_is_in, bool vector, hipStream_t stream);
-int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, int dtype,
-                int op, bool vector, hipStream_t stream);
+int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op, bool acc_is_in,
+                hipStream_t stream);
+int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, int dtype, int op,
+                hipStream_t stream);
 
 // Copies [src, src + bytes) to each of dests[0..ndest) (none overlapping the
 // source, any alignment); used where one result goes to several buffers.

@@ -66,8 +66,9 @@ struct Layout {
 };
 
 // Launches the fold or tree kernels for `order` over inputs `ins`.
+// `outs` has ALAMD_MAX_RANKS entries (unused ones null).
 int launch_order(void *const *outs, const void *const *ins, int P, const Layout &lay, int dtype, int op,
-                 int order, bool vector, hipStream_t stream) {
+                 int order, hipStream_t stream) {
   if (!is_float_dtype(dtype)) order = ALAMD_ORDER_RANK_ASC;  // integer ops: every order gives the same bits
   if (P == 1 && order_is_tree(order)) order = ALAMD_ORDER_RANK_ASC;
   if (order_is_tree(order)) {
@@ -78,7 +79,7 @@ int launch_order(void *const *outs, const void *const *ins, int P, const Layout 
     const int slots = build_tree(tp, ins, P, order);
     for (int j = 0; j < ALAMD_MAX_RANKS; ++j) tp.out[j] = static_cast<char *>(outs[j]);
     tp.seg = lay.seg;
-    return launch_tree(tp, slots, lay.nseg, lay.max_len, dtype, op, vector, stream);
+    return launch_tree(tp, slots, lay.nseg, lay.max_len, dtype, op, stream);
   }
   FoldParams fp;
   for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
@@ -90,7 +91,7 @@ int launch_order(void *const *outs, const void *const *ins, int P, const Layout 
   fp.start0 = lay.start0;
   fp.start_stride = lay.start_stride;
   fp.dir = order == ALAMD_ORDER_PAIRWISE_DESC ? -1 : 1;
-  return launch_fold(fp, lay.nseg, lay.max_len, dtype, op, order == ALAMD_ORDER_RING, vector, stream);
+  return launch_fold(fp, lay.nseg, lay.max_len, dtype, op, order == ALAMD_ORDER_RING, stream);
 }
 
 constexpr int kGatherU = 8, kGatherThreads = 128;
@@ -187,6 +188,10 @@ __global__ void __launch_bounds__(kGatherThreads) spread_kernel_vec(const char *
   }
 }
 
+int misaligned(const char *what, int index) {
+  return set_error(ALAMD_ERR_INVALID_ARG, "%s %d is not aligned to its element type", what, index);
+}
+
 int check_common(int P, size_t count, int dtype) {
   if (P < 1 || P > ALAMD_MAX_RANKS)
     return set_error(ALAMD_ERR_INVALID_ARG, "number of ranks %d outside [1, %d]", P, ALAMD_MAX_RANKS);
@@ -237,15 +242,14 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   if (!outs || !ins) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
   if (count == 0) return ALAMD_OK;
   const size_t es = alamd_dtype_size(dtype), bytes = count * es;
-  bool vector = true;
   for (int r = 0; r < P; ++r) {
     if (!ins[r]) return set_error(ALAMD_ERR_INVALID_ARG, "input %d is null", r);
-    vector = vector && aligned_to(ins[r], es);
+    if (!aligned_to(ins[r], es)) return misaligned("input", r);
   }
   void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
   for (int j = 0; j < nout; ++j) {
     if (!outs[j]) return set_error(ALAMD_ERR_INVALID_ARG, "output %d is null", j);
-    vector = vector && aligned_to(outs[j], es);
+    if (!aligned_to(outs[j], es)) return misaligned("output", j);
     for (int r = 0; r < P; ++r)
       if (outs[j] != ins[r] && ranges_overlap(outs[j], bytes, ins[r], bytes))
         return set_error(ALAMD_ERR_OVERLAP, "output %d partially overlaps input %d", j, r);
@@ -266,8 +270,8 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   lay.max_len = count;
   lay.start0 = start;
   lay.start_stride = 0;
-  if (nout == 1 || !vector || bytes < kSpreadMinBytes)
-    return launch_order(out_tab, ins, P, lay, dtype, op, order, vector, as_stream(stream));
+  if (nout == 1 || bytes < kSpreadMinBytes)
+    return launch_order(out_tab, ins, P, lay, dtype, op, order, as_stream(stream));
   // Several outputs of a large result: a workgroup that wrote its tile to every
   // output would interleave nout write streams (measured 69 % of peak).  Instead
   // the result goes to outs[0] and is then spread, 64 MiB at a time so that the
@@ -285,7 +289,7 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
     first[0] = static_cast<char *>(outs[0]) + e0 * es;
     lay.seg.seg_base = len;
     lay.max_len = len;
-    if ((rc = launch_order(first, in_tab, P, lay, dtype, op, order, vector, as_stream(stream)))) return rc;
+    if ((rc = launch_order(first, in_tab, P, lay, dtype, op, order, as_stream(stream)))) return rc;
     char *dests[ALAMD_MAX_RANKS];
     for (int j = 1; j < nout; ++j) dests[j - 1] = static_cast<char *>(outs[j]) + e0 * es;
     if ((rc = launch_spread(static_cast<char *>(first[0]), dests, nout - 1, len * es, as_stream(stream)))) return rc;
@@ -302,11 +306,11 @@ int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, si
   if (!recvs || !sends) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
   if (count == 0) return ALAMD_OK;
   const size_t es = alamd_dtype_size(dtype), blk = count * es, total = blk * (size_t)P;
-  bool vector = true, inplace = false;
+  bool inplace = false;
   void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
   for (int r = 0; r < P; ++r) {
     if (!sends[r] || !recvs[r]) return set_error(ALAMD_ERR_INVALID_ARG, "buffer %d is null", r);
-    vector = vector && aligned_to(sends[r], es) && aligned_to(recvs[r], es);
+    if (!aligned_to(sends[r], es) || !aligned_to(recvs[r], es)) return misaligned("buffer", r);
     out_tab[r] = recvs[r];
   }
   for (int b = 0; b < P; ++b) {
@@ -332,13 +336,13 @@ int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, si
   lay.start_stride = order_has_start(order) ? 1 : 0;
   if (!inplace || P == 1) {
     lay.nseg = (unsigned)P;
-    return launch_order(out_tab, sends, P, lay, dtype, op, order, vector, as_stream(stream));
+    return launch_order(out_tab, sends, P, lay, dtype, op, order, as_stream(stream));
   }
   // In place every result lands on block 0 of its own send buffer, which
   // block 0's fold still has to read: fold block 0 first (it overwrites only
   // what its own lanes have read), then the other blocks.
   lay.nseg = 1;
-  rc = launch_order(out_tab, sends, P, lay, dtype, op, order, vector, as_stream(stream));
+  rc = launch_order(out_tab, sends, P, lay, dtype, op, order, as_stream(stream));
   if (rc) return rc;
   // blocks 1..P-1: shift the tables by one block
   const void *in_shift[ALAMD_MAX_RANKS];
@@ -347,7 +351,7 @@ int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, si
   for (int b = 1; b < P; ++b) out_shift[b - 1] = recvs[b];
   lay.nseg = (unsigned)(P - 1);
   lay.start0 = order_has_start(order) ? 1 : 0;
-  return launch_order(out_shift, in_shift, P, lay, dtype, op, order, vector, as_stream(stream));
+  return launch_order(out_shift, in_shift, P, lay, dtype, op, order, as_stream(stream));
 }
 
 int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t count, int dtype,
@@ -420,11 +424,14 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, c
   }
   const size_t total = displ[P] * es;
   if (total == 0) return ALAMD_OK;
-  for (int r = 0; r < P; ++r)
+  for (int r = 0; r < P; ++r) {
     if (!sends[r]) return set_error(ALAMD_ERR_INVALID_ARG, "send buffer %d is null", r);
+    if (!aligned_to(sends[r], es)) return misaligned("send buffer", r);
+  }
   for (int b = 0; b < P; ++b) {
     if (counts[b] == 0) continue;
     if (!recvs[b]) return set_error(ALAMD_ERR_INVALID_ARG, "receive buffer %d is null", b);
+    if (!aligned_to(recvs[b], es)) return misaligned("receive buffer", b);
     for (int r = 0; r < P; ++r) {
       if (b == r && recvs[b] == sends[r]) continue;  // in place
       if (ranges_overlap(recvs[b], counts[b] * es, sends[r], total))
@@ -455,13 +462,8 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, c
       const size_t n = counts[b] - done < run ? counts[b] - done : run;
       const void *ins[ALAMD_MAX_RANKS];
       void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
-      bool vector = true;
-      for (int r = 0; r < P; ++r) {
-        ins[r] = static_cast<const char *>(sends[r]) + (displ[b] + done) * es;
-        vector = vector && aligned_to(ins[r], es);
-      }
+      for (int r = 0; r < P; ++r) ins[r] = static_cast<const char *>(sends[r]) + (displ[b] + done) * es;
       out_tab[0] = static_cast<char *>(recvs[b]) + done * es;
-      vector = vector && aligned_to(out_tab[0], es);
       Layout lay;
       lay.nseg = 1;
       lay.seg.seg_base = n;
@@ -474,7 +476,7 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, c
       lay.max_len = n;
       lay.start0 = order_has_start(order) ? b : 0;
       lay.start_stride = 0;
-      if ((rc = launch_order(out_tab, ins, P, lay, dtype, op, order, vector, as_stream(stream)))) return rc;
+      if ((rc = launch_order(out_tab, ins, P, lay, dtype, op, order, as_stream(stream)))) return rc;
     }
   }
   return ALAMD_OK;

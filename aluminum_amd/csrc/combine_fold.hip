@@ -2,10 +2,10 @@
 // contributions resident in HBM.  Bandwidth-bound: every input byte is read
 // once, every output byte written once.
 //
-// Vector path (all buffers 16-byte aligned): one workgroup per tile, all loads
-// of a lane issued before the first use, buffer instructions with per-tile
-// descriptors (see alamd_tile.h).  Element path (any alignment): one element
-// per access, grid-stride.
+// One workgroup per tile, all loads of a lane issued before the first use,
+// buffer instructions with per-tile descriptors (see alamd_tile.h); buffers
+// need only be aligned to their element type.  The len % N elements behind the
+// last whole vector of a segment are folded one per thread.
 #include "alamd_dispatch.h"
 #include "alamd_tile.h"
 
@@ -145,28 +145,10 @@ fold_vec_kernel(const FoldParams p) {
   if (p.seg.tile0 == 0 && blockIdx.x == 0 && e < len) fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
 }
 
-constexpr int kElemThreads = 256;
-
-template <typename T, int OP, bool ACC_IS_IN>
-__global__ void __launch_bounds__(kElemThreads) fold_elem_kernel(const FoldParams p) {
-  const int P = p.P;
-  const unsigned seg = blockIdx.y;
-  size_t off, len;
-  seg_range(p.seg, seg, off, len);
-  const size_t off_bytes = off * sizeof(T);
-  const size_t in_bytes = p.seg.in_blocked ? off_bytes : 0;
-  const int s = (p.start0 + (int)seg * p.start_stride) % P;
-  int j0, nj;
-  size_t out_bytes;
-  out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
-  for (size_t e = (size_t)blockIdx.x * kElemThreads + threadIdx.x; e < len; e += (size_t)gridDim.x * kElemThreads)
-    fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
-}
-
 }  // namespace
 
-int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op,
-                bool acc_is_in, bool vector, hipStream_t stream) {
+int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op, bool acc_is_in,
+                hipStream_t stream) {
   // operand roles only matter where a tie or a NaN can pick a side
   const bool roles = acc_is_in && is_float_dtype(dtype) && (op == ALAMD_MIN || op == ALAMD_MAX);
   return dispatch_any(dtype, op, [&](auto tt, auto ot) -> int {
@@ -176,33 +158,21 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
                                 std::is_same<T, f16_t>::value || std::is_same<T, bf16_t>::value) &&
                                (OP == ALAMD_MIN || OP == ALAMD_MAX);
     void (*kern)(const FoldParams) = nullptr;
-    if (vector) {
-      const size_t tile_elems = Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES / sizeof(T);
-      size_t tiles = (max_len + tile_elems - 1) / tile_elems;
-      if (tiles == 0) tiles = 1;
-      if (p.P == 8) {
-        if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 8> : fold_vec_kernel<T, OP, false, 8>;
-        else kern = fold_vec_kernel<T, OP, false, 8>;
-      } else {
-        if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 0> : fold_vec_kernel<T, OP, false, 0>;
-        else kern = fold_vec_kernel<T, OP, false, 0>;
-      }
-      FoldParams q = p;
-      for (size_t t0 = 0; t0 < tiles; t0 += kMaxTilesPerLaunch) {
-        const size_t nt = tiles - t0 < kMaxTilesPerLaunch ? tiles - t0 : kMaxTilesPerLaunch;
-        q.seg.tile0 = t0;
-        hipLaunchKernelGGL(kern, dim3((unsigned)nt, nseg, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
-      }
+    const size_t tile_elems = Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES / sizeof(T);
+    size_t tiles = (max_len + tile_elems - 1) / tile_elems;
+    if (tiles == 0) tiles = 1;
+    if (p.P == 8) {
+      if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 8> : fold_vec_kernel<T, OP, false, 8>;
+      else kern = fold_vec_kernel<T, OP, false, 8>;
     } else {
-      unsigned gx = stream_grid(max_len, (size_t)kElemThreads * 4, 8);
-      if (nseg > 1) {
-        unsigned per_seg = (stream_grid((size_t)-1 / 2, 1, 8) + nseg - 1) / nseg;
-        if (per_seg < 1) per_seg = 1;
-        if (gx > per_seg) gx = per_seg;
-      }
-      if constexpr (FP_MINMAX) kern = roles ? fold_elem_kernel<T, OP, true> : fold_elem_kernel<T, OP, false>;
-      else kern = fold_elem_kernel<T, OP, false>;
-      hipLaunchKernelGGL(kern, dim3(gx, nseg, 1), dim3(kElemThreads, 1, 1), 0, stream, p);
+      if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 0> : fold_vec_kernel<T, OP, false, 0>;
+      else kern = fold_vec_kernel<T, OP, false, 0>;
+    }
+    FoldParams q = p;
+    for (size_t t0 = 0; t0 < tiles; t0 += kMaxTilesPerLaunch) {
+      const size_t nt = tiles - t0 < kMaxTilesPerLaunch ? tiles - t0 : kMaxTilesPerLaunch;
+      q.seg.tile0 = t0;
+      hipLaunchKernelGGL(kern, dim3((unsigned)nt, nseg, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
     }
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;

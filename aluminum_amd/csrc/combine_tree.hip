@@ -8,8 +8,6 @@ namespace alamd {
 
 namespace {
 
-constexpr int kThreads = 256;
-
 __device__ __forceinline__ void seg_range(const SegParams &s, unsigned seg, size_t &off, size_t &len) {
   const unsigned long long sg = seg;
   off = sg * s.seg_base + (sg < s.seg_rem ? sg : s.seg_rem);
@@ -115,43 +113,19 @@ tree_vec_kernel(const TreeParams p) {
 }
 
 template <typename T, int OP, int SLOTS>
-__global__ void __launch_bounds__(kThreads) tree_elem_kernel(const TreeParams p) {
-  const unsigned seg = blockIdx.y;
-  size_t off, len;
-  seg_range(p.seg, seg, off, len);
-  const size_t off_bytes = off * sizeof(T);
-  const size_t in_bytes = p.seg.in_blocked ? off_bytes : 0;
-  int j0, nj;
-  size_t out_bytes;
-  tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
-  for (size_t e = (size_t)blockIdx.x * kThreads + threadIdx.x; e < len; e += (size_t)gridDim.x * kThreads)
-    tree_elem<T, OP, SLOTS>(p, in_bytes, j0, nj, out_bytes, e);
-}
-
-template <typename T, int OP, int SLOTS>
-int launch_tree_slots(const TreeParams &p, unsigned nseg, size_t max_len, bool vector, hipStream_t stream) {
-  if (vector) {
-    using S = TreeShape<T, OP, SLOTS>;
-    const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
-    size_t tiles = (max_len + tile_elems - 1) / tile_elems;
-    if (tiles == 0) tiles = 1;
-    TreeParams q = p;
-    bool full = p.nvalid == SLOTS;
-    for (int j = 0; j < SLOTS; ++j) full = full && p.b[j] == nullptr;
-    void (*kern)(const TreeParams) = full ? tree_vec_kernel<T, OP, SLOTS, true> : tree_vec_kernel<T, OP, SLOTS, false>;
-    for (size_t t0 = 0; t0 < tiles; t0 += kMaxTilesPerLaunch) {
-      const size_t nt = tiles - t0 < kMaxTilesPerLaunch ? tiles - t0 : kMaxTilesPerLaunch;
-      q.seg.tile0 = t0;
-      hipLaunchKernelGGL(kern, dim3((unsigned)nt, nseg, 1), dim3(S::THREADS, 1, 1), 0, stream, q);
-    }
-  } else {
-    unsigned gx = stream_grid(max_len, (size_t)kThreads * 4, 8);
-    if (nseg > 1) {
-      unsigned per_seg = (stream_grid((size_t)-1 / 2, 1, 8) + nseg - 1) / nseg;
-      if (per_seg < 1) per_seg = 1;
-      if (gx > per_seg) gx = per_seg;
-    }
-    hipLaunchKernelGGL((tree_elem_kernel<T, OP, SLOTS>), dim3(gx, nseg, 1), dim3(kThreads, 1, 1), 0, stream, p);
+int launch_tree_slots(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream) {
+  using S = TreeShape<T, OP, SLOTS>;
+  const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
+  size_t tiles = (max_len + tile_elems - 1) / tile_elems;
+  if (tiles == 0) tiles = 1;
+  TreeParams q = p;
+  bool full = p.nvalid == SLOTS;
+  for (int j = 0; j < SLOTS; ++j) full = full && p.b[j] == nullptr;
+  void (*kern)(const TreeParams) = full ? tree_vec_kernel<T, OP, SLOTS, true> : tree_vec_kernel<T, OP, SLOTS, false>;
+  for (size_t t0 = 0; t0 < tiles; t0 += kMaxTilesPerLaunch) {
+    const size_t nt = tiles - t0 < kMaxTilesPerLaunch ? tiles - t0 : kMaxTilesPerLaunch;
+    q.seg.tile0 = t0;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nt, nseg, 1), dim3(S::THREADS, 1, 1), 0, stream, q);
   }
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
@@ -159,17 +133,17 @@ int launch_tree_slots(const TreeParams &p, unsigned nseg, size_t max_len, bool v
 
 }  // namespace
 
-int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, int dtype,
-                int op, bool vector, hipStream_t stream) {
+int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, int dtype, int op,
+                hipStream_t stream) {
   return dispatch_float(dtype, op, [&](auto tt, auto ot) -> int {
     using T = typename decltype(tt)::type;
     constexpr int OP = decltype(ot)::value;
     switch (slots) {
-    case 2: return launch_tree_slots<T, OP, 2>(p, nseg, max_len, vector, stream);
-    case 4: return launch_tree_slots<T, OP, 4>(p, nseg, max_len, vector, stream);
-    case 8: return launch_tree_slots<T, OP, 8>(p, nseg, max_len, vector, stream);
-    case 16: return launch_tree_slots<T, OP, 16>(p, nseg, max_len, vector, stream);
-    case 32: return launch_tree_slots<T, OP, 32>(p, nseg, max_len, vector, stream);
+    case 2: return launch_tree_slots<T, OP, 2>(p, nseg, max_len, stream);
+    case 4: return launch_tree_slots<T, OP, 4>(p, nseg, max_len, stream);
+    case 8: return launch_tree_slots<T, OP, 8>(p, nseg, max_len, stream);
+    case 16: return launch_tree_slots<T, OP, 16>(p, nseg, max_len, stream);
+    case 32: return launch_tree_slots<T, OP, 32>(p, nseg, max_len, stream);
     default: return set_error(ALAMD_ERR_INVALID_ARG, "tree combine: bad slot count %d", slots);
     }
   });

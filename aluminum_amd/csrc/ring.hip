@@ -3,7 +3,8 @@
 // STEPWISE: one launch per ring step.  In reduce-scatter step t every rank r
 // (blockIdx.y) folds the segment it "receives" from rank r-1 into its own
 // copy; in allgather step t it copies the segment.  A segment is worked
-// through chunk by chunk: a chunk is owned by a fixed group of workgroups.
+// through chunk by chunk: a chunk is a run of tiles, no tile crosses a chunk
+// boundary.
 // FUSED: the fold kernels walk each segment once in ring order; an allreduce
 // then spreads every folded segment from its owner to the other ranks.
 #include "alamd_dispatch.h"
@@ -18,11 +19,10 @@ constexpr int kThreads = 256;
 struct RingParams {
   char *buf[ALAMD_MAX_RANKS];
   unsigned long long seg_base, seg_rem;
-  unsigned long long chunk_accesses;  // accesses (vectors or elements) per chunk
+  unsigned long long chunk_accesses;  // 128-bit vectors per chunk
   int P;
   int t;              // ring step
-  unsigned wg_per_chunk;    // element path: workgroups that share one chunk
-  unsigned tiles_per_chunk; // vector path: workgroups (tiles) per chunk
+  unsigned tiles_per_chunk;  // workgroups (tiles) per chunk
 };
 
 __device__ __forceinline__ void ring_seg(const RingParams &p, int seg, size_t &off, size_t &len) {
@@ -31,50 +31,8 @@ __device__ __forceinline__ void ring_seg(const RingParams &p, int seg, size_t &o
   len = p.seg_base + (sg < p.seg_rem ? 1u : 0u);
 }
 
-// Element path (any alignment).  OP < 0: plain copy (allgather step).
-template <typename T, int OP>
-__global__ void __launch_bounds__(kThreads) ring_step_elem_kernel(const RingParams p) {
-  constexpr int U = 4;
-  constexpr size_t TILE = (size_t)kThreads * U;
-  const int P = p.P, r = blockIdx.y;
-  // reduce-scatter step t receives segment r-t-1, allgather step t segment r-t
-  int seg = (OP >= 0 ? r - p.t - 1 : r - p.t) % P;
-  if (seg < 0) seg += P;
-  const int from = r == 0 ? P - 1 : r - 1;
-  size_t off, len;
-  ring_seg(p, seg, off, len);
-  char *local = p.buf[r] + off * sizeof(T);
-  const char *recv = p.buf[from] + off * sizeof(T);
-  const size_t n = len, cn = p.chunk_accesses;
-  const size_t nchunks = (n + cn - 1) / cn;
-  const unsigned wgpc = p.wg_per_chunk;
-  const unsigned lane_wg = blockIdx.x % wgpc;
-  for (size_t c = blockIdx.x / wgpc; c < nchunks; c += gridDim.x / wgpc) {
-    const size_t c0 = c * cn, c1 = (c0 + cn < n) ? c0 + cn : n;
-    for (size_t i0 = c0 + (size_t)lane_wg * TILE + threadIdx.x; i0 < c1; i0 += (size_t)wgpc * TILE) {
-      T a[U], b[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const size_t i = i0 + (size_t)u * kThreads;
-        if (i < c1) {
-          a[u] = ld_elem<T>(recv + i * sizeof(T));
-          if constexpr (OP >= 0) b[u] = ld_elem<T>(local + i * sizeof(T));
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const size_t i = i0 + (size_t)u * kThreads;
-        if (i < c1) {
-          if constexpr (OP >= 0) st_elem<T>(local + i * sizeof(T), Step<T, (OP >= 0 ? OP : 0)>::apply(a[u], b[u]));
-          else st_elem<T>(local + i * sizeof(T), a[u]);
-        }
-      }
-    }
-  }
-}
-
-// Vector path: a chunk is a run of tiles_per_chunk tiles; no tile crosses a
-// chunk boundary.  OP < 0: plain copy.
+// A chunk is a run of tiles_per_chunk tiles; no tile crosses a chunk boundary.
+// OP < 0: plain copy (allgather step).
 constexpr int kRingU = 8;
 template <typename T, int OP>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4)))
@@ -128,7 +86,6 @@ ring_step_vec_kernel(const RingParams p) {
 
 struct RingPlan {
   RingParams rp;
-  bool vector;
   unsigned gx;
   size_t es;
 };
@@ -142,12 +99,12 @@ int make_plan(RingPlan &pl, void *const *bufs, int P, size_t count, int dtype, s
   if (chunk_bytes == 0 || chunk_bytes % pl.es != 0)
     return set_error(ALAMD_ERR_INVALID_ARG, "chunk size %zu is not a positive multiple of the element size", chunk_bytes);
   const size_t bytes = count * pl.es;
-  pl.vector = true;  // any element-aligned buffers; ragged segments end in an element-wise tail
   for (int r = 0; r < ALAMD_MAX_RANKS; ++r) pl.rp.buf[r] = nullptr;
   for (int r = 0; r < P; ++r) {
     if (!bufs[r] && count) return set_error(ALAMD_ERR_INVALID_ARG, "buffer %d is null", r);
     pl.rp.buf[r] = static_cast<char *>(bufs[r]);
-    pl.vector = pl.vector && aligned_to(bufs[r], pl.es);
+    if (!aligned_to(bufs[r], pl.es))
+      return set_error(ALAMD_ERR_INVALID_ARG, "buffer %d is not aligned to its element type", r);
     for (int k = 0; k < r; ++k) {
       const uintptr_t x = reinterpret_cast<uintptr_t>(bufs[r]), y = reinterpret_cast<uintptr_t>(bufs[k]);
       if (count && x < y + bytes && y < x + bytes)
@@ -158,32 +115,19 @@ int make_plan(RingPlan &pl, void *const *bufs, int P, size_t count, int dtype, s
   pl.rp.seg_base = count / (size_t)P;
   pl.rp.seg_rem = count % (size_t)P;
   pl.rp.t = 0;
-  const size_t access = pl.vector ? 16 : pl.es;
-  size_t cn = chunk_bytes / access;
+  // a chunk is a whole number of 128-bit vectors (chunking never changes a bit: the step is element-wise)
+  size_t cn = chunk_bytes / 16;
   if (cn < 1) cn = 1;
   pl.rp.chunk_accesses = cn;
-  // workgroups: enough to fill the device across the P rows, a whole number per chunk
   const size_t seg_max = pl.rp.seg_base + (pl.rp.seg_rem ? 1 : 0);
-  const size_t n = seg_max / (pl.vector ? 16 / pl.es : 1);
+  const size_t n = seg_max / (16 / pl.es);  // whole vectors of the longest segment
   size_t nchunks = (n + cn - 1) / cn;
   if (nchunks < 1) nchunks = 1;
-  const size_t tiles_per_chunk = ((cn < n ? cn : (n ? n : 1)) + (size_t)kThreads * 4 - 1) / ((size_t)kThreads * 4);
-  const unsigned row_budget = (stream_grid((size_t)-1 / 2, 1, 8) + P - 1) / P;
-  size_t wgpc = row_budget / nchunks;
-  if (wgpc < 1) wgpc = 1;
-  if (wgpc > tiles_per_chunk) wgpc = tiles_per_chunk;
-  size_t chunk_rows = nchunks;
-  if (chunk_rows * wgpc > row_budget) chunk_rows = row_budget / wgpc ? row_budget / wgpc : 1;
-  pl.rp.wg_per_chunk = (unsigned)wgpc;
-  pl.rp.tiles_per_chunk = 1;
-  pl.gx = (unsigned)(chunk_rows * wgpc);
-  if (pl.vector) {
-    const size_t tile_vecs = Tile<kRingU, kThreads>::BYTES / 16;
-    const size_t tpc = ((cn < n ? cn : (n ? n : 1)) + tile_vecs - 1) / tile_vecs;
-    if (nchunks * tpc > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "too many chunks for one launch");
-    pl.rp.tiles_per_chunk = (unsigned)tpc;
-    pl.gx = (unsigned)(nchunks * tpc);
-  }
+  const size_t tile_vecs = Tile<kRingU, kThreads>::BYTES / 16;
+  const size_t tpc = ((cn < n ? cn : (n ? n : 1)) + tile_vecs - 1) / tile_vecs;
+  if (nchunks * tpc > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "too many chunks for one launch");
+  pl.rp.tiles_per_chunk = (unsigned)tpc;
+  pl.gx = (unsigned)(nchunks * tpc);
   return ALAMD_OK;
 }
 
@@ -193,10 +137,10 @@ int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, hipStream_t 
     // a copy only needs the element size
     void (*kern)(const RingParams) = nullptr;
     switch (pl.es) {
-    case 1: kern = pl.vector ? ring_step_vec_kernel<uint8_t, -1> : ring_step_elem_kernel<uint8_t, -1>; break;
-    case 2: kern = pl.vector ? ring_step_vec_kernel<uint16_t, -1> : ring_step_elem_kernel<uint16_t, -1>; break;
-    case 4: kern = pl.vector ? ring_step_vec_kernel<uint32_t, -1> : ring_step_elem_kernel<uint32_t, -1>; break;
-    default: kern = pl.vector ? ring_step_vec_kernel<uint64_t, -1> : ring_step_elem_kernel<uint64_t, -1>; break;
+    case 1: kern = ring_step_vec_kernel<uint8_t, -1>; break;
+    case 2: kern = ring_step_vec_kernel<uint16_t, -1>; break;
+    case 4: kern = ring_step_vec_kernel<uint32_t, -1>; break;
+    default: kern = ring_step_vec_kernel<uint64_t, -1>; break;
     }
     hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
     ALAMD_HIP(hipGetLastError());
@@ -205,15 +149,13 @@ int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, hipStream_t 
   return dispatch_any(dtype, op, [&](auto tt, auto ot) -> int {
     using T = typename decltype(tt)::type;
     constexpr int OP = decltype(ot)::value;
-    void (*kern)(const RingParams) = pl.vector ? ring_step_vec_kernel<T, OP> : ring_step_elem_kernel<T, OP>;
-    hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
+    hipLaunchKernelGGL((ring_step_vec_kernel<T, OP>), grid, block, 0, stream, pl.rp);
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;
   });
 }
 
-int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool all, bool vector,
-               hipStream_t stream) {
+int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool all, hipStream_t stream) {
   FoldParams fp;
   for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
     fp.in[r] = r < P ? static_cast<const char *>(bufs[r]) : nullptr;
@@ -233,8 +175,8 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   const size_t max_len = fp.seg.seg_base + (fp.seg.seg_rem ? 1 : 0);
   if (max_len == 0) return ALAMD_OK;
   const size_t es = alamd_dtype_size(dtype);
-  if (!all || !vector || fp.seg.seg_base * es < kSpreadMinBytes)
-    return launch_fold(fp, (unsigned)P, max_len, dtype, op, true, vector, stream);
+  if (!all || fp.seg.seg_base * es < kSpreadMinBytes)
+    return launch_fold(fp, (unsigned)P, max_len, dtype, op, true, stream);
   // Large allreduce: segment by segment, fold into the owner's buffer (what the
   // reduce-scatter leaves there), then spread the segment from the owner to the
   // other ranks while it is still in cache.  Writing each result tile to all P
@@ -254,7 +196,7 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
     fs.out[0] = static_cast<char *>(bufs[owner]) + off;
     fs.start0 = s;
     fs.seg.seg_base = len;
-    int rc = launch_fold(fs, 1, len, dtype, op, true, vector, stream);
+    int rc = launch_fold(fs, 1, len, dtype, op, true, stream);
     if (rc) return rc;
     char *dests[ALAMD_MAX_RANKS];
     int nd = 0;
@@ -290,7 +232,7 @@ int alamd_ring_reduce_scatter(void *const *bufs, int P, size_t count, int dtype,
   if (mode != ALAMD_RING_STEPWISE && mode != ALAMD_RING_FUSED)
     return set_error(ALAMD_ERR_INVALID_ALGO, "Invalid algorithm");
   if (count == 0 || P == 1) return ALAMD_OK;
-  if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, P, count, dtype, op, false, pl.vector, as_stream(stream));
+  if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, P, count, dtype, op, false, as_stream(stream));
   for (int t = 0; t < P - 1; ++t) {
     pl.rp.t = t;
     if ((rc = launch_step(pl, dtype, op, true, as_stream(stream)))) return rc;
@@ -320,7 +262,7 @@ int alamd_ring_allreduce(void *const *bufs, int P, size_t count, int dtype, int 
   if (mode != ALAMD_RING_STEPWISE && mode != ALAMD_RING_FUSED)
     return set_error(ALAMD_ERR_INVALID_ALGO, "Invalid algorithm");
   if (count == 0 || P == 1) return ALAMD_OK;
-  if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, P, count, dtype, op, true, pl.vector, as_stream(stream));
+  if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, P, count, dtype, op, true, as_stream(stream));
   rc = alamd_ring_reduce_scatter(bufs, P, count, dtype, op, chunk_bytes, mode, stream);
   if (rc) return rc;
   return alamd_ring_allgather(bufs, P, count, dtype, chunk_bytes, stream);

@@ -124,7 +124,9 @@ int alamd_init(void);
  * (include/aluminum/ht/reduce.hpp:72-82), nout = P an Allreduce over P
  * logical ranks.  An output may be identical to an input (in-place), but
  * must not overlap one partially.  `start` is the rank s of the orders that
- * have one and must be 0 otherwise. */
+ * have one and must be 0 otherwise.  Here and in every entry point below a
+ * buffer must be aligned to its element type (ALAMD_ERR_INVALID_ARG if not);
+ * no wider alignment is needed. */
 int alamd_combine(void *const *outs, int nout, const void *const *ins, int P,
                   size_t count, int dtype, int op, int order, int start,
                   void *stream);

@@ -287,6 +287,14 @@ def test_errors(al):
     assert e.value.code == 5
     with pytest.raises(al.AlError):
         al.combine(out, [a[0]] * 65, "sum")
+    # a pointer that is not aligned to its element type is refused (no kernel is launched)
+    raw = to_dev(np.zeros(80, np.uint8))
+    with pytest.raises(al.AlError, match="not aligned to its element type"):
+        al.combine(out, [a[0], raw[1:65]], "sum", dtype="f32", count=16)
+    with pytest.raises(al.AlError, match="not aligned to its element type"):
+        al.reduce_scatter([raw[2:10], raw[40:48]], [a[0], a[1]], "sum", dtype="f32", count=2)
+    with pytest.raises(al.AlError, match="not aligned to its element type"):
+        al.ring_allreduce([a[0], raw[1:65]], "sum", dtype="f32", count=16)
     # zero-length is a no-op
     al.combine(out, a, "sum", count=0)
     torch.cuda.synchronize()
