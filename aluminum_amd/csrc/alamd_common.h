@@ -193,11 +193,10 @@ template <typename T> __device__ __forceinline__ void st_elem(void *p, T v) {
   *reinterpret_cast<T *>(p) = v;
 }
 
-// The kernels issue 128-bit accesses at any element-aligned address: the
-// device runs in unaligned access mode, and a buffer of fp32 that starts 4
-// bytes off a 16-byte boundary is folded at the same rate as an aligned one
-// (2-byte and 1-byte offsets: about 80 %).  A pointer that is not even aligned
-// to its element type is refused.
+// The kernels issue 128-bit accesses at any element-aligned address (the
+// device runs in unaligned access mode; see head_elems in alamd_tile.h for
+// the one case that costs bandwidth).  A pointer that is not even aligned to
+// its element type is refused.
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
 // Grid size for a streaming kernel over `work_items` items with `per_block`

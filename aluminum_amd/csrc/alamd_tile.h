@@ -31,6 +31,20 @@ constexpr unsigned kRsrcFlags = 0x00020000u;
 // tile); longer inputs are cut into consecutive launches on the same stream.
 constexpr size_t kMaxTilesPerLaunch = 4096;
 
+// Loads of 128 bits run at full rate from any 4-byte-aligned address; from an
+// address that splits its dwords they lose about a fifth of the bandwidth
+// (stores do not care).  For element types narrower than 4 bytes the kernels
+// therefore handle up to three bytes' worth of leading elements one by one, so
+// that the vectors of the stream at `first` start on a dword boundary.
+template <typename T> __device__ __forceinline__ size_t head_elems(const char *first, size_t len) {
+  if constexpr (sizeof(T) >= 4) {
+    return 0;
+  } else {
+    const size_t h = ((4u - (unsigned)(reinterpret_cast<uintptr_t>(first) & 3u)) & 3u) / sizeof(T);
+    return h < len ? h : len;
+  }
+}
+
 template <int U, int THREADS> struct Tile {
   static constexpr size_t BYTES = (size_t)THREADS * U * 16;
   unsigned vo;

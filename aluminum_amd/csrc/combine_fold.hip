@@ -77,7 +77,10 @@ fold_vec_kernel(const FoldParams p) {
   size_t out_bytes;
   out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
 
-  const size_t vec_bytes = (len / N) * 16;
+  const size_t head = head_elems<T>(p.in[s] + in_bytes, len);
+  const size_t vlen = len - head;
+  const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
+  const size_t vec_bytes = (vlen / N) * 16;
   const size_t tb = ((size_t)p.seg.tile0 + blockIdx.x) * TL::BYTES;
   if (tb < vec_bytes) {
     const size_t rem = vec_bytes - tb;
@@ -88,7 +91,7 @@ fold_vec_kernel(const FoldParams p) {
       int idx = s;
 #pragma unroll
       for (int k = 0; k < PT; ++k) {
-        const auto r = TL::rsrc(p.in[idx] + in_bytes + tb, nrec);
+        const auto r = TL::rsrc(p.in[idx] + vin + tb, nrec);
 #pragma unroll
         for (int u = 0; u < U; ++u) x[k][u] = tl.load(r, u);
         idx = next_rank(idx, p.dir, PT);
@@ -107,7 +110,7 @@ fold_vec_kernel(const FoldParams p) {
       constexpr int B = 4;  // streams in flight between uses
       int idx = s;
       {
-        const auto r = TL::rsrc(p.in[idx] + in_bytes + tb, nrec);
+        const auto r = TL::rsrc(p.in[idx] + vin + tb, nrec);
 #pragma unroll
         for (int u = 0; u < U; ++u) acc[u] = tl.load(r, u);
       }
@@ -118,7 +121,7 @@ fold_vec_kernel(const FoldParams p) {
         for (int b = 0; b < B; ++b) {
           if (k + b < P) {
             id = next_rank(id, p.dir, P);
-            const auto r = TL::rsrc(p.in[id] + in_bytes + tb, nrec);
+            const auto r = TL::rsrc(p.in[id] + vin + tb, nrec);
 #pragma unroll
             for (int u = 0; u < U; ++u) x[b][u] = tl.load(r, u);
           }
@@ -135,14 +138,17 @@ fold_vec_kernel(const FoldParams p) {
       }
     }
     for (int j = j0; j < j0 + nj; ++j) {
-      const auto r = TL::rsrc(p.out[j] + out_bytes + tb, nrec);
+      const auto r = TL::rsrc(p.out[j] + vout + tb, nrec);
 #pragma unroll
       for (int u = 0; u < U; ++u) tl.store(r, u, acc[u]);
     }
   }
-  // the len % N trailing elements, one per thread of the first workgroup
-  const size_t e = (len / N) * N + threadIdx.x;
-  if (p.seg.tile0 == 0 && blockIdx.x == 0 && e < len) fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
+  // the head elements and the vlen % N elements behind the last whole vector, one per thread of the
+  // segment's first workgroup
+  if (p.seg.tile0 == 0 && blockIdx.x == 0 && threadIdx.x < head + vlen % N) {
+    const size_t e = threadIdx.x < head ? threadIdx.x : (vlen / N) * N + threadIdx.x;
+    fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
+  }
 }
 
 }  // namespace

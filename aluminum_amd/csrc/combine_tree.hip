@@ -69,7 +69,10 @@ tree_vec_kernel(const TreeParams p) {
   tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
   const int nvalid = FULL ? SLOTS : p.nvalid;
 
-  const size_t vec_bytes = (len / N) * 16;
+  const size_t head = head_elems<T>(p.a[0] + in_bytes, len);
+  const size_t vlen = len - head;
+  const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
+  const size_t vec_bytes = (vlen / N) * 16;
   const size_t tb = ((size_t)p.seg.tile0 + blockIdx.x) * TL::BYTES;
   if (tb < vec_bytes) {
     const size_t rem = vec_bytes - tb;
@@ -78,7 +81,7 @@ tree_vec_kernel(const TreeParams p) {
 #pragma unroll
     for (int j = 0; j < SLOTS; ++j) {
       if (j < nvalid) {
-        const auto r = TL::rsrc(p.a[j] + in_bytes + tb, nrec);
+        const auto r = TL::rsrc(p.a[j] + vin + tb, nrec);
 #pragma unroll
         for (int u = 0; u < U; ++u) v[j][u] = tl.load(r, u);
       }
@@ -87,7 +90,7 @@ tree_vec_kernel(const TreeParams p) {
 #pragma unroll
     for (int j = 0; j < SLOTS; ++j) {
       if (!FULL && j < nvalid && p.b[j] != nullptr) {
-        const auto r = TL::rsrc(p.b[j] + in_bytes + tb, nrec);
+        const auto r = TL::rsrc(p.b[j] + vin + tb, nrec);
 #pragma unroll
         for (int u = 0; u < U; ++u) v[j][u] = step_vec<T, OP>(v[j][u], tl.load(r, u));
       }
@@ -103,13 +106,16 @@ tree_vec_kernel(const TreeParams p) {
       }
     }
     for (int j = j0; j < j0 + nj; ++j) {
-      const auto r = TL::rsrc(p.out[j] + out_bytes + tb, nrec);
+      const auto r = TL::rsrc(p.out[j] + vout + tb, nrec);
 #pragma unroll
       for (int u = 0; u < U; ++u) tl.store(r, u, v[0][u]);
     }
   }
-  const size_t e = (len / N) * N + threadIdx.x;
-  if (p.seg.tile0 == 0 && blockIdx.x == 0 && e < len) tree_elem<T, OP, SLOTS>(p, in_bytes, j0, nj, out_bytes, e);
+  // the head elements and the vlen % N elements behind the last whole vector
+  if (p.seg.tile0 == 0 && blockIdx.x == 0 && threadIdx.x < head + vlen % N) {
+    const size_t e = threadIdx.x < head ? threadIdx.x : (vlen / N) * N + threadIdx.x;
+    tree_elem<T, OP, SLOTS>(p, in_bytes, j0, nj, out_bytes, e);
+  }
 }
 
 template <typename T, int OP, int SLOTS>

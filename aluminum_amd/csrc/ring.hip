@@ -48,9 +48,12 @@ ring_step_vec_kernel(const RingParams p) {
   char *local = p.buf[r] + off * sizeof(T);
   const char *recv = p.buf[from] + off * sizeof(T);
   constexpr size_t N = 16 / sizeof(T);
-  // the len % N elements after the last whole vector, one per thread of the segment's first workgroup
-  if (blockIdx.x == 0 && threadIdx.x < len % N) {
-    const size_t e = (len / N) * N + threadIdx.x;
+  const size_t head = head_elems<T>(recv, len);
+  const size_t vlen = len - head;
+  // the head elements and the vlen % N elements after the last whole vector, one per thread of the
+  // segment's first workgroup
+  if (blockIdx.x == 0 && threadIdx.x < head + vlen % N) {
+    const size_t e = threadIdx.x < head ? threadIdx.x : (vlen / N) * N + threadIdx.x;
     const T a = ld_elem<T>(recv + e * sizeof(T));
     if constexpr (OP >= 0) {
       const T b = ld_elem<T>(local + e * sizeof(T));
@@ -59,7 +62,9 @@ ring_step_vec_kernel(const RingParams p) {
       st_elem<T>(local + e * sizeof(T), a);
     }
   }
-  const size_t seg_bytes = (len / N) * 16;  // whole vectors
+  local += head * sizeof(T);
+  recv += head * sizeof(T);
+  const size_t seg_bytes = (vlen / N) * 16;  // whole vectors
   const size_t chunk_bytes = (size_t)p.chunk_accesses * 16;
   const size_t c = blockIdx.x / p.tiles_per_chunk, ti = blockIdx.x % p.tiles_per_chunk;
   const size_t c0 = c * chunk_bytes;
