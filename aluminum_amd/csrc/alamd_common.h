@@ -199,6 +199,18 @@ template <typename T> __device__ __forceinline__ void st_elem(void *p, T v) {
 // its element type is refused.
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
+// A byte range as the copy kernels walk it: `head` bytes up to the source's
+// next 4-byte boundary, `vec` bytes in whole 128-bit vectors, `tail` < 16.
+struct ByteSplit { size_t head, vec, tail; };
+inline ByteSplit split_bytes(const void *src, size_t bytes) {
+  ByteSplit b;
+  b.head = (4 - (reinterpret_cast<uintptr_t>(src) & 3)) & 3;
+  if (b.head > bytes) b.head = bytes;
+  b.vec = (bytes - b.head) & ~(size_t)15;
+  b.tail = bytes - b.head - b.vec;
+  return b;
+}
+
 // Grid size for a streaming kernel over `work_items` items with `per_block`
 // items per workgroup pass: enough workgroups to cover the work, capped at
 // `waves` workgroups per compute unit.

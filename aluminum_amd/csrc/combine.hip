@@ -163,8 +163,8 @@ __global__ void __launch_bounds__(kGatherThreads) bcast_kernel_vec(const char *s
 // of 32 MiB: 88 % of the HBM peak, against 67 % when every workgroup writes
 // its tile to all destinations (69 % for those writes alone).
 constexpr unsigned kSpreadChunkTiles = 512;
-__global__ void __launch_bounds__(kGatherThreads) spread_kernel_vec(const char *src, FoldParams p, size_t vec_bytes,
-                                                                    size_t tail_bytes, unsigned tpc, unsigned tiles) {
+__global__ void __launch_bounds__(kGatherThreads) spread_kernel_vec(const char *src, FoldParams p, ByteSplit b,
+                                                                    unsigned tpc, unsigned tiles) {
   using TL = Tile<kGatherU, kGatherThreads>;
   const TL tl;
   const unsigned ndest = (unsigned)p.P;
@@ -173,18 +173,20 @@ __global__ void __launch_bounds__(kGatherThreads) spread_kernel_vec(const char *
   const unsigned dest = rem / tpc, tile = chunk * tpc + rem % tpc;
   if (tile < tiles) {
     const size_t tb = (size_t)tile * TL::BYTES;
-    const int nrec = vec_bytes - tb > TL::BYTES ? (int)TL::BYTES : (int)(vec_bytes - tb);
-    const auto rs = TL::rsrc(src + tb, nrec);
-    const auto rd = TL::rsrc(p.out[dest] + tb, nrec);
+    const int nrec = b.vec - tb > TL::BYTES ? (int)TL::BYTES : (int)(b.vec - tb);
+    const auto rs = TL::rsrc(src + b.head + tb, nrec);
+    const auto rd = TL::rsrc(p.out[dest] + b.head + tb, nrec);
     u32x4 v[kGatherU];
 #pragma unroll
     for (int u = 0; u < kGatherU; ++u) v[u] = tl.load_cached(rs, u);
 #pragma unroll
     for (int u = 0; u < kGatherU; ++u) tl.store_nt(rd, u, v[u]);
   }
-  if (blockIdx.x == 0 && threadIdx.x < tail_bytes) {
-    const char c = src[vec_bytes + threadIdx.x];
-    for (unsigned r = 0; r < ndest; ++r) p.out[r][vec_bytes + threadIdx.x] = c;
+  // the bytes before the first and after the last whole vector
+  if (blockIdx.x == 0 && threadIdx.x < b.head + b.tail) {
+    const size_t i = threadIdx.x < b.head ? threadIdx.x : b.vec + threadIdx.x;
+    const char c = src[i];
+    for (unsigned r = 0; r < ndest; ++r) p.out[r][i] = c;
   }
 }
 
@@ -210,15 +212,16 @@ int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, 
     fp.out[r] = r < ndest ? dests[r] : nullptr;
   }
   fp.P = ndest;
-  const size_t vec_bytes = bytes & ~(size_t)15, tile = Tile<kGatherU, kGatherThreads>::BYTES;
-  size_t tiles = (vec_bytes + tile - 1) / tile;
+  const ByteSplit b = split_bytes(src, bytes);
+  const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
+  size_t tiles = (b.vec + tile - 1) / tile;
   if (tiles == 0) tiles = 1;
   const size_t tpc = tiles < kSpreadChunkTiles ? tiles : kSpreadChunkTiles;
   const size_t chunks = (tiles + tpc - 1) / tpc;
   const size_t blocks = chunks * tpc * (size_t)ndest;
   if (blocks > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
-  hipLaunchKernelGGL(spread_kernel_vec, dim3((unsigned)blocks), dim3(kGatherThreads), 0, stream, src, fp, vec_bytes,
-                     bytes - vec_bytes, (unsigned)tpc, (unsigned)tiles);
+  hipLaunchKernelGGL(spread_kernel_vec, dim3((unsigned)blocks), dim3(kGatherThreads), 0, stream, src, fp, b,
+                     (unsigned)tpc, (unsigned)tiles);
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
 }

@@ -94,17 +94,19 @@ __global__ void __launch_bounds__(256) widen_kernel(float *dst, const uint16_t *
 }
 
 constexpr int kCopyU = 8, kCopyThreads = 128;
-// vec_bytes (a multiple of 16) in tiles, then the tail_bytes < 16 that follow; any alignment.
-__global__ void __launch_bounds__(kCopyThreads) copy_kernel_vec(char *dst, const char *src, size_t vec_bytes,
-                                                                size_t tail_bytes) {
+// Any alignment: b.head + b.tail single bytes by the first workgroup, b.vec bytes in tiles.
+__global__ void __launch_bounds__(kCopyThreads) copy_kernel_vec(char *dst, const char *src, ByteSplit b) {
   using TL = Tile<kCopyU, kCopyThreads>;
   const TL tl;
-  if (blockIdx.x == 0 && threadIdx.x < tail_bytes) dst[vec_bytes + threadIdx.x] = src[vec_bytes + threadIdx.x];
+  if (blockIdx.x == 0 && threadIdx.x < b.head + b.tail) {
+    const size_t i = threadIdx.x < b.head ? threadIdx.x : b.vec + threadIdx.x;
+    dst[i] = src[i];
+  }
   const size_t tb = (size_t)blockIdx.x * TL::BYTES;
-  if (tb >= vec_bytes) return;
-  const int nrec = vec_bytes - tb > TL::BYTES ? (int)TL::BYTES : (int)(vec_bytes - tb);
-  const auto rs = TL::rsrc(src + tb, nrec);
-  const auto rd = TL::rsrc(dst + tb, nrec);
+  if (tb >= b.vec) return;
+  const int nrec = b.vec - tb > TL::BYTES ? (int)TL::BYTES : (int)(b.vec - tb);
+  const auto rs = TL::rsrc(src + b.head + tb, nrec);
+  const auto rd = TL::rsrc(dst + b.head + tb, nrec);
   u32x4 v[kCopyU];
 #pragma unroll
   for (int u = 0; u < kCopyU; ++u) v[u] = tl.load(rs, u);
@@ -167,12 +169,13 @@ int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void
 int alamd_copy(void *dst, const void *src, size_t bytes, void *stream) {
   if (bytes == 0) return ALAMD_OK;
   if (!dst || !src) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer");
-  const size_t vec_bytes = bytes & ~(size_t)15, tile = Tile<kCopyU, kCopyThreads>::BYTES;
-  size_t tiles = (vec_bytes + tile - 1) / tile;
+  const ByteSplit b = split_bytes(src, bytes);
+  const size_t tile = Tile<kCopyU, kCopyThreads>::BYTES;
+  size_t tiles = (b.vec + tile - 1) / tile;
   if (tiles == 0) tiles = 1;
   if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "copy too large for one launch");
   hipLaunchKernelGGL(copy_kernel_vec, dim3((unsigned)tiles), dim3(kCopyThreads), 0, as_stream(stream), (char *)dst,
-                     (const char *)src, vec_bytes, bytes - vec_bytes);
+                     (const char *)src, b);
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
 }

@@ -191,6 +191,20 @@ def test_allgather_large_slices(al):
     torch.cuda.synchronize()
     for r in range(P):
         assert torch.equal(bufs[r], want), "in place, rank %d" % r
+    # bytes: sources and receive buffers at odd addresses, slice length not a multiple of 16
+    count = (1 << 20) + 3
+    raw = [torch.empty(count + 8, dtype=torch.uint8, device="cuda") for _ in range(P)]
+    sends = [raw[r][1 + r % 3:1 + r % 3 + count] for r in range(P)]
+    for r in range(P):
+        al.fill(sends[r], "fullrange", 90 + r, dtype="u8", count=count)
+    rraw = [torch.full((P * count + 8,), 0xEE, dtype=torch.uint8, device="cuda") for _ in range(P)]
+    recvs = [rraw[r][3:3 + P * count] for r in range(P)]
+    al.allgather(recvs, sends, dtype="u8", count=count)
+    torch.cuda.synchronize()
+    want = torch.cat(sends)
+    for r in range(P):
+        assert torch.equal(recvs[r], want), "bytes, rank %d" % r
+        assert bool((rraw[r][:3] == 0xEE).all()) and bool((rraw[r][3 + P * count:] == 0xEE).all())
 
 
 @pytest.mark.parametrize("order", ("rank_asc", "tree_dbl"))
