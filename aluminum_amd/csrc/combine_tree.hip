@@ -36,10 +36,18 @@ __device__ __forceinline__ void tree_elem(const TreeParams &p, size_t in_bytes, 
   for (int j = j0; j < j0 + nj; ++j) st_elem<T>(p.out[j] + out_bytes + e * sizeof(T), v[0]);
 }
 
-template <typename T, int OP, int SLOTS> struct TreeShape {
+// Kernel variants: every slot occupied and none pre-folded (P a power of two:
+// straight-line code, no uniform branches between the loads and their uses);
+// some slots empty (binomial order, P not a power of two); some slots
+// pre-folded from a second rank (doubling / halving orders, P not a power of
+// two), which needs room for up to twice as many loads in flight.
+enum { TREE_FULL = 0, TREE_PARTIAL = 1, TREE_PREFOLD = 2 };
+
+template <typename T, int OP, int SLOTS, int MODE> struct TreeShape {
   static constexpr bool heavy = sizeof(T) <= 2;
   static constexpr int budget = heavy ? 32 : 64;  // 128-bit loads in flight per lane
-  static constexpr int U = budget / SLOTS >= 8 ? (heavy ? 4 : 8) : (budget / SLOTS >= 1 ? budget / SLOTS : 1);
+  static constexpr int streams = MODE == TREE_PREFOLD ? 2 * SLOTS : SLOTS;
+  static constexpr int U = budget / streams >= 8 ? (heavy ? 4 : 8) : (budget / streams >= 1 ? budget / streams : 1);
   static constexpr int THREADS = U == 8 ? 128 : 256;
 };
 
@@ -50,12 +58,10 @@ __device__ __forceinline__ void tree_out_select(const TreeParams &p, unsigned se
   else { j0 = ((int)seg + p.seg.owner_shift) % p.P; nj = 1; out_bytes = off_bytes; }
 }
 
-// FULL: every slot occupied and none pre-folded (P a power of two): straight-line
-// code, no uniform branches between the loads and their uses.
-template <typename T, int OP, int SLOTS, bool FULL>
-__global__ void __launch_bounds__((TreeShape<T, OP, SLOTS>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
+template <typename T, int OP, int SLOTS, int MODE>
+__global__ void __launch_bounds__((TreeShape<T, OP, SLOTS, MODE>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
 tree_vec_kernel(const TreeParams p) {
-  constexpr int U = TreeShape<T, OP, SLOTS>::U, THREADS = TreeShape<T, OP, SLOTS>::THREADS;
+  constexpr int U = TreeShape<T, OP, SLOTS, MODE>::U, THREADS = TreeShape<T, OP, SLOTS, MODE>::THREADS;
   constexpr int N = 16 / sizeof(T);
   using TL = Tile<U, THREADS>;
   const TL tl;
@@ -67,7 +73,7 @@ tree_vec_kernel(const TreeParams p) {
   int j0, nj;
   size_t out_bytes;
   tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
-  const int nvalid = FULL ? SLOTS : p.nvalid;
+  const int nvalid = MODE == TREE_FULL ? SLOTS : p.nvalid;
 
   const size_t head = head_elems<T>(p.a[0] + in_bytes, len);
   const size_t vlen = len - head;
@@ -86,13 +92,24 @@ tree_vec_kernel(const TreeParams p) {
         for (int u = 0; u < U; ++u) v[j][u] = tl.load(r, u);
       }
     }
-    // pre-folded slots: the odd rank keeps step(in = even rank, inout = odd rank)
+    if constexpr (MODE == TREE_PREFOLD) {
+      // pre-folded slots: the odd rank keeps step(in = even rank, inout = odd rank); all of
+      // their loads are issued before the first use, like the slots' own
+      u32x4 w[SLOTS][U];
 #pragma unroll
-    for (int j = 0; j < SLOTS; ++j) {
-      if (!FULL && j < nvalid && p.b[j] != nullptr) {
-        const auto r = TL::rsrc(p.b[j] + vin + tb, nrec);
+      for (int j = 0; j < SLOTS; ++j) {
+        if (j < nvalid && p.b[j] != nullptr) {
+          const auto r = TL::rsrc(p.b[j] + vin + tb, nrec);
 #pragma unroll
-        for (int u = 0; u < U; ++u) v[j][u] = step_vec<T, OP>(v[j][u], tl.load(r, u));
+          for (int u = 0; u < U; ++u) w[j][u] = tl.load(r, u);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < SLOTS; ++j) {
+        if (j < nvalid && p.b[j] != nullptr) {
+#pragma unroll
+          for (int u = 0; u < U; ++u) v[j][u] = step_vec<T, OP>(v[j][u], w[j][u]);
+        }
       }
     }
 #pragma unroll
@@ -118,23 +135,32 @@ tree_vec_kernel(const TreeParams p) {
   }
 }
 
-template <typename T, int OP, int SLOTS>
-int launch_tree_slots(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream) {
-  using S = TreeShape<T, OP, SLOTS>;
+template <typename T, int OP, int SLOTS, int MODE>
+int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream) {
+  using S = TreeShape<T, OP, SLOTS, MODE>;
   const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
   size_t tiles = (max_len + tile_elems - 1) / tile_elems;
   if (tiles == 0) tiles = 1;
+  // the launch cut is a number of bytes per stream, whatever the tile size
+  const size_t cut = kMaxTilesPerLaunch * (size_t)16384 / Tile<S::U, S::THREADS>::BYTES;
   TreeParams q = p;
-  bool full = p.nvalid == SLOTS;
-  for (int j = 0; j < SLOTS; ++j) full = full && p.b[j] == nullptr;
-  void (*kern)(const TreeParams) = full ? tree_vec_kernel<T, OP, SLOTS, true> : tree_vec_kernel<T, OP, SLOTS, false>;
-  for (size_t t0 = 0; t0 < tiles; t0 += kMaxTilesPerLaunch) {
-    const size_t nt = tiles - t0 < kMaxTilesPerLaunch ? tiles - t0 : kMaxTilesPerLaunch;
+  for (size_t t0 = 0; t0 < tiles; t0 += cut) {
+    const size_t nt = tiles - t0 < cut ? tiles - t0 : cut;
     q.seg.tile0 = t0;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nt, nseg, 1), dim3(S::THREADS, 1, 1), 0, stream, q);
+    hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE>), dim3((unsigned)nt, nseg, 1), dim3(S::THREADS, 1, 1), 0,
+                       stream, q);
   }
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
+}
+
+template <typename T, int OP, int SLOTS>
+int launch_tree_slots(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream) {
+  bool prefold = false;
+  for (int j = 0; j < SLOTS; ++j) prefold = prefold || p.b[j] != nullptr;
+  if (prefold) return launch_tree_mode<T, OP, SLOTS, TREE_PREFOLD>(p, nseg, max_len, stream);
+  if (p.nvalid == SLOTS) return launch_tree_mode<T, OP, SLOTS, TREE_FULL>(p, nseg, max_len, stream);
+  return launch_tree_mode<T, OP, SLOTS, TREE_PARTIAL>(p, nseg, max_len, stream);
 }
 
 }  // namespace
