@@ -162,15 +162,18 @@ __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
       r[j] = (__builtin_bit_cast(uint32_t, re) | (__builtin_bit_cast(uint32_t, ro) << 8)) ^ bias;
     }
     return r;
-  } else if constexpr (sizeof(T) == 1 && (OP == ALAMD_LOR || OP == ALAMD_LAND || OP == ALAMD_LXOR)) {
-    // four bytes at a time: 0x01 in every byte that is nonzero, then the bitwise op
+  } else if constexpr (sizeof(T) <= 2 && (OP == ALAMD_LOR || OP == ALAMD_LAND || OP == ALAMD_LXOR)) {
+    // a whole dword of bytes or halfwords at a time: a 1 in every element that
+    // is nonzero (the carry of low-bits + all-ones reaches the top bit iff a
+    // low bit is set), then the bitwise operator
+    constexpr uint32_t low = sizeof(T) == 1 ? 0x7f7f7f7fu : 0x7fff7fffu, top = ~low;
+    constexpr int shift = 8 * (int)sizeof(T) - 1;
+    auto nonzero = [](uint32_t x) { return ((((x & low) + low) | x) & top) >> shift; };
     u32x4 r;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t a = in[j], b = inout[j];
-      const uint32_t na = ((((a & 0x7f7f7f7fu) + 0x7f7f7f7fu) | a) & 0x80808080u) >> 7;
-      const uint32_t nb = ((((b & 0x7f7f7f7fu) + 0x7f7f7f7fu) | b) & 0x80808080u) >> 7;
-      r[j] = OP == ALAMD_LOR ? (nb | na) : OP == ALAMD_LAND ? (nb & na) : (nb ^ na);
+      r[j] = OP == ALAMD_LOR ? nonzero(b | a) : OP == ALAMD_LAND ? (nonzero(b) & nonzero(a)) : (nonzero(b) ^ nonzero(a));
     }
     return r;
   } else {
