@@ -145,6 +145,28 @@ __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
       r[j] = narrow_bf16x2(fp_step<float, OP>(a_lo, b_lo), fp_step<float, OP>(a_hi, b_hi));
     }
     return r;
+  } else if constexpr (sizeof(T) == 1 && OP == ALAMD_SUM) {
+    // four wrapping byte sums per dword: add the low seven bits of every byte
+    // (no carry leaves a byte), then put the top bits back with an xor
+    u32x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t a = in[j], b = inout[j];
+      r[j] = ((a & 0x7f7f7f7fu) + (b & 0x7f7f7f7fu)) ^ ((a ^ b) & 0x80808080u);
+    }
+    return r;
+  } else if constexpr (sizeof(T) == 1 && OP == ALAMD_PROD) {
+    // wrapping byte products as packed 16-bit products of the even and the odd bytes
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+    u32x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t a = in[j], b = inout[j];
+      const u16x2 pe = __builtin_bit_cast(u16x2, a & 0x00ff00ffu) * __builtin_bit_cast(u16x2, b & 0x00ff00ffu);
+      const u16x2 po = __builtin_bit_cast(u16x2, (a >> 8) & 0x00ff00ffu) * __builtin_bit_cast(u16x2, (b >> 8) & 0x00ff00ffu);
+      r[j] = (__builtin_bit_cast(uint32_t, pe) & 0x00ff00ffu) | ((__builtin_bit_cast(uint32_t, po) & 0x00ff00ffu) << 8);
+    }
+    return r;
   } else if constexpr (sizeof(T) == 1 && (OP == ALAMD_MIN || OP == ALAMD_MAX)) {
     // bytes compared as packed 16-bit pairs: even and odd bytes of a dword are
     // zero-extended into two 2 x u16 registers; signed bytes are first biased

@@ -48,13 +48,11 @@ __device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, siz
   for (int j = j0; j < j0 + nj; ++j) st_elem<T>(p.out[j] + out_bytes + e * sizeof(T), acc);
 }
 
-// Tile shape per element type: narrow arithmetic types spend many more ALU
-// operations per byte, so they keep fewer loads in flight per lane and more
-// waves resident to overlap arithmetic with memory.
+// Tile shape: 128 threads x 8 vectors per stream for every type (byte sums and
+// products, the most arithmetic per byte, are done a dword at a time and keep up).
 template <typename T, int OP> struct Shape {
-  static constexpr bool heavy = sizeof(T) == 1 && OP <= ALAMD_PROD;
-  static constexpr int U = heavy ? 4 : 8;
-  static constexpr int THREADS = heavy ? 256 : 128;
+  static constexpr int U = 8;
+  static constexpr int THREADS = 128;
 };
 
 // amdgpu_waves_per_eu(1, 2): the loads in flight are the point of this kernel;
