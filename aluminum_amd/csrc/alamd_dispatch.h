@@ -66,7 +66,8 @@ template <typename F> int dispatch_any(int dtype, int op, F &&f) {
 // ---- parameters of the two combine kernel families -------------------------
 
 // Work is a grid of segments (blockIdx.y) x tiles (blockIdx.x).  Segment s
-// covers elements [s*seg_base + min(s, seg_rem), +seg_base + (s < seg_rem)).
+// covers elements [s*seg_base + min(s, seg_rem), +seg_base + (s < seg_rem)),
+// or, when `ragged` is set, [seg_off[s], +seg_len[s]).
 struct SegParams {
   unsigned long long seg_base;
   unsigned long long seg_rem;
@@ -75,8 +76,33 @@ struct SegParams {
   int out_mode;     // OUT_ALL / OUT_SEG / OUT_OWNER
   int owner_shift;  // OUT_OWNER: output index is (segment + owner_shift) mod P
   int nout;         // OUT_ALL: number of outputs written
+  int ragged;       // 1: segments are given by the two tables below
+  unsigned long long seg_off[ALAMD_MAX_RANKS];
+  unsigned long long seg_len[ALAMD_MAX_RANKS];
 };
 enum { OUT_ALL = 0, OUT_SEG = 1, OUT_OWNER = 2 };
+
+// Equal segments (the first seg_rem of them one element longer), everything else zero.
+inline SegParams make_seg(size_t seg_base, size_t seg_rem, int in_blocked, int out_mode, int nout) {
+  SegParams s = {};
+  s.seg_base = seg_base;
+  s.seg_rem = seg_rem;
+  s.in_blocked = in_blocked;
+  s.out_mode = out_mode;
+  s.nout = nout;
+  return s;
+}
+
+__device__ __forceinline__ void seg_range(const SegParams &s, unsigned seg, size_t &off, size_t &len) {
+  if (s.ragged) {
+    off = s.seg_off[seg];
+    len = s.seg_len[seg];
+  } else {
+    const unsigned long long sg = seg;
+    off = sg * s.seg_base + (sg < s.seg_rem ? sg : s.seg_rem);
+    len = s.seg_base + (sg < s.seg_rem ? 1u : 0u);
+  }
+}
 
 // Left fold over a rotated rank sequence.
 struct FoldParams {

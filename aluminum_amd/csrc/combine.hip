@@ -263,13 +263,7 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   }
   Layout lay;
   lay.nseg = 1;
-  lay.seg.seg_base = count;
-  lay.seg.seg_rem = 0;
-  lay.seg.tile0 = 0;
-  lay.seg.in_blocked = 0;
-  lay.seg.out_mode = OUT_ALL;
-  lay.seg.owner_shift = 0;
-  lay.seg.nout = nout;
+  lay.seg = make_seg(count, 0, 0, OUT_ALL, nout);
   lay.max_len = count;
   lay.start0 = start;
   lay.start_stride = 0;
@@ -327,13 +321,7 @@ int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, si
         return set_error(ALAMD_ERR_OVERLAP, "receive buffers %d and %d overlap", k, b);
   }
   Layout lay;
-  lay.seg.seg_base = count;
-  lay.seg.seg_rem = 0;
-  lay.seg.tile0 = 0;
-  lay.seg.in_blocked = 1;
-  lay.seg.out_mode = OUT_SEG;
-  lay.seg.owner_shift = 0;
-  lay.seg.nout = 1;
+  lay.seg = make_seg(count, 0, 1, OUT_SEG, 1);
   lay.max_len = count;
   lay.start0 = 0;
   lay.start_stride = order_has_start(order) ? 1 : 0;
@@ -444,7 +432,30 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, c
       if (counts[k] && ranges_overlap(recvs[b], counts[b] * es, recvs[k], counts[k] * es))
         return set_error(ALAMD_ERR_OVERLAP, "receive buffers %d and %d overlap", k, b);
   }
-  // One fold per block, in ascending block order: in place, block b's result
+  bool any_inplace = false;
+  size_t max_count = 0;
+  for (int b = 0; b < P; ++b) {
+    any_inplace = any_inplace || (counts[b] && recvs[b] == sends[b]);
+    if (counts[b] > max_count) max_count = counts[b];
+  }
+  if (!any_inplace) {
+    // separate receive buffers: all blocks in one launch, one segment per block
+    Layout lay;
+    lay.nseg = (unsigned)P;
+    lay.seg = make_seg(0, 0, 1, OUT_SEG, 1);
+    lay.seg.ragged = 1;
+    void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
+    for (int b = 0; b < P; ++b) {
+      lay.seg.seg_off[b] = displ[b];
+      lay.seg.seg_len[b] = counts[b];
+      out_tab[b] = recvs[b];
+    }
+    lay.max_len = max_count;
+    lay.start0 = 0;
+    lay.start_stride = order_has_start(order) ? 1 : 0;
+    return launch_order(out_tab, sends, P, lay, dtype, op, order, as_stream(stream));
+  }
+  // In place: one fold per block, in ascending block order; block b's result
   // overwrites the start of rank b's buffer, which only blocks <= b read.
   for (int b = 0; b < P; ++b) {
     if (counts[b] == 0) continue;
@@ -469,13 +480,7 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, c
       out_tab[0] = static_cast<char *>(recvs[b]) + done * es;
       Layout lay;
       lay.nseg = 1;
-      lay.seg.seg_base = n;
-      lay.seg.seg_rem = 0;
-      lay.seg.tile0 = 0;
-      lay.seg.in_blocked = 0;
-      lay.seg.out_mode = OUT_ALL;
-      lay.seg.owner_shift = 0;
-      lay.seg.nout = 1;
+      lay.seg = make_seg(n, 0, 0, OUT_ALL, 1);
       lay.max_len = n;
       lay.start0 = order_has_start(order) ? b : 0;
       lay.start_stride = 0;

@@ -13,12 +13,6 @@ namespace alamd {
 
 namespace {
 
-__device__ __forceinline__ void seg_range(const SegParams &s, unsigned seg, size_t &off, size_t &len) {
-  const unsigned long long sg = seg;
-  off = sg * s.seg_base + (sg < s.seg_rem ? sg : s.seg_rem);
-  len = s.seg_base + (sg < s.seg_rem ? 1u : 0u);
-}
-
 // Which outputs a segment writes, and at which byte offset.
 __device__ __forceinline__ void out_select(const SegParams &s, int P, unsigned seg, size_t off_bytes,
                                            int &j0, int &nj, size_t &out_bytes) {

@@ -8,12 +8,6 @@ namespace alamd {
 
 namespace {
 
-__device__ __forceinline__ void seg_range(const SegParams &s, unsigned seg, size_t &off, size_t &len) {
-  const unsigned long long sg = seg;
-  off = sg * s.seg_base + (sg < s.seg_rem ? sg : s.seg_rem);
-  len = s.seg_base + (sg < s.seg_rem ? 1u : 0u);
-}
-
 // The tree over one element position, one element per access.
 template <typename T, int OP, int SLOTS>
 __device__ __forceinline__ void tree_elem(const TreeParams &p, size_t in_bytes, int j0, int nj,

@@ -167,13 +167,8 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
     fp.out[r] = r < P ? static_cast<char *>(bufs[r]) : nullptr;
   }
   fp.P = P;
-  fp.seg.seg_base = count / (size_t)P;
-  fp.seg.seg_rem = count % (size_t)P;
-  fp.seg.tile0 = 0;
-  fp.seg.in_blocked = 1;
-  fp.seg.out_mode = all ? OUT_ALL : OUT_OWNER;
+  fp.seg = make_seg(count / (size_t)P, count % (size_t)P, 1, all ? OUT_ALL : OUT_OWNER, P);
   fp.seg.owner_shift = P - 1;
-  fp.seg.nout = P;
   fp.start0 = 0;
   fp.start_stride = 1;
   fp.dir = 1;
