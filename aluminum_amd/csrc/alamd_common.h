@@ -227,7 +227,7 @@ inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintp
 // A byte range as the copy kernels walk it: `head` bytes up to the source's
 // next 4-byte boundary, `vec` bytes in whole 128-bit vectors, `tail` < 16.
 struct ByteSplit { size_t head, vec, tail; };
-inline ByteSplit split_bytes(const void *src, size_t bytes) {
+__host__ __device__ inline ByteSplit split_bytes(const void *src, size_t bytes) {
   ByteSplit b;
   b.head = (4 - (reinterpret_cast<uintptr_t>(src) & 3)) & 3;
   if (b.head > bytes) b.head = bytes;

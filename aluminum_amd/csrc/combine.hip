@@ -95,63 +95,40 @@ int launch_order(void *const *outs, const void *const *ins, int P, const Layout 
 }
 
 constexpr int kGatherU = 8, kGatherThreads = 128;
-__global__ void __launch_bounds__(kGatherThreads) gather_kernel_vec(FoldParams p, size_t blk_bytes) {
-  // blockIdx.y = source rank q; every destination gets a copy at block q
+
+// Slices below kSpreadMinBytes: one launch for all of them.  blockIdx.y = source
+// rank q, whose slice of seg_len[q] bytes goes to byte offset seg_off[q] of
+// every receive buffer; a workgroup copies one tile of the slice to all P
+// destinations (at these sizes the launch, not the write pattern, decides).
+// A destination that is the source itself (in place) is skipped.
+__global__ void __launch_bounds__(kGatherThreads) gather_kernel(FoldParams p) {
   using TL = Tile<kGatherU, kGatherThreads>;
   const TL tl;
   const int q = blockIdx.y;
   const char *src = p.in[q];
+  const size_t off = p.seg.seg_off[q];
+  const ByteSplit b = split_bytes(src, p.seg.seg_len[q]);
+  if (blockIdx.x == 0 && threadIdx.x < b.head + b.tail) {
+    const size_t i = threadIdx.x < b.head ? threadIdx.x : b.vec + threadIdx.x;
+    const char c = src[i];
+    for (int r = 0; r < p.P; ++r) {
+      char *dst = p.out[r] + off;
+      if (dst != src) dst[i] = c;
+    }
+  }
   const size_t tb = (size_t)blockIdx.x * TL::BYTES;
-  if (tb >= blk_bytes) return;
-  const int nrec = blk_bytes - tb > TL::BYTES ? (int)TL::BYTES : (int)(blk_bytes - tb);
-  const auto rs = TL::rsrc(src + tb, nrec);
+  if (tb >= b.vec) return;
+  const int nrec = b.vec - tb > TL::BYTES ? (int)TL::BYTES : (int)(b.vec - tb);
+  const auto rs = TL::rsrc(src + b.head + tb, nrec);
   u32x4 v[kGatherU];
 #pragma unroll
   for (int u = 0; u < kGatherU; ++u) v[u] = tl.load(rs, u);
   for (int r = 0; r < p.P; ++r) {
-    char *dst = p.out[r] + (size_t)q * blk_bytes;
+    char *dst = p.out[r] + off;
     if (dst == src) continue;
-    const auto rd = TL::rsrc(dst + tb, nrec);
+    const auto rd = TL::rsrc(dst + b.head + tb, nrec);
 #pragma unroll
     for (int u = 0; u < kGatherU; ++u) tl.store(rd, u, v[u]);
-  }
-}
-
-__global__ void __launch_bounds__(256) gather_kernel_bytes(FoldParams p, size_t blk_bytes) {
-  const int q = blockIdx.y;
-  const char *src = p.in[q];
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < blk_bytes; i += (size_t)gridDim.x * 256) {
-    const char c = src[i];
-    for (int r = 0; r < p.P; ++r) {
-      char *dst = p.out[r] + (size_t)q * blk_bytes;
-      if (dst != src) dst[i] = c;
-    }
-  }
-}
-
-// One source block copied to up to P destinations (allgatherv).
-__global__ void __launch_bounds__(kGatherThreads) bcast_kernel_vec(const char *src, FoldParams p, size_t vec_bytes,
-                                                                   size_t tail_bytes) {
-  using TL = Tile<kGatherU, kGatherThreads>;
-  const TL tl;
-  const size_t tb = (size_t)blockIdx.x * TL::BYTES;
-  if (tb < vec_bytes) {
-    const int nrec = vec_bytes - tb > TL::BYTES ? (int)TL::BYTES : (int)(vec_bytes - tb);
-    const auto rs = TL::rsrc(src + tb, nrec);
-    u32x4 v[kGatherU];
-#pragma unroll
-    for (int u = 0; u < kGatherU; ++u) v[u] = tl.load(rs, u);
-    for (int r = 0; r < p.P; ++r) {
-      if (p.out[r] == src) continue;
-      const auto rd = TL::rsrc(p.out[r] + tb, nrec);
-#pragma unroll
-      for (int u = 0; u < kGatherU; ++u) tl.store(rd, u, v[u]);
-    }
-  }
-  if (blockIdx.x == 0 && threadIdx.x < tail_bytes) {
-    const char c = src[vec_bytes + threadIdx.x];
-    for (int r = 0; r < p.P; ++r)
-      if (p.out[r] != src) p.out[r][vec_bytes + threadIdx.x] = c;
   }
 }
 
@@ -223,6 +200,40 @@ int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, 
   hipLaunchKernelGGL(spread_kernel_vec, dim3((unsigned)blocks), dim3(kGatherThreads), 0, stream, src, fp, b,
                      (unsigned)tpc, (unsigned)tiles);
   ALAMD_HIP(hipGetLastError());
+  return ALAMD_OK;
+}
+
+// Copies slice q (lens[q] bytes at sends[q]) to byte offset offs[q] of every
+// recvs[r]: slices of kSpreadMinBytes and more one by one through the spread
+// kernel, all smaller ones in a single launch.
+int launch_gather(void *const *recvs, const void *const *sends, int P, const size_t *offs, const size_t *lens,
+                  hipStream_t stream) {
+  FoldParams fp;
+  fp.seg = make_seg(0, 0, 0, OUT_ALL, 0);
+  fp.P = P;
+  size_t max_small = 0;
+  for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
+    fp.in[r] = r < P ? static_cast<const char *>(sends[r]) : nullptr;
+    fp.out[r] = r < P ? static_cast<char *>(recvs[r]) : nullptr;
+  }
+  for (int q = 0; q < P; ++q) {
+    fp.seg.seg_off[q] = offs[q];
+    fp.seg.seg_len[q] = lens[q] < kSpreadMinBytes ? lens[q] : 0;
+    if (fp.seg.seg_len[q] > max_small) max_small = fp.seg.seg_len[q];
+    if (lens[q] < kSpreadMinBytes) continue;
+    char *dests[ALAMD_MAX_RANKS];
+    int nd = 0;
+    for (int r = 0; r < P; ++r)
+      if (fp.out[r] + offs[q] != fp.in[q]) dests[nd++] = fp.out[r] + offs[q];  // in place: already there
+    const int rc = launch_spread(fp.in[q], dests, nd, lens[q], stream);
+    if (rc) return rc;
+  }
+  if (max_small) {
+    const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
+    hipLaunchKernelGGL(gather_kernel, dim3((unsigned)((max_small + tile - 1) / tile), P, 1),
+                       dim3(kGatherThreads, 1, 1), 0, stream, fp);
+    ALAMD_HIP(hipGetLastError());
+  }
   return ALAMD_OK;
 }
 
@@ -352,13 +363,8 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
   if (!recvs || !sends) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
   if (count == 0) return ALAMD_OK;
   const size_t es = alamd_dtype_size(dtype), blk = count * es;
-  FoldParams fp;
-  for (int r = 0; r < ALAMD_MAX_RANKS; ++r) { fp.in[r] = nullptr; fp.out[r] = nullptr; }
-  for (int r = 0; r < P; ++r) {
+  for (int r = 0; r < P; ++r)
     if (!sends[r] || !recvs[r]) return set_error(ALAMD_ERR_INVALID_ARG, "buffer %d is null", r);
-    fp.in[r] = static_cast<const char *>(sends[r]);
-    fp.out[r] = static_cast<char *>(recvs[r]);
-  }
   for (int r = 0; r < P; ++r) {
     for (int q = 0; q < P; ++q) {
       const char *slot = static_cast<const char *>(recvs[r]) + (size_t)q * blk;
@@ -370,33 +376,9 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
       if (ranges_overlap(recvs[r], blk * (size_t)P, recvs[k], blk * (size_t)P))
         return set_error(ALAMD_ERR_OVERLAP, "receive buffers %d and %d overlap", k, r);
   }
-  fp.P = P;
-  hipStream_t st = as_stream(stream);
-  if (blk >= kSpreadMinBytes) {
-    // large slices: one launch per source, one destination stream at a time
-    for (int q = 0; q < P; ++q) {
-      char *dests[ALAMD_MAX_RANKS];
-      int nd = 0;
-      for (int r = 0; r < P; ++r) {
-        char *slot = fp.out[r] + (size_t)q * blk;
-        if (slot != fp.in[q]) dests[nd++] = slot;  // in place: rank q's own slice is already there
-      }
-      if ((rc = launch_spread(fp.in[q], dests, nd, blk, st))) return rc;
-    }
-    return ALAMD_OK;
-  } else if (blk % 16 == 0) {
-    const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
-    const size_t tiles = (blk + tile - 1) / tile;
-    if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
-    hipLaunchKernelGGL(gather_kernel_vec, dim3((unsigned)tiles, P, 1), dim3(kGatherThreads, 1, 1), 0, st, fp, blk);
-  } else {
-    unsigned per = (stream_grid((size_t)-1 / 2, 1, 8) + P - 1) / P;
-    unsigned gx = stream_grid(blk, 256, 8);
-    if (gx > per) gx = per < 1 ? 1 : per;
-    hipLaunchKernelGGL(gather_kernel_bytes, dim3(gx, P, 1), dim3(256, 1, 1), 0, st, fp, blk);
-  }
-  ALAMD_HIP(hipGetLastError());
-  return ALAMD_OK;
+  size_t offs[ALAMD_MAX_RANKS], lens[ALAMD_MAX_RANKS];
+  for (int q = 0; q < P; ++q) { offs[q] = (size_t)q * blk; lens[q] = blk; }
+  return launch_gather(recvs, sends, P, offs, lens, as_stream(stream));
 }
 
 int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, const size_t *counts, int dtype,
@@ -520,30 +502,9 @@ int alamd_allgatherv(void *const *recvs, const void *const *sends, int P, const 
       if (ranges_overlap(recvs[r], extent * es, recvs[k], extent * es))
         return set_error(ALAMD_ERR_OVERLAP, "receive buffers %d and %d overlap", k, r);
   }
-  hipStream_t st = as_stream(stream);
-  for (int q = 0; q < P; ++q) {
-    if (counts[q] == 0) continue;
-    const size_t bytes = counts[q] * es;
-    const char *src = static_cast<const char *>(sends[q]);
-    FoldParams fp;
-    for (int r = 0; r < ALAMD_MAX_RANKS; ++r) { fp.in[r] = nullptr; fp.out[r] = nullptr; }
-    for (int r = 0; r < P; ++r) fp.out[r] = static_cast<char *>(recvs[r]) + displs[q] * es;
-    fp.P = P;
-    if (bytes >= kSpreadMinBytes) {
-      char *dests[ALAMD_MAX_RANKS];
-      int nd = 0;
-      for (int r = 0; r < P; ++r)
-        if (fp.out[r] != src) dests[nd++] = fp.out[r];
-      if ((rc = launch_spread(src, dests, nd, bytes, st))) return rc;
-    } else {
-      const size_t vec_bytes = bytes & ~(size_t)15, tile = Tile<kGatherU, kGatherThreads>::BYTES;
-      const size_t tiles = (vec_bytes + tile - 1) / tile;
-      hipLaunchKernelGGL(bcast_kernel_vec, dim3((unsigned)(tiles ? tiles : 1)), dim3(kGatherThreads), 0, st, src, fp,
-                         vec_bytes, bytes - vec_bytes);
-    }
-    ALAMD_HIP(hipGetLastError());
-  }
-  return ALAMD_OK;
+  size_t offs[ALAMD_MAX_RANKS], lens[ALAMD_MAX_RANKS];
+  for (int q = 0; q < P; ++q) { offs[q] = displs[q] * es; lens[q] = counts[q] * es; }
+  return launch_gather(recvs, sends, P, offs, lens, as_stream(stream));
 }
 
 }  // extern "C"
