@@ -322,3 +322,54 @@ def test_combine_in_a_hip_graph(al):
         torch.cuda.synchronize()
         want = oracle.combine(fresh, "f32", "sum", "tree_dbl")
         assert_bits_equal(to_host(out, np.float32), want, "f32", "graph replay %d" % rep)
+
+
+def test_collectives_in_a_hip_graph(al):
+    """An allreduce to every rank (fold + spread), a Reduce_scatterv (ragged segments), an Allgatherv
+    (spread for the large slice, the table-driven kernel for the small ones) and a fused ring captured
+    into one graph; every replay, with fresh inputs, gives what the oracle gives."""
+    import torch
+    P, n = 4, (1 << 19) + 36
+    counts = [300000, 0, 5, n - 300005]
+    displs = [0, 300000, 300000, 300005]
+    ins = [dev_empty(n, np.float32) for _ in range(P)]
+    all_out = [dev_empty(n, np.float32) for _ in range(P)]
+    rs_out = [dev_empty(max(c, 1), np.float32) for c in counts]
+    ag_out = [dev_empty(n, np.float32) for _ in range(P)]
+    ring = [dev_empty(n, np.float32) for _ in range(P)]
+
+    def run():
+        al.combine(all_out, ins, "sum", order="tree_dbl")
+        al.reduce_scatterv(rs_out, ins, counts, "sum", order="pairwise_desc")
+        al.allgatherv(ag_out, rs_out, counts, displs)
+        for r in range(P):
+            al.copy(ring[r], ins[r])
+        al.ring_allreduce(ring, "sum", mode="fused")
+
+    fresh = make_inputs(P, n, "f32", "sum", seed=900)
+    for t, a in zip(ins, fresh):
+        t.copy_(torch.from_numpy(a))
+    run()  # eager warm-up outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        run()
+    for rep in range(3):
+        fresh = make_inputs(P, n, "f32", "sum", seed=910 + 10 * rep)
+        for t, a in zip(ins, fresh):
+            t.copy_(torch.from_numpy(a))
+        for t in all_out + ag_out + ring:
+            t.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        want_all = oracle.combine(fresh, "f32", "sum", "tree_dbl")
+        want_rs = oracle.reduce_scatterv(fresh, counts, "f32", "sum", "pairwise_desc")
+        want_ag = np.concatenate([want_rs[q][:counts[q]] for q in range(P)])
+        want_ring = oracle.ring_allreduce(fresh, "f32", "sum", (4 << 20) // 4)[0]
+        for r in range(P):
+            assert_bits_equal(to_host(all_out[r], np.float32), want_all, "f32", "replay %d allreduce rank %d" % (rep, r))
+            assert_bits_equal(to_host(rs_out[r], np.float32)[:counts[r]], want_rs[r][:counts[r]], "f32",
+                              "replay %d reduce_scatterv rank %d" % (rep, r))
+            assert_bits_equal(to_host(ag_out[r], np.float32), want_ag, "f32", "replay %d allgatherv rank %d" % (rep, r))
+            assert_bits_equal(to_host(ring[r], np.float32), want_ring, "f32", "replay %d ring rank %d" % (rep, r))
