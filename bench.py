@@ -293,7 +293,21 @@ def c2_port_sample():
         return {"error": str(e)[:200]}
 
 
-def cpu_baseline():
+def c1_gpu_checksum(al, torch):
+    """C1 on the GPU: the combine of the same four generated 2^20-element buffers, in the order
+    MPI_Allreduce applies above 2 KiB; returns the oracle's checksum of the result."""
+    import oracle
+    n, ranks = 1 << 20, 4
+    ins = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(ranks)]
+    out = torch.empty(n, dtype=torch.float32, device="cuda")
+    for r in range(ranks):
+        al.fill(ins[r], "uniform_pm1", 1000 + r)
+    al.combine([out], ins, "sum", order="tree_dbl")
+    torch.cuda.synchronize()
+    return "%016x" % oracle.checksum(out.cpu().numpy())
+
+
+def cpu_baseline(al=None, torch=None):
     """The reference's MPI-backend host combine on this box's host cores."""
     exe = os.path.join(ROOT, "oracle", "mpi_baseline")
     mpiexec = "/opt/conda/bin/mpiexec"
@@ -304,12 +318,16 @@ def cpu_baseline():
             line = [l for l in p.stdout.splitlines() if l.startswith("{")]
             if p.returncode == 0 and line:
                 r = json.loads(line[-1])
+                same = None
+                if al is not None and "checksum" in r:
+                    # the bits MPI_Allreduce produced on the host against the GPU's for the same inputs
+                    same = c1_gpu_checksum(al, torch) == r["checksum"]
                 return {"value": r["gbps_median"], "unit": "GB/s", "cores": 4, "kind": "port",
                         "sample": "MPI_Allreduce(MPI_SUM, MPI_FLOAT) on a dup'd communicator, the call "
                                   "Al::Allreduce<MPIBackend> forwards to; 4 MPICH ranks on this host, "
                                   "2^20 elements per rank, uniform[-1,1] seed 1000+rank, 10 warm-up + 3000 "
                                   "timed (about 10 s), median of max-over-ranks; GB/s over (P+1)*n*4 bytes",
-                        "median_ms": r["median_ms"], "min_ms": r["min_ms"],
+                        "median_ms": r["median_ms"], "min_ms": r["min_ms"], "gpu_result_identical": same,
                         "host_cpus": os.cpu_count(), "same_workload_port": c2_port_sample()}
         except Exception:
             pass
@@ -414,7 +432,7 @@ def main():
         "also": also,
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"] = cpu_baseline(al, torch)
     print(json.dumps(out))
 
 
