@@ -100,3 +100,31 @@ def test_reduce_scatterv_vectors_on_the_gpu(al, path):
         for b in range(P):
             want = arr(c["out"][b], dt)[:counts[b]]
             assert_bits_equal(to_host(d_recvs[b], npdt)[:counts[b]], want, dt, "reduce_scatterv P=%d rank %d" % (P, b))
+
+
+MPIEXEC = "/opt/conda/bin/mpiexec"
+MPI_PROGRAM = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "mpi_baseline")
+
+
+@pytest.mark.skipif(not (os.path.exists(MPIEXEC) and os.path.exists(MPI_PROGRAM)),
+                    reason="needs mpiexec and the built oracle/mpi_baseline")
+@pytest.mark.parametrize("P", (2, 3, 5, 8))
+def test_live_mpi_allreduce_against_the_gpu(al, P):
+    """MPI_Allreduce(MPI_SUM, MPI_FLOAT) run now, on this machine's host cores, over generated inputs
+    (uniform[-1,1), seed 1000+rank), against the GPU's combine of the same inputs: equal checksums."""
+    import subprocess
+    import torch
+    for n in (300, 513, (1 << 16) + 1, 1 << 20):
+        p = subprocess.run([MPIEXEC, "-n", str(P), MPI_PROGRAM, str(n), "0", "1"], capture_output=True, text=True,
+                           timeout=120)
+        line = [l for l in p.stdout.splitlines() if l.startswith("{")]
+        assert p.returncode == 0 and line, (p.stdout, p.stderr)
+        want = json.loads(line[-1])["checksum"]
+        ins = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(P)]
+        out = torch.empty(n, dtype=torch.float32, device="cuda")
+        for r in range(P):
+            al.fill(ins[r], "uniform_pm1", 1000 + r)
+        order = "tree_binomial" if n * 4 <= 2048 else "tree_dbl"
+        al.combine([out], ins, "sum", order=order)
+        torch.cuda.synchronize()
+        assert "%016x" % oracle.checksum(out.cpu().numpy()) == want, "P=%d n=%d" % (P, n)
