@@ -136,7 +136,10 @@ __global__ void __launch_bounds__(kGatherThreads) gather_kernel(FoldParams p) {
 // Block ids run chunk by chunk (tpc tiles, 8 MiB); inside a chunk all tiles of
 // destination 0 come first, then destination 1, ...: at any time the device
 // writes one contiguous stream per chunk instead of P interleaved ones, and
-// re-reads the chunk of the source from cache.  Measured for 1 read + 8 writes
+// re-reads the chunk of the source from cache (workgroups are dealt to the eight
+// XCDs round-robin and tpc is a multiple of 8, so the workgroups that copy one
+// source tile to the different destinations run on the same XCD and share its
+// L2).  Measured for 1 read + 8 writes
 // of 32 MiB: 88 % of the HBM peak, against 67 % when every workgroup writes
 // its tile to all destinations (69 % for those writes alone).
 constexpr unsigned kSpreadChunkTiles = 512;
