@@ -96,78 +96,51 @@ int launch_order(void *const *outs, const void *const *ins, int P, const Layout 
 
 constexpr int kGatherU = 8, kGatherThreads = 128;
 
-// Slices below kSpreadMinBytes: one launch for all of them.  blockIdx.y = source
-// rank q, whose slice of seg_len[q] bytes goes to byte offset seg_off[q] of
-// every receive buffer; a workgroup copies one tile of the slice to all P
-// destinations (at these sizes the launch, not the write pattern, decides).
-// A destination that is the source itself (in place) is skipped.
-__global__ void __launch_bounds__(kGatherThreads) gather_kernel(FoldParams p) {
+// Slices to several destinations: blockIdx.y = source q, whose seg_len[q] bytes
+// go to byte offset seg_off[q] of every destination p.out[0..P) (a destination
+// that is the source itself, the in-place form, is skipped).  One workgroup
+// per (destination, tile).  blockIdx.x runs chunk by chunk (tpc tiles, 8 MiB);
+// inside a chunk all tiles of destination 0 come first, then destination 1,
+// ...: at any time the device writes one contiguous stream per chunk instead
+// of P interleaved ones, and re-reads the chunk of the source from cache:
+// workgroups are dealt to the eight XCDs round-robin and tpc is a multiple of
+// 8, so the workgroups that copy one source tile to the different destinations
+// run on the same XCD and share its L2 (88 % of peak; 79 % with tpc a multiple
+// of 4 only, 49 % with an odd tpc).  Measured for 1 read + 8 writes of 32 MiB:
+// 88 % of the HBM peak, against 67 % when every workgroup writes its tile to
+// all destinations (69 % for those writes alone).
+constexpr unsigned kSpreadChunkTiles = 512;
+__global__ void __launch_bounds__(kGatherThreads) spread_kernel(FoldParams p, unsigned tpc) {
   using TL = Tile<kGatherU, kGatherThreads>;
   const TL tl;
   const int q = blockIdx.y;
   const char *src = p.in[q];
   const size_t off = p.seg.seg_off[q];
   const ByteSplit b = split_bytes(src, p.seg.seg_len[q]);
-  if (blockIdx.x == 0 && threadIdx.x < b.head + b.tail) {
-    const size_t i = threadIdx.x < b.head ? threadIdx.x : b.vec + threadIdx.x;
-    const char c = src[i];
-    for (int r = 0; r < p.P; ++r) {
-      char *dst = p.out[r] + off;
-      if (dst != src) dst[i] = c;
-    }
-  }
-  const size_t tb = (size_t)blockIdx.x * TL::BYTES;
-  if (tb >= b.vec) return;
-  const int nrec = b.vec - tb > TL::BYTES ? (int)TL::BYTES : (int)(b.vec - tb);
-  const auto rs = TL::rsrc(src + b.head + tb, nrec);
-  u32x4 v[kGatherU];
-#pragma unroll
-  for (int u = 0; u < kGatherU; ++u) v[u] = tl.load(rs, u);
-  for (int r = 0; r < p.P; ++r) {
-    char *dst = p.out[r] + off;
-    if (dst == src) continue;
-    const auto rd = TL::rsrc(dst + b.head + tb, nrec);
-#pragma unroll
-    for (int u = 0; u < kGatherU; ++u) tl.store(rd, u, v[u]);
-  }
-}
-
-// One source region to p.P destinations, one workgroup per (destination, tile).
-// Block ids run chunk by chunk (tpc tiles, 8 MiB); inside a chunk all tiles of
-// destination 0 come first, then destination 1, ...: at any time the device
-// writes one contiguous stream per chunk instead of P interleaved ones, and
-// re-reads the chunk of the source from cache (workgroups are dealt to the eight
-// XCDs round-robin and tpc is a multiple of 8, so the workgroups that copy one
-// source tile to the different destinations run on the same XCD and share its
-// L2).  Measured for 1 read + 8 writes
-// of 32 MiB: 88 % of the HBM peak, against 67 % when every workgroup writes
-// its tile to all destinations (69 % for those writes alone).
-constexpr unsigned kSpreadChunkTiles = 512;
-__global__ void __launch_bounds__(kGatherThreads) spread_kernel_vec(const char *src, FoldParams p, ByteSplit b,
-                                                                    unsigned tpc, unsigned tiles) {
-  using TL = Tile<kGatherU, kGatherThreads>;
-  const TL tl;
   const unsigned ndest = (unsigned)p.P;
-  const unsigned per_chunk = tpc * ndest;
-  const unsigned chunk = blockIdx.x / per_chunk, rem = blockIdx.x % per_chunk;
-  const unsigned dest = rem / tpc, tile = chunk * tpc + rem % tpc;
-  if (tile < tiles) {
-    const size_t tb = (size_t)tile * TL::BYTES;
-    const int nrec = b.vec - tb > TL::BYTES ? (int)TL::BYTES : (int)(b.vec - tb);
-    const auto rs = TL::rsrc(src + b.head + tb, nrec);
-    const auto rd = TL::rsrc(p.out[dest] + b.head + tb, nrec);
-    u32x4 v[kGatherU];
-#pragma unroll
-    for (int u = 0; u < kGatherU; ++u) v[u] = tl.load_cached(rs, u);
-#pragma unroll
-    for (int u = 0; u < kGatherU; ++u) tl.store_nt(rd, u, v[u]);
-  }
   // the bytes before the first and after the last whole vector
   if (blockIdx.x == 0 && threadIdx.x < b.head + b.tail) {
     const size_t i = threadIdx.x < b.head ? threadIdx.x : b.vec + threadIdx.x;
     const char c = src[i];
-    for (unsigned r = 0; r < ndest; ++r) p.out[r][i] = c;
+    for (unsigned r = 0; r < ndest; ++r) {
+      char *dst = p.out[r] + off;
+      if (dst != src) dst[i] = c;
+    }
   }
+  const unsigned per_chunk = tpc * ndest;
+  const unsigned chunk = blockIdx.x / per_chunk, rem = blockIdx.x % per_chunk;
+  const unsigned dest = rem / tpc;
+  const size_t tb = ((size_t)chunk * tpc + rem % tpc) * TL::BYTES;
+  char *dst = p.out[dest] + off;
+  if (tb >= b.vec || dst == src) return;
+  const int nrec = b.vec - tb > TL::BYTES ? (int)TL::BYTES : (int)(b.vec - tb);
+  const auto rs = TL::rsrc(src + b.head + tb, nrec);
+  const auto rd = TL::rsrc(dst + b.head + tb, nrec);
+  u32x4 v[kGatherU];
+#pragma unroll
+  for (int u = 0; u < kGatherU; ++u) v[u] = tl.load_cached(rs, u);
+#pragma unroll
+  for (int u = 0; u < kGatherU; ++u) tl.store_nt(rd, u, v[u]);
 }
 
 int misaligned(const char *what, int index) {
@@ -182,63 +155,73 @@ int check_common(int P, size_t count, int dtype) {
   return ALAMD_OK;
 }
 
+// fp.in[q], fp.out[r], fp.P (destinations), fp.seg.seg_off / seg_len (bytes) set for nsrc sources.
+int launch_spread_table(const FoldParams &fp, int nsrc, hipStream_t stream) {
+  size_t max_len = 0;
+  for (int q = 0; q < nsrc; ++q)
+    if (fp.seg.seg_len[q] > max_len) max_len = fp.seg.seg_len[q];
+  if (max_len == 0 || fp.P <= 0) return ALAMD_OK;
+  const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
+  const size_t tiles = (max_len + tile - 1) / tile;
+  // always a multiple of 8 (see spread_kernel); workgroups past the last tile exit at once
+  const size_t tpc = tiles < kSpreadChunkTiles ? (tiles + 7) & ~(size_t)7 : kSpreadChunkTiles;
+  const size_t chunks = (tiles + tpc - 1) / tpc;
+  const size_t blocks = chunks * tpc * (size_t)fp.P;
+  if (blocks > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
+  hipLaunchKernelGGL(spread_kernel, dim3((unsigned)blocks, (unsigned)nsrc, 1), dim3(kGatherThreads, 1, 1), 0, stream,
+                     fp, (unsigned)tpc);
+  ALAMD_HIP(hipGetLastError());
+  return ALAMD_OK;
+}
+
 }  // namespace
 
 int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, hipStream_t stream) {
   if (ndest <= 0 || bytes == 0) return ALAMD_OK;
   FoldParams fp;
+  fp.seg = make_seg(0, 0, 0, OUT_ALL, 0);
   for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
     fp.in[r] = nullptr;
     fp.out[r] = r < ndest ? dests[r] : nullptr;
   }
+  fp.in[0] = src;
   fp.P = ndest;
-  const ByteSplit b = split_bytes(src, bytes);
-  const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
-  size_t tiles = (b.vec + tile - 1) / tile;
-  if (tiles == 0) tiles = 1;
-  const size_t tpc = tiles < kSpreadChunkTiles ? tiles : kSpreadChunkTiles;
-  const size_t chunks = (tiles + tpc - 1) / tpc;
-  const size_t blocks = chunks * tpc * (size_t)ndest;
-  if (blocks > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
-  hipLaunchKernelGGL(spread_kernel_vec, dim3((unsigned)blocks), dim3(kGatherThreads), 0, stream, src, fp, b,
-                     (unsigned)tpc, (unsigned)tiles);
-  ALAMD_HIP(hipGetLastError());
-  return ALAMD_OK;
+  fp.seg.seg_len[0] = bytes;
+  return launch_spread_table(fp, 1, stream);
 }
 
-// Copies slice q (lens[q] bytes at sends[q]) to byte offset offs[q] of every
-// recvs[r]: slices of kSpreadMinBytes and more one by one through the spread
-// kernel, all smaller ones in a single launch.
+namespace {
+
+// Copies slice q (lens[q] bytes at sends[q]) to byte offset offs[q] of every recvs[r].  Slices of two
+// chunks (16 MiB) and more get a launch each - one launch over all of them is long enough for the XCDs
+// to drift apart (32 MiB slices: 88 % of peak one by one, 83 % together) - the smaller ones share one
+// (8 MiB slices: 85 us together, 98 us one by one; 1 MiB slices: 15 us against 43 us).
 int launch_gather(void *const *recvs, const void *const *sends, int P, const size_t *offs, const size_t *lens,
                   hipStream_t stream) {
   FoldParams fp;
   fp.seg = make_seg(0, 0, 0, OUT_ALL, 0);
   fp.P = P;
-  size_t max_small = 0;
   for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
     fp.in[r] = r < P ? static_cast<const char *>(sends[r]) : nullptr;
     fp.out[r] = r < P ? static_cast<char *>(recvs[r]) : nullptr;
   }
+  const size_t big = 2 * (size_t)kSpreadChunkTiles * Tile<kGatherU, kGatherThreads>::BYTES;
   for (int q = 0; q < P; ++q) {
     fp.seg.seg_off[q] = offs[q];
-    fp.seg.seg_len[q] = lens[q] < kSpreadMinBytes ? lens[q] : 0;
-    if (fp.seg.seg_len[q] > max_small) max_small = fp.seg.seg_len[q];
-    if (lens[q] < kSpreadMinBytes) continue;
-    char *dests[ALAMD_MAX_RANKS];
-    int nd = 0;
-    for (int r = 0; r < P; ++r)
-      if (fp.out[r] + offs[q] != fp.in[q]) dests[nd++] = fp.out[r] + offs[q];  // in place: already there
-    const int rc = launch_spread(fp.in[q], dests, nd, lens[q], stream);
+    fp.seg.seg_len[q] = lens[q];
+    if (lens[q] < big) continue;
+    FoldParams one = fp;
+    one.in[0] = fp.in[q];
+    one.seg.seg_off[0] = offs[q];
+    one.seg.seg_len[0] = lens[q];
+    const int rc = launch_spread_table(one, 1, stream);
     if (rc) return rc;
+    fp.seg.seg_len[q] = 0;
   }
-  if (max_small) {
-    const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
-    hipLaunchKernelGGL(gather_kernel, dim3((unsigned)((max_small + tile - 1) / tile), P, 1),
-                       dim3(kGatherThreads, 1, 1), 0, stream, fp);
-    ALAMD_HIP(hipGetLastError());
-  }
-  return ALAMD_OK;
+  return launch_spread_table(fp, P, stream);
 }
+
+}  // namespace
 
 }  // namespace alamd
 
