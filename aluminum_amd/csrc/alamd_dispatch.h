@@ -132,9 +132,19 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
 int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, int dtype, int op,
                 hipStream_t stream);
 
+// A result that goes to several buffers is folded into one of them and then
+// spread (one write stream per workgroup) when that is faster than writing
+// every tile to all of them from the fold kernel: from three outputs and 40 MiB
+// up (measured at P = 8: 32 MiB 81 us in one kernel / 86 us in two steps, 48 MiB
+// 146 / 128, 256 MiB 773 / 667; two outputs 437 / 455, four 544 / 529).
+constexpr size_t kTwoStepMinBytes = (size_t)40 << 20;
+constexpr int kTwoStepMinOutputs = 3;
+
 // Copies [src, src + bytes) to each of dests[0..ndest) (none overlapping the
-// source, any alignment); used where one result goes to several buffers.
-constexpr size_t kSpreadMinBytes = (size_t)1 << 20;  // below this the all-in-one kernels are used
+// source, any alignment).
 int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, hipStream_t stream);
+// The general form: source q = fp.in[q], fp.seg.seg_len[q] bytes, copied to byte offset
+// fp.seg.seg_off[q] of every fp.out[0..fp.P) except where that is the source itself.
+int launch_spread_table(const FoldParams &fp, int nsrc, hipStream_t stream);
 
 }  // namespace alamd

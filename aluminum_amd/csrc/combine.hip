@@ -155,7 +155,8 @@ int check_common(int P, size_t count, int dtype) {
   return ALAMD_OK;
 }
 
-// fp.in[q], fp.out[r], fp.P (destinations), fp.seg.seg_off / seg_len (bytes) set for nsrc sources.
+}  // namespace
+
 int launch_spread_table(const FoldParams &fp, int nsrc, hipStream_t stream) {
   size_t max_len = 0;
   for (int q = 0; q < nsrc; ++q)
@@ -173,8 +174,6 @@ int launch_spread_table(const FoldParams &fp, int nsrc, hipStream_t stream) {
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
 }
-
-}  // namespace
 
 int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, hipStream_t stream) {
   if (ndest <= 0 || bytes == 0) return ALAMD_OK;
@@ -264,7 +263,7 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   lay.max_len = count;
   lay.start0 = start;
   lay.start_stride = 0;
-  if (nout == 1 || bytes < kSpreadMinBytes)
+  if (nout < kTwoStepMinOutputs || bytes < kTwoStepMinBytes)
     return launch_order(out_tab, ins, P, lay, dtype, op, order, as_stream(stream));
   // Several outputs of a large result: a workgroup that wrote its tile to every
   // output would interleave nout write streams (measured 69 % of peak).  Instead

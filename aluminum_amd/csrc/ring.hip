@@ -15,6 +15,8 @@ namespace alamd {
 namespace {
 
 constexpr int kThreads = 256;
+// fused allreduce: segments of this size and more are folded and spread one by one
+constexpr size_t kRingSegmentwiseMinBytes = (size_t)16 << 20;
 
 struct RingParams {
   char *buf[ALAMD_MAX_RANKS];
@@ -175,12 +177,38 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   const size_t max_len = fp.seg.seg_base + (fp.seg.seg_rem ? 1 : 0);
   if (max_len == 0) return ALAMD_OK;
   const size_t es = alamd_dtype_size(dtype);
-  if (!all || fp.seg.seg_base * es < kSpreadMinBytes)
+  if (!all || P < kTwoStepMinOutputs || count * es < kTwoStepMinBytes)
     return launch_fold(fp, (unsigned)P, max_len, dtype, op, true, stream);
-  // Large allreduce: segment by segment, fold into the owner's buffer (what the
-  // reduce-scatter leaves there), then spread the segment from the owner to the
-  // other ranks while it is still in cache.  Writing each result tile to all P
-  // buffers from one workgroup interleaves P write streams and is slower.
+  // Large allreduce.  Writing each result tile to all P buffers from the fold
+  // kernel interleaves P write streams; instead every segment is folded into
+  // its owner's buffer (what the reduce-scatter leaves there) and then spread
+  // from the owner to the other ranks.
+  auto seg_off = [&](int s) {
+    const size_t sg = (size_t)s, rem = (size_t)fp.seg.seg_rem;
+    return (sg * fp.seg.seg_base + (sg < rem ? sg : rem)) * es;
+  };
+  auto seg_len = [&](int s) { return fp.seg.seg_base + ((size_t)s < fp.seg.seg_rem ? 1 : 0); };
+  if (max_len * es < kRingSegmentwiseMinBytes) {
+    // one launch folds all segments, one launch spreads them all
+    FoldParams fo = fp;
+    fo.seg.out_mode = OUT_OWNER;
+    int rc = launch_fold(fo, (unsigned)P, max_len, dtype, op, true, stream);
+    if (rc) return rc;
+    FoldParams sp;
+    sp.seg = make_seg(0, 0, 0, OUT_ALL, 0);
+    sp.P = P;
+    for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
+      sp.in[r] = nullptr;
+      sp.out[r] = r < P ? static_cast<char *>(bufs[r]) : nullptr;
+    }
+    for (int s = 0; s < P; ++s) {
+      sp.in[s] = static_cast<const char *>(bufs[(s + P - 1) % P]) + seg_off(s);
+      sp.seg.seg_off[s] = seg_off(s);
+      sp.seg.seg_len[s] = seg_len(s) * es;
+    }
+    return launch_spread_table(sp, P, stream);
+  }
+  // larger segments one by one, so that the spread reads the segment while it is still in cache
   FoldParams fs = fp;
   fs.seg.seg_rem = 0;
   fs.seg.in_blocked = 0;
@@ -188,9 +216,7 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   fs.seg.nout = 1;
   fs.start_stride = 0;
   for (int s = 0; s < P; ++s) {
-    const size_t sg = (size_t)s, rem = (size_t)fp.seg.seg_rem;
-    const size_t off = (sg * fp.seg.seg_base + (sg < rem ? sg : rem)) * es;
-    const size_t len = fp.seg.seg_base + (sg < rem ? 1 : 0);
+    const size_t off = seg_off(s), len = seg_len(s);
     const int owner = (s + P - 1) % P;
     for (int r = 0; r < P; ++r) fs.in[r] = static_cast<const char *>(bufs[r]) + off;
     fs.out[0] = static_cast<char *>(bufs[owner]) + off;
