@@ -145,6 +145,7 @@ constexpr int kTwoStepMinOutputs = 3;
 int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, hipStream_t stream);
 // The general form: source q = fp.in[q], fp.seg.seg_len[q] bytes, copied to byte offset
 // fp.seg.seg_off[q] of every fp.out[0..fp.P) except where that is the source itself.
-int launch_spread_table(const FoldParams &fp, int nsrc, hipStream_t stream);
+// split_large: give every slice of 16 MiB and more a launch of its own.
+int launch_spread_table(const FoldParams &fp, int nsrc, bool split_large, hipStream_t stream);
 
 }  // namespace alamd

@@ -157,7 +157,9 @@ int check_common(int P, size_t count, int dtype) {
 
 }  // namespace
 
-int launch_spread_table(const FoldParams &fp, int nsrc, hipStream_t stream) {
+namespace {
+
+int launch_spread_once(const FoldParams &fp, int nsrc, hipStream_t stream) {
   size_t max_len = 0;
   for (int q = 0; q < nsrc; ++q)
     if (fp.seg.seg_len[q] > max_len) max_len = fp.seg.seg_len[q];
@@ -175,6 +177,29 @@ int launch_spread_table(const FoldParams &fp, int nsrc, hipStream_t stream) {
   return ALAMD_OK;
 }
 
+}  // namespace
+
+// split_large: slices of two chunks (16 MiB) and more get a launch each, the smaller ones share one.
+// For an allgather of separate send buffers one launch over large slices is long enough for the XCDs to
+// drift apart (32 MiB slices: 88 % of peak one by one, 83 % together; 8 MiB slices: 85 us together,
+// 98 us one by one; 1 MiB: 15 us against 43 us).  Segments that a fold has just written are spread
+// faster in one launch (eight 32 MiB segments: 650 us for the whole allreduce against 667 us).
+int launch_spread_table(const FoldParams &fp, int nsrc, bool split_large, hipStream_t stream) {
+  const size_t big = 2 * (size_t)kSpreadChunkTiles * Tile<kGatherU, kGatherThreads>::BYTES;
+  FoldParams rest = fp;
+  for (int q = 0; q < nsrc && nsrc > 1 && split_large; ++q) {
+    if (fp.seg.seg_len[q] < big) continue;
+    FoldParams one = fp;
+    one.in[0] = fp.in[q];
+    one.seg.seg_off[0] = fp.seg.seg_off[q];
+    one.seg.seg_len[0] = fp.seg.seg_len[q];
+    const int rc = launch_spread_once(one, 1, stream);
+    if (rc) return rc;
+    rest.seg.seg_len[q] = 0;
+  }
+  return launch_spread_once(rest, nsrc, stream);
+}
+
 int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, hipStream_t stream) {
   if (ndest <= 0 || bytes == 0) return ALAMD_OK;
   FoldParams fp;
@@ -186,15 +211,12 @@ int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, 
   fp.in[0] = src;
   fp.P = ndest;
   fp.seg.seg_len[0] = bytes;
-  return launch_spread_table(fp, 1, stream);
+  return launch_spread_table(fp, 1, false, stream);
 }
 
 namespace {
 
-// Copies slice q (lens[q] bytes at sends[q]) to byte offset offs[q] of every recvs[r].  Slices of two
-// chunks (16 MiB) and more get a launch each - one launch over all of them is long enough for the XCDs
-// to drift apart (32 MiB slices: 88 % of peak one by one, 83 % together) - the smaller ones share one
-// (8 MiB slices: 85 us together, 98 us one by one; 1 MiB slices: 15 us against 43 us).
+// Copies slice q (lens[q] bytes at sends[q]) to byte offset offs[q] of every recvs[r].
 int launch_gather(void *const *recvs, const void *const *sends, int P, const size_t *offs, const size_t *lens,
                   hipStream_t stream) {
   FoldParams fp;
@@ -204,20 +226,11 @@ int launch_gather(void *const *recvs, const void *const *sends, int P, const siz
     fp.in[r] = r < P ? static_cast<const char *>(sends[r]) : nullptr;
     fp.out[r] = r < P ? static_cast<char *>(recvs[r]) : nullptr;
   }
-  const size_t big = 2 * (size_t)kSpreadChunkTiles * Tile<kGatherU, kGatherThreads>::BYTES;
   for (int q = 0; q < P; ++q) {
     fp.seg.seg_off[q] = offs[q];
     fp.seg.seg_len[q] = lens[q];
-    if (lens[q] < big) continue;
-    FoldParams one = fp;
-    one.in[0] = fp.in[q];
-    one.seg.seg_off[0] = offs[q];
-    one.seg.seg_len[0] = lens[q];
-    const int rc = launch_spread_table(one, 1, stream);
-    if (rc) return rc;
-    fp.seg.seg_len[q] = 0;
   }
-  return launch_spread_table(fp, P, stream);
+  return launch_spread_table(fp, P, true, stream);
 }
 
 }  // namespace

@@ -15,8 +15,6 @@ namespace alamd {
 namespace {
 
 constexpr int kThreads = 256;
-// fused allreduce: segments of this size and more are folded and spread one by one
-constexpr size_t kRingSegmentwiseMinBytes = (size_t)16 << 20;
 
 struct RingParams {
   char *buf[ALAMD_MAX_RANKS];
@@ -188,49 +186,24 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
     return (sg * fp.seg.seg_base + (sg < rem ? sg : rem)) * es;
   };
   auto seg_len = [&](int s) { return fp.seg.seg_base + ((size_t)s < fp.seg.seg_rem ? 1 : 0); };
-  if (max_len * es < kRingSegmentwiseMinBytes) {
-    // one launch folds all segments, one launch spreads them all
-    FoldParams fo = fp;
-    fo.seg.out_mode = OUT_OWNER;
-    int rc = launch_fold(fo, (unsigned)P, max_len, dtype, op, true, stream);
-    if (rc) return rc;
-    FoldParams sp;
-    sp.seg = make_seg(0, 0, 0, OUT_ALL, 0);
-    sp.P = P;
-    for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
-      sp.in[r] = nullptr;
-      sp.out[r] = r < P ? static_cast<char *>(bufs[r]) : nullptr;
-    }
-    for (int s = 0; s < P; ++s) {
-      sp.in[s] = static_cast<const char *>(bufs[(s + P - 1) % P]) + seg_off(s);
-      sp.seg.seg_off[s] = seg_off(s);
-      sp.seg.seg_len[s] = seg_len(s) * es;
-    }
-    return launch_spread_table(sp, P, stream);
+  // one launch folds all segments (8 reads + 1 write), then the segments are spread
+  FoldParams fo = fp;
+  fo.seg.out_mode = OUT_OWNER;
+  const int rc = launch_fold(fo, (unsigned)P, max_len, dtype, op, true, stream);
+  if (rc) return rc;
+  FoldParams sp;
+  sp.seg = make_seg(0, 0, 0, OUT_ALL, 0);
+  sp.P = P;
+  for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
+    sp.in[r] = nullptr;
+    sp.out[r] = r < P ? static_cast<char *>(bufs[r]) : nullptr;
   }
-  // larger segments one by one, so that the spread reads the segment while it is still in cache
-  FoldParams fs = fp;
-  fs.seg.seg_rem = 0;
-  fs.seg.in_blocked = 0;
-  fs.seg.out_mode = OUT_ALL;
-  fs.seg.nout = 1;
-  fs.start_stride = 0;
   for (int s = 0; s < P; ++s) {
-    const size_t off = seg_off(s), len = seg_len(s);
-    const int owner = (s + P - 1) % P;
-    for (int r = 0; r < P; ++r) fs.in[r] = static_cast<const char *>(bufs[r]) + off;
-    fs.out[0] = static_cast<char *>(bufs[owner]) + off;
-    fs.start0 = s;
-    fs.seg.seg_base = len;
-    int rc = launch_fold(fs, 1, len, dtype, op, true, stream);
-    if (rc) return rc;
-    char *dests[ALAMD_MAX_RANKS];
-    int nd = 0;
-    for (int r = 0; r < P; ++r)
-      if (r != owner) dests[nd++] = static_cast<char *>(bufs[r]) + off;
-    if ((rc = launch_spread(fs.out[0], dests, nd, len * es, stream))) return rc;
+    sp.in[s] = static_cast<const char *>(bufs[(s + P - 1) % P]) + seg_off(s);
+    sp.seg.seg_off[s] = seg_off(s);
+    sp.seg.seg_len[s] = seg_len(s) * es;
   }
-  return ALAMD_OK;
+  return launch_spread_table(sp, P, false, stream);
 }
 
 }  // namespace
