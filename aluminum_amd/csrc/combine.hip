@@ -280,27 +280,16 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
     return launch_order(out_tab, ins, P, lay, dtype, op, order, as_stream(stream));
   // Several outputs of a large result: a workgroup that wrote its tile to every
   // output would interleave nout write streams (measured 69 % of peak).  Instead
-  // the result goes to outs[0] and is then spread, 64 MiB at a time so that the
-  // spread reads what the fold has just written while it is still in cache.
-  // In place (outs[j] == ins[j]) this is safe: a piece of an input is
-  // overwritten only after the fold of that piece has been launched before it
-  // on the same stream.
-  const size_t piece = kMaxTilesPerLaunch * (size_t)16384 / es;  // elements; a multiple of every tile size
+  // the result goes to outs[0] and is then spread from there.  In place
+  // (outs[j] == ins[j]) this is safe: the inputs are overwritten by a launch
+  // that follows the whole fold on the same stream.
   lay.seg.nout = 1;
-  const void *in_tab[ALAMD_MAX_RANKS];
-  for (size_t e0 = 0; e0 < count; e0 += piece) {
-    const size_t len = count - e0 < piece ? count - e0 : piece;
-    for (int r = 0; r < P; ++r) in_tab[r] = static_cast<const char *>(ins[r]) + e0 * es;
-    void *first[ALAMD_MAX_RANKS] = {nullptr};
-    first[0] = static_cast<char *>(outs[0]) + e0 * es;
-    lay.seg.seg_base = len;
-    lay.max_len = len;
-    if ((rc = launch_order(first, in_tab, P, lay, dtype, op, order, as_stream(stream)))) return rc;
-    char *dests[ALAMD_MAX_RANKS];
-    for (int j = 1; j < nout; ++j) dests[j - 1] = static_cast<char *>(outs[j]) + e0 * es;
-    if ((rc = launch_spread(static_cast<char *>(first[0]), dests, nout - 1, len * es, as_stream(stream)))) return rc;
-  }
-  return ALAMD_OK;
+  void *first[ALAMD_MAX_RANKS] = {nullptr};
+  first[0] = outs[0];
+  if ((rc = launch_order(first, ins, P, lay, dtype, op, order, as_stream(stream)))) return rc;
+  char *dests[ALAMD_MAX_RANKS];
+  for (int j = 1; j < nout; ++j) dests[j - 1] = static_cast<char *>(outs[j]);
+  return launch_spread(static_cast<const char *>(outs[0]), dests, nout - 1, bytes, as_stream(stream));
 }
 
 int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, size_t count, int dtype,
