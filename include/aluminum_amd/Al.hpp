@@ -27,13 +27,17 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstddef>
+#include <chrono>
+#include <condition_variable>
 #include <cstdint>
 #include <deque>
 #include <exception>
+#include <functional>
 #include <memory>
 #include <mutex>
 #include <sstream>
 #include <string>
+#include <thread>
 #include <type_traits>
 #include <vector>
 
@@ -921,6 +925,95 @@ class GPUStatusFlag {
 
  private:
   alamd_flag *flag_ = nullptr;
+};
+
+
+/** Host steps in stream order, on one background thread: the four phases of the
+ *  reference's host-transfer state machine
+ *  (HostTransferCollectiveSignalAtEndState::step, include/aluminum/ht/base_state.hpp:86-117;
+ *  the thread itself: src/progress.cpp) built from the two flag types above.
+ *  enqueue(stream, fn) returns at once; then
+ *    1. the stream, when it gets there, sets a start flag           (GPUStatusFlag::record)
+ *    2. the thread sees it and runs fn() - the reference's MPI call; here whatever
+ *       the caller needs between two pieces of GPU work, e.g. an exchange with another host
+ *    3. the thread lets the stream go on                            (GPUWait::signal)
+ *    4. the stream sets an end flag, after which the state is freed (GPUStatusFlag::record)
+ *  fn must not make a HIP call that waits for `stream` (it is blocked until fn returns).
+ *  The combine itself never takes this path: it runs on the GPU. */
+class ProgressEngine {
+ public:
+  ProgressEngine() : thread_([this] { run(); }) {}
+  ~ProgressEngine() {
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      stop_ = true;
+    }
+    wake_.notify_all();
+    thread_.join();
+  }
+  ProgressEngine(const ProgressEngine &) = delete;
+  ProgressEngine &operator=(const ProgressEngine &) = delete;
+
+  void enqueue(hipStream_t stream, std::function<void()> fn) {
+    auto st = std::make_unique<State>();
+    st->fn = std::move(fn);
+    st->start.record(stream);
+    st->go.wait(stream);
+    st->end.record(stream);
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      states_.push_back(std::move(st));
+    }
+    wake_.notify_all();
+  }
+  /** Host steps enqueued and not yet retired. */
+  size_t pending() {
+    std::lock_guard<std::mutex> lock(mutex_);
+    return states_.size();
+  }
+
+ private:
+  struct State {
+    GPUStatusFlag start, end;
+    GPUWait go;
+    std::function<void()> fn;
+    bool ran = false;
+  };
+  void run() {
+    std::unique_lock<std::mutex> lock(mutex_);
+    for (;;) {
+      wake_.wait(lock, [this] { return stop_ || !states_.empty(); });
+      if (states_.empty()) return;  // stop requested and nothing left to retire
+      bool progressed = false;
+      for (size_t i = 0; i < states_.size();) {
+        State *st = states_[i].get();
+        if (!st->ran && st->start.query()) {
+          lock.unlock();
+          st->fn();          // phase 2, outside the lock: enqueue() may be called meanwhile
+          st->go.signal();   // phase 3
+          lock.lock();
+          st->ran = true;
+          progressed = true;
+        }
+        if (st->ran && st->end.query()) {  // phase 4: the wait has been consumed
+          states_.erase(states_.begin() + static_cast<long>(i));
+          progressed = true;
+        } else {
+          ++i;
+        }
+      }
+      if (!progressed) {
+        lock.unlock();
+        std::this_thread::sleep_for(std::chrono::microseconds(5));
+        lock.lock();
+      }
+    }
+  }
+  std::mutex mutex_;
+  std::condition_variable wake_;
+  std::deque<std::unique_ptr<State>> states_;
+  bool stop_ = false;
+  std::thread thread_;  // last: started when everything above exists
 };
 
 }  // namespace amd

@@ -104,6 +104,44 @@ static void test_flags(hipStream_t stream) {
   EXPECT(x.down()[0] == 0x01010101, "work behind the wait ran");
 }
 
+// The host-transfer shape end to end: device -> pinned host copy, a host step in stream order,
+// pinned host -> device copy; all enqueued before anything has run.
+static void test_progress_engine(hipStream_t stream) {
+  const size_t n = 1000;
+  DevBuf<int> x(n);
+  std::vector<int> init(n);
+  for (size_t i = 0; i < n; ++i) init[i] = (int)i;
+  x.up(init);
+  int *pinned = nullptr;
+  HIPCHK(hipHostMalloc(reinterpret_cast<void **>(&pinned), n * sizeof(int), hipHostMallocDefault));
+  std::memset(pinned, 0, n * sizeof(int));
+  int order_seen[2] = {0, 0}, step = 0;
+  {
+    Al::amd::ProgressEngine pe;
+    Al::amd::GPUWait gate;
+    gate.wait(stream, 1u << 24);  // nothing below may run before the host opens the gate
+    HIPCHK(hipMemcpyAsync(pinned, x.p, n * sizeof(int), hipMemcpyDeviceToHost, stream));
+    pe.enqueue(stream, [&] {
+      order_seen[0] = ++step;
+      for (size_t i = 0; i < n; ++i) pinned[i] = 2 * pinned[i] + 1;  // sees what the copy before it brought
+    });
+    HIPCHK(hipMemcpyAsync(x.p, pinned, n * sizeof(int), hipMemcpyHostToDevice, stream));
+    pe.enqueue(stream, [&] { order_seen[1] = ++step; });
+    EXPECT(pe.pending() == 2, "two host steps pending");
+    EXPECT(step == 0, "no host step before the stream got there");
+    gate.signal();
+    HIPCHK(hipStreamSynchronize(stream));
+    EXPECT(order_seen[0] == 1 && order_seen[1] == 2, "host steps ran once each, in stream order");
+    for (int spin = 0; spin < 2000 && pe.pending(); ++spin) std::this_thread::sleep_for(std::chrono::milliseconds(1));
+    EXPECT(pe.pending() == 0, "states retired after their end flags");
+  }
+  const auto got = x.down();
+  bool ok = true;
+  for (size_t i = 0; i < n; ++i) ok = ok && got[i] == 2 * (int)i + 1;
+  EXPECT(ok, "device data went through the host step");
+  HIPCHK(hipHostFree(pinned));
+}
+
 int main() {
   int ndev = 0;
   if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) { std::printf("no GPU\n"); return 2; }
@@ -157,6 +195,7 @@ int main() {
   test_errors(stream);
   test_threads_and_streams();
   test_flags(stream);
+  test_progress_engine(stream);
 
   HIPCHK(hipStreamDestroy(stream));
   Al::Finalize();
