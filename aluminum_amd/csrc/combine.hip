@@ -170,7 +170,8 @@ int launch_spread_once(const FoldParams &fp, int nsrc, hipStream_t stream) {
   const size_t tpc = tiles < kSpreadChunkTiles ? (tiles + 7) & ~(size_t)7 : kSpreadChunkTiles;
   const size_t chunks = (tiles + tpc - 1) / tpc;
   const size_t blocks = chunks * tpc * (size_t)fp.P;
-  if (blocks > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
+  // a launch holds fewer than 2^32 threads in x
+  if (blocks * kGatherThreads > 0xffffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
   hipLaunchKernelGGL(spread_kernel, dim3((unsigned)blocks, (unsigned)nsrc, 1), dim3(kGatherThreads, 1, 1), 0, stream,
                      fp, (unsigned)tpc);
   ALAMD_HIP(hipGetLastError());

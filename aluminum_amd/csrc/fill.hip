@@ -173,7 +173,7 @@ int alamd_copy(void *dst, const void *src, size_t bytes, void *stream) {
   const size_t tile = Tile<kCopyU, kCopyThreads>::BYTES;
   size_t tiles = (b.vec + tile - 1) / tile;
   if (tiles == 0) tiles = 1;
-  if (tiles > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "copy too large for one launch");
+  if (tiles * kCopyThreads > 0xffffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "copy too large for one launch");
   hipLaunchKernelGGL(copy_kernel_vec, dim3((unsigned)tiles), dim3(kCopyThreads), 0, as_stream(stream), (char *)dst,
                      (const char *)src, b);
   ALAMD_HIP(hipGetLastError());

@@ -130,7 +130,8 @@ int make_plan(RingPlan &pl, void *const *bufs, int P, size_t count, int dtype, s
   if (nchunks < 1) nchunks = 1;
   const size_t tile_vecs = Tile<kRingU, kThreads>::BYTES / 16;
   const size_t tpc = ((cn < n ? cn : (n ? n : 1)) + tile_vecs - 1) / tile_vecs;
-  if (nchunks * tpc > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "too many chunks for one launch");
+  if (nchunks * tpc * kThreads > 0xffffffffull)
+    return set_error(ALAMD_ERR_INVALID_ARG, "too many chunks for one launch");
   pl.rp.tiles_per_chunk = (unsigned)tpc;
   pl.gx = (unsigned)(nchunks * tpc);
   return ALAMD_OK;
