@@ -158,7 +158,10 @@ def run_layout_workload(al, torch, name, steps, warmup):
     c2_f32_allreduce - the combine delivered to all eight ranks' receive buffers (8 reads + 8 writes of
     2^26 elements, order tree_dbl: what Al::Allreduce yields above 2 KiB);
     c2_f32_allgather - eight slices of 2^23 elements gathered into eight receive buffers of 2^26
-    (each slice read once, written eight times)."""
+    (each slice read once, written eight times);
+    c2_f32_reduce_scatter - eight send buffers of 2^26 elements, block b folded into receive buffer b of
+    2^23 elements (order pairwise_desc from the receiving rank: what MPI_Reduce_scatter_block yields above
+    512 KiB)."""
     import numpy as np
     import oracle
     m = 1 << 18
@@ -178,6 +181,23 @@ def run_layout_workload(al, torch, name, steps, warmup):
             for lo in (0, count - m):
                 want = oracle.combine_generated(P, m, "f32", "sum", "tree_dbl", 0, "uniform_pm1", 1000, lo)
                 ok = ok and outs[j][lo:lo + m].cpu().numpy().tobytes() == want.tobytes()
+    elif name == "c2_f32_reduce_scatter":
+        count = 1 << 23
+        sends = [torch.empty(P * count, dtype=torch.float32, device="cuda") for _ in range(P)]
+        recvs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+        for r in range(P):
+            al.fill(sends[r], "uniform_pm1", 1000 + r)
+        fn = lambda: al.reduce_scatter(recvs, sends, "sum", order="pairwise_desc", count=count)
+        alg = (P + 1) * P * count * 4
+        launches = 1
+        fn()
+        torch.cuda.synchronize()
+        ok = True
+        for b in (0, P - 1):
+            for lo in (0, count - m):
+                want = oracle.combine_generated(P, m, "f32", "sum", "pairwise_desc", b, "uniform_pm1", 1000,
+                                                b * count + lo)
+                ok = ok and recvs[b][lo:lo + m].cpu().numpy().tobytes() == want.tobytes()
     else:
         count = 1 << 23
         sends = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
@@ -355,8 +375,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2_f32_sum",
                     choices=sorted(WORKLOADS) + ["c3_ring_stepwise", "c3_ring_fused", "c5_halo", "flags",
-                                               "c2_f32_allreduce", "c2_f32_allgather"])
-    ap.add_argument("--also", default="c2_bf16_sum,c2_f32_sum_rotating,c2_f32_allreduce,c2_f32_allgather,c3_ring_fused",
+                                               "c2_f32_allreduce", "c2_f32_allgather", "c2_f32_reduce_scatter"])
+    ap.add_argument("--also", default="c2_bf16_sum,c2_f32_sum_rotating,c2_f32_allreduce,c2_f32_reduce_scatter,c2_f32_allgather,c3_ring_fused",
                     help="comma-separated extra workloads reported under 'also' ('' for none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--raw", action="store_true", help="print only the workload's own measurement record")
@@ -388,7 +408,7 @@ def main():
         main_res = run_halo_workload(al, torch, args.steps, args.warmup)
     elif args.workload == "flags":
         main_res = run_flag_workload()
-    elif args.workload in ("c2_f32_allreduce", "c2_f32_allgather"):
+    elif args.workload in ("c2_f32_allreduce", "c2_f32_allgather", "c2_f32_reduce_scatter"):
         main_res = run_layout_workload(al, torch, args.workload, args.steps, args.warmup)
     else:
         main_res = run_combine_workload(al, torch, args.workload, args.steps, args.warmup)
