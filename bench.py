@@ -327,6 +327,17 @@ def c1_gpu_checksum(al, torch):
     return "%016x" % oracle.checksum(out.cpu().numpy())
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return None
+
+
 def cpu_baseline(al=None, torch=None):
     """The reference's MPI-backend host combine on this box's host cores."""
     exe = os.path.join(ROOT, "oracle", "mpi_baseline")
@@ -348,7 +359,7 @@ def cpu_baseline(al=None, torch=None):
                                   "2^20 elements per rank, uniform[-1,1] seed 1000+rank, 10 warm-up + 3000 "
                                   "timed (about 10 s), median of max-over-ranks; GB/s over (P+1)*n*4 bytes",
                         "median_ms": r["median_ms"], "min_ms": r["min_ms"], "gpu_result_identical": same,
-                        "host_cpus": os.cpu_count(), "same_workload_port": c2_port_sample()}
+                        "host_cpus": os.cpu_count(), "cpu_model": cpu_model(), "same_workload_port": c2_port_sample()}
         except Exception:
             pass
     # MPI-free restatement: the oracle's threaded tree combine on the same shape
@@ -365,7 +376,7 @@ def cpu_baseline(al=None, torch=None):
     return {"value": (ranks + 1) * n * 4 / med * 1e-9, "unit": "GB/s", "cores": oracle.num_threads(),
             "kind": "port", "sample": "MPI-free restatement: CPU oracle TREE_DBL combine, 4 buffers of 2^20 "
                                       "fp32, median of 30", "median_ms": med * 1e3,
-            "host_cpus": os.cpu_count()}
+            "host_cpus": os.cpu_count(), "cpu_model": cpu_model()}
 
 
 def main():
