@@ -452,7 +452,10 @@ def main():
         "parity_vs_oracle": main_res.get("parity_vs_oracle"),
         "roofline": {"bound": "hbm", "achieved": main_res["gbps_kernel"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": main_res["gbps_kernel"] / HBM_PEAK_GBPS,
+                     # measured HBM bytes (fetched + written) per call, and per launch of the kernel
                      "traffic": MEASURED_TRAFFIC.get(args.workload),
+                     "traffic_per_launch": (MEASURED_TRAFFIC[args.workload] // main_res["launches_per_step"]
+                                            if args.workload in MEASURED_TRAFFIC else None),
                      "kernel": KERNEL_NAME.get(args.workload, "alamd::fold_vec_kernel"),
                      "kernel_ms": main_res["kernel_ms"],
                      # one call is cut into launches of at most 4096 tiles of 16 KiB per stream
