@@ -36,10 +36,12 @@ template <> struct unit_of<4> { using type = uint32_t; };
 template <> struct unit_of<8> { using type = uint64_t; };
 template <> struct unit_of<16> { using type = u32x4; };
 
-template <int UB, bool PACK>
+// U = independent accesses per thread: the short rows of the x faces need
+// several in flight, but a launch also needs a few workgroups per CU, so the
+// host picks the largest U that leaves enough of them.
+template <int UB, bool PACK, int U>
 __global__ void __launch_bounds__(kThreads) halo_kernel(const HaloParams p) {
   using Unit = typename unit_of<UB>::type;
-  constexpr int U = 4;  // independent accesses per thread: the short rows of the x faces need them in flight
   const HaloFace &f = p.f[blockIdx.y];
   const unsigned long long n = f.nunits;
   const unsigned upr = f.upr, rows_y = f.rows_y;
@@ -122,17 +124,26 @@ int halo_launch(void *grid, void *const bufs[6], const size_t dims[3], size_t ha
     if (f.nunits > max_units) max_units = f.nunits;
   }
   for (int k = nf; k < 6; ++k) hp.f[k] = hp.f[0];
+  // 8 accesses per thread if that still gives two workgroups per CU over all faces, else 2
+  const unsigned two_per_cu = stream_grid((size_t)-1 / 2, 1, 2);
+  const bool wide = (max_units + kThreads * 8 - 1) / (kThreads * 8) * nf >= two_per_cu;
+  const int acc = wide ? 8 : 2;
   unsigned per_face = (stream_grid((size_t)-1 / 2, 1, 8) + nf - 1) / nf;
-  unsigned gx = stream_grid((size_t)max_units, (size_t)kThreads * 4, 8);
+  unsigned gx = stream_grid((size_t)max_units, (size_t)kThreads * acc, 8);
   if (gx > per_face) gx = per_face < 1 ? 1 : per_face;
   const dim3 grid_dim(gx, nf, 1), block(kThreads, 1, 1);
   void (*kern)(const HaloParams) = nullptr;
+  auto pick = [&](auto ub) {
+    constexpr int UB = decltype(ub)::value;
+    if (wide) return pack ? halo_kernel<UB, true, 8> : halo_kernel<UB, false, 8>;
+    return pack ? halo_kernel<UB, true, 2> : halo_kernel<UB, false, 2>;
+  };
   switch (unit) {
-  case 16: kern = pack ? halo_kernel<16, true> : halo_kernel<16, false>; break;
-  case 8: kern = pack ? halo_kernel<8, true> : halo_kernel<8, false>; break;
-  case 4: kern = pack ? halo_kernel<4, true> : halo_kernel<4, false>; break;
-  case 2: kern = pack ? halo_kernel<2, true> : halo_kernel<2, false>; break;
-  default: kern = pack ? halo_kernel<1, true> : halo_kernel<1, false>; break;
+  case 16: kern = pick(std::integral_constant<int, 16>{}); break;
+  case 8: kern = pick(std::integral_constant<int, 8>{}); break;
+  case 4: kern = pick(std::integral_constant<int, 4>{}); break;
+  case 2: kern = pick(std::integral_constant<int, 2>{}); break;
+  default: kern = pick(std::integral_constant<int, 1>{}); break;
   }
   hipLaunchKernelGGL(kern, grid_dim, block, 0, stream, hp);
   ALAMD_HIP(hipGetLastError());
