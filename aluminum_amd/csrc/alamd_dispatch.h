@@ -72,6 +72,7 @@ struct SegParams {
   unsigned long long seg_base;
   unsigned long long seg_rem;
   unsigned long long tile0;  // index of the first tile of this launch
+  unsigned seg0;             // index of the first segment of this launch
   int in_blocked;   // 1: inputs are read at the segment's offset, 0: at 0
   int out_mode;     // OUT_ALL / OUT_SEG / OUT_OWNER
   int owner_shift;  // OUT_OWNER: output index is (segment + owner_shift) mod P

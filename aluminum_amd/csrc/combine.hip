@@ -99,7 +99,7 @@ constexpr int kGatherU = 8, kGatherThreads = 128;
 // Slices to several destinations: blockIdx.y = source q, whose seg_len[q] bytes
 // go to byte offset seg_off[q] of every destination p.out[0..P) (a destination
 // that is the source itself, the in-place form, is skipped).  One workgroup
-// per (destination, tile).  blockIdx.x runs chunk by chunk (tpc tiles, 8 MiB);
+// per (destination, tile).  blockIdx.x runs chunk by chunk (tpc tiles, 16 MiB);
 // inside a chunk all tiles of destination 0 come first, then destination 1,
 // ...: at any time the device writes one contiguous stream per chunk instead
 // of P interleaved ones, and re-reads the chunk of the source from cache:
@@ -109,8 +109,17 @@ constexpr int kGatherU = 8, kGatherThreads = 128;
 // of 4 only, 49 % with an odd tpc).  Measured for 1 read + 8 writes of 32 MiB:
 // 88 % of the HBM peak, against 67 % when every workgroup writes its tile to
 // all destinations (69 % for those writes alone).
-constexpr unsigned kSpreadChunkTiles = 512;
-__global__ void __launch_bounds__(kGatherThreads) spread_kernel(FoldParams p, unsigned tpc) {
+// A chunk's share per XCD (2 MiB) has to stay in that XCD's 4 MiB L2 between
+// the destinations: 32 MiB chunks run at 64 %.  A launch covers at most
+// kSpreadLaunchChunks chunks of every source: in longer launches the XCDs
+// drift apart.  Measured on buffers that no earlier call has touched (1 GiB to
+// 7 destinations): 84 % with 16 MiB chunks and launches of one or two chunks,
+// 80 % with four chunks per launch, 76 % with the whole GiB in one launch,
+// 77 % / 81 % with 8 MiB chunks in one launch / one launch per two chunks.
+constexpr unsigned kSpreadChunkTiles = 1024;
+constexpr unsigned kSpreadLaunchChunks = 2;
+__global__ void __launch_bounds__(kGatherThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
+spread_kernel(FoldParams p, unsigned tpc, unsigned tile0) {
   using TL = Tile<kGatherU, kGatherThreads>;
   const TL tl;
   const int q = blockIdx.y;
@@ -119,7 +128,7 @@ __global__ void __launch_bounds__(kGatherThreads) spread_kernel(FoldParams p, un
   const ByteSplit b = split_bytes(src, p.seg.seg_len[q]);
   const unsigned ndest = (unsigned)p.P;
   // the bytes before the first and after the last whole vector
-  if (blockIdx.x == 0 && threadIdx.x < b.head + b.tail) {
+  if (tile0 == 0 && blockIdx.x == 0 && threadIdx.x < b.head + b.tail) {
     const size_t i = threadIdx.x < b.head ? threadIdx.x : b.vec + threadIdx.x;
     const char c = src[i];
     for (unsigned r = 0; r < ndest; ++r) {
@@ -130,7 +139,7 @@ __global__ void __launch_bounds__(kGatherThreads) spread_kernel(FoldParams p, un
   const unsigned per_chunk = tpc * ndest;
   const unsigned chunk = blockIdx.x / per_chunk, rem = blockIdx.x % per_chunk;
   const unsigned dest = rem / tpc;
-  const size_t tb = ((size_t)chunk * tpc + rem % tpc) * TL::BYTES;
+  const size_t tb = ((size_t)tile0 + (size_t)chunk * tpc + rem % tpc) * TL::BYTES;
   char *dst = p.out[dest] + off;
   if (tb >= b.vec || dst == src) return;
   const int nrec = b.vec - tb > TL::BYTES ? (int)TL::BYTES : (int)(b.vec - tb);
@@ -168,25 +177,29 @@ int launch_spread_once(const FoldParams &fp, int nsrc, hipStream_t stream) {
   const size_t tiles = (max_len + tile - 1) / tile;
   // always a multiple of 8 (see spread_kernel); workgroups past the last tile exit at once
   const size_t tpc = tiles < kSpreadChunkTiles ? (tiles + 7) & ~(size_t)7 : kSpreadChunkTiles;
-  const size_t chunks = (tiles + tpc - 1) / tpc;
-  const size_t blocks = chunks * tpc * (size_t)fp.P;
+  const size_t per_launch = tpc * kSpreadLaunchChunks;
   // a launch holds fewer than 2^32 threads in x
-  if (blocks * kGatherThreads > 0xffffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
-  hipLaunchKernelGGL(spread_kernel, dim3((unsigned)blocks, (unsigned)nsrc, 1), dim3(kGatherThreads, 1, 1), 0, stream,
-                     fp, (unsigned)tpc);
+  if (per_launch * (size_t)fp.P * kGatherThreads > 0xffffffffull || tiles > 0xffffffffull)
+    return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
+  for (size_t t0 = 0; t0 < tiles; t0 += per_launch) {
+    const size_t nt = tiles - t0 < per_launch ? tiles - t0 : per_launch;
+    const size_t chunks = (nt + tpc - 1) / tpc;
+    hipLaunchKernelGGL(spread_kernel, dim3((unsigned)(chunks * tpc * (size_t)fp.P), (unsigned)nsrc, 1),
+                       dim3(kGatherThreads, 1, 1), 0, stream, fp, (unsigned)tpc, (unsigned)t0);
+  }
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
 }
 
 }  // namespace
 
-// split_large: slices of two chunks (16 MiB) and more get a launch each, the smaller ones share one.
+// split_large: slices of one chunk (16 MiB) and more get launches of their own, the smaller ones share one.
 // For an allgather of separate send buffers one launch over large slices is long enough for the XCDs to
 // drift apart (32 MiB slices: 88 % of peak one by one, 83 % together; 8 MiB slices: 85 us together,
 // 98 us one by one; 1 MiB: 15 us against 43 us).  Segments that a fold has just written are spread
 // faster in one launch (eight 32 MiB segments: 650 us for the whole allreduce against 667 us).
 int launch_spread_table(const FoldParams &fp, int nsrc, bool split_large, hipStream_t stream) {
-  const size_t big = 2 * (size_t)kSpreadChunkTiles * Tile<kGatherU, kGatherThreads>::BYTES;
+  const size_t big = (size_t)kSpreadChunkTiles * Tile<kGatherU, kGatherThreads>::BYTES;
   FoldParams rest = fp;
   for (int q = 0; q < nsrc && nsrc > 1 && split_large; ++q) {
     if (fp.seg.seg_len[q] < big) continue;

@@ -59,7 +59,7 @@ fold_vec_kernel(const FoldParams p) {
   using TL = Tile<U, THREADS>;
   const TL tl;
   const int P = PT ? PT : p.P;
-  const unsigned seg = blockIdx.y;
+  const unsigned seg = blockIdx.y + p.seg.seg0;
   size_t off, len;
   seg_range(p.seg, seg, off, len);
   const size_t off_bytes = off * sizeof(T);
@@ -167,10 +167,19 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
       else kern = fold_vec_kernel<T, OP, false, 0>;
     }
     FoldParams q = p;
-    for (size_t t0 = 0; t0 < tiles; t0 += kMaxTilesPerLaunch) {
-      const size_t nt = tiles - t0 < kMaxTilesPerLaunch ? tiles - t0 : kMaxTilesPerLaunch;
+    // about kMaxTilesPerLaunch workgroups per launch, whatever the number of segments: small work in
+    // one launch; otherwise up to eight segments side by side (blockIdx.y), the rest in further launches
+    const bool small = tiles * nseg <= kMaxTilesPerLaunch;
+    const unsigned segs = small || nseg < 8 ? nseg : 8;
+    const size_t cut = small ? tiles : kMaxTilesPerLaunch / segs;
+    for (size_t t0 = 0; t0 < tiles; t0 += cut) {
+      const size_t nt = tiles - t0 < cut ? tiles - t0 : cut;
       q.seg.tile0 = t0;
-      hipLaunchKernelGGL(kern, dim3((unsigned)nt, nseg, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
+      for (unsigned s0 = 0; s0 < nseg; s0 += segs) {
+        q.seg.seg0 = s0;
+        hipLaunchKernelGGL(kern, dim3((unsigned)nt, nseg - s0 < segs ? nseg - s0 : segs, 1),
+                           dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
+      }
     }
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;

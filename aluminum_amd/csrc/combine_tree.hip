@@ -59,7 +59,7 @@ tree_vec_kernel(const TreeParams p) {
   constexpr int N = 16 / sizeof(T);
   using TL = Tile<U, THREADS>;
   const TL tl;
-  const unsigned seg = blockIdx.y;
+  const unsigned seg = blockIdx.y + p.seg.seg0;
   size_t off, len;
   seg_range(p.seg, seg, off, len);
   const size_t off_bytes = off * sizeof(T);
@@ -135,14 +135,21 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
   size_t tiles = (max_len + tile_elems - 1) / tile_elems;
   if (tiles == 0) tiles = 1;
-  // the launch cut is a number of bytes per stream, whatever the tile size
-  const size_t cut = kMaxTilesPerLaunch * (size_t)16384 / Tile<S::U, S::THREADS>::BYTES;
+  // the launch cut is a number of bytes over all segments of a launch, whatever the tile size: small
+  // work in one launch; otherwise up to eight segments side by side (blockIdx.y)
+  const size_t per_launch = kMaxTilesPerLaunch * (size_t)16384 / Tile<S::U, S::THREADS>::BYTES;
+  const bool small = tiles * nseg <= per_launch;
+  const unsigned segs = small || nseg < 8 ? nseg : 8;
+  const size_t cut = small ? tiles : per_launch / segs;
   TreeParams q = p;
   for (size_t t0 = 0; t0 < tiles; t0 += cut) {
     const size_t nt = tiles - t0 < cut ? tiles - t0 : cut;
     q.seg.tile0 = t0;
-    hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE>), dim3((unsigned)nt, nseg, 1), dim3(S::THREADS, 1, 1), 0,
-                       stream, q);
+    for (unsigned s0 = 0; s0 < nseg; s0 += segs) {
+      q.seg.seg0 = s0;
+      hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE>), dim3((unsigned)nt, nseg - s0 < segs ? nseg - s0 : segs, 1),
+                         dim3(S::THREADS, 1, 1), 0, stream, q);
+    }
   }
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;

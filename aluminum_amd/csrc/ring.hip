@@ -204,7 +204,7 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
     sp.seg.seg_off[s] = seg_off(s);
     sp.seg.seg_len[s] = seg_len(s) * es;
   }
-  return launch_spread_table(sp, P, false, stream);
+  return launch_spread_table(sp, P, true, stream);
 }
 
 }  // namespace

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import oracle
-from util import assert_bits_equal
+from util import assert_bits_equal, to_dev
 
 pytestmark = pytest.mark.gpu
 P = 8
@@ -341,3 +341,51 @@ def test_every_pair_of_bytes_in_every_lane(al, dtype):
         al.combine([out], [a_dev, b_dev], op, order="rank_asc", dtype=dtype)
         torch.cuda.synchronize()
         assert_bits_equal(out.cpu().numpy().view(npdt), oracle.step(a, b, dtype, op), dtype, "%s %s" % (dtype, op))
+
+
+def test_allgather_slices_over_several_launches(al):
+    """Slices longer than one spread launch covers (32 MiB of a source), byte counts that are not
+    multiples of 16, sources and receive buffers at odd addresses; separate buffers and in place."""
+    import torch
+    P = 3
+    count = (40 << 20) + 5
+    raw = [torch.empty(count + 8, dtype=torch.uint8, device="cuda") for _ in range(P)]
+    sends = [raw[r][1 + r:1 + r + count] for r in range(P)]
+    for r in range(P):
+        al.fill(sends[r], "fullrange", 170 + r, dtype="u8", count=count)
+    rraw = [torch.full((P * count + 8,), 0xEE, dtype=torch.uint8, device="cuda") for _ in range(P)]
+    recvs = [rraw[r][3:3 + P * count] for r in range(P)]
+    al.allgather(recvs, sends, dtype="u8", count=count)
+    torch.cuda.synchronize()
+    want = torch.cat(sends)
+    for q in range(P):
+        host = oracle.fill(count, "u8", "fullrange", 170 + q)
+        assert want[q * count:(q + 1) * count].cpu().numpy().tobytes() == host.tobytes()
+    for r in range(P):
+        assert torch.equal(recvs[r], want), "rank %d" % r
+        assert bool((rraw[r][:3] == 0xEE).all()) and bool((rraw[r][3 + P * count:] == 0xEE).all())
+    # in place: rank r's slice already sits at r * count of its own buffer
+    bufs = [torch.full((P * count,), 0x11, dtype=torch.uint8, device="cuda") for _ in range(P)]
+    for r in range(P):
+        bufs[r][r * count:(r + 1) * count].copy_(sends[r])
+    al.allgather(bufs, [bufs[r][r * count:(r + 1) * count] for r in range(P)], dtype="u8", count=count)
+    torch.cuda.synchronize()
+    for r in range(P):
+        assert torch.equal(bufs[r], want), "in place, rank %d" % r
+
+
+@pytest.mark.parametrize("order", ("rank_asc", "tree_halv"))
+def test_reduce_scatter_more_than_eight_large_segments(al, order):
+    """Twelve blocks of 6 MB: more segments than one launch takes side by side, each longer than
+    one launch's share of tiles, with a ragged tail."""
+    import torch
+    P = 12
+    count = 1500000 + 3
+    sends = [oracle.fill(P * count, "f32", "uniform_pm1", 900 + r) for r in range(P)]
+    d_sends = [to_dev(s) for s in sends]
+    recvs = [torch.zeros(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+    al.reduce_scatter(recvs, d_sends, "sum", order=order, count=count)
+    torch.cuda.synchronize()
+    want = oracle.reduce_scatter(sends, "f32", "sum", order)
+    for r in range(P):
+        assert_bits_equal(recvs[r].cpu().numpy(), want[r], "f32", "%s rank %d" % (order, r))
