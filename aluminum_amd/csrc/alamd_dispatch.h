@@ -140,6 +140,18 @@ int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, i
 // 146 / 128, 256 MiB 773 / 667; two outputs 437 / 455, four 544 / 529).
 constexpr size_t kTwoStepMinBytes = (size_t)40 << 20;
 constexpr int kTwoStepMinOutputs = 3;
+// The two steps alternate over pieces of the result of this many bytes, so that
+// the spread reads what the fold has just written from the 256 MiB memory-side
+// cache instead of HBM (P = 8, 1 GiB per rank, buffers no earlier call has
+// touched: 80 % of peak with pieces of 64 to 256 MiB, 75 % with the whole
+// result folded first; no difference up to 256 MiB per rank, which stay one piece).
+constexpr size_t kTwoStepPieceBytes = (size_t)128 << 20;
+// The fused ring allreduce does the same over pieces of this many bytes in all
+// (8 MiB of each of eight segments: one fold launch of 4096 workgroups, one
+// spread launch).  P = 8, untouched buffers, 256 MiB / 1 GiB per rank: 81.6 % /
+// 81.3 % of peak; 80 % / 80 % with pieces of 32 MiB or 256 MiB, 75 % with 16 or
+// 48 MiB, 80 % / 77 % with the whole result folded first.
+constexpr size_t kRingPieceBytes = (size_t)64 << 20;
 
 // Copies [src, src + bytes) to each of dests[0..ndest) (none overlapping the
 // source, any alignment).

@@ -294,16 +294,26 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
     return launch_order(out_tab, ins, P, lay, dtype, op, order, as_stream(stream));
   // Several outputs of a large result: a workgroup that wrote its tile to every
   // output would interleave nout write streams (measured 69 % of peak).  Instead
-  // the result goes to outs[0] and is then spread from there.  In place
-  // (outs[j] == ins[j]) this is safe: the inputs are overwritten by a launch
-  // that follows the whole fold on the same stream.
-  lay.seg.nout = 1;
-  void *first[ALAMD_MAX_RANKS] = {nullptr};
-  first[0] = outs[0];
-  if ((rc = launch_order(first, ins, P, lay, dtype, op, order, as_stream(stream)))) return rc;
-  char *dests[ALAMD_MAX_RANKS];
-  for (int j = 1; j < nout; ++j) dests[j - 1] = static_cast<char *>(outs[j]);
-  return launch_spread(static_cast<const char *>(outs[0]), dests, nout - 1, bytes, as_stream(stream));
+  // the result goes to outs[0] and is then spread from there, piece by piece.
+  // In place (outs[j] == ins[j]) this is safe: a piece of the inputs is
+  // overwritten by a launch that follows the fold of that piece on the same
+  // stream, and no other piece reads it.
+  const size_t piece = bytes > 2 * kTwoStepPieceBytes ? kTwoStepPieceBytes / es : count;
+  for (size_t e0 = 0; e0 < count; e0 += piece) {
+    const size_t n = count - e0 < piece ? count - e0 : piece;
+    Layout pl = lay;
+    pl.seg = make_seg(n, 0, 0, OUT_ALL, 1);
+    pl.max_len = n;
+    void *first[ALAMD_MAX_RANKS] = {nullptr};
+    first[0] = static_cast<char *>(outs[0]) + e0 * es;
+    const void *pin[ALAMD_MAX_RANKS];
+    for (int r = 0; r < P; ++r) pin[r] = static_cast<const char *>(ins[r]) + e0 * es;
+    if ((rc = launch_order(first, pin, P, pl, dtype, op, order, as_stream(stream)))) return rc;
+    char *dests[ALAMD_MAX_RANKS];
+    for (int j = 1; j < nout; ++j) dests[j - 1] = static_cast<char *>(outs[j]) + e0 * es;
+    if ((rc = launch_spread(static_cast<const char *>(first[0]), dests, nout - 1, n * es, as_stream(stream)))) return rc;
+  }
+  return ALAMD_OK;
 }
 
 int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, size_t count, int dtype,

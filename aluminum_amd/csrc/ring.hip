@@ -187,24 +187,38 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
     return (sg * fp.seg.seg_base + (sg < rem ? sg : rem)) * es;
   };
   auto seg_len = [&](int s) { return fp.seg.seg_base + ((size_t)s < fp.seg.seg_rem ? 1 : 0); };
-  // one launch folds all segments (8 reads + 1 write), then the segments are spread
-  FoldParams fo = fp;
-  fo.seg.out_mode = OUT_OWNER;
-  const int rc = launch_fold(fo, (unsigned)P, max_len, dtype, op, true, stream);
-  if (rc) return rc;
-  FoldParams sp;
-  sp.seg = make_seg(0, 0, 0, OUT_ALL, 0);
-  sp.P = P;
-  for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
-    sp.in[r] = nullptr;
-    sp.out[r] = r < P ? static_cast<char *>(bufs[r]) : nullptr;
+  // piece by piece: fold the same range of every segment (P reads + 1 write), then spread it
+  // (kRingPieceBytes over all segments: one fold launch and one spread launch per piece)
+  const size_t tile_elems = Tile<8, 128>::BYTES / es;
+  size_t piece = kRingPieceBytes / (size_t)P / es / tile_elems * tile_elems;
+  if (piece == 0) piece = tile_elems;
+  for (size_t e0 = 0; e0 < max_len; e0 += piece) {
+    FoldParams fo = fp;
+    fo.seg.out_mode = OUT_OWNER;
+    fo.seg.ragged = 1;
+    FoldParams sp;
+    sp.seg = make_seg(0, 0, 0, OUT_ALL, 0);
+    sp.P = P;
+    for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
+      sp.in[r] = nullptr;
+      sp.out[r] = r < P ? static_cast<char *>(bufs[r]) : nullptr;
+    }
+    size_t longest = 0;
+    for (int s = 0; s < P; ++s) {
+      const size_t len = seg_len(s) > e0 ? (seg_len(s) - e0 < piece ? seg_len(s) - e0 : piece) : 0;
+      const size_t off = seg_off(s) + e0 * es;
+      fo.seg.seg_off[s] = off / es;
+      fo.seg.seg_len[s] = len;
+      sp.in[s] = static_cast<const char *>(bufs[(s + P - 1) % P]) + off;
+      sp.seg.seg_off[s] = off;
+      sp.seg.seg_len[s] = len * es;
+      if (len > longest) longest = len;
+    }
+    int rc = launch_fold(fo, (unsigned)P, longest, dtype, op, true, stream);
+    if (rc) return rc;
+    if ((rc = launch_spread_table(sp, P, true, stream))) return rc;
   }
-  for (int s = 0; s < P; ++s) {
-    sp.in[s] = static_cast<const char *>(bufs[(s + P - 1) % P]) + seg_off(s);
-    sp.seg.seg_off[s] = seg_off(s);
-    sp.seg.seg_len[s] = seg_len(s) * es;
-  }
-  return launch_spread_table(sp, P, true, stream);
+  return ALAMD_OK;
 }
 
 }  // namespace

@@ -153,6 +153,9 @@ def run_ring_workload(al, torch, mode, steps, warmup):
             "parity_vs_oracle": bool(ok)}
 
 
+LAYOUTS = [w + r for w in ("c2_f32_allreduce", "c2_f32_allgather", "c2_f32_reduce_scatter") for r in ("", "_rotating")]
+
+
 def run_layout_workload(al, torch, name, steps, warmup):
     """The two write-heavy layouts at the C2 shape (P = 8 fp32 ranks, seed 1000+rank):
     c2_f32_allreduce - the combine delivered to all eight ranks' receive buffers (8 reads + 8 writes of
@@ -161,63 +164,74 @@ def run_layout_workload(al, torch, name, steps, warmup):
     (each slice read once, written eight times);
     c2_f32_reduce_scatter - eight send buffers of 2^26 elements, block b folded into receive buffer b of
     2^23 elements (order pairwise_desc from the receiving rank: what MPI_Reduce_scatter_block yields above
-    512 KiB)."""
-    import numpy as np
+    512 KiB).
+    With the suffix _rotating the calls go round four sets of buffers, so that nothing a call reads or
+    writes was touched by the three calls before it (no help from the 256 MiB memory-side cache)."""
     import oracle
     m = 1 << 18
-    if name == "c2_f32_allreduce":
-        count = 1 << 26
-        ins = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
-        outs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
-        for r in range(P):
-            al.fill(ins[r], "uniform_pm1", 1000 + r)
-        fn = lambda: al.combine(outs, ins, "sum", order="tree_dbl")
-        alg = 2 * P * count * 4
-        launches = count * 4 // (64 << 20) + 1
-        fn()
-        torch.cuda.synchronize()
-        ok = True
-        for j in (0, P - 1):
-            for lo in (0, count - m):
-                want = oracle.combine_generated(P, m, "f32", "sum", "tree_dbl", 0, "uniform_pm1", 1000, lo)
-                ok = ok and outs[j][lo:lo + m].cpu().numpy().tobytes() == want.tobytes()
-    elif name == "c2_f32_reduce_scatter":
-        count = 1 << 23
-        sends = [torch.empty(P * count, dtype=torch.float32, device="cuda") for _ in range(P)]
-        recvs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
-        for r in range(P):
-            al.fill(sends[r], "uniform_pm1", 1000 + r)
-        fn = lambda: al.reduce_scatter(recvs, sends, "sum", order="pairwise_desc", count=count)
-        alg = (P + 1) * P * count * 4
-        launches = 1
-        fn()
-        torch.cuda.synchronize()
-        ok = True
-        for b in (0, P - 1):
-            for lo in (0, count - m):
-                want = oracle.combine_generated(P, m, "f32", "sum", "pairwise_desc", b, "uniform_pm1", 1000,
-                                                b * count + lo)
-                ok = ok and recvs[b][lo:lo + m].cpu().numpy().tobytes() == want.tobytes()
-    else:
-        count = 1 << 23
-        sends = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
-        recvs = [torch.empty(P * count, dtype=torch.float32, device="cuda") for _ in range(P)]
-        for r in range(P):
-            al.fill(sends[r], "uniform_pm1", 1000 + r)
-        fn = lambda: al.allgather(recvs, sends, count=count)
-        alg = (P + P * P) * count * 4
-        launches = P
-        fn()
-        torch.cuda.synchronize()
-        ok = True
-        for j in (0, P - 1):
-            for q in (0, P - 1):
-                want = oracle.fill(m, "f32", "uniform_pm1", 1000 + q, count - m)
-                got = recvs[j][(q + 1) * count - m:(q + 1) * count].cpu().numpy()
-                ok = ok and got.tobytes() == want.tobytes()
-    wall, kms = timed(torch, fn, steps, warmup)
+    rotating = name.endswith("_rotating")
+    base = name[:-len("_rotating")] if rotating else name
+    fns, ok = [], True
+    for s in range(4 if rotating else 1):
+        if base == "c2_f32_allreduce":
+            count = 1 << 26
+            ins = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+            outs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+            for r in range(P):
+                al.fill(ins[r], "uniform_pm1", 1000 + r)
+            fn = lambda ins=ins, outs=outs: al.combine(outs, ins, "sum", order="tree_dbl")
+            alg = 2 * P * count * 4
+            launches = count * 4 // (64 << 20) + count * 4 // (32 << 20)
+            fn()
+            torch.cuda.synchronize()
+            for j in (0, P - 1):
+                for lo in (0, count - m):
+                    want = oracle.combine_generated(P, m, "f32", "sum", "tree_dbl", 0, "uniform_pm1", 1000, lo)
+                    ok = ok and outs[j][lo:lo + m].cpu().numpy().tobytes() == want.tobytes()
+        elif base == "c2_f32_reduce_scatter":
+            count = 1 << 23
+            sends = [torch.empty(P * count, dtype=torch.float32, device="cuda") for _ in range(P)]
+            recvs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+            for r in range(P):
+                al.fill(sends[r], "uniform_pm1", 1000 + r)
+            fn = lambda sends=sends, recvs=recvs: al.reduce_scatter(recvs, sends, "sum", order="pairwise_desc",
+                                                                    count=count)
+            alg = (P + 1) * P * count * 4
+            launches = P * count * 4 // (64 << 20)
+            fn()
+            torch.cuda.synchronize()
+            for b in (0, P - 1):
+                for lo in (0, count - m):
+                    want = oracle.combine_generated(P, m, "f32", "sum", "pairwise_desc", b, "uniform_pm1", 1000,
+                                                    b * count + lo)
+                    ok = ok and recvs[b][lo:lo + m].cpu().numpy().tobytes() == want.tobytes()
+        elif base == "c2_f32_allgather":
+            count = 1 << 23
+            sends = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+            recvs = [torch.empty(P * count, dtype=torch.float32, device="cuda") for _ in range(P)]
+            for r in range(P):
+                al.fill(sends[r], "uniform_pm1", 1000 + r)
+            fn = lambda sends=sends, recvs=recvs: al.allgather(recvs, sends, count=count)
+            alg = (P + P * P) * count * 4
+            launches = P
+            fn()
+            torch.cuda.synchronize()
+            for j in (0, P - 1):
+                for q in (0, P - 1):
+                    want = oracle.fill(m, "f32", "uniform_pm1", 1000 + q, count - m)
+                    got = recvs[j][(q + 1) * count - m:(q + 1) * count].cpu().numpy()
+                    ok = ok and got.tobytes() == want.tobytes()
+        else:
+            raise SystemExit("unknown workload %s" % name)
+        fns.append(fn)
+    turn = [0]
+
+    def step():
+        fns[turn[0] % len(fns)]()
+        turn[0] += 1
+    wall, kms = timed(torch, step, steps, warmup)
     return {"workload": name, "dtype": "f32", "op": "sum", "P": P, "count": count, "launches_per_step": launches,
-            "algorithmic_bytes": alg, "ms_per_step": wall * 1e3, "kernel_ms": kms,
+            "buffer_sets": len(fns), "algorithmic_bytes": alg, "ms_per_step": wall * 1e3, "kernel_ms": kms,
             "gbps_wall": alg / wall * 1e-9, "gbps_kernel": alg / (kms * 1e-3) * 1e-9, "parity_vs_oracle": bool(ok)}
 
 
@@ -385,9 +399,10 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2_f32_sum",
-                    choices=sorted(WORKLOADS) + ["c3_ring_stepwise", "c3_ring_fused", "c5_halo", "flags",
-                                               "c2_f32_allreduce", "c2_f32_allgather", "c2_f32_reduce_scatter"])
-    ap.add_argument("--also", default="c2_bf16_sum,c2_f32_sum_rotating,c2_f32_allreduce,c2_f32_reduce_scatter,c2_f32_allgather,c3_ring_fused",
+                    choices=sorted(WORKLOADS) + ["c3_ring_stepwise", "c3_ring_fused", "c5_halo", "flags"] + LAYOUTS)
+    ap.add_argument("--also", default="c2_bf16_sum,c2_f32_sum_rotating,c2_f32_allreduce,c2_f32_allreduce_rotating,"
+                                      "c2_f32_reduce_scatter,c2_f32_reduce_scatter_rotating,c2_f32_allgather,"
+                                      "c2_f32_allgather_rotating,c3_ring_fused",
                     help="comma-separated extra workloads reported under 'also' ('' for none)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--raw", action="store_true", help="print only the workload's own measurement record")
@@ -419,7 +434,7 @@ def main():
         main_res = run_halo_workload(al, torch, args.steps, args.warmup)
     elif args.workload == "flags":
         main_res = run_flag_workload()
-    elif args.workload in ("c2_f32_allreduce", "c2_f32_allgather", "c2_f32_reduce_scatter"):
+    elif args.workload in LAYOUTS:
         main_res = run_layout_workload(al, torch, args.workload, args.steps, args.warmup)
     else:
         main_res = run_combine_workload(al, torch, args.workload, args.steps, args.warmup)

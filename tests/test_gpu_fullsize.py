@@ -253,7 +253,7 @@ def test_allgatherv_large_slices_with_tails(al):
 
 @pytest.mark.parametrize("P,count", [(3, 3 * 300000), (8, 8 * 262144 + 8 * 4)])
 def test_fused_ring_large_segments(al, P, count):
-    """Segments above 1 MiB: fold into the owner, then spread; same bits as the stepwise ring."""
+    """Segments above 1 MiB, one fold launch; same bits as the stepwise ring."""
     import torch
     bufs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
     for r in range(P):
@@ -389,3 +389,46 @@ def test_reduce_scatter_more_than_eight_large_segments(al, order):
     want = oracle.reduce_scatter(sends, "f32", "sum", order)
     for r in range(P):
         assert_bits_equal(recvs[r].cpu().numpy(), want[r], "f32", "%s rank %d" % (order, r))
+
+
+@pytest.mark.parametrize("inplace", (False, True))
+def test_combine_to_several_outputs_in_pieces(al, inplace):
+    """A result above 256 MiB for three outputs alternates fold and spread over 128 MiB pieces:
+    300 MiB + 5 elements, every output equal to the one-output result, windows against the oracle."""
+    import torch
+    P = 3
+    n = (300 << 20) // 4 + 5
+    ins = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(P)]
+    for r in range(P):
+        al.fill(ins[r], "uniform_pm1", 1500 + r)
+    single = torch.empty(n, dtype=torch.float32, device="cuda")
+    al.combine([single], ins, "sum", order="tree_dbl")
+    outs = ins if inplace else [torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(P)]
+    al.combine(outs, ins, "sum", order="tree_dbl")
+    torch.cuda.synchronize()
+    for j in range(P):
+        assert torch.equal(outs[j].view(torch.int32), single.view(torch.int32)), "output %d" % j
+    m = 1 << 16
+    piece = (128 << 20) // 4
+    for lo in (0, piece - m // 2, 2 * piece - m // 2, n - m):
+        want = oracle.combine_generated(P, m, "f32", "sum", "tree_dbl", 0, "uniform_pm1", 1500, lo)
+        assert_bits_equal(single[lo:lo + m].cpu().numpy(), want, "f32", "window at %d" % lo)
+
+
+@pytest.mark.parametrize("P,count", [(3, 3 * 6000000 + 2), (5, 5 * 4200000 + 3)])
+def test_fused_ring_in_pieces(al, P, count):
+    """Fused ring allreduce above 40 MiB: 64 MiB pieces over ragged segments; same bits as the oracle's
+    chunk-by-chunk ring and as the stepwise mode."""
+    import torch
+    bufs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+    for r in range(P):
+        al.fill(bufs[r], "uniform_pm1", 1600 + r)
+    step = [b.clone() for b in bufs]
+    al.ring_allreduce(bufs, "sum", mode="fused")
+    al.ring_allreduce(step, "sum", mode="stepwise")
+    torch.cuda.synchronize()
+    host = [oracle.fill(count, "f32", "uniform_pm1", 1600 + r) for r in range(P)]
+    want = oracle.ring_allreduce(host, "f32", "sum", (4 << 20) // 4)[0]
+    for r in range(P):
+        assert_bits_equal(bufs[r].cpu().numpy(), want, "f32", "fused rank %d" % r)
+        assert torch.equal(step[r].view(torch.int32), bufs[r].view(torch.int32))
