@@ -110,14 +110,16 @@ constexpr int kGatherU = 8, kGatherThreads = 128;
 // 88 % of the HBM peak, against 67 % when every workgroup writes its tile to
 // all destinations (69 % for those writes alone).
 // A chunk's share per XCD (2 MiB) has to stay in that XCD's 4 MiB L2 between
-// the destinations: 32 MiB chunks run at 64 %.  A launch covers at most
-// kSpreadLaunchChunks chunks of every source: in longer launches the XCDs
-// drift apart.  Measured on buffers that no earlier call has touched (1 GiB to
-// 7 destinations): 84 % with 16 MiB chunks and launches of one or two chunks,
-// 80 % with four chunks per launch, 76 % with the whole GiB in one launch,
-// 77 % / 81 % with 8 MiB chunks in one launch / one launch per two chunks.
+// the destinations (a stand-alone copy of this kernel, 1 GiB to 7 destinations
+// that no earlier launch has touched: 32 MiB chunks 64 % of peak, 8 and 16 MiB
+// chunks 76 to 84 % depending on the launch length).  Two waves per SIMD: with
+// the default occupancy the same calls run 4 to 10 points lower on untouched
+// buffers (allgather of 128 MiB slices 69 % against 77 to 86 %).  A launch
+// covers at most kSpreadLaunchChunks chunks of every source; between launch
+// lengths of 32 MiB and the whole source the differences measured through the
+// library (+-2 points) are smaller than those between two runs of one setting.
 constexpr unsigned kSpreadChunkTiles = 1024;
-constexpr unsigned kSpreadLaunchChunks = 2;
+constexpr unsigned kSpreadLaunchChunks = 8;
 __global__ void __launch_bounds__(kGatherThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
 spread_kernel(FoldParams p, unsigned tpc, unsigned tile0) {
   using TL = Tile<kGatherU, kGatherThreads>;

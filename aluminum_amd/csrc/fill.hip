@@ -95,14 +95,19 @@ __global__ void __launch_bounds__(256) widen_kernel(float *dst, const uint16_t *
 
 constexpr int kCopyU = 8, kCopyThreads = 128;
 // Any alignment: b.head + b.tail single bytes by the first workgroup, b.vec bytes in tiles.
-__global__ void __launch_bounds__(kCopyThreads) copy_kernel_vec(char *dst, const char *src, ByteSplit b) {
+// Two waves per SIMD and launches of 256 MiB: measured on 8 GiB that no earlier
+// launch has touched, 81.6 % of the HBM peak (one launch 76 %, 64 MiB launches
+// 76 %, four or eight waves per SIMD 73 % / 70 %).
+constexpr size_t kCopyTilesPerLaunch = 16384;
+__global__ void __launch_bounds__(kCopyThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
+copy_kernel_vec(char *dst, const char *src, ByteSplit b, size_t tile0) {
   using TL = Tile<kCopyU, kCopyThreads>;
   const TL tl;
-  if (blockIdx.x == 0 && threadIdx.x < b.head + b.tail) {
+  if (tile0 == 0 && blockIdx.x == 0 && threadIdx.x < b.head + b.tail) {
     const size_t i = threadIdx.x < b.head ? threadIdx.x : b.vec + threadIdx.x;
     dst[i] = src[i];
   }
-  const size_t tb = (size_t)blockIdx.x * TL::BYTES;
+  const size_t tb = (tile0 + blockIdx.x) * TL::BYTES;
   if (tb >= b.vec) return;
   const int nrec = b.vec - tb > TL::BYTES ? (int)TL::BYTES : (int)(b.vec - tb);
   const auto rs = TL::rsrc(src + b.head + tb, nrec);
@@ -173,9 +178,11 @@ int alamd_copy(void *dst, const void *src, size_t bytes, void *stream) {
   const size_t tile = Tile<kCopyU, kCopyThreads>::BYTES;
   size_t tiles = (b.vec + tile - 1) / tile;
   if (tiles == 0) tiles = 1;
-  if (tiles * kCopyThreads > 0xffffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "copy too large for one launch");
-  hipLaunchKernelGGL(copy_kernel_vec, dim3((unsigned)tiles), dim3(kCopyThreads), 0, as_stream(stream), (char *)dst,
-                     (const char *)src, b);
+  for (size_t t0 = 0; t0 < tiles; t0 += kCopyTilesPerLaunch) {
+    const size_t nt = tiles - t0 < kCopyTilesPerLaunch ? tiles - t0 : kCopyTilesPerLaunch;
+    hipLaunchKernelGGL(copy_kernel_vec, dim3((unsigned)nt), dim3(kCopyThreads), 0, as_stream(stream), (char *)dst,
+                       (const char *)src, b, t0);
+  }
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
 }
