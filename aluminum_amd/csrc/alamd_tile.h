@@ -26,10 +26,27 @@ constexpr unsigned kRsrcFlags = 0x00020000u;
 
 // Workgroups are handed to the eight XCDs round-robin and each XCD then works
 // through its share at its own pace, so over a long launch the XCDs drift
-// apart and the addresses in flight spread over more DRAM pages.  A launch
-// therefore covers at most this many tiles per stream (64 MiB at 16 KiB per
-// tile); longer inputs are cut into consecutive launches on the same stream.
-constexpr size_t kMaxTilesPerLaunch = 4096;
+// apart and the addresses in flight spread over more DRAM pages.  Longer inputs
+// are therefore cut into consecutive launches on the same stream.  The best
+// cut shrinks with the number of streams, and cuts that are not powers of two
+// run 1 to 2 points lower than their power-of-two neighbours.  Measured on
+// untouched buffers of 256 MiB per rank, % of the HBM peak by tiles of 16 KiB
+// per stream and launch (2048 / 4096 / 8192 / 16384 / 32768):
+//   P = 2: 68 75 78 79 79     P = 3: 72 76 77 77 77     P = 4: 73 76 77 76 77
+//   P = 6: 74 76 76 75 74     P = 8: 76 77 76 75 75     P = 12: 76 75 74 72 72
+// The rule below picks 16384, 8192, 8192, 4096, 4096 and 2048 for these.
+constexpr size_t kLaunchBytes = (size_t)800 << 20;
+// Tiles (of `tile_bytes` per stream) in one launch of a kernel that reads `nin` streams and
+// writes one: the largest power of two that keeps the launch within kLaunchBytes.
+inline size_t floor_pow2(size_t v) {
+  size_t t = 1;
+  while (t * 2 <= v) t *= 2;
+  return t;
+}
+inline size_t launch_tiles(int nin, size_t tile_bytes) {
+  const size_t t = floor_pow2(kLaunchBytes / ((size_t)(nin + 1) * tile_bytes));
+  return t < 8 ? 8 : t;
+}
 
 // Loads of 128 bits run at full rate from any 4-byte-aligned address; from an
 // address that splits its dwords they lose about a fifth of the bandwidth

@@ -137,10 +137,10 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   if (tiles == 0) tiles = 1;
   // the launch cut is a number of bytes over all segments of a launch, whatever the tile size: small
   // work in one launch; otherwise up to eight segments side by side (blockIdx.y)
-  const size_t per_launch = kMaxTilesPerLaunch * (size_t)16384 / Tile<S::U, S::THREADS>::BYTES;
+  const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES);
   const bool small = tiles * nseg <= per_launch;
   const unsigned segs = small || nseg < 8 ? nseg : 8;
-  const size_t cut = small ? tiles : per_launch / segs;
+  const size_t cut = small ? tiles : floor_pow2(per_launch / segs);
   TreeParams q = p;
   for (size_t t0 = 0; t0 < tiles; t0 += cut) {
     const size_t nt = tiles - t0 < cut ? tiles - t0 : cut;

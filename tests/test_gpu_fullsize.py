@@ -128,19 +128,22 @@ def test_c5_halo_full_size(al):
     assert (g3[:h, h:-h, h:-h] == b3[h:2 * h, h:-h, h:-h]).all()
 
 
-def test_multi_launch_boundaries(al):
-    """Counts around the 4096-tile launch cut (64 MiB per stream) and a ragged tail."""
+@pytest.mark.parametrize("P,cut", [(2, 16384), (8, 4096), (12, 2048)])
+def test_multi_launch_boundaries(al, P, cut):
+    """Counts around the launch cut (a power of two of 16 KiB tiles that depends on the number of
+    ranks) and a ragged tail."""
     import torch
     tile = 16384 // 4
-    for n in (4096 * tile - 1, 4096 * tile, 4096 * tile + 1, 2 * 4096 * tile + 4099):
-        ins = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(2)]
-        for r in range(2):
+    for n in (cut * tile - 1, cut * tile + 1, 2 * cut * tile + 4099):
+        ins = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(P)]
+        for r in range(P):
             al.fill(ins[r], "uniform_pm1", 77 + r)
         out = torch.empty(n, dtype=torch.float32, device="cuda")
         al.combine([out], ins, "sum")
         torch.cuda.synchronize()
-        want = oracle.combine_generated(2, n, "f32", "sum", "rank_asc", 0, "uniform_pm1", 77)
+        want = oracle.combine_generated(P, n, "f32", "sum", "rank_asc", 0, "uniform_pm1", 77)
         assert_bits_equal(out.cpu().numpy(), want, "f32", "n=%d" % n)
+        del ins, out
 
 
 def test_buffers_beyond_4_gib(al):
