@@ -159,6 +159,6 @@ int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, 
 // The general form: source q = fp.in[q], fp.seg.seg_len[q] bytes, copied to byte offset
 // fp.seg.seg_off[q] of every fp.out[0..fp.P) except where that is the source itself.
 // split_large: give every slice of 16 MiB and more a launch of its own.
-int launch_spread_table(const FoldParams &fp, int nsrc, bool split_large, hipStream_t stream);
+int launch_spread_table(const FoldParams &fp, int nsrc, bool from_hbm, hipStream_t stream);
 
 }  // namespace alamd

@@ -99,7 +99,7 @@ constexpr int kGatherU = 8, kGatherThreads = 128;
 // Slices to several destinations: blockIdx.y = source q, whose seg_len[q] bytes
 // go to byte offset seg_off[q] of every destination p.out[0..P) (a destination
 // that is the source itself, the in-place form, is skipped).  One workgroup
-// per (destination, tile).  blockIdx.x runs chunk by chunk (tpc tiles, 16 MiB);
+// per (destination, tile).  blockIdx.x runs chunk by chunk (tpc tiles, 8 or 16 MiB);
 // inside a chunk all tiles of destination 0 come first, then destination 1,
 // ...: at any time the device writes one contiguous stream per chunk instead
 // of P interleaved ones, and re-reads the chunk of the source from cache:
@@ -109,17 +109,24 @@ constexpr int kGatherU = 8, kGatherThreads = 128;
 // of 4 only, 49 % with an odd tpc).  Measured for 1 read + 8 writes of 32 MiB:
 // 88 % of the HBM peak, against 67 % when every workgroup writes its tile to
 // all destinations (69 % for those writes alone).
-// A chunk's share per XCD (2 MiB) has to stay in that XCD's 4 MiB L2 between
-// the destinations (a stand-alone copy of this kernel, 1 GiB to 7 destinations
-// that no earlier launch has touched: 32 MiB chunks 64 % of peak, 8 and 16 MiB
-// chunks 76 to 84 % depending on the launch length).  Two waves per SIMD: with
-// the default occupancy the same calls run 4 to 10 points lower on untouched
-// buffers (allgather of 128 MiB slices 69 % against 77 to 86 %).  A launch
-// covers at most kSpreadLaunchChunks chunks of every source; between launch
-// lengths of 32 MiB and the whole source the differences measured through the
-// library (+-2 points) are smaller than those between two runs of one setting.
-constexpr unsigned kSpreadChunkTiles = 1024;
-constexpr unsigned kSpreadLaunchChunks = 8;
+// A chunk's share per XCD (at most 2 MiB) has to stay in that XCD's 4 MiB L2
+// between the destinations: 32 MiB chunks run at 64 to 79 % of peak.  Two
+// waves per SIMD: with the default occupancy the same calls run 4 to 10 points
+// lower on buffers that no earlier call has touched.  Chunk length and launch
+// length depend on where the source comes from (settings compared in one
+// process, alternating, on separately allocated buffers; chunk tiles / chunks
+// per launch):
+//  - slices read from HBM (an allgather): 16 MiB chunks, launches of two chunks
+//    per source.  Untouched 128 MiB slices: 1024/1 and 1024/2 83 %, 1024/4
+//    79 %, 1024/8 77 %, 512/4 79 %, whole slice in one launch 77 %; untouched
+//    32 MiB slices: 1024/any 83 %, 512/any 79 %; repeated buffers: 92 to 94 %.
+//  - a result that a fold has just written, still in the memory-side cache (the
+//    second step of a combine into several buffers): 8 MiB chunks, launches of
+//    sixteen.  Allreduce at 256 MiB / 1 GiB per rank, untouched: 512/16 82 % /
+//    81.5 %, 1024/8 81.5 % / 80 %, 1024/2 79.6 % / 78.8 %, whole piece in one
+//    launch 80.4 % / 80.5 %; repeated: 512/16 86 %, 1024/2 83 %.
+struct SpreadShape { unsigned chunk_tiles, launch_chunks; };
+constexpr SpreadShape kSpreadFromHbm = {1024, 2}, kSpreadFromCache = {512, 16};
 __global__ void __launch_bounds__(kGatherThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
 spread_kernel(FoldParams p, unsigned tpc, unsigned tile0) {
   using TL = Tile<kGatherU, kGatherThreads>;
@@ -170,7 +177,7 @@ int check_common(int P, size_t count, int dtype) {
 
 namespace {
 
-int launch_spread_once(const FoldParams &fp, int nsrc, hipStream_t stream) {
+int launch_spread_once(const FoldParams &fp, int nsrc, SpreadShape shape, hipStream_t stream) {
   size_t max_len = 0;
   for (int q = 0; q < nsrc; ++q)
     if (fp.seg.seg_len[q] > max_len) max_len = fp.seg.seg_len[q];
@@ -178,8 +185,8 @@ int launch_spread_once(const FoldParams &fp, int nsrc, hipStream_t stream) {
   const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
   const size_t tiles = (max_len + tile - 1) / tile;
   // always a multiple of 8 (see spread_kernel); workgroups past the last tile exit at once
-  const size_t tpc = tiles < kSpreadChunkTiles ? (tiles + 7) & ~(size_t)7 : kSpreadChunkTiles;
-  const size_t per_launch = tpc * kSpreadLaunchChunks;
+  const size_t tpc = tiles < shape.chunk_tiles ? (tiles + 7) & ~(size_t)7 : shape.chunk_tiles;
+  const size_t per_launch = tpc * shape.launch_chunks;
   // a launch holds fewer than 2^32 threads in x
   if (per_launch * (size_t)fp.P * kGatherThreads > 0xffffffffull || tiles > 0xffffffffull)
     return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
@@ -195,25 +202,26 @@ int launch_spread_once(const FoldParams &fp, int nsrc, hipStream_t stream) {
 
 }  // namespace
 
-// split_large: slices of one chunk (16 MiB) and more get launches of their own, the smaller ones share one.
-// For an allgather of separate send buffers one launch over large slices is long enough for the XCDs to
-// drift apart (32 MiB slices: 88 % of peak one by one, 83 % together; 8 MiB slices: 85 us together,
-// 98 us one by one; 1 MiB: 15 us against 43 us).  Segments that a fold has just written are spread
-// faster in one launch (eight 32 MiB segments: 650 us for the whole allreduce against 667 us).
-int launch_spread_table(const FoldParams &fp, int nsrc, bool split_large, hipStream_t stream) {
-  const size_t big = (size_t)kSpreadChunkTiles * Tile<kGatherU, kGatherThreads>::BYTES;
+// from_hbm: the sources are slices that no launch has just written (an allgather).  Slices of one
+// chunk (16 MiB) and more then get launches of their own, the smaller ones share one: one launch over
+// several large slices is long enough for the XCDs to drift apart (32 MiB slices: 88 % of peak one by
+// one, 83 % together; 8 MiB slices: 85 us together, 98 us one by one; 1 MiB: 15 us against 43 us).
+// Otherwise the sources are what a fold has just written, and all of them share the launches.
+int launch_spread_table(const FoldParams &fp, int nsrc, bool from_hbm, hipStream_t stream) {
+  if (!from_hbm) return launch_spread_once(fp, nsrc, kSpreadFromCache, stream);
+  const size_t big = (size_t)kSpreadFromHbm.chunk_tiles * Tile<kGatherU, kGatherThreads>::BYTES;
   FoldParams rest = fp;
-  for (int q = 0; q < nsrc && nsrc > 1 && split_large; ++q) {
+  for (int q = 0; q < nsrc && nsrc > 1; ++q) {
     if (fp.seg.seg_len[q] < big) continue;
     FoldParams one = fp;
     one.in[0] = fp.in[q];
     one.seg.seg_off[0] = fp.seg.seg_off[q];
     one.seg.seg_len[0] = fp.seg.seg_len[q];
-    const int rc = launch_spread_once(one, 1, stream);
+    const int rc = launch_spread_once(one, 1, kSpreadFromHbm, stream);
     if (rc) return rc;
     rest.seg.seg_len[q] = 0;
   }
-  return launch_spread_once(rest, nsrc, stream);
+  return launch_spread_once(rest, nsrc, kSpreadFromHbm, stream);
 }
 
 int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, hipStream_t stream) {

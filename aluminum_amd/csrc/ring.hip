@@ -216,7 +216,7 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
     }
     int rc = launch_fold(fo, (unsigned)P, longest, dtype, op, true, stream);
     if (rc) return rc;
-    if ((rc = launch_spread_table(sp, P, true, stream))) return rc;
+    if ((rc = launch_spread_table(sp, P, false, stream))) return rc;
   }
   return ALAMD_OK;
 }
