@@ -168,10 +168,11 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
     }
     FoldParams q = p;
     // about per_launch workgroups per launch, whatever the number of segments: small work in one
-    // launch; otherwise up to eight segments side by side (blockIdx.y), the rest in further launches
+    // launch; otherwise up to four segments side by side (blockIdx.y), the rest in further launches
+    // (eight side by side run 0.5 to 1 point lower on untouched buffers, one or two the same)
     const size_t per_launch = launch_tiles(p.P, Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES);
     const bool small = tiles * nseg <= per_launch;
-    const unsigned segs = small || nseg < 8 ? nseg : 8;
+    const unsigned segs = small || nseg < 4 ? nseg : 4;
     const size_t cut = small ? tiles : floor_pow2(per_launch / segs);
     for (size_t t0 = 0; t0 < tiles; t0 += cut) {
       const size_t nt = tiles - t0 < cut ? tiles - t0 : cut;

@@ -136,10 +136,10 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   size_t tiles = (max_len + tile_elems - 1) / tile_elems;
   if (tiles == 0) tiles = 1;
   // the launch cut is a number of bytes over all segments of a launch, whatever the tile size: small
-  // work in one launch; otherwise up to eight segments side by side (blockIdx.y)
+  // work in one launch; otherwise up to four segments side by side (blockIdx.y)
   const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES);
   const bool small = tiles * nseg <= per_launch;
-  const unsigned segs = small || nseg < 8 ? nseg : 8;
+  const unsigned segs = small || nseg < 4 ? nseg : 4;
   const size_t cut = small ? tiles : floor_pow2(per_launch / segs);
   TreeParams q = p;
   for (size_t t0 = 0; t0 < tiles; t0 += cut) {
