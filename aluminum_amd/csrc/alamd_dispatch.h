@@ -135,10 +135,15 @@ int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, i
 
 // A result that goes to several buffers is folded into one of them and then
 // spread (one write stream per workgroup) when that is faster than writing
-// every tile to all of them from the fold kernel: from three outputs and 40 MiB
-// up (measured at P = 8: 32 MiB 81 us in one kernel / 86 us in two steps, 48 MiB
-// 146 / 128, 256 MiB 773 / 667; two outputs 437 / 455, four 544 / 529).
-constexpr size_t kTwoStepMinBytes = (size_t)40 << 20;
+// every tile to all of them from the fold kernel: from three outputs and 16 MiB
+// up.  Measured at P = 8, eight outputs, us per call in one kernel / in two
+// steps, on buffers that no earlier call has touched: 8 MiB 25 / 24, 16 MiB
+// 50 / 44, 32 MiB 99 / 85, 64 MiB 197 / 165, 128 MiB 393 / 328 (4 MiB: 12 / 15);
+// on the same buffers again and again: 8 MiB 20 / 24, 16 MiB 40 / 44, 32 MiB
+// 77 / 84, 40 MiB 119 / 103, 64 MiB 196 / 162, 128 MiB 394 / 318 (the two steps
+// take the same time either way).  At 256 MiB: two outputs 437 / 455, four
+// 544 / 529.
+constexpr size_t kTwoStepMinBytes = (size_t)16 << 20;
 constexpr int kTwoStepMinOutputs = 3;
 // The two steps alternate over pieces of the result of this many bytes, so that
 // the spread reads what the fold has just written from the 256 MiB memory-side

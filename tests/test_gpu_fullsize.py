@@ -168,7 +168,7 @@ def test_buffers_beyond_4_gib(al):
 
 
 def test_allgather_large_slices(al):
-    """Slices above 1 MiB take the one-launch-per-source path; also in place."""
+    """Slices of a few MB (below the 16 MiB from which a slice gets launches of its own); also in place."""
     import torch
     P = 5
     for count in (700001, 700004):  # 2.8 MB fp32 slices: byte path, then 16-byte aligned vector path
@@ -213,8 +213,8 @@ def test_allgather_large_slices(al):
 @pytest.mark.parametrize("order", ("rank_asc", "tree_dbl"))
 @pytest.mark.parametrize("inplace", (False, True))
 def test_large_combine_to_several_outputs(al, order, inplace):
-    """Above 1 MiB a result for several outputs is folded into the first and then spread,
-    64 MiB at a time: counts around that piece size, three ranks, separate and in-place outputs."""
+    """From 16 MiB up a result for several outputs is folded into the first and then spread: one
+    count below that and three around 64 MiB, three ranks, separate and in-place outputs."""
     import torch
     P = 3
     piece = (64 << 20) // 4
@@ -231,7 +231,7 @@ def test_large_combine_to_several_outputs(al, order, inplace):
 
 
 def test_allgatherv_large_slices_with_tails(al):
-    """Slices above 1 MiB whose byte counts are not multiples of 16, placed back to front."""
+    """Slices of 1 to 2 MB whose byte counts are not multiples of 16, placed back to front."""
     import torch
     P = 4
     counts = [300001, 0, 262147, 500003]
@@ -420,7 +420,7 @@ def test_combine_to_several_outputs_in_pieces(al, inplace):
 
 @pytest.mark.parametrize("P,count", [(3, 3 * 6000000 + 2), (5, 5 * 4200000 + 3)])
 def test_fused_ring_in_pieces(al, P, count):
-    """Fused ring allreduce above 40 MiB: 64 MiB pieces over ragged segments; same bits as the oracle's
+    """Fused ring allreduce above 16 MiB: 64 MiB pieces over ragged segments; same bits as the oracle's
     chunk-by-chunk ring and as the stepwise mode."""
     import torch
     bufs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
