@@ -224,12 +224,17 @@ template <typename T> __device__ __forceinline__ void st_elem(void *p, T v) {
 // its element type is refused.
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
-// A byte range as the copy kernels walk it: `head` bytes up to the source's
-// next 4-byte boundary, `vec` bytes in whole 128-bit vectors, `tail` < 16.
+// A byte range as the copy kernel walks it: `head` single bytes, `vec` bytes in
+// whole 128-bit vectors, `tail` < 16.  The vectors start where the destination
+// reaches a 64-byte boundary, so that every line is stored whole, if that
+// leaves the loads 4-byte aligned (128-bit loads run at full rate from any
+// 4-byte boundary and lose a fifth when they split dwords); otherwise at the
+// source's next 4-byte boundary.
 struct ByteSplit { size_t head, vec, tail; };
-__host__ __device__ inline ByteSplit split_bytes(const void *src, size_t bytes) {
+inline ByteSplit split_bytes(const void *dst, const void *src, size_t bytes) {
+  const uintptr_t d = reinterpret_cast<uintptr_t>(dst), s = reinterpret_cast<uintptr_t>(src);
   ByteSplit b;
-  b.head = (4 - (reinterpret_cast<uintptr_t>(src) & 3)) & 3;
+  b.head = ((d ^ s) & 3) == 0 ? (64 - (d & 63)) & 63 : (4 - (s & 3)) & 3;
   if (b.head > bytes) b.head = bytes;
   b.vec = (bytes - b.head) & ~(size_t)15;
   b.tail = bytes - b.head - b.vec;

@@ -49,17 +49,18 @@ inline size_t launch_tiles(int nin, size_t tile_bytes) {
 }
 
 // Loads of 128 bits run at full rate from any 4-byte-aligned address; from an
-// address that splits its dwords they lose about a fifth of the bandwidth
-// (stores do not care).  For element types narrower than 4 bytes the kernels
-// therefore handle up to three bytes' worth of leading elements one by one, so
-// that the vectors of the stream at `first` start on a dword boundary.
-template <typename T> __device__ __forceinline__ size_t head_elems(const char *first, size_t len) {
-  if constexpr (sizeof(T) >= 4) {
-    return 0;
-  } else {
-    const size_t h = ((4u - (unsigned)(reinterpret_cast<uintptr_t>(first) & 3u)) & 3u) / sizeof(T);
-    return h < len ? h : len;
-  }
+// address that splits its dwords they lose about a fifth of the bandwidth.
+// Stores want whole 64-byte lines: on buffers that no earlier launch has
+// touched, a fold whose output starts 4, 16 or 32 bytes off a 64-byte boundary
+// runs at 70.6 % of the HBM peak against 79 %.  The kernels therefore handle
+// the leading elements one by one up to the output's next 64-byte boundary
+// (at most 63 bytes' worth), if that leaves the first input's vectors on a
+// dword boundary; otherwise up to the first input's next dword boundary.
+template <typename T> __device__ __forceinline__ size_t head_elems(const char *out, const char *first, size_t len) {
+  const uintptr_t o = reinterpret_cast<uintptr_t>(out), f = reinterpret_cast<uintptr_t>(first);
+  const size_t bytes = ((o ^ f) & 3u) == 0 ? (64u - (unsigned)(o & 63u)) & 63u : (4u - (unsigned)(f & 3u)) & 3u;
+  const size_t h = bytes / sizeof(T);
+  return h < len ? h : len;
 }
 
 template <int U, int THREADS> struct Tile {

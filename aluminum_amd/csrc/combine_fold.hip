@@ -69,7 +69,7 @@ fold_vec_kernel(const FoldParams p) {
   size_t out_bytes;
   out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
 
-  const size_t head = head_elems<T>(p.in[s] + in_bytes, len);
+  const size_t head = head_elems<T>(p.out[j0] + out_bytes, p.in[s] + in_bytes, len);
   const size_t vlen = len - head;
   const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
   const size_t vec_bytes = (vlen / N) * 16;

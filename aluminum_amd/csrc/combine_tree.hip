@@ -69,7 +69,7 @@ tree_vec_kernel(const TreeParams p) {
   tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
   const int nvalid = MODE == TREE_FULL ? SLOTS : p.nvalid;
 
-  const size_t head = head_elems<T>(p.a[0] + in_bytes, len);
+  const size_t head = head_elems<T>(p.out[j0] + out_bytes, p.a[0] + in_bytes, len);
   const size_t vlen = len - head;
   const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
   const size_t vec_bytes = (vlen / N) * 16;

@@ -174,7 +174,7 @@ int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void
 int alamd_copy(void *dst, const void *src, size_t bytes, void *stream) {
   if (bytes == 0) return ALAMD_OK;
   if (!dst || !src) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer");
-  const ByteSplit b = split_bytes(src, bytes);
+  const ByteSplit b = split_bytes(dst, src, bytes);
   const size_t tile = Tile<kCopyU, kCopyThreads>::BYTES;
   size_t tiles = (b.vec + tile - 1) / tile;
   if (tiles == 0) tiles = 1;

@@ -48,7 +48,7 @@ ring_step_vec_kernel(const RingParams p) {
   char *local = p.buf[r] + off * sizeof(T);
   const char *recv = p.buf[from] + off * sizeof(T);
   constexpr size_t N = 16 / sizeof(T);
-  const size_t head = head_elems<T>(recv, len);
+  const size_t head = head_elems<T>(local, recv, len);
   const size_t vlen = len - head;
   // the head elements and the vlen % N elements after the last whole vector, one per thread of the
   // segment's first workgroup

@@ -118,6 +118,36 @@ def test_vector_path_at_any_element_alignment(al, dtype):
             assert_bits_equal(to_host(o, ins[0].dtype), want, dtype, "%s %s" % (dtype, order))
 
 
+@pytest.mark.parametrize("dtype", ("u8", "i16", "bf16", "f32", "f64"))
+def test_head_up_to_the_outputs_64_byte_boundary(al, dtype):
+    """The kernels walk the leading elements one by one until the output reaches a 64-byte boundary:
+    outputs 1 element to 60 bytes past a boundary, inputs at the same or at other offsets, counts
+    shorter than the head, equal to it and far beyond; fold and tree orders, combine and allgather."""
+    import torch
+    P = 3
+    es = oracle.dtype_size(dtype)
+    for out_off in (1, 60 // es, max(1, 36 // es)):
+        for in_off in (out_off, 0, out_off + 4 // min(es, 4)):
+            for n in (1, 64 // es - out_off, 64 // es, 3 * 4096 + 5):
+                if n < 1:
+                    continue
+                ins = make_inputs(P, n, dtype, "sum", seed=90 + out_off)
+                views = [_offset_view(a, in_off) for a in ins]
+                for order in ("rank_asc", "tree_halv"):
+                    want = oracle.combine(ins, dtype, "sum", order)
+                    raw = dev_empty(n + out_off + 16, ins[0].dtype)
+                    al.combine([raw[out_off:out_off + n]], views, "sum", order=order, dtype=dtype, count=n)
+                    torch.cuda.synchronize()
+                    assert_bits_equal(to_host(raw, ins[0].dtype)[out_off:out_off + n], want, dtype,
+                                      "%s %s out+%d in+%d n=%d" % (dtype, order, out_off, in_off, n))
+                recvs = [dev_empty(P * n + out_off + 16, ins[0].dtype) for _ in range(P)]
+                al.allgather([r[out_off:out_off + P * n] for r in recvs], views, dtype=dtype, count=n)
+                torch.cuda.synchronize()
+                for r in recvs:
+                    got = to_host(r, ins[0].dtype)[out_off:out_off + P * n]
+                    assert got.tobytes() == np.concatenate(ins).tobytes(), "allgather out+%d n=%d" % (out_off, n)
+
+
 @pytest.mark.parametrize("dtype", ("u8", "bf16", "f32", "f64"))
 @pytest.mark.parametrize("inplace", (False, True))
 def test_reduce_scatter_odd_block_sizes(al, dtype, inplace):
