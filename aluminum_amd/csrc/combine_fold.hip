@@ -157,8 +157,6 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
                                (OP == ALAMD_MIN || OP == ALAMD_MAX);
     void (*kern)(const FoldParams) = nullptr;
     const size_t tile_elems = Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES / sizeof(T);
-    size_t tiles = (max_len + tile_elems - 1) / tile_elems;
-    if (tiles == 0) tiles = 1;
     if (p.P == 8) {
       if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 8> : fold_vec_kernel<T, OP, false, 8>;
       else kern = fold_vec_kernel<T, OP, false, 8>;
@@ -167,22 +165,12 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
       else kern = fold_vec_kernel<T, OP, false, 0>;
     }
     FoldParams q = p;
-    // about per_launch workgroups per launch, whatever the number of segments: small work in one
-    // launch; otherwise up to four segments side by side (blockIdx.y), the rest in further launches
-    // (eight side by side run 0.5 to 1 point lower on untouched buffers, one or two the same)
     const size_t per_launch = launch_tiles(p.P, Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES);
-    const bool small = tiles * nseg <= per_launch;
-    const unsigned segs = small || nseg < 4 ? nseg : 4;
-    const size_t cut = small ? tiles : floor_pow2(per_launch / segs);
-    for (size_t t0 = 0; t0 < tiles; t0 += cut) {
-      const size_t nt = tiles - t0 < cut ? tiles - t0 : cut;
+    plan_launches(p.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
       q.seg.tile0 = t0;
-      for (unsigned s0 = 0; s0 < nseg; s0 += segs) {
-        q.seg.seg0 = s0;
-        hipLaunchKernelGGL(kern, dim3((unsigned)nt, nseg - s0 < segs ? nseg - s0 : segs, 1),
-                           dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
-      }
-    }
+      q.seg.seg0 = s0;
+      hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
+    });
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;
   });

@@ -133,24 +133,14 @@ template <typename T, int OP, int SLOTS, int MODE>
 int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream) {
   using S = TreeShape<T, OP, SLOTS, MODE>;
   const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
-  size_t tiles = (max_len + tile_elems - 1) / tile_elems;
-  if (tiles == 0) tiles = 1;
-  // the launch cut is a number of bytes over all segments of a launch, whatever the tile size: small
-  // work in one launch; otherwise up to four segments side by side (blockIdx.y)
   const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES);
-  const bool small = tiles * nseg <= per_launch;
-  const unsigned segs = small || nseg < 4 ? nseg : 4;
-  const size_t cut = small ? tiles : floor_pow2(per_launch / segs);
   TreeParams q = p;
-  for (size_t t0 = 0; t0 < tiles; t0 += cut) {
-    const size_t nt = tiles - t0 < cut ? tiles - t0 : cut;
+  plan_launches(p.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
     q.seg.tile0 = t0;
-    for (unsigned s0 = 0; s0 < nseg; s0 += segs) {
-      q.seg.seg0 = s0;
-      hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE>), dim3((unsigned)nt, nseg - s0 < segs ? nseg - s0 : segs, 1),
-                         dim3(S::THREADS, 1, 1), 0, stream, q);
-    }
-  }
+    q.seg.seg0 = s0;
+    hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE>), dim3((unsigned)nt, ns, 1), dim3(S::THREADS, 1, 1), 0,
+                       stream, q);
+  });
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
 }

@@ -435,3 +435,21 @@ def test_fused_ring_in_pieces(al, P, count):
     for r in range(P):
         assert_bits_equal(bufs[r].cpu().numpy(), want, "f32", "fused rank %d" % r)
         assert torch.equal(step[r].view(torch.int32), bufs[r].view(torch.int32))
+
+
+@pytest.mark.parametrize("order", ("rank_asc", "tree_halv"))
+def test_reduce_scatterv_very_unequal_blocks(al, order):
+    """One block of 144 MB beside blocks of 20 bytes, nothing and 36 MB: the long blocks get launches of
+    their own (several each), the short ones theirs."""
+    import torch
+    P = 4
+    counts = [36000000, 5, 0, 9000001]
+    total = sum(counts)
+    sends = [oracle.fill(total, "f32", "uniform_pm1", 1700 + r) for r in range(P)]
+    d_sends = [to_dev(s) for s in sends]
+    recvs = [torch.zeros(max(c, 1), dtype=torch.float32, device="cuda") for c in counts]
+    al.reduce_scatterv(recvs, d_sends, counts, "sum", order=order)
+    torch.cuda.synchronize()
+    want = oracle.reduce_scatterv(sends, counts, "f32", "sum", order)
+    for b in range(P):
+        assert_bits_equal(recvs[b].cpu().numpy()[:counts[b]], want[b], "f32", "%s block %d" % (order, b))
