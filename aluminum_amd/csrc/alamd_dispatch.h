@@ -161,7 +161,12 @@ void plan_launches(const SegParams &seg, unsigned nseg, size_t max_len, size_t t
     }
     if (hi > 0) {
       const size_t cut = hi * n <= per_launch ? hi : floor_pow2(per_launch / n);
-      for (size_t t0 = 0; t0 < hi; t0 += cut) launch(t0, hi - t0 < cut ? hi - t0 : cut, s0, n);
+      // a remainder of less than half a cut rides with the launch before it
+      for (size_t t0 = 0; t0 < hi;) {
+        const size_t nt = hi - t0 < cut + cut / 2 ? hi - t0 : cut;
+        launch(t0, nt, s0, n);
+        t0 += nt;
+      }
     }
     s0 += n;
   }

@@ -191,13 +191,15 @@ int launch_spread_once(const FoldParams &fp, int nsrc, SpreadShape shape, hipStr
   const size_t tpc = tiles < shape.chunk_tiles ? (tiles + 7) & ~(size_t)7 : shape.chunk_tiles;
   const size_t per_launch = tpc * shape.launch_chunks;
   // a launch holds fewer than 2^32 threads in x
-  if (per_launch * (size_t)fp.P * kGatherThreads > 0xffffffffull || tiles > 0xffffffffull)
+  if (2 * per_launch * (size_t)fp.P * kGatherThreads > 0xffffffffull || tiles > 0xffffffffull)
     return set_error(ALAMD_ERR_INVALID_ARG, "count too large for one launch");
-  for (size_t t0 = 0; t0 < tiles; t0 += per_launch) {
-    const size_t nt = tiles - t0 < per_launch ? tiles - t0 : per_launch;
+  // a remainder of less than half a launch rides with the launch before it
+  for (size_t t0 = 0; t0 < tiles;) {
+    const size_t nt = tiles - t0 < per_launch + per_launch / 2 ? tiles - t0 : per_launch;
     const size_t chunks = (nt + tpc - 1) / tpc;
     hipLaunchKernelGGL(spread_kernel, dim3((unsigned)(chunks * tpc * (size_t)fp.P), (unsigned)nsrc, 1),
                        dim3(kGatherThreads, 1, 1), 0, stream, fp, (unsigned)tpc, (unsigned)t0);
+    t0 += nt;
   }
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
@@ -312,8 +314,8 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   // overwritten by a launch that follows the fold of that piece on the same
   // stream, and no other piece reads it.
   const size_t piece = bytes > 2 * kTwoStepPieceBytes ? kTwoStepPieceBytes / es : count;
-  for (size_t e0 = 0; e0 < count; e0 += piece) {
-    const size_t n = count - e0 < piece ? count - e0 : piece;
+  for (size_t e0 = 0, n; e0 < count; e0 += n) {
+    n = count - e0 < piece + piece / 2 ? count - e0 : piece;  // no short last piece
     Layout pl = lay;
     pl.seg = make_seg(n, 0, 0, OUT_ALL, 1);
     pl.max_len = n;

@@ -178,10 +178,12 @@ int alamd_copy(void *dst, const void *src, size_t bytes, void *stream) {
   const size_t tile = Tile<kCopyU, kCopyThreads>::BYTES;
   size_t tiles = (b.vec + tile - 1) / tile;
   if (tiles == 0) tiles = 1;
-  for (size_t t0 = 0; t0 < tiles; t0 += kCopyTilesPerLaunch) {
-    const size_t nt = tiles - t0 < kCopyTilesPerLaunch ? tiles - t0 : kCopyTilesPerLaunch;
+  // a remainder of less than half a launch rides with the launch before it
+  for (size_t t0 = 0; t0 < tiles;) {
+    const size_t nt = tiles - t0 < kCopyTilesPerLaunch + kCopyTilesPerLaunch / 2 ? tiles - t0 : kCopyTilesPerLaunch;
     hipLaunchKernelGGL(copy_kernel_vec, dim3((unsigned)nt), dim3(kCopyThreads), 0, as_stream(stream), (char *)dst,
                        (const char *)src, b, t0);
+    t0 += nt;
   }
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;

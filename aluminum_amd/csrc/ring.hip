@@ -192,7 +192,8 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   const size_t tile_elems = Tile<8, 128>::BYTES / es;
   size_t piece = kRingPieceBytes / (size_t)P / es / tile_elems * tile_elems;
   if (piece == 0) piece = tile_elems;
-  for (size_t e0 = 0; e0 < max_len; e0 += piece) {
+  for (size_t e0 = 0, pn; e0 < max_len; e0 += pn) {
+    pn = max_len - e0 < piece + piece / 2 ? max_len - e0 : piece;  // no short last piece
     FoldParams fo = fp;
     fo.seg.out_mode = OUT_OWNER;
     fo.seg.ragged = 1;
@@ -205,7 +206,7 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
     }
     size_t longest = 0;
     for (int s = 0; s < P; ++s) {
-      const size_t len = seg_len(s) > e0 ? (seg_len(s) - e0 < piece ? seg_len(s) - e0 : piece) : 0;
+      const size_t len = seg_len(s) > e0 ? (seg_len(s) - e0 < pn ? seg_len(s) - e0 : pn) : 0;
       const size_t off = seg_off(s) + e0 * es;
       fo.seg.seg_off[s] = off / es;
       fo.seg.seg_len[s] = len;
