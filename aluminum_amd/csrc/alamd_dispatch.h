@@ -132,7 +132,7 @@ struct TreeParams {
 // The launches of a kernel whose grid is (tiles, segments): `launch(tile0, ntiles, seg0, nsegs)` is
 // called for each.  About `per_launch` workgroups per launch (see launch_tiles), whatever the number of
 // segments: small work goes in one launch; otherwise up to four consecutive segments of similar
-// length run side by side (blockIdx.y) - eight side by side run 0.5 to 1 point lower on untouched
+// length (more when they are short enough for the launch to hold them) run side by side (blockIdx.y) - eight side by side run 0.5 to 1 point lower on untouched
 // buffers, one or two the same - and a segment much longer than its neighbours gets launches of its
 // own, so that no launch consists mostly of workgroups that find nothing to do (one block of 256 MiB
 // beside seven of 4 KB in a Reduce_scatterv: 70 % of the HBM peak when all ran side by side).
@@ -152,7 +152,10 @@ void plan_launches(const SegParams &seg, unsigned nseg, size_t max_len, size_t t
   for (unsigned s0 = 0; s0 < nseg;) {
     size_t lo = tiles_of(s0), hi = lo;
     unsigned n = 1;
-    while (s0 + n < nseg && n < 4) {
+    // four side by side, or as many as it takes to fill a launch when the segments are short
+    const size_t fill = per_launch / (lo ? lo : 1);
+    const unsigned most_side = fill > 4 ? (unsigned)fill : 4;
+    while (s0 + n < nseg && n < most_side) {
       const size_t t = tiles_of(s0 + n), nlo = t < lo ? t : lo, nhi = t > hi ? t : hi;
       if (nhi > 2 * nlo) break;
       lo = nlo;
@@ -160,7 +163,7 @@ void plan_launches(const SegParams &seg, unsigned nseg, size_t max_len, size_t t
       ++n;
     }
     if (hi > 0) {
-      const size_t cut = hi * n <= per_launch ? hi : floor_pow2(per_launch / n);
+      const size_t cut = hi * n <= per_launch + per_launch / 2 ? hi : floor_pow2(per_launch / n);
       // a remainder of less than half a cut rides with the launch before it
       for (size_t t0 = 0; t0 < hi;) {
         const size_t nt = hi - t0 < cut + cut / 2 ? hi - t0 : cut;

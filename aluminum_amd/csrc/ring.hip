@@ -188,9 +188,12 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   };
   auto seg_len = [&](int s) { return fp.seg.seg_base + ((size_t)s < fp.seg.seg_rem ? 1 : 0); };
   // piece by piece: fold the same range of every segment (P reads + 1 write), then spread it
-  // (kRingPieceBytes over all segments: one fold launch and one spread launch per piece)
+  // (one fold launch's worth of tiles over all segments: one fold launch and one spread launch per piece)
   const size_t tile_elems = Tile<8, 128>::BYTES / es;
-  size_t piece = kRingPieceBytes / (size_t)P / es / tile_elems * tile_elems;
+  // (64 MiB from P = 8 up, where that is what one fold launch covers; more below: 128 MiB at P = 3 and 4)
+  size_t piece_bytes = launch_tiles(P, Tile<8, 128>::BYTES) * Tile<8, 128>::BYTES;
+  if (piece_bytes < kRingPieceBytes) piece_bytes = kRingPieceBytes;
+  size_t piece = piece_bytes / (size_t)P / es / tile_elems * tile_elems;
   if (piece == 0) piece = tile_elems;
   for (size_t e0 = 0, pn; e0 < max_len; e0 += pn) {
     pn = max_len - e0 < piece + piece / 2 ? max_len - e0 : piece;  // no short last piece
