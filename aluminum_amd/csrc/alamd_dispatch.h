@@ -132,10 +132,11 @@ struct TreeParams {
 // The launches of a kernel whose grid is (tiles, segments): `launch(tile0, ntiles, seg0, nsegs)` is
 // called for each.  About `per_launch` workgroups per launch (see launch_tiles), whatever the number of
 // segments: small work goes in one launch; otherwise up to four consecutive segments of similar
-// length (more when they are short enough for the launch to hold them) run side by side (blockIdx.y) - eight side by side run 0.5 to 1 point lower on untouched
-// buffers, one or two the same - and a segment much longer than its neighbours gets launches of its
-// own, so that no launch consists mostly of workgroups that find nothing to do (one block of 256 MiB
-// beside seven of 4 KB in a Reduce_scatterv: 70 % of the HBM peak when all ran side by side).
+// length run side by side (blockIdx.y), more when they are short enough for one launch to hold
+// them (eight long ones side by side run 0.5 to 1 point lower on untouched buffers, one or two the
+// same), and a segment much longer than its neighbours gets launches of its own, so that no launch
+// consists mostly of workgroups that find nothing to do (one block of 256 MiB beside seven of 4 KB in
+// a Reduce_scatterv: 70 % of the HBM peak when all ran side by side, 79 % now).
 template <typename F>
 void plan_launches(const SegParams &seg, unsigned nseg, size_t max_len, size_t tile_elems, size_t per_launch,
                    F launch) {
@@ -210,7 +211,7 @@ constexpr size_t kRingPieceBytes = (size_t)64 << 20;
 int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, hipStream_t stream);
 // The general form: source q = fp.in[q], fp.seg.seg_len[q] bytes, copied to byte offset
 // fp.seg.seg_off[q] of every fp.out[0..fp.P) except where that is the source itself.
-// split_large: give every slice of 16 MiB and more a launch of its own.
+// from_hbm: the sources are slices no launch has just written (see launch_spread_table's definition).
 int launch_spread_table(const FoldParams &fp, int nsrc, bool from_hbm, hipStream_t stream);
 
 }  // namespace alamd
