@@ -42,7 +42,7 @@ def main():
     t0, fails = time.time(), 0
     for k in range(args.runs):
         op, dt = rng.choice(OPS), rng.choice(DATATYPES)
-        ranks = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16])
+        ranks = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16, 24, 32])
         cmd = [exe, "--op", op, "--datatype", dt,
                "--reduction-op", rng.choice(FP_REDUCTIONS if dt in FLOATS else INT_REDUCTIONS),
                "--algorithm", rng.choice(ALGORITHMS[op]), "--ranks", str(ranks), "--root", str(rng.randrange(ranks)),
