@@ -453,3 +453,50 @@ def test_reduce_scatterv_very_unequal_blocks(al, order):
     want = oracle.reduce_scatterv(sends, counts, "f32", "sum", order)
     for b in range(P):
         assert_bits_equal(recvs[b].cpu().numpy()[:counts[b]], want[b], "f32", "%s block %d" % (order, b))
+
+
+@pytest.mark.parametrize("P", (24, 64))
+def test_many_ranks_medium_sizes(al, P):
+    """Sixty-four (and twenty-four) ranks at sizes where the launch planner puts many short segments side by
+    side and the allgather groups several short slices per launch: allgather of odd-sized byte slices,
+    Reduce_scatter, fused and stepwise ring allreduce, combine into every rank's buffer."""
+    import torch
+    # allgather: slices of about 300 KB, byte counts not multiples of 16
+    count = 300007
+    sends = [oracle.fill(count, "u8", "fullrange", 2100 + r) for r in range(P)]
+    recvs = [torch.full((P * count,), 0xEE, dtype=torch.uint8, device="cuda") for _ in range(P)]
+    al.allgather(recvs, [to_dev(s) for s in sends], dtype="u8", count=count)
+    torch.cuda.synchronize()
+    want = np.concatenate(sends)
+    for r in (0, P // 2, P - 1):
+        assert recvs[r].cpu().numpy().tobytes() == want.tobytes(), "allgather rank %d" % r
+    del recvs
+    # reduce_scatter: blocks of about 600 KB
+    blk = 150001
+    host = [oracle.fill(P * blk, "i32", "fullrange", 2200 + r) for r in range(P)]
+    d_sends = [to_dev(h) for h in host]
+    outs = [torch.zeros(blk, dtype=torch.int32, device="cuda") for _ in range(P)]
+    al.reduce_scatter(outs, d_sends, "sum", dtype="i32", count=blk)
+    torch.cuda.synchronize()
+    want_rs = oracle.reduce_scatter(host, "i32", "sum", "rank_asc")
+    for r in range(P):
+        assert_bits_equal(outs[r].cpu().numpy().view(np.int32), want_rs[r], "i32", "reduce_scatter rank %d" % r)
+    # ring allreduce over the same buffers (in place), fused against stepwise against the oracle
+    n = P * blk
+    step = [d.clone() for d in d_sends]
+    al.ring_allreduce(d_sends, "sum", mode="fused", dtype="i32")
+    al.ring_allreduce(step, "sum", mode="stepwise", dtype="i32")
+    torch.cuda.synchronize()
+    want_ar = oracle.combine(host, "i32", "sum", "rank_asc")
+    for r in (0, 1, P - 1):
+        assert_bits_equal(d_sends[r].cpu().numpy().view(np.int32), want_ar, "i32", "fused ring rank %d" % r)
+        assert torch.equal(step[r], d_sends[r])
+    # combine of float inputs into every rank's buffer (two steps: fold, then spread to P - 1 buffers)
+    m = 4200011
+    fin = [oracle.fill(m, "f32", "uniform_pm1", 2300 + r) for r in range(P)]
+    d_in = [to_dev(f) for f in fin]
+    al.combine(d_in, d_in, "sum", order="rank_asc")
+    torch.cuda.synchronize()
+    want_c = oracle.combine(fin, "f32", "sum", "rank_asc")
+    for r in (0, P - 1):
+        assert_bits_equal(d_in[r].cpu().numpy(), want_c, "f32", "combine rank %d" % r)
