@@ -73,7 +73,9 @@ struct SegParams {
   unsigned long long seg_base;
   unsigned long long seg_rem;
   unsigned long long tile0;  // index of the first tile of this launch
-  unsigned seg0;             // index of the first segment of this launch
+  unsigned seg0;             // position of the first segment of this launch
+  int mapped;                // 1: the segment at position i is order[i], 0: it is i
+  unsigned char order[ALAMD_MAX_RANKS];
   int in_blocked;   // 1: inputs are read at the segment's offset, 0: at 0
   int out_mode;     // OUT_ALL / OUT_SEG / OUT_OWNER
   int owner_shift;  // OUT_OWNER: output index is (segment + owner_shift) mod P
@@ -93,6 +95,11 @@ inline SegParams make_seg(size_t seg_base, size_t seg_rem, int in_blocked, int o
   s.out_mode = out_mode;
   s.nout = nout;
   return s;
+}
+
+// The segment a workgroup works on: launches walk positions, which the host may have sorted by length.
+__device__ __forceinline__ unsigned seg_of(const SegParams &s, unsigned pos) {
+  return s.mapped ? s.order[pos] : pos;
 }
 
 __device__ __forceinline__ void seg_range(const SegParams &s, unsigned seg, size_t &off, size_t &len) {
@@ -138,42 +145,73 @@ struct TreeParams {
 // consists mostly of workgroups that find nothing to do (one block of 256 MiB beside seven of 4 KB in
 // a Reduce_scatterv: 70 % of the HBM peak when all ran side by side, 79 % now).
 template <typename F>
-void plan_launches(const SegParams &seg, unsigned nseg, size_t max_len, size_t tile_elems, size_t per_launch,
-                   F launch) {
-  auto tiles_of = [&](unsigned s) {
-    const size_t len = seg.ragged ? (size_t)seg.seg_len[s] : max_len;
-    return (len + tile_elems - 1) / tile_elems;
-  };
+void plan_launches(SegParams &seg, unsigned nseg, size_t max_len, size_t tile_elems, size_t per_launch, F launch) {
+  seg.mapped = 0;
   size_t most = (max_len + tile_elems - 1) / tile_elems;
   if (most == 0) most = 1;
   if (most * nseg <= per_launch) {
     launch((size_t)0, most, 0u, nseg);
     return;
   }
-  for (unsigned s0 = 0; s0 < nseg;) {
-    size_t lo = tiles_of(s0), hi = lo;
-    unsigned n = 1;
-    // four side by side, or as many as it takes to fill a launch when the segments are short
-    const size_t fill = per_launch / (lo ? lo : 1);
-    const unsigned most_side = fill > 4 ? (unsigned)fill : 4;
-    while (s0 + n < nseg && n < most_side) {
-      const size_t t = tiles_of(s0 + n), nlo = t < lo ? t : lo, nhi = t > hi ? t : hi;
-      if (nhi > 2 * nlo) break;
-      lo = nlo;
-      hi = nhi;
-      ++n;
-    }
-    if (hi > 0) {
-      const size_t cut = hi * n <= per_launch + per_launch / 2 ? hi : floor_pow2(per_launch / n);
-      // a remainder of less than half a cut rides with the launch before it
-      for (size_t t0 = 0; t0 < hi;) {
-        const size_t nt = hi - t0 < cut + cut / 2 ? hi - t0 : cut;
-        launch(t0, nt, s0, n);
-        t0 += nt;
-      }
-    }
-    s0 += n;
+  size_t tiles_at[ALAMD_MAX_RANKS];
+  unsigned char sorted[ALAMD_MAX_RANKS], rank_order[ALAMD_MAX_RANKS];
+  for (unsigned s = 0; s < nseg; ++s) {
+    const size_t len = seg.ragged ? (size_t)seg.seg_len[s] : max_len;
+    tiles_at[s] = (len + tile_elems - 1) / tile_elems;
+    sorted[s] = rank_order[s] = (unsigned char)s;
   }
+  // Walks the positions of `order` in runs of similar length; calls visit(t0, nt, s0, n) per launch
+  // and returns their number.
+  auto walk = [&](const unsigned char *order, auto visit) {
+    unsigned launches = 0;
+    for (unsigned s0 = 0; s0 < nseg;) {
+      size_t lo = tiles_at[order[s0]], hi = lo;
+      unsigned n = 1;
+      // four side by side, or as many as it takes to fill a launch when the segments are short
+      const size_t fill = per_launch / (lo ? lo : 1);
+      const unsigned most_side = fill > 4 ? (unsigned)fill : 4;
+      while (s0 + n < nseg && n < most_side) {
+        const size_t t = tiles_at[order[s0 + n]], nlo = t < lo ? t : lo, nhi = t > hi ? t : hi;
+        if (nhi > 2 * nlo) break;
+        lo = nlo;
+        hi = nhi;
+        ++n;
+      }
+      if (hi > 0) {
+        const size_t cut = hi * n <= per_launch + per_launch / 2 ? hi : floor_pow2(per_launch / n);
+        // a remainder of less than half a cut rides with the launch before it
+        for (size_t t0 = 0; t0 < hi;) {
+          const size_t nt = hi - t0 < cut + cut / 2 ? hi - t0 : cut;
+          visit(t0, nt, s0, n);
+          ++launches;
+          t0 += nt;
+        }
+      }
+      s0 += n;
+    }
+    return launches;
+  };
+  auto nothing = [](size_t, size_t, unsigned, unsigned) {};
+  // Ragged segments may be taken longest first instead of in rank order, so that neighbours are
+  // alike: worth it when that saves a quarter of the launches (64 blocks of random lengths up to
+  // 4 MB: 37 % of peak in rank order, where most runs are one or two segments and each launch too
+  // short to fill the device, 54 % sorted; 16 blocks up to 16 MB: 62 % and 67 %).  Eight large blocks
+  // need about as many launches either way and run 1 to 2 points better in rank order.
+  if (seg.ragged) {
+    for (unsigned i = 1; i < nseg; ++i) {  // insertion sort, stable
+      const unsigned char o = sorted[i];
+      unsigned k = i;
+      for (; k > 0 && tiles_at[sorted[k - 1]] < tiles_at[o]; --k) sorted[k] = sorted[k - 1];
+      sorted[k] = o;
+    }
+    if (4 * walk(sorted, nothing) <= 3 * walk(rank_order, nothing)) {
+      seg.mapped = 1;
+      for (unsigned s = 0; s < nseg; ++s) seg.order[s] = sorted[s];
+      walk(sorted, launch);
+      return;
+    }
+  }
+  walk(rank_order, launch);
 }
 
 int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op, bool acc_is_in,

@@ -59,7 +59,7 @@ fold_vec_kernel(const FoldParams p) {
   using TL = Tile<U, THREADS>;
   const TL tl;
   const int P = PT ? PT : p.P;
-  const unsigned seg = blockIdx.y + p.seg.seg0;
+  const unsigned seg = seg_of(p.seg, blockIdx.y + p.seg.seg0);
   size_t off, len;
   seg_range(p.seg, seg, off, len);
   const size_t off_bytes = off * sizeof(T);
@@ -166,7 +166,7 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
     }
     FoldParams q = p;
     const size_t per_launch = launch_tiles(p.P, Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES);
-    plan_launches(p.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
+    plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
       q.seg.tile0 = t0;
       q.seg.seg0 = s0;
       hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);

@@ -59,7 +59,7 @@ tree_vec_kernel(const TreeParams p) {
   constexpr int N = 16 / sizeof(T);
   using TL = Tile<U, THREADS>;
   const TL tl;
-  const unsigned seg = blockIdx.y + p.seg.seg0;
+  const unsigned seg = seg_of(p.seg, blockIdx.y + p.seg.seg0);
   size_t off, len;
   seg_range(p.seg, seg, off, len);
   const size_t off_bytes = off * sizeof(T);
@@ -135,7 +135,7 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
   const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES);
   TreeParams q = p;
-  plan_launches(p.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
+  plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
     q.seg.tile0 = t0;
     q.seg.seg0 = s0;
     hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE>), dim3((unsigned)nt, ns, 1), dim3(S::THREADS, 1, 1), 0,

@@ -500,3 +500,23 @@ def test_many_ranks_medium_sizes(al, P):
     want_c = oracle.combine(fin, "f32", "sum", "rank_asc")
     for r in (0, P - 1):
         assert_bits_equal(d_in[r].cpu().numpy(), want_c, "f32", "combine rank %d" % r)
+
+
+@pytest.mark.parametrize("order", ("rank_asc", "tree_dbl"))
+def test_reduce_scatterv_blocks_taken_longest_first(al, order):
+    """Sixteen blocks that alternate between about 10 MB and a few KB: in rank order every launch would
+    hold one long block, so the launches take the blocks sorted by length; every block still lands in
+    its own rank's buffer, folded from its own starting rank."""
+    import torch
+    P = 16
+    counts = [2600000 + 4099 * r if r % 2 == 0 else 700 + r for r in range(P)]
+    counts[5] = 0
+    total = sum(counts)
+    sends = [oracle.fill(total, "f32", "uniform_pm1", 2500 + r) for r in range(P)]
+    d_sends = [to_dev(s) for s in sends]
+    recvs = [torch.zeros(max(c, 1), dtype=torch.float32, device="cuda") for c in counts]
+    al.reduce_scatterv(recvs, d_sends, counts, "sum", order=order)
+    torch.cuda.synchronize()
+    want = oracle.reduce_scatterv(sends, counts, "f32", "sum", order)
+    for b in range(P):
+        assert_bits_equal(recvs[b].cpu().numpy()[:counts[b]], want[b], "f32", "%s block %d" % (order, b))
