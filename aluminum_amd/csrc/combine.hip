@@ -256,7 +256,34 @@ int launch_spread_table(const FoldParams &fp, int nsrc, bool from_hbm, hipStream
     if (rc) return rc;
     rest.seg.seg_len[q] = 0;
   }
-  return launch_spread_once(rest, nsrc, kSpreadFromHbm, stream);
+  // The short slices share launches.  Equal ones (an allgather) go in rank order; unequal ones
+  // (an allgatherv) longest first, in runs whose lengths differ by at most a factor of two, so that
+  // a launch sized for its longest slice is not mostly workgroups with nothing to copy.
+  int idx[ALAMD_MAX_RANKS], m = 0;
+  for (int q = 0; q < nsrc; ++q)
+    if (rest.seg.seg_len[q] > 0) idx[m++] = q;
+  for (int i = 1; i < m; ++i) {  // insertion sort, stable
+    const int o = idx[i];
+    int k = i;
+    for (; k > 0 && rest.seg.seg_len[idx[k - 1]] < rest.seg.seg_len[o]; --k) idx[k] = idx[k - 1];
+    idx[k] = o;
+  }
+  for (int i0 = 0; i0 < m;) {
+    FoldParams run = fp;
+    int n = 0;
+    const size_t longest = rest.seg.seg_len[idx[i0]];
+    while (i0 + n < m && 2 * rest.seg.seg_len[idx[i0 + n]] >= longest) {
+      const int q = idx[i0 + n];
+      run.in[n] = fp.in[q];
+      run.seg.seg_off[n] = fp.seg.seg_off[q];
+      run.seg.seg_len[n] = fp.seg.seg_len[q];
+      ++n;
+    }
+    const int rc = launch_spread_once(run, n, kSpreadFromHbm, stream);
+    if (rc) return rc;
+    i0 += n;
+  }
+  return ALAMD_OK;
 }
 
 int launch_spread(const char *src, char *const *dests, int ndest, size_t bytes, hipStream_t stream) {
