@@ -76,6 +76,9 @@ struct SegParams {
   unsigned seg0;             // position of the first segment of this launch
   int mapped;                // 1: the segment at position i is order[i], 0: it is i
   unsigned char order[ALAMD_MAX_RANKS];
+  // leading elements of each segment handled one by one (see head_count); the host fills this in, so
+  // that no workgroup has to wait for the output pointer before it can issue its loads
+  unsigned char seg_head[ALAMD_MAX_RANKS];
   int in_blocked;   // 1: inputs are read at the segment's offset, 0: at 0
   int out_mode;     // OUT_ALL / OUT_SEG / OUT_OWNER
   int owner_shift;  // OUT_OWNER: output index is (segment + owner_shift) mod P
@@ -102,7 +105,7 @@ __device__ __forceinline__ unsigned seg_of(const SegParams &s, unsigned pos) {
   return s.mapped ? s.order[pos] : pos;
 }
 
-__device__ __forceinline__ void seg_range(const SegParams &s, unsigned seg, size_t &off, size_t &len) {
+__host__ __device__ inline void seg_range(const SegParams &s, unsigned seg, size_t &off, size_t &len) {
   if (s.ragged) {
     off = s.seg_off[seg];
     len = s.seg_len[seg];
@@ -111,6 +114,14 @@ __device__ __forceinline__ void seg_range(const SegParams &s, unsigned seg, size
     off = sg * s.seg_base + (sg < s.seg_rem ? sg : s.seg_rem);
     len = s.seg_base + (sg < s.seg_rem ? 1u : 0u);
   }
+}
+
+// Which outputs a segment writes (out[j0 .. j0 + nj)), and at which byte offset.
+__host__ __device__ inline void out_select(const SegParams &s, int P, unsigned seg, size_t off_bytes, int &j0, int &nj,
+                                           size_t &out_bytes) {
+  if (s.out_mode == OUT_ALL) { j0 = 0; nj = s.nout; out_bytes = s.in_blocked ? off_bytes : 0; }
+  else if (s.out_mode == OUT_SEG) { j0 = (int)seg; nj = 1; out_bytes = 0; }
+  else { j0 = ((int)seg + s.owner_shift) % P; nj = 1; out_bytes = off_bytes; }
 }
 
 // Left fold over a rotated rank sequence.

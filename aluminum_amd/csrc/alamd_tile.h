@@ -56,11 +56,14 @@ inline size_t launch_tiles(int nin, size_t tile_bytes) {
 // the leading elements one by one up to the output's next 64-byte boundary
 // (at most 63 bytes' worth), if that leaves the first input's vectors on a
 // dword boundary; otherwise up to the first input's next dword boundary.
-template <typename T> __device__ __forceinline__ size_t head_elems(const char *out, const char *first, size_t len) {
+__host__ __device__ inline size_t head_count(size_t elem_size, const char *out, const char *first, size_t len) {
   const uintptr_t o = reinterpret_cast<uintptr_t>(out), f = reinterpret_cast<uintptr_t>(first);
   const size_t bytes = ((o ^ f) & 3u) == 0 ? (64u - (unsigned)(o & 63u)) & 63u : (4u - (unsigned)(f & 3u)) & 3u;
-  const size_t h = bytes / sizeof(T);
+  const size_t h = bytes / elem_size;
   return h < len ? h : len;
+}
+template <typename T> __device__ __forceinline__ size_t head_elems(const char *out, const char *first, size_t len) {
+  return head_count(sizeof(T), out, first, len);
 }
 
 template <int U, int THREADS> struct Tile {

@@ -13,14 +13,6 @@ namespace alamd {
 
 namespace {
 
-// Which outputs a segment writes, and at which byte offset.
-__device__ __forceinline__ void out_select(const SegParams &s, int P, unsigned seg, size_t off_bytes,
-                                           int &j0, int &nj, size_t &out_bytes) {
-  if (s.out_mode == OUT_ALL) { j0 = 0; nj = s.nout; out_bytes = s.in_blocked ? off_bytes : 0; }
-  else if (s.out_mode == OUT_SEG) { j0 = (int)seg; nj = 1; out_bytes = 0; }
-  else { j0 = ((int)seg + s.owner_shift) % P; nj = 1; out_bytes = off_bytes; }
-}
-
 __device__ __forceinline__ int next_rank(int idx, int dir, int P) {
   idx += dir;
   if (idx >= P) idx -= P;
@@ -69,7 +61,7 @@ fold_vec_kernel(const FoldParams p) {
   size_t out_bytes;
   out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
 
-  const size_t head = head_elems<T>(p.out[j0] + out_bytes, p.in[s] + in_bytes, len);
+  const size_t head = p.seg.seg_head[seg];
   const size_t vlen = len - head;
   const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
   const size_t vec_bytes = (vlen / N) * 16;
@@ -165,6 +157,15 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
       else kern = fold_vec_kernel<T, OP, false, 0>;
     }
     FoldParams q = p;
+    for (unsigned sg = 0; sg < nseg; ++sg) {
+      size_t off, len, out_bytes;
+      int j0, nj;
+      seg_range(p.seg, sg, off, len);
+      out_select(p.seg, p.P, sg, off * sizeof(T), j0, nj, out_bytes);
+      const int first = (p.start0 + (int)sg * p.start_stride) % p.P;
+      q.seg.seg_head[sg] = (unsigned char)head_count(sizeof(T), p.out[j0] + out_bytes,
+                                                     p.in[first] + (p.seg.in_blocked ? off * sizeof(T) : 0), len);
+    }
     const size_t per_launch = launch_tiles(p.P, Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES);
     plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
       q.seg.tile0 = t0;

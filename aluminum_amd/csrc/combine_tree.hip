@@ -45,7 +45,7 @@ template <typename T, int OP, int SLOTS, int MODE> struct TreeShape {
   static constexpr int THREADS = U == 8 ? 128 : 256;
 };
 
-__device__ __forceinline__ void tree_out_select(const TreeParams &p, unsigned seg, size_t off_bytes,
+__host__ __device__ inline void tree_out_select(const TreeParams &p, unsigned seg, size_t off_bytes,
                                                 size_t in_bytes, int &j0, int &nj, size_t &out_bytes) {
   if (p.seg.out_mode == OUT_ALL) { j0 = 0; nj = p.seg.nout; out_bytes = in_bytes; }
   else if (p.seg.out_mode == OUT_SEG) { j0 = (int)seg; nj = 1; out_bytes = 0; }
@@ -69,7 +69,7 @@ tree_vec_kernel(const TreeParams p) {
   tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
   const int nvalid = MODE == TREE_FULL ? SLOTS : p.nvalid;
 
-  const size_t head = head_elems<T>(p.out[j0] + out_bytes, p.a[0] + in_bytes, len);
+  const size_t head = p.seg.seg_head[seg];
   const size_t vlen = len - head;
   const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
   const size_t vec_bytes = (vlen / N) * 16;
@@ -135,6 +135,14 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
   const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES);
   TreeParams q = p;
+  for (unsigned sg = 0; sg < nseg; ++sg) {
+    size_t off, len, out_bytes;
+    int j0, nj;
+    seg_range(p.seg, sg, off, len);
+    const size_t in_bytes = p.seg.in_blocked ? off * sizeof(T) : 0;
+    tree_out_select(p, sg, off * sizeof(T), in_bytes, j0, nj, out_bytes);
+    q.seg.seg_head[sg] = (unsigned char)head_count(sizeof(T), p.out[j0] + out_bytes, p.a[0] + in_bytes, len);
+  }
   plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
     q.seg.tile0 = t0;
     q.seg.seg0 = s0;
