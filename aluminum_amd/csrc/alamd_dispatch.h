@@ -79,6 +79,7 @@ struct SegParams {
   // leading elements of each segment handled one by one (see head_count); the host fills this in, so
   // that no workgroup has to wait for the output pointer before it can issue its loads
   unsigned char seg_head[ALAMD_MAX_RANKS];
+  int any_head;              // 0: every seg_head is zero (all buffers 64-byte aligned: the usual case)
   int in_blocked;   // 1: inputs are read at the segment's offset, 0: at 0
   int out_mode;     // OUT_ALL / OUT_SEG / OUT_OWNER
   int owner_shift;  // OUT_OWNER: output index is (segment + owner_shift) mod P

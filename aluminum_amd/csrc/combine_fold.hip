@@ -43,7 +43,13 @@ template <typename T, int OP> struct Shape {
 
 // amdgpu_waves_per_eu(1, 2): the loads in flight are the point of this kernel;
 // the register allocator must not trade them away for more resident waves.
-template <typename T, int OP, bool ACC_IS_IN, int PT>
+// HEAD = false: no segment has leading elements to handle one by one (every buffer on a 64-byte
+// boundary).  With the head a compile-time zero the fp32 fold runs 1.6 points faster (83.8 % of the HBM
+// peak against 82.2 %) and the fp32 tree 2.8; both bodies in one kernel behind a uniform branch ran slower
+// than either (82.7 %, bf16 80.8 % against 82.2 %), so there are two kernels and the host picks.
+// (The body must stay in the kernel itself: moved into an inlined device function it was compiled
+// with 161 instead of 249 VGPRs, i.e. with fewer loads in flight, and lost 1.5 points.)
+template <typename T, int OP, bool ACC_IS_IN, int PT, bool HEAD>
 __global__ void __launch_bounds__((Shape<T, OP>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
 fold_vec_kernel(const FoldParams p) {
   constexpr int U = Shape<T, OP>::U, THREADS = Shape<T, OP>::THREADS;
@@ -61,7 +67,7 @@ fold_vec_kernel(const FoldParams p) {
   size_t out_bytes;
   out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
 
-  const size_t head = p.seg.seg_head[seg];
+  const size_t head = HEAD ? p.seg.seg_head[seg] : 0;
   const size_t vlen = len - head;
   const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
   const size_t vec_bytes = (vlen / N) * 16;
@@ -135,6 +141,7 @@ fold_vec_kernel(const FoldParams p) {
   }
 }
 
+
 }  // namespace
 
 int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op, bool acc_is_in,
@@ -147,15 +154,7 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
     constexpr bool FP_MINMAX = (std::is_same<T, float>::value || std::is_same<T, double>::value ||
                                 std::is_same<T, f16_t>::value || std::is_same<T, bf16_t>::value) &&
                                (OP == ALAMD_MIN || OP == ALAMD_MAX);
-    void (*kern)(const FoldParams) = nullptr;
     const size_t tile_elems = Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES / sizeof(T);
-    if (p.P == 8) {
-      if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 8> : fold_vec_kernel<T, OP, false, 8>;
-      else kern = fold_vec_kernel<T, OP, false, 8>;
-    } else {
-      if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 0> : fold_vec_kernel<T, OP, false, 0>;
-      else kern = fold_vec_kernel<T, OP, false, 0>;
-    }
     FoldParams q = p;
     for (unsigned sg = 0; sg < nseg; ++sg) {
       size_t off, len, out_bytes;
@@ -165,6 +164,24 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
       const int first = (p.start0 + (int)sg * p.start_stride) % p.P;
       q.seg.seg_head[sg] = (unsigned char)head_count(sizeof(T), p.out[j0] + out_bytes,
                                                      p.in[first] + (p.seg.in_blocked ? off * sizeof(T) : 0), len);
+      if (q.seg.seg_head[sg]) q.seg.any_head = 1;
+    }
+    auto pick = [&](auto acc_is_in_t, auto pt_t) -> void (*)(const FoldParams) {
+      constexpr bool A = decltype(acc_is_in_t)::value;
+      constexpr int PT = decltype(pt_t)::value;
+      return q.seg.any_head ? fold_vec_kernel<T, OP, A, PT, true> : fold_vec_kernel<T, OP, A, PT, false>;
+    };
+    using No = std::false_type;
+    using Yes = std::true_type;
+    using P8 = std::integral_constant<int, 8>;
+    using PN = std::integral_constant<int, 0>;
+    void (*kern)(const FoldParams) = nullptr;
+    if (p.P == 8) {
+      if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, P8{}) : pick(No{}, P8{});
+      else kern = pick(No{}, P8{});
+    } else {
+      if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, PN{}) : pick(No{}, PN{});
+      else kern = pick(No{}, PN{});
     }
     const size_t per_launch = launch_tiles(p.P, Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES);
     plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {

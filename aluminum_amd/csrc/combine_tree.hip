@@ -52,7 +52,8 @@ __host__ __device__ inline void tree_out_select(const TreeParams &p, unsigned se
   else { j0 = ((int)seg + p.seg.owner_shift) % p.P; nj = 1; out_bytes = off_bytes; }
 }
 
-template <typename T, int OP, int SLOTS, int MODE>
+// HEAD = false: no segment has leading elements to handle one by one (see the fold kernel).
+template <typename T, int OP, int SLOTS, int MODE, bool HEAD>
 __global__ void __launch_bounds__((TreeShape<T, OP, SLOTS, MODE>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
 tree_vec_kernel(const TreeParams p) {
   constexpr int U = TreeShape<T, OP, SLOTS, MODE>::U, THREADS = TreeShape<T, OP, SLOTS, MODE>::THREADS;
@@ -69,7 +70,7 @@ tree_vec_kernel(const TreeParams p) {
   tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
   const int nvalid = MODE == TREE_FULL ? SLOTS : p.nvalid;
 
-  const size_t head = p.seg.seg_head[seg];
+  const size_t head = HEAD ? p.seg.seg_head[seg] : 0;
   const size_t vlen = len - head;
   const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
   const size_t vec_bytes = (vlen / N) * 16;
@@ -129,6 +130,7 @@ tree_vec_kernel(const TreeParams p) {
   }
 }
 
+
 template <typename T, int OP, int SLOTS, int MODE>
 int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream) {
   using S = TreeShape<T, OP, SLOTS, MODE>;
@@ -142,12 +144,14 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
     const size_t in_bytes = p.seg.in_blocked ? off * sizeof(T) : 0;
     tree_out_select(p, sg, off * sizeof(T), in_bytes, j0, nj, out_bytes);
     q.seg.seg_head[sg] = (unsigned char)head_count(sizeof(T), p.out[j0] + out_bytes, p.a[0] + in_bytes, len);
+    if (q.seg.seg_head[sg]) q.seg.any_head = 1;
   }
+  void (*kern)(const TreeParams) =
+      q.seg.any_head ? tree_vec_kernel<T, OP, SLOTS, MODE, true> : tree_vec_kernel<T, OP, SLOTS, MODE, false>;
   plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
     q.seg.tile0 = t0;
     q.seg.seg0 = s0;
-    hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE>), dim3((unsigned)nt, ns, 1), dim3(S::THREADS, 1, 1), 0,
-                       stream, q);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(S::THREADS, 1, 1), 0, stream, q);
   });
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
