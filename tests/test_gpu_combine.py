@@ -359,7 +359,7 @@ def test_collectives_in_a_hip_graph(al):
     (spread for the large slice, the table-driven kernel for the small ones) and a fused ring captured
     into one graph; every replay, with fresh inputs, gives what the oracle gives."""
     import torch
-    P, n = 4, (1 << 19) + 36
+    P, n = 4, (1 << 22) + 36  # 16 MiB and a bit: the combine takes its two steps, the ring its pieces
     counts = [300000, 0, 5, n - 300005]
     displs = [0, 300000, 300000, 300005]
     ins = [dev_empty(n, np.float32) for _ in range(P)]
