@@ -35,7 +35,7 @@ __device__ __forceinline__ void ring_seg(const RingParams &p, int seg, size_t &o
 // OP < 0: plain copy (allgather step).
 constexpr int kRingU = 8;
 template <typename T, int OP>
-__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 4)))
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
 ring_step_vec_kernel(const RingParams p) {
   using TL = Tile<kRingU, kThreads>;
   const TL tl;
