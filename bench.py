@@ -46,7 +46,7 @@ P = 8
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
 # the same counter's reading for the 1 GiB copy kernel (profiles/fold_vec_kernel_f32_sum_P8_c2.md).
-MEASURED_TRAFFIC = {"c2_f32_sum": 2416031701}
+MEASURED_TRAFFIC = {"c2_f32_sum": 2416032085}
 KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false, 8, false>"}
 
 
