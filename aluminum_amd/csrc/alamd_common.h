@@ -77,6 +77,10 @@ template <> __device__ __forceinline__ bf16_t narrow<bf16_t>(float f) {
 
 // ---- the pairwise step ----------------------------------------------------
 //
+// avg is sum followed by one division by the number of ranks (see Divisor
+// below), so its pairwise step is the step of sum.
+constexpr bool op_is_sum(int op) { return op == ALAMD_SUM || op == ALAMD_AVG; }
+//
 // step<T, OP>(in, inout) is one application of an MPI reduction function to
 // one element: the value stored back to inoutvec.  For the native types it
 // is OP(inout, in) with MIN(x, y) = (x < y) ? x : y and MAX(x, y) =
@@ -94,7 +98,7 @@ template <typename T, int OP> struct Step {
   // integer types
   static __device__ __forceinline__ T apply(T in, T inout) {
     using U = typename unsigned_of<T>::type;
-    if constexpr (OP == ALAMD_SUM) return static_cast<T>(static_cast<U>(static_cast<U>(inout) + static_cast<U>(in)));
+    if constexpr (op_is_sum(OP)) return static_cast<T>(static_cast<U>(static_cast<U>(inout) + static_cast<U>(in)));
     else if constexpr (OP == ALAMD_PROD) return static_cast<T>(static_cast<U>(static_cast<U>(inout) * static_cast<U>(in)));
     else if constexpr (OP == ALAMD_MIN) return (inout < in) ? inout : in;
     else if constexpr (OP == ALAMD_MAX) return (inout > in) ? inout : in;
@@ -108,7 +112,7 @@ template <typename T, int OP> struct Step {
 };
 
 template <typename F, int OP> __device__ __forceinline__ F fp_step(F in, F inout) {
-  if constexpr (OP == ALAMD_SUM) return inout + in;
+  if constexpr (op_is_sum(OP)) return inout + in;
   else if constexpr (OP == ALAMD_PROD) return inout * in;
   else if constexpr (OP == ALAMD_MIN) return (inout < in) ? inout : in;
   else return (inout > in) ? inout : in;
@@ -145,7 +149,7 @@ __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
       r[j] = narrow_bf16x2(fp_step<float, OP>(a_lo, b_lo), fp_step<float, OP>(a_hi, b_hi));
     }
     return r;
-  } else if constexpr (sizeof(T) == 1 && OP == ALAMD_SUM) {
+  } else if constexpr (sizeof(T) == 1 && op_is_sum(OP)) {
     // four wrapping byte sums per dword: add the low seven bits of every byte
     // (no carry leaves a byte), then put the top bits back with an xor
     u32x4 r;
@@ -207,6 +211,86 @@ __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
     for (int j = 0; j < N; ++j) b.e[j] = Step<T, OP>::apply(a.e[j], b.e[j]);
     return b.v;
   }
+}
+
+// ---- the division that ends an avg ------------------------------------------
+//
+// avg = the sum in the named order (rounded, or wrapped, after every step
+// exactly as for sum), then one division by the number of ranks d in the
+// element type's own arithmetic: IEEE division for fp32 / fp64; widen, fp32
+// division, round-to-nearest-even narrowing for fp16 / bf16 (one more step of
+// the rule of src/mpi_impl.cpp:61-145); C integer division (truncation toward
+// zero) for the integer types.  The reference forwards avg to the
+// communication library of its NCCL backend (include/aluminum/nccl_impl.hpp:176)
+// and rejects it elsewhere.
+//
+// Integer division by the uniform d without a divide instruction (Granlund and
+// Montgomery, "Division by invariant integers using multiplication"): with
+// l = ceil(log2 d), m = floor(2^N (2^l - d) / d) + 1, t = mulhi(m, n),
+// n / d = (t + ((n - t) >> min(l, 1))) >> max(l - 1, 0) for every N-bit n.
+struct Divisor {
+  unsigned long long m64;
+  unsigned m32;
+  unsigned sh1, sh2;
+  float f;
+  double d;
+};
+
+inline Divisor make_divisor(int ranks) {
+  Divisor dv;
+  const unsigned d = ranks > 0 ? (unsigned)ranks : 1u;
+  unsigned l = 0;
+  while ((1u << l) < d) ++l;
+  const unsigned long long k = (1ull << l) - d;
+  dv.m32 = (unsigned)(((k << 32) / d) + 1);
+  dv.m64 = (unsigned long long)((((unsigned __int128)k << 64) / d) + 1);
+  dv.sh1 = l < 1 ? l : 1;
+  dv.sh2 = l > 1 ? l - 1 : 0;
+  dv.f = (float)d;
+  dv.d = (double)d;
+  return dv;
+}
+
+__device__ __forceinline__ uint32_t udiv_by(uint32_t n, const Divisor &dv) {
+  const uint32_t t = __umulhi(dv.m32, n);
+  return (t + ((n - t) >> dv.sh1)) >> dv.sh2;
+}
+__device__ __forceinline__ uint64_t udiv_by(uint64_t n, const Divisor &dv) {
+  const uint64_t t = __umul64hi(dv.m64, n);
+  return (t + ((n - t) >> dv.sh1)) >> dv.sh2;
+}
+
+template <typename T> __device__ __forceinline__ T div_elem(T x, const Divisor &dv) {
+  if constexpr (std::is_same<T, float>::value) return x / dv.f;
+  else if constexpr (std::is_same<T, double>::value) return x / dv.d;
+  else if constexpr (std::is_same<T, f16_t>::value || std::is_same<T, bf16_t>::value) return narrow<T>(widen(x) / dv.f);
+  else {
+    // magnitude in 32 or 64 bits, unsigned division, sign put back
+    using W = typename std::conditional<sizeof(T) == 8, uint64_t, uint32_t>::type;
+    using SW = typename std::make_signed<W>::type;
+    const bool neg = std::is_signed<T>::value && x < 0;
+    const W a = neg ? (W)0 - (W)(SW)x : (W)x;
+    const W q = udiv_by(a, dv);
+    return (T)(neg ? (W)0 - q : q);
+  }
+}
+
+// The end of a combine: for avg every element of the folded vector is divided
+// by the number of ranks; for every other operator nothing happens.
+template <typename T, int OP> __device__ __forceinline__ u32x4 finish_vec(u32x4 acc, const Divisor &dv) {
+  if constexpr (OP != ALAMD_AVG) return acc;
+  else {
+    constexpr int N = 16 / sizeof(T);
+    union U { u32x4 v; T e[N]; __device__ U() {} } a;
+    a.v = acc;
+#pragma unroll
+    for (int j = 0; j < N; ++j) a.e[j] = div_elem<T>(a.e[j], dv);
+    return a.v;
+  }
+}
+template <typename T, int OP> __device__ __forceinline__ T finish_elem(T acc, const Divisor &dv) {
+  if constexpr (OP != ALAMD_AVG) return acc;
+  else return div_elem<T>(acc, dv);
 }
 
 // ---- element access (any alignment) --------------------------------------

@@ -25,6 +25,7 @@ template <typename S, typename F> int dispatch_int_op(int op, F &&f) {
   case ALAMD_BOR: return f(TypeTag<U>{}, OpTag<ALAMD_BOR>{});
   case ALAMD_BAND: return f(TypeTag<U>{}, OpTag<ALAMD_BAND>{});
   case ALAMD_BXOR: return f(TypeTag<U>{}, OpTag<ALAMD_BXOR>{});
+  case ALAMD_AVG: return f(TypeTag<S>{}, OpTag<ALAMD_AVG>{});  // the final division depends on the sign
   default: return set_error(ALAMD_ERR_UNSUPPORTED_OP, "Reduction operator not supported");
   }
 }
@@ -35,6 +36,7 @@ template <typename T, typename F> int dispatch_fp_op(int op, F &&f) {
   case ALAMD_PROD: return f(TypeTag<T>{}, OpTag<ALAMD_PROD>{});
   case ALAMD_MIN: return f(TypeTag<T>{}, OpTag<ALAMD_MIN>{});
   case ALAMD_MAX: return f(TypeTag<T>{}, OpTag<ALAMD_MAX>{});
+  case ALAMD_AVG: return f(TypeTag<T>{}, OpTag<ALAMD_AVG>{});
   default: return set_error(ALAMD_ERR_UNSUPPORTED_OP, "Reduction operator not supported");
   }
 }
@@ -134,18 +136,21 @@ struct FoldParams {
   int start0;        // first operand of segment s is rank (start0 + s*start_stride) mod P
   int start_stride;
   int dir;           // +1: next operand is rank+1, -1: rank-1 (with wrap)
+  Divisor div;       // avg: the number of ranks as a divisor
 };
 
-// Balanced pairwise tree over up to 32 slots.  Slot j holds a[j], or
-// step(in = a[j], inout = b[j]) when b[j] is set; slots >= nvalid are empty.
+// Balanced pairwise tree over up to 64 slots.  Slot j holds a[j], or
+// step(in = a[j], inout = b[j]) when b[j] is set (only among the first 32: a
+// pre-fold leaves at most 32 slots); slots >= nvalid are empty.
 // Level d = 1,2,4..: slot i (multiple of 2d) = step(in = slot i+d, inout = slot i).
 struct TreeParams {
-  const char *a[32];
-  const char *b[32];
+  const char *a[ALAMD_MAX_RANKS];
+  const char *b[ALAMD_MAX_RANKS];
   char *out[ALAMD_MAX_RANKS];
   SegParams seg;
   int P;        // number of ranks (for OUT_OWNER)
   int nvalid;   // occupied slots
+  Divisor div;  // avg: the number of ranks as a divisor
 };
 
 // The launches of a kernel whose grid is (tiles, segments): `launch(tile0, ntiles, seg0, nsegs)` is

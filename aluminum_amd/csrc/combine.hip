@@ -32,7 +32,7 @@ bool order_valid(int order) { return order >= ALAMD_ORDER_RANK_ASC && order <= A
 
 // Fills the slot tables of a tree order over the P inputs `ins`.
 int build_tree(TreeParams &tp, const void *const *ins, int P, int order) {
-  for (int j = 0; j < 32; ++j) { tp.a[j] = nullptr; tp.b[j] = nullptr; }
+  for (int j = 0; j < ALAMD_MAX_RANKS; ++j) { tp.a[j] = nullptr; tp.b[j] = nullptr; }
   tp.P = P;
   if (order == ALAMD_ORDER_TREE_BINOMIAL) {
     for (int j = 0; j < P; ++j) tp.a[j] = static_cast<const char *>(ins[j]);
@@ -40,7 +40,7 @@ int build_tree(TreeParams &tp, const void *const *ins, int P, int order) {
     return ceil_pow2(P);
   }
   const int pof2 = floor_pow2(P), rem = P - pof2;
-  const char *la[32], *lb[32];
+  const char *la[ALAMD_MAX_RANKS], *lb[ALAMD_MAX_RANKS];
   for (int j = 0; j < pof2; ++j) {
     if (j < rem) { la[j] = static_cast<const char *>(ins[2 * j]); lb[j] = static_cast<const char *>(ins[2 * j + 1]); }
     else { la[j] = static_cast<const char *>(ins[j + rem]); lb[j] = nullptr; }
@@ -72,9 +72,6 @@ int launch_order(void *const *outs, const void *const *ins, int P, const Layout 
   if (!is_float_dtype(dtype)) order = ALAMD_ORDER_RANK_ASC;  // integer ops: every order gives the same bits
   if (P == 1 && order_is_tree(order)) order = ALAMD_ORDER_RANK_ASC;
   if (order_is_tree(order)) {
-    if (P > ALAMD_MAX_TREE_RANKS)
-      return set_error(ALAMD_ERR_INVALID_ARG, "tree orders support at most %d ranks (got %d)",
-                       ALAMD_MAX_TREE_RANKS, P);
     TreeParams tp;
     const int slots = build_tree(tp, ins, P, order);
     for (int j = 0; j < ALAMD_MAX_RANKS; ++j) tp.out[j] = static_cast<char *>(outs[j]);

@@ -31,6 +31,7 @@ __device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, siz
     const T x = ld_elem<T>(p.in[idx] + in_bytes + e * sizeof(T));
     acc = ACC_IS_IN ? Step<T, OP>::apply(acc, x) : Step<T, OP>::apply(x, acc);
   }
+  acc = finish_elem<T, OP>(acc, p.div);
   for (int j = j0; j < j0 + nj; ++j) st_elem<T>(p.out[j] + out_bytes + e * sizeof(T), acc);
 }
 
@@ -127,6 +128,8 @@ fold_vec_kernel(const FoldParams p) {
         idx = id;
       }
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc[u] = finish_vec<T, OP>(acc[u], p.div);
     for (int j = j0; j < j0 + nj; ++j) {
       const auto r = TL::rsrc(p.out[j] + vout + tb, nrec);
 #pragma unroll
@@ -156,6 +159,7 @@ int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, i
                                (OP == ALAMD_MIN || OP == ALAMD_MAX);
     const size_t tile_elems = Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES / sizeof(T);
     FoldParams q = p;
+    q.div = make_divisor(p.P);
     for (unsigned sg = 0; sg < nseg; ++sg) {
       size_t off, len, out_bytes;
       int j0, nj;

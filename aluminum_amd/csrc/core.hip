@@ -59,9 +59,9 @@ unsigned stream_grid(size_t work_items, size_t per_block, int waves) {
 int check_type_op(int dtype, int op) {
   if (dtype < 0 || dtype >= ALAMD_NUM_DTYPES)
     return set_error(ALAMD_ERR_UNSUPPORTED_TYPE, "unknown dtype %d", dtype);
-  if (op < ALAMD_SUM || op > ALAMD_BXOR)
+  if (op < ALAMD_SUM || op > ALAMD_AVG)
     return set_error(ALAMD_ERR_UNSUPPORTED_OP, "Reduction operator not supported");
-  if (is_float_dtype(dtype) && op > ALAMD_MAX)
+  if (is_float_dtype(dtype) && op > ALAMD_MAX && op != ALAMD_AVG)
     return set_error(ALAMD_ERR_UNSUPPORTED_OP, "Reduction operator not supported");
   return ALAMD_OK;
 }

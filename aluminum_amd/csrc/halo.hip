@@ -1,11 +1,24 @@
 // Halo face pack / unpack for a 3-D grid with x fastest.  A face is a list of
 // rows (runs along x); rows of the y and z faces are whole interior lines,
 // rows of the x faces are only `halo` elements long and one allocation line
-// apart.  All selected faces are handled by one launch (blockIdx.y = face):
-// at these sizes (a few MiB per face) launch latency is a large part of the
-// cost.  Data moves in the widest power-of-two unit (up to 128 bits) that the
-// row length, row pitch and base addresses allow, so that the contiguous side
-// of every face is accessed in whole coalesced runs.
+// apart.  All selected faces are handled by one launch over a flat grid of
+// workgroups (at these sizes, a few MiB per face, launch latency is a large
+// part of the cost): every face owns a range of workgroups, the x faces first.
+//
+// Data moves in the widest power-of-two unit (up to 128 bits) that the row
+// length, row pitch and base addresses allow.  A workgroup covers a tile of
+// rows x units: LX = 2^k lanes side by side along a row, 256 / LX rows per
+// pass, U passes, so a thread finds its place with shifts and one 32-bit
+// division per access (by the number of rows in a plane).
+//
+// The short runs of an x face cost a whole cache line each, whatever is done
+// with the rest of the line, so the x faces are bound by the number of lines
+// the device can move, not by bytes.  When both x faces are selected they are
+// handled as one face of twice the row length: neighbouring lanes take the -x
+// and the +x run of a row, and the +x run of row y usually lies in the same
+// 128-byte line as the -x run of row y+1, which a wave then fetches once
+// (516^3 fp64 grid, halo 2: 1.25 lines per row instead of 2; both faces
+// together 12.2 us against 14.4 us).
 #include "alamd_common.h"
 
 namespace alamd {
@@ -13,20 +26,28 @@ namespace alamd {
 namespace {
 
 constexpr int kThreads = 256;
+constexpr int kPasses = 2;  // rows in flight per thread (1, 2, 4 within 5 %; 8 is 10-25 % slower)
 
 struct HaloFace {
-  char *buf;                      // contiguous face buffer
-  unsigned long long grid_off;    // byte offset of the face's first element in the grid
-  unsigned long long pitch_y;     // bytes between rows adjacent in y
-  unsigned long long pitch_z;     // bytes between rows adjacent in z
-  unsigned long long nunits;      // units in the face
-  unsigned upr;                   // units per row
-  unsigned rows_y;                // rows per z-plane of the face
+  char *buf;                   // contiguous face buffer (of a pair: the -x face's)
+  char *buf2;                  // of a pair: the +x face's buffer
+  unsigned long long goff;     // byte offset in the grid of the face's first element
+  unsigned long long pitch_z;  // bytes between planes
+  unsigned long long pitch_y;  // bytes between rows
+  unsigned upr;                // units per row of one face buffer
+  unsigned cols;               // units per row handled here: upr, or 2 * upr for a pair
+  unsigned delta2;             // of a pair: bytes from the -x run of a row to its +x run
+  unsigned ny;                 // rows per plane of the face
+  unsigned nslots;             // rows * column tiles
+  unsigned lx_log2;            // lanes side by side along a row: 1 << lx_log2
+  unsigned ctiles;             // column tiles (of 1 << lx_log2 units) per row
+  unsigned blk0;               // first workgroup of this face
 };
 
 struct HaloParams {
   HaloFace f[6];
   char *grid;
+  int nf;
 };
 
 template <int UB> struct unit_of;
@@ -36,38 +57,61 @@ template <> struct unit_of<4> { using type = uint32_t; };
 template <> struct unit_of<8> { using type = uint64_t; };
 template <> struct unit_of<16> { using type = u32x4; };
 
-// U = independent accesses per thread: the short rows of the x faces need
-// several in flight, but a launch also needs a few workgroups per CU, so the
-// host picks the largest U that leaves enough of them.
-template <int UB, bool PACK, int U>
+// Store written through to memory (sc0 sc1).  The ghost cells of an x face are
+// runs of a few bytes in lines of their own: kept in L2 as dirty partial lines
+// they cost more when they are evicted later (six-face unpack of the 516^3
+// fp64 grid 15.5 us with plain stores, 13.6 us written through; non-temporal
+// stores of such runs take 45 us).
+template <int UB> __device__ __forceinline__ void store_through(char *p, typename unit_of<UB>::type v) {
+  if constexpr (UB == 16) asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+  else if constexpr (UB == 8) asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+  else if constexpr (UB == 4) asm volatile("global_store_dword %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+  else if constexpr (UB == 2) asm volatile("global_store_short %0, %1, off sc0 sc1" ::"v"(p), "v"((uint32_t)v) : "memory");
+  else asm volatile("global_store_byte %0, %1, off sc0 sc1" ::"v"(p), "v"((uint32_t)v) : "memory");
+}
+
+template <int UB, bool PACK>
 __global__ void __launch_bounds__(kThreads) halo_kernel(const HaloParams p) {
   using Unit = typename unit_of<UB>::type;
-  const HaloFace &f = p.f[blockIdx.y];
-  const unsigned long long n = f.nunits;
-  const unsigned upr = f.upr, rows_y = f.rows_y;
-  for (unsigned long long i0 = (unsigned long long)blockIdx.x * (kThreads * U) + threadIdx.x; i0 < n;
-       i0 += (unsigned long long)gridDim.x * (kThreads * U)) {
-    Unit v[U];
-    char *g[U];
-    char *b[U];
+  constexpr int U = kPasses;
+  int fi = 0;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const unsigned long long i = i0 + (unsigned long long)u * kThreads;
-      if (i < n) {
-        // faces hold fewer than 2^32 rows
-        const unsigned long long row = i / upr;
-        const unsigned col = (unsigned)(i - row * upr);
-        const unsigned long long z = row / rows_y;
-        const unsigned y = (unsigned)(row - z * rows_y);
-        g[u] = p.grid + f.grid_off + z * f.pitch_z + (unsigned long long)y * f.pitch_y + (unsigned long long)col * UB;
-        b[u] = f.buf + i * UB;
-        v[u] = *reinterpret_cast<const Unit *>(PACK ? g[u] : b[u]);
-      }
+  for (int k = 1; k < 6; ++k)
+    if (k < p.nf && blockIdx.x >= p.f[k].blk0) fi = k;
+  const HaloFace &f = p.f[fi];
+  const unsigned lx = 1u << f.lx_log2, ly = (unsigned)kThreads >> f.lx_log2;
+  const unsigned tx = threadIdx.x & (lx - 1), ty = threadIdx.x >> f.lx_log2;
+  // a slot is (row, column tile); consecutive slots of a row are consecutive column tiles
+  const unsigned s0 = (blockIdx.x - f.blk0) * (ly * U) + ty;
+  Unit v[U];
+  char *g[U], *b[U];
+  bool ok[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const unsigned s = s0 + (unsigned)u * ly;
+    ok[u] = s < f.nslots;
+    unsigned r = s, ct = 0;
+    if (f.ctiles > 1) {
+      r = s / f.ctiles;
+      ct = s - r * f.ctiles;
     }
+    const unsigned col = ct * lx + tx;
+    ok[u] = ok[u] && col < f.cols;
+    const bool second = col >= f.upr;  // the +x face of a pair
+    const unsigned c1 = second ? col - f.upr : col;
+    const unsigned z = r / f.ny, y = r - z * f.ny;
+    g[u] = p.grid + f.goff + (unsigned long long)z * f.pitch_z + (unsigned long long)y * f.pitch_y +
+           (unsigned long long)c1 * UB + (second ? f.delta2 : 0u);
+    b[u] = (second ? f.buf2 : f.buf) + ((unsigned long long)r * f.upr + c1) * UB;
+  }
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const unsigned long long i = i0 + (unsigned long long)u * kThreads;
-      if (i < n) *reinterpret_cast<Unit *>(PACK ? b[u] : g[u]) = v[u];
+  for (int u = 0; u < U; ++u)
+    if (ok[u]) v[u] = *reinterpret_cast<const Unit *>(PACK ? g[u] : b[u]);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (ok[u]) {
+      if (PACK) *reinterpret_cast<Unit *>(b[u]) = v[u];
+      else store_through<UB>(g[u], v[u]);
     }
   }
 }
@@ -84,68 +128,75 @@ int halo_launch(void *grid, void *const bufs[6], const size_t dims[3], size_t ha
   if (halo == 0 || face_mask == 0) return ALAMD_OK;
   if (!grid || !bufs) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer");
   const size_t sx = dims[0] + 2 * halo, sy = dims[1] + 2 * halo;
-  HaloParams hp;
-  hp.grid = static_cast<char *>(grid);
+  if (sx * es > 0xffffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "grid extent too large");
   // widest unit every selected face allows
   size_t unit = 16;
   auto shrink = [&unit](size_t v) { while (unit > 1 && v % unit != 0) unit /= 2; };
   shrink(reinterpret_cast<uintptr_t>(grid));
   shrink(sx * es);
-  int nf = 0;
-  unsigned long long max_units = 0;
   size_t lo[6][3], ext[6][3];
-  int sel[6];
   for (int face = 0; face < 6; ++face) {
     if (!(face_mask & (1u << face))) continue;
     if (!bufs[face]) return set_error(ALAMD_ERR_INVALID_ARG, "buffer of face %d is null", face);
     const int axis = face / 2, plus = face % 2;
-    for (int d = 0; d < 3; ++d) { lo[nf][d] = halo; ext[nf][d] = dims[d]; }
-    ext[nf][axis] = halo;
+    for (int d = 0; d < 3; ++d) { lo[face][d] = halo; ext[face][d] = dims[d]; }
+    ext[face][axis] = halo;
     // pack reads the interior boundary slab, unpack writes the ghost slab
-    if (pack) lo[nf][axis] = plus ? dims[axis] : halo;
-    else lo[nf][axis] = plus ? halo + dims[axis] : 0;
+    if (pack) lo[face][axis] = plus ? dims[axis] : halo;
+    else lo[face][axis] = plus ? halo + dims[axis] : 0;
     shrink(reinterpret_cast<uintptr_t>(bufs[face]));
-    shrink(ext[nf][0] * es);
-    shrink(lo[nf][0] * es);
-    sel[nf] = face;
-    ++nf;
+    shrink(ext[face][0] * es);
+    shrink(lo[face][0] * es);
   }
-  for (int k = 0; k < nf; ++k) {
-    HaloFace &f = hp.f[k];
-    f.buf = static_cast<char *>(bufs[sel[k]]);
-    f.grid_off = ((lo[k][2] * sy + lo[k][1]) * sx + lo[k][0]) * es;
+  HaloParams hp;
+  hp.grid = static_cast<char *>(grid);
+  hp.nf = 0;
+  unsigned long long blocks = 0;
+  const bool pair = (face_mask & 3u) == 3u;
+  for (int face = 0; face < 6; ++face) {
+    if (!(face_mask & (1u << face)) || (pair && face == 1)) continue;
+    HaloFace &f = hp.f[hp.nf++];
+    f.buf = f.buf2 = static_cast<char *>(bufs[face]);
+    f.goff = ((lo[face][2] * sy + lo[face][1]) * sx + lo[face][0]) * es;
     f.pitch_y = sx * es;
     f.pitch_z = sx * sy * es;
-    f.upr = (unsigned)(ext[k][0] * es / unit);
-    f.rows_y = (unsigned)ext[k][1];
-    f.nunits = (unsigned long long)f.upr * ext[k][1] * ext[k][2];
-    if (ext[k][0] * es / unit > 0xffffffffull || ext[k][1] > 0xffffffffull)
+    f.upr = f.cols = (unsigned)(ext[face][0] * es / unit);
+    f.delta2 = 0;
+    if (pair && face == 0) {
+      f.buf2 = static_cast<char *>(bufs[1]);
+      f.cols = 2 * f.upr;
+      f.delta2 = (unsigned)((lo[1][0] - lo[0][0]) * es);
+    }
+    f.ny = (unsigned)ext[face][1];
+    // lanes along a row: the largest power of two that divides the row length (so that no lane
+    // of a column tile is idle), at most the workgroup
+    unsigned l = 0;
+    while (l < 8 && f.cols % (2u << l) == 0) ++l;
+    f.lx_log2 = l;
+    f.ctiles = f.cols >> l;
+    const unsigned long long rows = (unsigned long long)ext[face][1] * ext[face][2];
+    const unsigned long long slots = rows * f.ctiles;
+    if (ext[face][1] > 0xffffffffull || slots > 0xfff00000ull)
       return set_error(ALAMD_ERR_INVALID_ARG, "grid extent too large");
-    if (f.nunits > max_units) max_units = f.nunits;
+    f.nslots = (unsigned)slots;
+    const unsigned per_block = ((unsigned)kThreads >> l) * kPasses;
+    f.blk0 = (unsigned)blocks;
+    blocks += (slots + per_block - 1) / per_block;
+    if (blocks > 0x7fffffffull) return set_error(ALAMD_ERR_INVALID_ARG, "grid extent too large");
   }
-  for (int k = nf; k < 6; ++k) hp.f[k] = hp.f[0];
-  // 8 accesses per thread if that still gives two workgroups per CU over all faces, else 2
-  const unsigned two_per_cu = stream_grid((size_t)-1 / 2, 1, 2);
-  const bool wide = (max_units + kThreads * 8 - 1) / (kThreads * 8) * nf >= two_per_cu;
-  const int acc = wide ? 8 : 2;
-  unsigned per_face = (stream_grid((size_t)-1 / 2, 1, 8) + nf - 1) / nf;
-  unsigned gx = stream_grid((size_t)max_units, (size_t)kThreads * acc, 8);
-  if (gx > per_face) gx = per_face < 1 ? 1 : per_face;
-  const dim3 grid_dim(gx, nf, 1), block(kThreads, 1, 1);
+  for (int k = hp.nf; k < 6; ++k) {
+    hp.f[k] = hp.f[0];
+    hp.f[k].blk0 = 0xffffffffu;
+  }
   void (*kern)(const HaloParams) = nullptr;
-  auto pick = [&](auto ub) {
-    constexpr int UB = decltype(ub)::value;
-    if (wide) return pack ? halo_kernel<UB, true, 8> : halo_kernel<UB, false, 8>;
-    return pack ? halo_kernel<UB, true, 2> : halo_kernel<UB, false, 2>;
-  };
   switch (unit) {
-  case 16: kern = pick(std::integral_constant<int, 16>{}); break;
-  case 8: kern = pick(std::integral_constant<int, 8>{}); break;
-  case 4: kern = pick(std::integral_constant<int, 4>{}); break;
-  case 2: kern = pick(std::integral_constant<int, 2>{}); break;
-  default: kern = pick(std::integral_constant<int, 1>{}); break;
+  case 16: kern = pack ? halo_kernel<16, true> : halo_kernel<16, false>; break;
+  case 8: kern = pack ? halo_kernel<8, true> : halo_kernel<8, false>; break;
+  case 4: kern = pack ? halo_kernel<4, true> : halo_kernel<4, false>; break;
+  case 2: kern = pack ? halo_kernel<2, true> : halo_kernel<2, false>; break;
+  default: kern = pack ? halo_kernel<1, true> : halo_kernel<1, false>; break;
   }
-  hipLaunchKernelGGL(kern, grid_dim, block, 0, stream, hp);
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1, 1), dim3(kThreads, 1, 1), 0, stream, hp);
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
 }

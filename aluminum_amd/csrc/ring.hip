@@ -23,6 +23,7 @@ struct RingParams {
   int P;
   int t;              // ring step
   unsigned tiles_per_chunk;  // workgroups (tiles) per chunk
+  Divisor div;        // avg: the number of ranks as a divisor
 };
 
 __device__ __forceinline__ void ring_seg(const RingParams &p, int seg, size_t &off, size_t &len) {
@@ -32,9 +33,10 @@ __device__ __forceinline__ void ring_seg(const RingParams &p, int seg, size_t &o
 }
 
 // A chunk is a run of tiles_per_chunk tiles; no tile crosses a chunk boundary.
-// OP < 0: plain copy (allgather step).
+// OP < 0: plain copy (allgather step).  FIN: the last reduce-scatter step of an
+// avg, which ends with the division by the number of ranks.
 constexpr int kRingU = 8;
-template <typename T, int OP>
+template <typename T, int OP, bool FIN>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
 ring_step_vec_kernel(const RingParams p) {
   using TL = Tile<kRingU, kThreads>;
@@ -57,7 +59,9 @@ ring_step_vec_kernel(const RingParams p) {
     const T a = ld_elem<T>(recv + e * sizeof(T));
     if constexpr (OP >= 0) {
       const T b = ld_elem<T>(local + e * sizeof(T));
-      st_elem<T>(local + e * sizeof(T), Step<T, (OP >= 0 ? OP : 0)>::apply(a, b));
+      T v = Step<T, (OP >= 0 ? OP : 0)>::apply(a, b);
+      if constexpr (FIN) v = finish_elem<T, OP>(v, p.div);
+      st_elem<T>(local + e * sizeof(T), v);
     } else {
       st_elem<T>(local + e * sizeof(T), a);
     }
@@ -82,7 +86,11 @@ ring_step_vec_kernel(const RingParams p) {
 #pragma unroll
     for (int u = 0; u < kRingU; ++u) b[u] = tl.load(rl, u);
 #pragma unroll
-    for (int u = 0; u < kRingU; ++u) tl.store(rl, u, step_vec<T, (OP >= 0 ? OP : 0)>(a[u], b[u]));
+    for (int u = 0; u < kRingU; ++u) {
+      u32x4 v = step_vec<T, (OP >= 0 ? OP : 0)>(a[u], b[u]);
+      if constexpr (FIN) v = finish_vec<T, OP>(v, p.div);
+      tl.store(rl, u, v);
+    }
   } else {
 #pragma unroll
     for (int u = 0; u < kRingU; ++u) tl.store(rl, u, a[u]);
@@ -117,6 +125,7 @@ int make_plan(RingPlan &pl, void *const *bufs, int P, size_t count, int dtype, s
     }
   }
   pl.rp.P = P;
+  pl.rp.div = make_divisor(P);
   pl.rp.seg_base = count / (size_t)P;
   pl.rp.seg_rem = count % (size_t)P;
   pl.rp.t = 0;
@@ -137,16 +146,17 @@ int make_plan(RingPlan &pl, void *const *bufs, int P, size_t count, int dtype, s
   return ALAMD_OK;
 }
 
-int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, hipStream_t stream) {
+// last: the final reduce-scatter step, after which every rank holds its fully reduced segment
+int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, bool last, hipStream_t stream) {
   const dim3 grid(pl.gx, pl.rp.P, 1), block(kThreads, 1, 1);
   if (!reduce) {
     // a copy only needs the element size
     void (*kern)(const RingParams) = nullptr;
     switch (pl.es) {
-    case 1: kern = ring_step_vec_kernel<uint8_t, -1>; break;
-    case 2: kern = ring_step_vec_kernel<uint16_t, -1>; break;
-    case 4: kern = ring_step_vec_kernel<uint32_t, -1>; break;
-    default: kern = ring_step_vec_kernel<uint64_t, -1>; break;
+    case 1: kern = ring_step_vec_kernel<uint8_t, -1, false>; break;
+    case 2: kern = ring_step_vec_kernel<uint16_t, -1, false>; break;
+    case 4: kern = ring_step_vec_kernel<uint32_t, -1, false>; break;
+    default: kern = ring_step_vec_kernel<uint64_t, -1, false>; break;
     }
     hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
     ALAMD_HIP(hipGetLastError());
@@ -155,7 +165,11 @@ int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, hipStream_t 
   return dispatch_any(dtype, op, [&](auto tt, auto ot) -> int {
     using T = typename decltype(tt)::type;
     constexpr int OP = decltype(ot)::value;
-    hipLaunchKernelGGL((ring_step_vec_kernel<T, OP>), grid, block, 0, stream, pl.rp);
+    void (*kern)(const RingParams) = ring_step_vec_kernel<T, OP, false>;
+    if constexpr (OP == ALAMD_AVG) {
+      if (last) kern = ring_step_vec_kernel<T, OP, true>;
+    }
+    hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;
   });
@@ -253,7 +267,7 @@ int alamd_ring_reduce_scatter(void *const *bufs, int P, size_t count, int dtype,
   if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, P, count, dtype, op, false, as_stream(stream));
   for (int t = 0; t < P - 1; ++t) {
     pl.rp.t = t;
-    if ((rc = launch_step(pl, dtype, op, true, as_stream(stream)))) return rc;
+    if ((rc = launch_step(pl, dtype, op, true, t == P - 2, as_stream(stream)))) return rc;
   }
   return ALAMD_OK;
 }
@@ -266,7 +280,7 @@ int alamd_ring_allgather(void *const *bufs, int P, size_t count, int dtype, size
   if (count == 0 || P == 1) return ALAMD_OK;
   for (int t = 0; t < P - 1; ++t) {
     pl.rp.t = t;
-    if ((rc = launch_step(pl, dtype, 0, false, as_stream(stream)))) return rc;
+    if ((rc = launch_step(pl, dtype, 0, false, false, as_stream(stream)))) return rc;
   }
   return ALAMD_OK;
 }

@@ -30,10 +30,8 @@ extern "C" {
 #define ALAMD_VERSION_MAJOR 0
 #define ALAMD_VERSION_MINOR 1
 
-/* Largest number of logical ranks one call can combine. */
+/* Largest number of logical ranks one call can combine, under every order. */
 #define ALAMD_MAX_RANKS 64
-/* Largest number of logical ranks under the tree orders. */
-#define ALAMD_MAX_TREE_RANKS 32
 
 typedef enum {
   ALAMD_OK = 0,
@@ -59,9 +57,15 @@ typedef enum {
 } alamd_dtype;
 
 /* Numerically identical to Al::ReductionOperator
- * (include/aluminum/base.hpp:103-105), so the C++ shim casts.  avg is
- * rejected with ALAMD_ERR_UNSUPPORTED_OP exactly as the reference's MPI and
- * host-transfer backends reject it. */
+ * (include/aluminum/base.hpp:103-105), so the C++ shim casts.
+ * avg (the reference has it on its NCCL backend only,
+ * include/aluminum/nccl_impl.hpp:176; its MPI and host-transfer backends throw,
+ * include/aluminum/mpi/utils.hpp:192-194) is defined for every type as the sum
+ * in the call's order, rounded or wrapped after every step exactly as for
+ * ALAMD_SUM, followed by one division by the number of ranks P in the element
+ * type's own arithmetic: IEEE division for fp32 / fp64; for fp16 / bf16 the
+ * sum is widened, divided in fp32 and narrowed round-to-nearest-even; for the
+ * integer types C division, which truncates toward zero. */
 typedef enum {
   ALAMD_SUM = 0, ALAMD_PROD = 1, ALAMD_MIN = 2, ALAMD_MAX = 3, ALAMD_LOR = 4,
   ALAMD_LAND = 5, ALAMD_LXOR = 6, ALAMD_BOR = 7, ALAMD_BAND = 8, ALAMD_BXOR = 9,
@@ -104,9 +108,9 @@ int alamd_version(void);
 /* Bytes per element, 0 for an unknown dtype. */
 size_t alamd_dtype_size(int dtype);
 /* ALAMD_OK if `op` is defined for `dtype`
- * (include/aluminum/mpi/utils.hpp:169-269: every op but avg for the native
- * types; sum, prod, min, max for fp16 / bf16; MPI defines the logical and
- * bitwise ops for integers only). */
+ * (include/aluminum/mpi/utils.hpp:169-269: sum, prod, min, max for every type;
+ * MPI defines the logical and bitwise ops for integers only; avg for every
+ * type, see alamd_op). */
 int alamd_check_op(int dtype, int op);
 /* Selects nothing and allocates nothing; checks that the current device is a
  * gfx950 and caches its compute-unit count.  Optional: every entry point

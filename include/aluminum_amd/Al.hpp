@@ -714,10 +714,11 @@ struct IsOpSupported<Op, HipCombineBackend> : std::integral_constant<bool, amd::
 template <typename Backend, typename T> struct IsTypeSupported : std::false_type {};
 template <typename T> struct IsTypeSupported<HipCombineBackend, T> : amd::HasTypeMap<T> {};
 
-/** Every operator but avg, like the MPI and host-transfer backends (mpi/utils.hpp:192-194). */
+/** Every operator, avg included: the sum in the collective's order followed by one division by
+ *  comm.size() in the element type's arithmetic (the reference has avg on its NCCL backend only,
+ *  include/aluminum/nccl_impl.hpp:176; its MPI and host-transfer backends throw, mpi/utils.hpp:192-194). */
 template <typename Backend, ReductionOperator op> struct IsReductionOpSupported : std::false_type {};
-template <ReductionOperator op>
-struct IsReductionOpSupported<HipCombineBackend, op> : std::integral_constant<bool, op != ReductionOperator::avg> {};
+template <ReductionOperator op> struct IsReductionOpSupported<HipCombineBackend, op> : std::true_type {};
 
 template <AlOperation Op, typename Backend, typename = void> struct OpAlgoType {};
 template <AlOperation Op>

@@ -59,6 +59,7 @@ def lib():
             getattr(L, name).restype = None
             getattr(L, name).argtypes = [vp, vp, sz]
         L.alo_step.argtypes = [vp, vp, sz, i, i]
+        L.alo_divide.argtypes = [vp, sz, i, i]
         L.alo_schedule.argtypes = [i, i, i, C.POINTER(C.c_int), C.POINTER(C.c_int)]
         L.alo_combine.argtypes = [vp, C.POINTER(vp), i, sz, i, i, i, i]
         L.alo_combine_generated.argtypes = [vp, i, sz, i, i, i, i, i, u64, u64]
@@ -167,6 +168,15 @@ def step(inout, inn, dtype, op):
     rc = lib().alo_step(_ptr(res), _ptr(inn), res.size, _dt(dtype), _op(op))
     if rc:
         raise ValueError("Reduction operator not supported")
+    return res
+
+
+def divide(x, dtype, ranks):
+    """Returns x / ranks (a new array): the division that ends an avg."""
+    res = np.array(x, copy=True)
+    rc = lib().alo_divide(_ptr(res), res.size, _dt(dtype), ranks)
+    if rc:
+        raise ValueError("bad divide arguments")
     return res
 
 

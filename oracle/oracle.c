@@ -30,14 +30,17 @@ static int is_float_dtype(int dtype) {
          dtype == ALO_F64;
 }
 
-/* include/aluminum/mpi/utils.hpp:169-233: the generic map accepts sum..bxor
- * and throws on avg; the __half / bfloat specialisations accept only
- * sum, prod, min, max.  MPI itself defines the logical and bitwise ops for
- * integer types only, so fp32/fp64 with them is an error at the MPI call. */
+/* include/aluminum/mpi/utils.hpp:169-233: the generic map accepts sum..bxor;
+ * the __half / bfloat specialisations accept only sum, prod, min, max.  MPI
+ * itself defines the logical and bitwise ops for integer types only, so
+ * fp32/fp64 with them is an error at the MPI call.  avg exists on the
+ * reference's NCCL path only (include/aluminum/nccl_impl.hpp:176); the MPI and
+ * host-transfer backends throw on it (mpi/utils.hpp:192-194).  Here it is
+ * defined for every type as the sum followed by alo_divide. */
 int alo_check_op(int dtype, int op) {
   if (alo_dtype_size(dtype) == 0) return 2;
-  if (op < ALO_SUM || op > ALO_BXOR) return 1;
-  if (is_float_dtype(dtype) && op > ALO_MAX) return 1;
+  if (op < ALO_SUM || op > ALO_AVG) return 1;
+  if (is_float_dtype(dtype) && op > ALO_MAX && op != ALO_AVG) return 1;
   return 0;
 }
 
@@ -250,7 +253,8 @@ void alo_fill(void *dst, size_t n, int dtype, int dist, uint64_t seed,
   static int step_##NAME(T *b, const T *a, size_t n, int op) {                  \
     size_t i;                                                                   \
     switch (op) {                                                               \
-    case ALO_SUM: for (i = 0; i < n; i++) b[i] = (T)((uint64_t)a[i] + (uint64_t)b[i]); break; \
+    case ALO_SUM: /* and avg: the sum comes first */                            \
+    case ALO_AVG: for (i = 0; i < n; i++) b[i] = (T)((uint64_t)a[i] + (uint64_t)b[i]); break; \
     case ALO_PROD: for (i = 0; i < n; i++) b[i] = (T)((uint64_t)a[i] * (uint64_t)b[i]); break; \
     case ALO_MIN: for (i = 0; i < n; i++) b[i] = (b[i] < a[i]) ? b[i] : a[i]; break; \
     case ALO_MAX: for (i = 0; i < n; i++) b[i] = (b[i] > a[i]) ? b[i] : a[i]; break; \
@@ -281,7 +285,7 @@ DEF_INT_STEP(u64, uint64_t)
   static int step_##NAME(T *b, const T *a, size_t n, int op) {                  \
     size_t i;                                                                   \
     switch (op) {                                                               \
-    case ALO_SUM: for (i = 0; i < n; i++) b[i] = a[i] + b[i]; break;            \
+    case ALO_SUM: case ALO_AVG: for (i = 0; i < n; i++) b[i] = a[i] + b[i]; break; \
     case ALO_PROD: for (i = 0; i < n; i++) b[i] = a[i] * b[i]; break;           \
     case ALO_MIN: for (i = 0; i < n; i++) b[i] = (b[i] < a[i]) ? b[i] : a[i]; break; \
     case ALO_MAX: for (i = 0; i < n; i++) b[i] = (b[i] > a[i]) ? b[i] : a[i]; break; \
@@ -300,7 +304,7 @@ DEF_FP_STEP(f64, double)
   static int step_##NAME(uint16_t *b, const uint16_t *a, size_t n, int op) {    \
     size_t i;                                                                   \
     switch (op) {                                                               \
-    case ALO_SUM: for (i = 0; i < n; i++) b[i] = NARROW(WIDEN(a[i]) + WIDEN(b[i])); break; \
+    case ALO_SUM: case ALO_AVG: for (i = 0; i < n; i++) b[i] = NARROW(WIDEN(a[i]) + WIDEN(b[i])); break; \
     case ALO_PROD: for (i = 0; i < n; i++) b[i] = NARROW(WIDEN(a[i]) * WIDEN(b[i])); break; \
     case ALO_MIN: for (i = 0; i < n; i++) { float x = WIDEN(a[i]), y = WIDEN(b[i]); b[i] = NARROW((y < x) ? y : x); } break; \
     case ALO_MAX: for (i = 0; i < n; i++) { float x = WIDEN(a[i]), y = WIDEN(b[i]); b[i] = NARROW((x < y) ? y : x); } break; \
@@ -341,6 +345,42 @@ int alo_step(void *inout, const void *in, size_t n, int dtype, int op) {
   for (size_t t = 0; t < ntiles; t++) {
     size_t lo = t * ALO_TILE, len = n - lo < ALO_TILE ? n - lo : ALO_TILE;
     step_serial((char *)inout + lo * es, (const char *)in + lo * es, len, dtype, op);
+  }
+  return 0;
+}
+
+/* The division that ends an avg: x[i] /= ranks in the element type's own
+ * arithmetic.  fp32 / fp64: IEEE division.  fp16 / bf16: widen, fp32 division,
+ * narrow (one more step of the rule of src/mpi_impl.cpp:61-145).  Integers: C
+ * division, which truncates toward zero. */
+static void divide_serial(void *x, size_t n, int dtype, int ranks) {
+  size_t i;
+  switch (dtype) {
+  case ALO_I8: { int8_t *p = (int8_t *)x; for (i = 0; i < n; i++) p[i] = (int8_t)(p[i] / ranks); } break;
+  case ALO_U8: { uint8_t *p = (uint8_t *)x; for (i = 0; i < n; i++) p[i] = (uint8_t)(p[i] / ranks); } break;
+  case ALO_I16: { int16_t *p = (int16_t *)x; for (i = 0; i < n; i++) p[i] = (int16_t)(p[i] / ranks); } break;
+  case ALO_U16: { uint16_t *p = (uint16_t *)x; for (i = 0; i < n; i++) p[i] = (uint16_t)(p[i] / ranks); } break;
+  case ALO_I32: { int32_t *p = (int32_t *)x; for (i = 0; i < n; i++) p[i] = p[i] / (int32_t)ranks; } break;
+  case ALO_U32: { uint32_t *p = (uint32_t *)x; for (i = 0; i < n; i++) p[i] = p[i] / (uint32_t)ranks; } break;
+  case ALO_I64: { int64_t *p = (int64_t *)x; for (i = 0; i < n; i++) p[i] = p[i] / (int64_t)ranks; } break;
+  case ALO_U64: { uint64_t *p = (uint64_t *)x; for (i = 0; i < n; i++) p[i] = p[i] / (uint64_t)ranks; } break;
+  case ALO_F16: { uint16_t *p = (uint16_t *)x; for (i = 0; i < n; i++) p[i] = alo_f32_to_f16(alo_f16_to_f32(p[i]) / (float)ranks); } break;
+  case ALO_BF16: { uint16_t *p = (uint16_t *)x; for (i = 0; i < n; i++) p[i] = alo_f32_to_bf16(alo_bf16_to_f32(p[i]) / (float)ranks); } break;
+  case ALO_F32: { float *p = (float *)x; for (i = 0; i < n; i++) p[i] = p[i] / (float)ranks; } break;
+  case ALO_F64: { double *p = (double *)x; for (i = 0; i < n; i++) p[i] = p[i] / (double)ranks; } break;
+  default: break;
+  }
+}
+
+int alo_divide(void *x, size_t n, int dtype, int ranks) {
+  const size_t es = alo_dtype_size(dtype);
+  if (es == 0) return 2;
+  if (ranks < 1) return 4;
+  const size_t ntiles = (n + ALO_TILE - 1) / ALO_TILE;
+#pragma omp parallel for schedule(static)
+  for (size_t t = 0; t < ntiles; t++) {
+    size_t lo = t * ALO_TILE, len = n - lo < ALO_TILE ? n - lo : ALO_TILE;
+    divide_serial((char *)x + lo * es, len, dtype, ranks);
   }
   return 0;
 }
@@ -461,6 +501,7 @@ static int combine_impl(void *out, const void *const *in, int P, size_t n,
             memcpy(slots[r], (const char *)in[r] + lo * es, len * es);
         }
         run_schedule(slots, pairs, np, len, dtype, op);
+        if (op == ALO_AVG) divide_serial(slots[result], len, dtype, P);
         memcpy((char *)out + lo * es, slots[result], len * es);
       }
     }
@@ -566,6 +607,9 @@ int alo_ring_reduce_scatter(void *const *bufs, int P, size_t n, int dtype,
         size_t m = len - c < chunk_elems ? len - c : chunk_elems;
         memcpy(wire, (const char *)bufs[from] + (off + c) * es, m * es); /* the message */
         alo_step((char *)bufs[r] + (off + c) * es, wire, m, dtype, op);
+        /* avg: the last step leaves the full sum in place; divide it there */
+        if (op == ALO_AVG && t == P - 2)
+          alo_divide((char *)bufs[r] + (off + c) * es, m, dtype, P);
       }
     }
   free(wire);

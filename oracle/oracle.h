@@ -37,6 +37,12 @@
  *   Ring RS+AG emulation: moved literally chunk by chunk here and compared
  *     with the closed-form rotated fold, plus invariants (all ranks equal,
  *     chunk size does not change a bit).
+ *   alo_divide (avg): numpy / torch division of the same sums (float32,
+ *     float64, float16 and bfloat16 arithmetic; Python integers for the
+ *     truncating integer division), closed forms (equal contributions).  The
+ *     rounding rule itself is this build's: the reference hands avg to NCCL
+ *     and holds no vectors for it, so against the reference avg is "parity
+ *     unpinned".
  *   Halo pack/unpack: numpy slicing of the same grid.
  *   NaN payload bits are outside every parity claim (tests compare NaN-ness).
  *   Float min/max with NaN or +-0 operands under an order with more than two
@@ -90,8 +96,10 @@ enum {
 };
 
 size_t alo_dtype_size(int dtype);
-/* 0 if `op` is defined for `dtype` on the reference's MPI / HT path
- * (include/aluminum/mpi/utils.hpp:169-233), else nonzero. */
+/* 0 if `op` is defined for `dtype`: the pairs of the reference's MPI / HT path
+ * (include/aluminum/mpi/utils.hpp:169-233) plus avg for every type (the
+ * reference has it on its NCCL path only, include/aluminum/nccl_impl.hpp:176),
+ * else nonzero. */
 int alo_check_op(int dtype, int op);
 
 /* Counter-based generator: element `idx` of stream `seed`. */
@@ -113,6 +121,13 @@ void alo_f16_to_f32_array(float *dst, const uint16_t *src, size_t n);
  * inout[i] = in[i] OP inout[i].  Returns 0, or nonzero for an undefined
  * (dtype, op) pair. */
 int alo_step(void *inout, const void *in, size_t n, int dtype, int op);
+
+/* The division that ends an avg: x[i] = x[i] / ranks.  fp32 / fp64: IEEE
+ * division; fp16 / bf16: widen, fp32 division, round-to-nearest-even
+ * narrowing; integers: C division (truncation toward zero).  With op =
+ * ALO_AVG every combine below is the sum in the named order (rounded or wrapped
+ * after every step as for sum) followed by this division by P. */
+int alo_divide(void *x, size_t n, int dtype, int ranks);
 
 /* The schedule of a named order over P operands: `pairs` receives up to P-1
  * (inout_slot, in_slot) pairs, executed in sequence; the result ends in

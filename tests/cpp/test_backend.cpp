@@ -14,7 +14,7 @@ static_assert(!Al::IsOpSupported<Al::AlOperation::alltoall, Backend>::value, "al
 static_assert(Al::IsTypeSupported<Backend, float>::value && Al::IsTypeSupported<Backend, unsigned long long>::value &&
                   Al::IsTypeSupported<Backend, Al::amd::bfloat16_bits>::value, "types");
 static_assert(!Al::IsTypeSupported<Backend, long double>::value, "long double has no device type");
-static_assert(Al::IsReductionOpSupported<Backend, Op::bxor>::value && !Al::IsReductionOpSupported<Backend, Op::avg>::value,
+static_assert(Al::IsReductionOpSupported<Backend, Op::bxor>::value && Al::IsReductionOpSupported<Backend, Op::avg>::value,
               "operators");
 static_assert(std::is_same<Al::OpAlgoType<Al::AlOperation::allgather, Backend>::type, Algo>::value, "algo type");
 
@@ -23,12 +23,12 @@ static void test_errors(hipStream_t stream) {
   Al::amd::World world(2, stream);
   bool threw = false;
   try {
-    Al::Allreduce<Backend>(a.p, 64, Op::avg, world.comm(0));
-    Al::Allreduce<Backend>(b.p, 64, Op::avg, world.comm(1));
+    Al::Allreduce<Backend>(a.p, 64, Op::band, world.comm(0));
+    Al::Allreduce<Backend>(b.p, 64, Op::band, world.comm(1));
   } catch (const Al::al_exception &e) {
     threw = std::string(e.what()).find("Reduction operator not supported") != std::string::npos;
   }
-  EXPECT(threw, "avg must throw 'Reduction operator not supported'");
+  EXPECT(threw, "band on float must throw 'Reduction operator not supported'");
   Al::amd::World w2(2, stream);
   threw = false;
   try {

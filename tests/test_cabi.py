@@ -64,7 +64,7 @@ def test_argument_checks_need_no_gpu():
     f32, SUM, AVG = al.DTYPES.index("f32"), 0, 10
     assert L.alamd_combine(one, 1, two, 0, 16, f32, SUM, 0, 0, None) == 1          # P = 0
     assert L.alamd_combine(one, 1, two, 65, 16, f32, SUM, 0, 0, None) == 1         # P too large
-    assert L.alamd_combine(one, 1, two, 2, 16, f32, AVG, 0, 0, None) == 2
+    assert L.alamd_combine(one, 1, two, 2, 16, f32, AVG + 1, 0, 0, None) == 2
     assert b"Reduction operator not supported" in L.alamd_last_error()
     assert L.alamd_combine(one, 1, two, 2, 16, f32, 7, 0, 0, None) == 2            # bor on fp32
     assert L.alamd_combine(one, 1, two, 2, 16, 42, SUM, 0, 0, None) == 3

@@ -54,7 +54,7 @@ def test_benchmark_sweep_rows():
     for r in rows:
         assert r[0] == "HipCombineBackend" and r[2] == "allreduce" and r[4] == "1" and r[7] == "4"
         assert 0 < float(r[10]) < 1.0
-    bad = subprocess.run([exe, "--op", "allreduce", "--reduction-op", "avg", "--max-size", "4"], capture_output=True,
+    bad = subprocess.run([exe, "--op", "allreduce", "--reduction-op", "bxor", "--max-size", "4"], capture_output=True,
                          text=True, timeout=60)
     assert bad.returncode == 1 and "Reduction operator not supported" in bad.stderr
 
@@ -70,6 +70,14 @@ OPS_SWEEPS = [
     "--op allreduce --datatype uchar --reduction-op lxor --inplace --odd-sizes --max-size 65536 --ranks 5",
     "--op allreduce --datatype longlong --reduction-op band --nonblocking --max-size 65536 --ranks 8",
     "--op allreduce --datatype double --reduction-op prod --algorithm ring --min-size 0 --max-size 32768 --ranks 8",
+    # more than 32 logical ranks: the default algorithm is a tree order there too
+    "--op allreduce --datatype float --odd-sizes --max-size 16384 --ranks 33",
+    "--op allreduce --datatype bfloat16 --inplace --max-size 16384 --ranks 64",
+    "--op reduce --datatype double --root 40 --algorithm tree_binomial --max-size 4096 --ranks 48",
+    "--op reduce_scatter --datatype float --max-size 256 --ranks 40",
+    "--op allreduce --datatype float --reduction-op avg --inplace --odd-sizes --max-size 65536 --ranks 6",
+    "--op allreduce --datatype bfloat16 --reduction-op avg --algorithm ring --max-size 32768 --ranks 8",
+    "--op reduce_scatter --datatype int --reduction-op avg --nonblocking --odd-sizes --max-size 16384 --ranks 7",
     "--op reduce --datatype float --root 2 --inplace --odd-sizes --max-size 65536 --ranks 4",
     "--op reduce --datatype int --reduction-op min --root 0 --nonblocking --max-size 65536 --ranks 7",
     "--op reduce_scatter --datatype float --inplace --nonblocking --odd-sizes --max-size 65536 --ranks 8",

@@ -12,12 +12,12 @@ pytestmark = pytest.mark.gpu
 
 DIST_FOR = {"sum": "uniform_pm1", "prod": "uniform_09_11", "min": "uniform_pm1", "max": "uniform_pm1",
             "lor": "bool01", "land": "bool01", "lxor": "bool01", "bor": "fullrange",
-            "band": "fullrange", "bxor": "fullrange"}
+            "band": "fullrange", "bxor": "fullrange", "avg": "uniform_pm1"}
 
 
 def make_inputs(P, n, dtype, op, seed=1000):
     dist = DIST_FOR[op]
-    if dtype in INT_DTYPES and op in ("sum", "prod", "min", "max"):
+    if dtype in INT_DTYPES and op in ("sum", "prod", "min", "max", "avg"):
         dist = "fullrange"
     return [oracle.fill(n, dtype, dist, seed + r) for r in range(P)]
 
@@ -46,7 +46,7 @@ def test_combine_all_ops_orders(al, dtype):
 
 
 @pytest.mark.parametrize("dtype", ("f32", "bf16", "i32"))
-@pytest.mark.parametrize("P", (4, 6, 7, 8, 13, 16, 31, 32))
+@pytest.mark.parametrize("P", (4, 6, 7, 8, 13, 16, 31, 32, 33, 40, 48, 63, 64))
 def test_combine_many_ranks(al, dtype, P):
     n = 5000
     for order in ORDERS:
@@ -301,12 +301,76 @@ def test_allgatherv(al, dtype):
     assert e.value.code == 5
 
 
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_avg_division_every_rank_count(al, dtype):
+    """avg ends with one division by P: every 8- and 16-bit pattern (and edge values plus random ones of
+    the wider types) as the sum, for every P up to 64, against the oracle's C division."""
+    import torch
+    np_dt = oracle.NP_CARRIER[dtype]
+    es = oracle.dtype_size(dtype)
+    if es <= 2:
+        x = np.arange(1 << (8 * es), dtype=np.uint32).astype(np.uint8 if es == 1 else np.uint16).view(np_dt)
+    else:
+        x = oracle.fill(20000, dtype, "fullrange" if dtype in INT_DTYPES else "uniform_pm1", 77)
+        if dtype in INT_DTYPES:
+            info = np.iinfo(np_dt)
+            edge = [info.min, info.min + 1, info.max, info.max - 1, 0, 1, 2, 63, 64, 65, 127, 128, 129]
+            edge += [-1, -2, -63, -64, -65] if info.min < 0 else []
+            x[:len(edge)] = np.array(edge, dtype=np_dt)
+        else:
+            tiny = np.finfo(np_dt).tiny
+            x[:6] = np.array([0.0, -0.0, tiny, -tiny * 0.5, np.inf, np.nan], dtype=np_dt)
+            x[6:100] *= tiny  # subnormal quotients
+    zero = np.zeros_like(x)
+    d_x, d_zero = to_dev(x), to_dev(zero)
+    out = dev_empty(x.size, x.dtype)
+    for P in list(range(1, 18)) + [24, 31, 32, 33, 48, 63, 64]:
+        ins = [d_x] + [d_zero] * (P - 1)
+        al.combine([out], ins, "avg", order="rank_asc", dtype=dtype, count=x.size)
+        torch.cuda.synchronize()
+        want = oracle.combine([x] + [zero] * (P - 1), dtype, "avg", "rank_asc")
+        assert_bits_equal(to_host(out, x.dtype), want, dtype, "avg %s P=%d" % (dtype, P))
+
+
+def test_avg_in_every_collective(al):
+    """avg through reduce_scatter, reduce_scatterv (in place too), the combine into several buffers
+    and the tree orders."""
+    import torch
+    P, n = 5, 7001
+    for dtype in ("f32", "bf16", "i16", "u64"):
+        ins = make_inputs(P, P * n, dtype, "avg")
+        np_dt = ins[0].dtype
+        want = oracle.reduce_scatter(ins, dtype, "avg", "pairwise_desc")
+        recvs = [dev_empty(n, np_dt) for _ in range(P)]
+        al.reduce_scatter(recvs, [to_dev(a) for a in ins], "avg", order="pairwise_desc", dtype=dtype, count=n)
+        torch.cuda.synchronize()
+        for b in range(P):
+            assert_bits_equal(to_host(recvs[b], np_dt), want[b], dtype, "reduce_scatter avg %s block %d" % (dtype, b))
+        bufs = [to_dev(a) for a in ins]
+        al.reduce_scatter(bufs, bufs, "avg", order="pairwise_desc", dtype=dtype, count=n)
+        torch.cuda.synchronize()
+        for b in range(P):
+            assert_bits_equal(to_host(bufs[b], np_dt)[:n], want[b], dtype, "in-place reduce_scatter avg %s" % dtype)
+        counts = [n + 3, 0, 2 * n, 17, P * n - (n + 3) - 2 * n - 17]
+        wantv = oracle.reduce_scatterv(ins, counts, dtype, "avg", "tree_halv")
+        recvs = [dev_empty(max(c, 1), np_dt) for c in counts]
+        al.reduce_scatterv(recvs, [to_dev(a) for a in ins], counts, "avg", order="tree_halv", dtype=dtype)
+        torch.cuda.synchronize()
+        for b in range(P):
+            assert_bits_equal(to_host(recvs[b], np_dt)[:counts[b]], wantv[b], dtype, "reduce_scatterv avg %s" % dtype)
+        for order in ("tree_dbl", "tree_binomial", "ring"):
+            wanta = oracle.combine(ins, dtype, "avg", order, 2 if order == "ring" else 0)
+            outs = run_combine(al, ins, dtype, "avg", order, 2 if order == "ring" else 0, nout=P)
+            for o in outs:
+                assert_bits_equal(o, wanta, dtype, "avg %s %s to %d buffers" % (dtype, order, P))
+
+
 def test_errors(al):
     import torch
     a = [to_dev(np.zeros(16, np.float32)) for _ in range(2)]
     out = [dev_empty(16, np.float32)]
     with pytest.raises(al.AlError, match="Reduction operator not supported"):
-        al.combine(out, a, "avg")
+        al.combine(out, a, 11)  # one past avg
     with pytest.raises(al.AlError, match="Reduction operator not supported"):
         al.combine(out, a, "band")
     with pytest.raises(al.AlError, match="Invalid algorithm"):

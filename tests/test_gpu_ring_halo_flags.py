@@ -14,14 +14,15 @@ pytestmark = pytest.mark.gpu
 
 def ring_inputs(P, n, dtype, op):
     dist = {"sum": "normal", "prod": "uniform_09_11", "min": "uniform_pm1", "max": "uniform_pm1",
-            "bxor": "fullrange", "lor": "bool01"}[op]
-    if dtype not in FLOAT_DTYPES and op in ("sum", "prod", "min", "max"):
+            "bxor": "fullrange", "lor": "bool01", "avg": "normal"}[op]
+    if dtype not in FLOAT_DTYPES and op in ("sum", "prod", "min", "max", "avg"):
         dist = "fullrange"
     return [oracle.fill(n, dtype, dist, 2000 + r) for r in range(P)]
 
 
 @pytest.mark.parametrize("dtype,op", [("bf16", "sum"), ("f32", "sum"), ("f16", "prod"), ("f64", "max"),
-                                      ("bf16", "min"), ("i32", "sum"), ("u8", "lor"), ("u64", "bxor")])
+                                      ("bf16", "min"), ("i32", "sum"), ("u8", "lor"), ("u64", "bxor"),
+                                      ("bf16", "avg"), ("f32", "avg"), ("i8", "avg"), ("i64", "avg")])
 @pytest.mark.parametrize("mode", ("stepwise", "fused"))
 def test_ring_allreduce(al, dtype, op, mode):
     import torch
@@ -93,7 +94,7 @@ def test_ring_errors(al):
     with pytest.raises(al.AlError):
         al.ring_allreduce(bufs, "sum", chunk_bytes=0)
     with pytest.raises(al.AlError, match="Reduction operator not supported"):
-        al.ring_allreduce(bufs, "avg")
+        al.ring_allreduce(bufs, "lor")  # a logical operator on a float type
     with pytest.raises(al.AlError):
         al.ring_allreduce([bufs[0], bufs[0]], "sum")
 

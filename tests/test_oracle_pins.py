@@ -48,9 +48,10 @@ def test_fp_step_against_numpy(dtype):
 
 
 def test_unsupported_pairs():
-    # include/aluminum/mpi/utils.hpp:169-269
+    # include/aluminum/mpi/utils.hpp:169-269; avg (NCCL path only in the reference) is defined for every type
     for dt in ALL_DTYPES:
-        assert oracle.check_op(dt, "avg") != 0
+        assert oracle.check_op(dt, "avg") == 0
+        assert oracle.check_op(dt, 11) != 0
         for op in ("lor", "land", "lxor", "bor", "band", "bxor"):
             assert (oracle.check_op(dt, op) != 0) == (dt in FLOAT_DTYPES)
         for op in ("sum", "prod", "min", "max"):
@@ -60,6 +61,50 @@ def test_unsupported_pairs():
 
 
 # ---- 16-bit floats -----------------------------------------------------------
+
+def trunc_div(a, d):
+    """C integer division of a numpy integer array by d, through Python integers."""
+    return np.array([abs(int(v)) // d * (1 if v >= 0 else -1) for v in a.tolist()], dtype=a.dtype)
+
+
+@pytest.mark.parametrize("dtype", ALL_DTYPES)
+def test_avg_is_sum_then_divide(dtype):
+    """avg = the sum of the same order, then one division by P: pinned with numpy / torch division of
+    the oracle's own sum (itself pinned above) and with closed forms."""
+    import torch
+    n = 3000
+    np_dt = oracle.NP_CARRIER[dtype]
+    for P in (1, 2, 3, 7, 8, 64):
+        dist = "fullrange" if dtype in INT_DTYPES else "uniform_pm1"
+        ins = [oracle.fill(n, dtype, dist, 50 + r) for r in range(P)]
+        for order in ("rank_asc", "tree_dbl"):
+            s = oracle.combine(ins, dtype, "sum", order)
+            got = oracle.combine(ins, dtype, "avg", order)
+            if dtype in INT_DTYPES:
+                want = trunc_div(s, P)   # truncation toward zero
+            elif dtype == "f32":
+                want = s / np.float32(P)
+            elif dtype == "f64":
+                want = s / np.float64(P)
+            elif dtype == "f16":
+                want = (s.view(np.float16).astype(np.float32) / np.float32(P)).astype(np.float16).view(np.uint16)
+            else:  # bf16: widen, fp32 division, torch's round-to-nearest-even narrowing
+                wide = torch.from_numpy(s.view(np.int16).copy()).view(torch.bfloat16).float()
+                want = (wide / float(P)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+            assert_bits_equal(got, want, dtype, "avg %s P=%d %s" % (dtype, P, order))
+            assert_bits_equal(oracle.divide(s, dtype, P), want, dtype, "divide %s P=%d" % (dtype, P))
+    # closed forms: equal contributions whose sum is exact average to the contribution itself
+    x = oracle.fill(n, dtype, "smallint", 9)
+    for P in (2, 4, 5, 8):
+        assert_bits_equal(oracle.combine([x] * P, dtype, "avg", "rank_asc"), x, dtype, "avg of equals")
+    # truncation toward zero, not flooring: (-7) / 2 = -3; unsigned wraps before it divides
+    if dtype in ("i8", "i16", "i32", "i64"):
+        a = np.array([-7, 7, -1, 1], dtype=np_dt)
+        assert oracle.combine([a, np.zeros(4, np_dt)], dtype, "avg", "rank_asc").tolist() == [-3, 3, 0, 0]
+    if dtype == "u8":
+        a = np.array([200, 100], dtype=np_dt)
+        assert oracle.combine([a, a], dtype, "avg", "rank_asc").tolist() == [(400 % 256) // 2, 100]
+
 
 def test_f16_widen_all_patterns_against_numpy():
     bits = np.arange(1 << 16, dtype=np.uint32).astype(np.uint16)

@@ -7,8 +7,8 @@ SIGNED_VIEW = {np.dtype(np.uint16): np.int16, np.dtype(np.uint32): np.int32,
 FLOAT_DTYPES = ("f16", "bf16", "f32", "f64")
 INT_DTYPES = ("i8", "u8", "i16", "u16", "i32", "u32", "i64", "u64")
 ALL_DTYPES = INT_DTYPES + FLOAT_DTYPES
-FP_OPS = ("sum", "prod", "min", "max")
-INT_OPS = ("sum", "prod", "min", "max", "lor", "land", "lxor", "bor", "band", "bxor")
+FP_OPS = ("sum", "prod", "min", "max", "avg")
+INT_OPS = ("sum", "prod", "min", "max", "lor", "land", "lxor", "bor", "band", "bxor", "avg")
 ORDERS = ("rank_asc", "tree_dbl", "tree_halv", "pairwise_desc", "ring", "tree_binomial")
 
 
