@@ -127,6 +127,71 @@ __host__ __device__ inline void out_select(const SegParams &s, int P, unsigned s
   else { j0 = ((int)seg + s.owner_shift) % P; nj = 1; out_bytes = off_bytes; }
 }
 
+// ---- a fold whose output overlaps one of its inputs at a displacement ---------
+//
+// An in-place Reduce_scatterv writes block b's result to elements [0, n) of
+// rank b's buffer while that rank's contribution is read from [displ, displ + n)
+// of the same buffer: with 0 < displ < n the tile that writes a range must not
+// store before the tiles that read that range have loaded it.  One launch does
+// this without any order among workgroups being assumed:
+//  - a workgroup takes its tile from a ticket counter, so every tile with a
+//    lower number is held by a workgroup that is already running;
+//  - when the loads of a tile have landed (values in registers) its workgroup
+//    sets the tile's flag, and only then waits for the flags of the (at most
+//    two) lower-numbered tiles whose reads overlap its own writes; a flag is set
+//    before any wait, so no wait can be circular;
+//  - the elements behind the last whole vector are one more ticket, handled
+//    the same way.
+// The counter and the flags are scratch memory in HBM, cleared on the stream
+// before the launch.  A wait is bounded: if it expires (it cannot, unless the
+// device loses a workgroup) the error word is set and the workgroup goes on.
+struct ChainParams {
+  unsigned *ticket;                 // next tile; null: not a chained launch
+  unsigned *flags;                  // flags[t] != 0: tile t has loaded its inputs
+  unsigned *error;                  // set to 1 by a wait that expired
+  unsigned long long displ_bytes;   // the overlapping input starts this far behind the output
+  unsigned nvec_tiles;              // whole-vector tiles (the tail is ticket nvec_tiles)
+};
+constexpr unsigned kChainMaxSpins = 1u << 24;
+
+__device__ __forceinline__ unsigned chain_take_tile(const ChainParams &c) {
+  __shared__ unsigned s_tile;
+  if (threadIdx.x == 0) s_tile = __hip_atomic_fetch_add(c.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  return s_tile;
+}
+
+// Called by every thread of the workgroup that holds tile `self`, between the last use of the loaded
+// values and the first store to bytes [w0, w0 + wlen) of the output.
+__device__ __forceinline__ void chain_gate(const ChainParams &c, unsigned self, unsigned long long w0,
+                                           unsigned long long wlen, unsigned tile_bytes) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads have returned
+  __syncthreads();                                  // ... and every other wave's of the workgroup
+  if (threadIdx.x == 0) {
+    if (self < c.nvec_tiles) __hip_atomic_store(&c.flags[self], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    // tiles t that read output bytes [w0, w0 + wlen): displ + t*TB < w0 + wlen and displ + (t+1)*TB > w0
+    const long long tb = (long long)tile_bytes;
+    const long long a0 = (long long)w0 - (long long)c.displ_bytes, a1 = a0 + (long long)wlen;
+    if (a1 > 0 && self > 0) {
+      long long lo = a0 <= 0 ? 0 : a0 / tb;            // floor
+      long long hi = (a1 + tb - 1) / tb - 1;           // ceil - 1
+      if (hi > (long long)self - 1) hi = (long long)self - 1;
+      if (hi > (long long)c.nvec_tiles - 1) hi = (long long)c.nvec_tiles - 1;
+      for (long long t = lo; t <= hi; ++t) {
+        unsigned spins = 0;
+        while (__hip_atomic_load(&c.flags[t], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
+          __builtin_amdgcn_s_sleep(2);
+          if (++spins > kChainMaxSpins) {
+            __hip_atomic_store(c.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+}
+
 // Left fold over a rotated rank sequence.
 struct FoldParams {
   const char *in[ALAMD_MAX_RANKS];
@@ -137,6 +202,7 @@ struct FoldParams {
   int start_stride;
   int dir;           // +1: next operand is rank+1, -1: rank-1 (with wrap)
   Divisor div;       // avg: the number of ranks as a divisor
+  ChainParams chain; // set for a chained launch only
 };
 
 // Balanced pairwise tree over up to 64 slots.  Slot j holds a[j], or
@@ -151,6 +217,7 @@ struct TreeParams {
   int P;        // number of ranks (for OUT_OWNER)
   int nvalid;   // occupied slots
   Divisor div;  // avg: the number of ranks as a divisor
+  ChainParams chain;  // set for a chained launch only
 };
 
 // The launches of a kernel whose grid is (tiles, segments): `launch(tile0, ntiles, seg0, nsegs)` is
@@ -231,10 +298,16 @@ void plan_launches(SegParams &seg, unsigned nseg, size_t max_len, size_t tile_el
   walk(rank_order, launch);
 }
 
+// chain: null for an ordinary launch; else the scratch of a chained launch (one segment, one output,
+// every tile in one launch; displ_bytes and nvec_tiles are filled in here).
+struct ChainScratch { unsigned *ticket, *flags, *error; size_t max_tiles; };
 int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op, bool acc_is_in,
-                hipStream_t stream);
+                hipStream_t stream, const ChainScratch *chain = nullptr, size_t displ_bytes = 0);
 int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, int dtype, int op,
-                hipStream_t stream);
+                hipStream_t stream, const ChainScratch *chain = nullptr, size_t displ_bytes = 0);
+// Clears the ticket counter, the error word and the first `tiles` flags on `stream` (a kernel, not a
+// memset, so that the call may be captured into a graph).
+int chain_clear(const ChainScratch &cs, size_t tiles, hipStream_t stream);
 
 // A result that goes to several buffers is folded into one of them and then
 // spread (one write stream per workgroup) when that is faster than writing

@@ -1,7 +1,11 @@
 // Host side of the combine entry points: argument checks, the mapping of a
 // named order onto one of the two kernel families, the Reduce_scatter and
 // Allgather layouts.
+#include <map>
+#include <mutex>
 #include <string>
+#include <utility>
+#include <vector>
 
 #include "alamd_dispatch.h"
 #include "alamd_tile.h"
@@ -67,8 +71,9 @@ struct Layout {
 
 // Launches the fold or tree kernels for `order` over inputs `ins`.
 // `outs` has ALAMD_MAX_RANKS entries (unused ones null).
+// chain / displ_bytes: see launch_fold.
 int launch_order(void *const *outs, const void *const *ins, int P, const Layout &lay, int dtype, int op,
-                 int order, hipStream_t stream) {
+                 int order, hipStream_t stream, const ChainScratch *chain = nullptr, size_t displ_bytes = 0) {
   if (!is_float_dtype(dtype)) order = ALAMD_ORDER_RANK_ASC;  // integer ops: every order gives the same bits
   if (P == 1 && order_is_tree(order)) order = ALAMD_ORDER_RANK_ASC;
   if (order_is_tree(order)) {
@@ -76,7 +81,7 @@ int launch_order(void *const *outs, const void *const *ins, int P, const Layout 
     const int slots = build_tree(tp, ins, P, order);
     for (int j = 0; j < ALAMD_MAX_RANKS; ++j) tp.out[j] = static_cast<char *>(outs[j]);
     tp.seg = lay.seg;
-    return launch_tree(tp, slots, lay.nseg, lay.max_len, dtype, op, stream);
+    return launch_tree(tp, slots, lay.nseg, lay.max_len, dtype, op, stream, chain, displ_bytes);
   }
   FoldParams fp;
   for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
@@ -88,7 +93,66 @@ int launch_order(void *const *outs, const void *const *ins, int P, const Layout 
   fp.start0 = lay.start0;
   fp.start_stride = lay.start_stride;
   fp.dir = order == ALAMD_ORDER_PAIRWISE_DESC ? -1 : 1;
-  return launch_fold(fp, lay.nseg, lay.max_len, dtype, op, order == ALAMD_ORDER_RING, stream);
+  return launch_fold(fp, lay.nseg, lay.max_len, dtype, op, order == ALAMD_ORDER_RING, stream, chain, displ_bytes);
+}
+
+// ---- scratch of the chained launches -----------------------------------------
+
+__global__ void chain_clear_kernel(unsigned *ticket, unsigned *flags, unsigned long long n) {
+  const unsigned long long i0 = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i0 == 0) *ticket = 0u;
+  for (unsigned long long i = i0; i < n; i += (unsigned long long)gridDim.x * blockDim.x) flags[i] = 0u;
+}
+
+// Bytes in front of the flags: the ticket counter and the error word, on a line of their own.
+constexpr size_t kChainHeaderBytes = 256;
+// The smallest tile of any kernel that can run chained (256 threads x one 128-bit vector).
+constexpr size_t kChainMinTileBytes = 4096;
+
+// One scratch buffer per (device, stream): calls on different streams may overlap in time.  A buffer
+// that turns out too small is replaced by a larger one and kept until the process ends, because work
+// already enqueued may still use it.
+struct ChainPool {
+  std::mutex mutex;
+  std::map<std::pair<int, hipStream_t>, ChainScratch> live;
+  std::vector<void *> retired;
+};
+ChainPool &chain_pool() {
+  static ChainPool *pool = new ChainPool;  // never destroyed: device memory outlives static destruction order
+  return *pool;
+}
+
+ChainScratch scratch_at(void *base, size_t bytes) {
+  ChainScratch cs;
+  char *b = static_cast<char *>(base);
+  cs.ticket = reinterpret_cast<unsigned *>(b);
+  cs.error = reinterpret_cast<unsigned *>(b + 4);
+  cs.flags = reinterpret_cast<unsigned *>(b + kChainHeaderBytes);
+  cs.max_tiles = (bytes - kChainHeaderBytes) / sizeof(unsigned);
+  return cs;
+}
+
+int chain_scratch_for(hipStream_t stream, size_t tiles, ChainScratch &out) {
+  int dev = 0;
+  ALAMD_HIP(hipGetDevice(&dev));
+  ChainPool &pool = chain_pool();
+  std::lock_guard<std::mutex> lock(pool.mutex);
+  auto key = std::make_pair(dev, stream);
+  auto it = pool.live.find(key);
+  if (it != pool.live.end() && it->second.max_tiles >= tiles) {
+    out = it->second;
+    return ALAMD_OK;
+  }
+  size_t cap = (size_t)1 << 16;
+  while (cap < tiles) cap *= 2;
+  const size_t bytes = kChainHeaderBytes + cap * sizeof(unsigned);
+  void *mem = nullptr;
+  ALAMD_HIP(hipMalloc(&mem, bytes));
+  ALAMD_HIP(hipMemset(mem, 0, kChainHeaderBytes));
+  if (it != pool.live.end()) pool.retired.push_back(it->second.ticket);
+  out = scratch_at(mem, bytes);
+  pool.live[key] = out;
+  return ALAMD_OK;
 }
 
 constexpr int kGatherU = 8, kGatherThreads = 128;
@@ -185,6 +249,15 @@ int check_common(int P, size_t count, int dtype) {
 }
 
 }  // namespace
+
+int chain_clear(const ChainScratch &cs, size_t tiles, hipStream_t stream) {
+  if (tiles > cs.max_tiles) return set_error(ALAMD_ERR_INVALID_ARG, "chain scratch too small");
+  const unsigned blocks = (unsigned)((tiles + 255) / 256 < 1 ? 1 : ((tiles + 255) / 256 > 1024 ? 1024 : (tiles + 255) / 256));
+  hipLaunchKernelGGL(chain_clear_kernel, dim3(blocks, 1, 1), dim3(256, 1, 1), 0, stream, cs.ticket, cs.flags,
+                     (unsigned long long)tiles);
+  ALAMD_HIP(hipGetLastError());
+  return ALAMD_OK;
+}
 
 namespace {
 
@@ -314,6 +387,64 @@ int launch_gather(void *const *recvs, const void *const *sends, int P, const siz
     fp.seg.seg_len[q] = lens[q];
   }
   return launch_spread_table(fp, P, true, stream);
+}
+
+}  // namespace
+
+namespace {
+
+// The in-place part of Reduce_scatterv: one fold per block, in ascending block order; block b's
+// result overwrites the start of rank b's buffer, which only blocks <= b read.  A block that is in
+// place and starts displ elements into its own buffer with 0 < displ < count reads its own rank's
+// elements displ + i while it writes element i of the same buffer; it runs as a chained launch (see
+// ChainParams), with scratch from `fixed` if given, else from the pool of the stream.
+int reduce_scatterv_in_place(void *const *recvs, const void *const *sends, int P, const size_t *counts,
+                             const size_t *displ, int dtype, int op, int order, hipStream_t stream,
+                             const ChainScratch *fixed) {
+  const size_t es = alamd_dtype_size(dtype);
+  for (int b = 0; b < P; ++b) {
+    if (counts[b] == 0) continue;
+    const bool inplace = recvs[b] == sends[b];
+    const bool overlapped = inplace && displ[b] != 0 && displ[b] < counts[b];
+    // A few runs no longer than the displacement, each launched after the one before it, never read
+    // what an unfinished launch writes and run at the full rate (a chained launch reaches about a third
+    // of it: 1.9 to 2.5 TB/s at P = 8); more than kMaxRuns of them would be launch-bound.
+    constexpr size_t kMaxRuns = 32;
+    const bool chained = overlapped && (counts[b] + displ[b] - 1) / displ[b] > kMaxRuns;
+    const size_t run = overlapped && !chained ? displ[b] : counts[b];
+    int rc = ALAMD_OK;
+    for (size_t done = 0; done < counts[b] && rc == ALAMD_OK; done += run) {
+      const size_t n = counts[b] - done < run ? counts[b] - done : run;
+      const void *ins[ALAMD_MAX_RANKS];
+      void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
+      for (int r = 0; r < P; ++r) ins[r] = static_cast<const char *>(sends[r]) + (displ[b] + done) * es;
+      out_tab[0] = static_cast<char *>(recvs[b]) + done * es;
+      Layout lay;
+      lay.nseg = 1;
+      lay.seg = make_seg(n, 0, 0, OUT_ALL, 1);
+      lay.max_len = n;
+      lay.start0 = order_has_start(order) ? b : 0;
+      lay.start_stride = 0;
+      if (chained) {
+        ChainScratch cs;
+        const size_t tiles = (n * es + kChainMinTileBytes - 1) / kChainMinTileBytes;
+        if (fixed) {
+          cs = *fixed;
+          if (tiles > cs.max_tiles)
+            return set_error(ALAMD_ERR_INVALID_ARG,
+                             "in-place block %d of %zu bytes is beyond the %zu bytes the fixed scratch covers", b,
+                             n * es, cs.max_tiles * kChainMinTileBytes);
+        } else if ((rc = chain_scratch_for(stream, tiles, cs))) {
+          return rc;
+        }
+        rc = launch_order(out_tab, ins, P, lay, dtype, op, order, stream, &cs, displ[b] * es);
+      } else {
+        rc = launch_order(out_tab, ins, P, lay, dtype, op, order, stream);
+      }
+    }
+    if (rc) return rc;
+  }
+  return ALAMD_OK;
 }
 
 }  // namespace
@@ -517,39 +648,7 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, c
     lay.start_stride = order_has_start(order) ? 1 : 0;
     return launch_order(out_tab, sends, P, lay, dtype, op, order, as_stream(stream));
   }
-  // In place: one fold per block, in ascending block order; block b's result
-  // overwrites the start of rank b's buffer, which only blocks <= b read.
-  for (int b = 0; b < P; ++b) {
-    if (counts[b] == 0) continue;
-    const bool inplace = recvs[b] == sends[b];
-    // In place, block b reads its own rank's elements displ[b] + i while writing
-    // element i of the same buffer: go through the block in runs no longer than
-    // displ[b], each launched after the previous one, so no run reads what an
-    // unfinished run writes.
-    size_t run = counts[b];
-    if (inplace && displ[b] != 0 && displ[b] < counts[b]) {
-      run = displ[b];
-      if ((counts[b] + run - 1) / run > 4096)
-        return set_error(ALAMD_ERR_OVERLAP,
-                         "in-place reduce_scatterv: block %d of %zu elements starts only %zu elements into its own "
-                         "buffer; use separate receive buffers", b, counts[b], displ[b]);
-    }
-    for (size_t done = 0; done < counts[b]; done += run) {
-      const size_t n = counts[b] - done < run ? counts[b] - done : run;
-      const void *ins[ALAMD_MAX_RANKS];
-      void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
-      for (int r = 0; r < P; ++r) ins[r] = static_cast<const char *>(sends[r]) + (displ[b] + done) * es;
-      out_tab[0] = static_cast<char *>(recvs[b]) + done * es;
-      Layout lay;
-      lay.nseg = 1;
-      lay.seg = make_seg(n, 0, 0, OUT_ALL, 1);
-      lay.max_len = n;
-      lay.start0 = order_has_start(order) ? b : 0;
-      lay.start_stride = 0;
-      if ((rc = launch_order(out_tab, ins, P, lay, dtype, op, order, as_stream(stream)))) return rc;
-    }
-  }
-  return ALAMD_OK;
+  return reduce_scatterv_in_place(recvs, sends, P, counts, displ, dtype, op, order, as_stream(stream), nullptr);
 }
 
 int alamd_allgatherv(void *const *recvs, const void *const *sends, int P, const size_t *counts,

@@ -1,201 +1,30 @@
-// The fold kernels: out[i] = (((x_s . x_s+-1) . x_s+-2) ...)[i] over P rank
-// contributions resident in HBM.  Bandwidth-bound: every input byte is read
-// once, every output byte written once.
-//
-// One workgroup per tile, all loads of a lane issued before the first use,
-// buffer instructions with per-tile descriptors (see alamd_tile.h); buffers
-// need only be aligned to their element type.  The len % N elements behind the
-// last whole vector of a segment are folded one per thread.
-#include "alamd_dispatch.h"
-#include "alamd_tile.h"
+// Fold kernels of the floating-point types, and the entry of the fold family:
+// the integer types are built in combine_fold_narrow.hip and combine_fold_wide.hip.
+#include "combine_fold_impl.h"
 
 namespace alamd {
-
 namespace {
-
-__device__ __forceinline__ int next_rank(int idx, int dir, int P) {
-  idx += dir;
-  if (idx >= P) idx -= P;
-  if (idx < 0) idx += P;
-  return idx;
+ALAMD_FOLD_GROUP(group, case ALAMD_F16: return dispatch_fp_op<f16_t>(op, run);
+                 case ALAMD_BF16: return dispatch_fp_op<bf16_t>(op, run);
+                 case ALAMD_F32: return dispatch_fp_op<float>(op, run);
+                 case ALAMD_F64: return dispatch_fp_op<double>(op, run);)
 }
-
-// The fold of one element position, one element per access.
-template <typename T, int OP, bool ACC_IS_IN>
-__device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, size_t in_bytes, int j0, int nj,
-                                          size_t out_bytes, size_t e) {
-  int idx = s;
-  T acc = ld_elem<T>(p.in[idx] + in_bytes + e * sizeof(T));
-  for (int k = 1; k < P; ++k) {
-    idx = next_rank(idx, p.dir, P);
-    const T x = ld_elem<T>(p.in[idx] + in_bytes + e * sizeof(T));
-    acc = ACC_IS_IN ? Step<T, OP>::apply(acc, x) : Step<T, OP>::apply(x, acc);
-  }
-  acc = finish_elem<T, OP>(acc, p.div);
-  for (int j = j0; j < j0 + nj; ++j) st_elem<T>(p.out[j] + out_bytes + e * sizeof(T), acc);
-}
-
-// Tile shape: 128 threads x 8 vectors per stream for every type (byte sums and
-// products, the most arithmetic per byte, are done a dword at a time and keep up).
-template <typename T, int OP> struct Shape {
-  static constexpr int U = 8;
-  static constexpr int THREADS = 128;
-};
-
-// amdgpu_waves_per_eu(1, 2): the loads in flight are the point of this kernel;
-// the register allocator must not trade them away for more resident waves.
-// HEAD = false: no segment has leading elements to handle one by one (every buffer on a 64-byte
-// boundary).  With the head a compile-time zero the fp32 fold runs 1.6 points faster (83.8 % of the HBM
-// peak against 82.2 %) and the fp32 tree 2.8; both bodies in one kernel behind a uniform branch ran slower
-// than either (82.7 %, bf16 80.8 % against 82.2 %), so there are two kernels and the host picks.
-// (The body must stay in the kernel itself: moved into an inlined device function it was compiled
-// with 161 instead of 249 VGPRs, i.e. with fewer loads in flight, and lost 1.5 points.)
-template <typename T, int OP, bool ACC_IS_IN, int PT, bool HEAD>
-__global__ void __launch_bounds__((Shape<T, OP>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
-fold_vec_kernel(const FoldParams p) {
-  constexpr int U = Shape<T, OP>::U, THREADS = Shape<T, OP>::THREADS;
-  constexpr int N = 16 / sizeof(T);
-  using TL = Tile<U, THREADS>;
-  const TL tl;
-  const int P = PT ? PT : p.P;
-  const unsigned seg = seg_of(p.seg, blockIdx.y + p.seg.seg0);
-  size_t off, len;
-  seg_range(p.seg, seg, off, len);
-  const size_t off_bytes = off * sizeof(T);
-  const size_t in_bytes = p.seg.in_blocked ? off_bytes : 0;
-  const int s = (p.start0 + (int)seg * p.start_stride) % P;
-  int j0, nj;
-  size_t out_bytes;
-  out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
-
-  const size_t head = HEAD ? p.seg.seg_head[seg] : 0;
-  const size_t vlen = len - head;
-  const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
-  const size_t vec_bytes = (vlen / N) * 16;
-  const size_t tb = ((size_t)p.seg.tile0 + blockIdx.x) * TL::BYTES;
-  if (tb < vec_bytes) {
-    const size_t rem = vec_bytes - tb;
-    const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
-    u32x4 acc[U];
-    if constexpr (PT > 0) {
-      u32x4 x[PT][U];
-      int idx = s;
-#pragma unroll
-      for (int k = 0; k < PT; ++k) {
-        const auto r = TL::rsrc(p.in[idx] + vin + tb, nrec);
-#pragma unroll
-        for (int u = 0; u < U; ++u) x[k][u] = tl.load(r, u);
-        idx = next_rank(idx, p.dir, PT);
-      }
-      // stream-major, the order the loads were issued in (they return in
-      // order): every accumulator advances as soon as a stream has arrived
-#pragma unroll
-      for (int u = 0; u < U; ++u) acc[u] = x[0][u];
-#pragma unroll
-      for (int k = 1; k < PT; ++k) {
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-          acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[k][u]) : step_vec<T, OP>(x[k][u], acc[u]);
-      }
-    } else {
-      constexpr int B = 4;  // streams in flight between uses
-      int idx = s;
-      {
-        const auto r = TL::rsrc(p.in[idx] + vin + tb, nrec);
-#pragma unroll
-        for (int u = 0; u < U; ++u) acc[u] = tl.load(r, u);
-      }
-      for (int k = 1; k < P; k += B) {
-        u32x4 x[B][U];
-        int id = idx;
-#pragma unroll
-        for (int b = 0; b < B; ++b) {
-          if (k + b < P) {
-            id = next_rank(id, p.dir, P);
-            const auto r = TL::rsrc(p.in[id] + vin + tb, nrec);
-#pragma unroll
-            for (int u = 0; u < U; ++u) x[b][u] = tl.load(r, u);
-          }
-        }
-#pragma unroll
-        for (int b = 0; b < B; ++b) {
-          if (k + b < P) {
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-              acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[b][u]) : step_vec<T, OP>(x[b][u], acc[u]);
-          }
-        }
-        idx = id;
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) acc[u] = finish_vec<T, OP>(acc[u], p.div);
-    for (int j = j0; j < j0 + nj; ++j) {
-      const auto r = TL::rsrc(p.out[j] + vout + tb, nrec);
-#pragma unroll
-      for (int u = 0; u < U; ++u) tl.store(r, u, acc[u]);
-    }
-  }
-  // the head elements and the vlen % N elements behind the last whole vector, one per thread of the
-  // segment's first workgroup
-  if (p.seg.tile0 == 0 && blockIdx.x == 0 && threadIdx.x < head + vlen % N) {
-    const size_t e = threadIdx.x < head ? threadIdx.x : (vlen / N) * N + threadIdx.x;
-    fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
-  }
-}
-
-
-}  // namespace
+int launch_fold_narrow(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op, bool roles,
+                       hipStream_t stream, const ChainScratch *chain, size_t displ_bytes);
+int launch_fold_wide(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op, bool roles,
+                     hipStream_t stream, const ChainScratch *chain, size_t displ_bytes);
 
 int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op, bool acc_is_in,
-                hipStream_t stream) {
+                hipStream_t stream, const ChainScratch *chain, size_t displ_bytes) {
   // operand roles only matter where a tie or a NaN can pick a side
   const bool roles = acc_is_in && is_float_dtype(dtype) && (op == ALAMD_MIN || op == ALAMD_MAX);
-  return dispatch_any(dtype, op, [&](auto tt, auto ot) -> int {
-    using T = typename decltype(tt)::type;
-    constexpr int OP = decltype(ot)::value;
-    constexpr bool FP_MINMAX = (std::is_same<T, float>::value || std::is_same<T, double>::value ||
-                                std::is_same<T, f16_t>::value || std::is_same<T, bf16_t>::value) &&
-                               (OP == ALAMD_MIN || OP == ALAMD_MAX);
-    const size_t tile_elems = Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES / sizeof(T);
-    FoldParams q = p;
-    q.div = make_divisor(p.P);
-    for (unsigned sg = 0; sg < nseg; ++sg) {
-      size_t off, len, out_bytes;
-      int j0, nj;
-      seg_range(p.seg, sg, off, len);
-      out_select(p.seg, p.P, sg, off * sizeof(T), j0, nj, out_bytes);
-      const int first = (p.start0 + (int)sg * p.start_stride) % p.P;
-      q.seg.seg_head[sg] = (unsigned char)head_count(sizeof(T), p.out[j0] + out_bytes,
-                                                     p.in[first] + (p.seg.in_blocked ? off * sizeof(T) : 0), len);
-      if (q.seg.seg_head[sg]) q.seg.any_head = 1;
-    }
-    auto pick = [&](auto acc_is_in_t, auto pt_t) -> void (*)(const FoldParams) {
-      constexpr bool A = decltype(acc_is_in_t)::value;
-      constexpr int PT = decltype(pt_t)::value;
-      return q.seg.any_head ? fold_vec_kernel<T, OP, A, PT, true> : fold_vec_kernel<T, OP, A, PT, false>;
-    };
-    using No = std::false_type;
-    using Yes = std::true_type;
-    using P8 = std::integral_constant<int, 8>;
-    using PN = std::integral_constant<int, 0>;
-    void (*kern)(const FoldParams) = nullptr;
-    if (p.P == 8) {
-      if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, P8{}) : pick(No{}, P8{});
-      else kern = pick(No{}, P8{});
-    } else {
-      if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, PN{}) : pick(No{}, PN{});
-      else kern = pick(No{}, PN{});
-    }
-    const size_t per_launch = launch_tiles(p.P, Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES);
-    plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
-      q.seg.tile0 = t0;
-      q.seg.seg0 = s0;
-      hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
-    });
-    ALAMD_HIP(hipGetLastError());
-    return ALAMD_OK;
-  });
+  switch (dtype) {
+  case ALAMD_I8: case ALAMD_U8: case ALAMD_I16: case ALAMD_U16:
+    return launch_fold_narrow(p, nseg, max_len, dtype, op, roles, stream, chain, displ_bytes);
+  case ALAMD_I32: case ALAMD_U32: case ALAMD_I64: case ALAMD_U64:
+    return launch_fold_wide(p, nseg, max_len, dtype, op, roles, stream, chain, displ_bytes);
+  default:
+    return group(p, nseg, max_len, dtype, op, roles, stream, chain, displ_bytes);
+  }
 }
-
 }  // namespace alamd

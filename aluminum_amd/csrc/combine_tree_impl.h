@@ -1,0 +1,278 @@
+// The tree kernels (included by the translation units that build them, one per
+// element type): balanced pairwise combine of up to 32 slots held in
+// registers (64 slots as two halves of 32).  Used for floating-point types under the TREE_* orders, where
+// the pairing decides the rounding; integer types never need it.
+#pragma once
+
+#include "alamd_dispatch.h"
+#include "alamd_tile.h"
+
+namespace alamd {
+
+namespace {
+
+// The tree over one element position, one element per access.  HALVES = 2: 2 * SLOTS slots, the
+// two halves reduced one after the other and combined by the tree's top level.
+template <typename T, int OP, int SLOTS, int HALVES>
+__device__ __forceinline__ T tree_elem_value(const TreeParams &p, size_t in_bytes, size_t e) {
+  T res;
+#pragma unroll
+  for (int h = 0; h < HALVES; ++h) {
+    const int base = h * SLOTS;
+    const int nvalid = p.nvalid - base;
+    if (h > 0 && nvalid <= 0) break;
+    T v[SLOTS];
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j)
+      if (j < nvalid) v[j] = ld_elem<T>(p.a[base + j] + in_bytes + e * sizeof(T));
+#pragma unroll
+    for (int j = 0; j < SLOTS; ++j)
+      if (j < nvalid && p.b[base + j] != nullptr)
+        v[j] = Step<T, OP>::apply(v[j], ld_elem<T>(p.b[base + j] + in_bytes + e * sizeof(T)));
+#pragma unroll
+    for (int d = 1; d < SLOTS; d *= 2) {
+#pragma unroll
+      for (int i = 0; i + d < SLOTS; i += 2 * d)
+        if (i + d < nvalid) v[i] = Step<T, OP>::apply(v[i + d], v[i]);
+    }
+    res = h == 0 ? v[0] : Step<T, OP>::apply(v[0], res);
+  }
+  return finish_elem<T, OP>(res, p.div);
+}
+template <typename T, int OP, int SLOTS, int HALVES>
+__device__ __forceinline__ void tree_elem(const TreeParams &p, size_t in_bytes, int j0, int nj,
+                                          size_t out_bytes, size_t e) {
+  const T res = tree_elem_value<T, OP, SLOTS, HALVES>(p, in_bytes, e);
+  for (int j = j0; j < j0 + nj; ++j) st_elem<T>(p.out[j] + out_bytes + e * sizeof(T), res);
+}
+
+// Kernel variants: every slot occupied and none pre-folded (P a power of two:
+// straight-line code, no uniform branches between the loads and their uses);
+// some slots empty (binomial order, P not a power of two); some slots
+// pre-folded from a second rank (doubling / halving orders, P not a power of
+// two), which needs room for up to twice as many loads in flight.
+enum { TREE_FULL = 0, TREE_PARTIAL = 1, TREE_PREFOLD = 2 };
+
+template <typename T, int OP, int SLOTS, int MODE> struct TreeShape {
+  static constexpr bool heavy = sizeof(T) <= 2;
+  static constexpr int budget = heavy ? 32 : 64;  // 128-bit loads in flight per lane
+  static constexpr int streams = MODE == TREE_PREFOLD ? 2 * SLOTS : SLOTS;
+  static constexpr int U = budget / streams >= 8 ? (heavy ? 4 : 8) : (budget / streams >= 1 ? budget / streams : 1);
+  static constexpr int THREADS = U == 8 ? 128 : 256;
+};
+
+__host__ __device__ inline void tree_out_select(const TreeParams &p, unsigned seg, size_t off_bytes,
+                                                size_t in_bytes, int &j0, int &nj, size_t &out_bytes) {
+  if (p.seg.out_mode == OUT_ALL) { j0 = 0; nj = p.seg.nout; out_bytes = in_bytes; }
+  else if (p.seg.out_mode == OUT_SEG) { j0 = (int)seg; nj = 1; out_bytes = 0; }
+  else { j0 = ((int)seg + p.seg.owner_shift) % p.P; nj = 1; out_bytes = off_bytes; }
+}
+
+// HEAD = false: no segment has leading elements to handle one by one (see the fold kernel).
+// HALVES = 2: 2 * SLOTS slots (33 to 64 ranks under the binomial order, 64 under the other two).  The
+// top level of a tree over 2 * SLOTS slots combines slot 0 with slot SLOTS, each the root of a tree
+// over SLOTS slots, so the two halves are loaded and reduced one after the other with the registers
+// of one.
+// CHAIN: the output overlaps one of the inputs at a displacement (see ChainParams and the fold kernel).
+template <typename T, int OP, int SLOTS, int MODE, bool HEAD, int HALVES, bool CHAIN = false>
+__global__ void __launch_bounds__((TreeShape<T, OP, SLOTS, MODE>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
+tree_vec_kernel(const TreeParams p) {
+  static_assert(!(CHAIN && HEAD), "a chained launch has no head");
+  constexpr int U = TreeShape<T, OP, SLOTS, MODE>::U, THREADS = TreeShape<T, OP, SLOTS, MODE>::THREADS;
+  constexpr int N = 16 / sizeof(T);
+  static_assert(HALVES == 1 || MODE != TREE_PREFOLD, "a pre-fold never meets more than 32 slots");
+  using TL = Tile<U, THREADS>;
+  const TL tl;
+  const unsigned seg = seg_of(p.seg, blockIdx.y + p.seg.seg0);
+  size_t off, len;
+  seg_range(p.seg, seg, off, len);
+  const size_t off_bytes = off * sizeof(T);
+  const size_t in_bytes = p.seg.in_blocked ? off_bytes : 0;
+  int j0, nj;
+  size_t out_bytes;
+  tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
+
+  const size_t head = HEAD ? p.seg.seg_head[seg] : 0;
+  const size_t vlen = len - head;
+  const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
+  const size_t vec_bytes = (vlen / N) * 16;
+  unsigned bx = blockIdx.x;
+  if constexpr (CHAIN) bx = chain_take_tile(p.chain);
+  const size_t tb = ((size_t)p.seg.tile0 + bx) * TL::BYTES;
+  if (tb < vec_bytes) {
+    const size_t rem = vec_bytes - tb;
+    const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
+    u32x4 res[U];
+#pragma unroll
+    for (int h = 0; h < HALVES; ++h) {
+      const int base = h * SLOTS;
+      const int nvalid = MODE == TREE_FULL ? SLOTS : p.nvalid - base;
+      if (h > 0 && nvalid <= 0) break;
+      u32x4 v[SLOTS][U];
+#pragma unroll
+      for (int j = 0; j < SLOTS; ++j) {
+        if (j < nvalid) {
+          const auto r = TL::rsrc(p.a[base + j] + vin + tb, nrec);
+#pragma unroll
+          for (int u = 0; u < U; ++u) v[j][u] = tl.load(r, u);
+        }
+      }
+      if constexpr (MODE == TREE_PREFOLD) {
+        // pre-folded slots: the odd rank keeps step(in = even rank, inout = odd rank); all of
+        // their loads are issued before the first use, like the slots' own
+        u32x4 w[SLOTS][U];
+#pragma unroll
+        for (int j = 0; j < SLOTS; ++j) {
+          if (j < nvalid && p.b[j] != nullptr) {
+            const auto r = TL::rsrc(p.b[j] + vin + tb, nrec);
+#pragma unroll
+            for (int u = 0; u < U; ++u) w[j][u] = tl.load(r, u);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < SLOTS; ++j) {
+          if (j < nvalid && p.b[j] != nullptr) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[j][u] = step_vec<T, OP>(v[j][u], w[j][u]);
+          }
+        }
+      }
+#pragma unroll
+      for (int d = 1; d < SLOTS; d *= 2) {
+#pragma unroll
+        for (int i = 0; i + d < SLOTS; i += 2 * d) {
+          if (i + d < nvalid) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[i][u] = step_vec<T, OP>(v[i + d][u], v[i][u]);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) res[u] = h == 0 ? v[0][u] : step_vec<T, OP>(v[0][u], res[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) res[u] = finish_vec<T, OP>(res[u], p.div);
+    if constexpr (CHAIN) chain_gate(p.chain, bx, tb, (unsigned long long)nrec, (unsigned)TL::BYTES);
+    for (int j = j0; j < j0 + nj; ++j) {
+      const auto r = TL::rsrc(p.out[j] + vout + tb, nrec);
+#pragma unroll
+      for (int u = 0; u < U; ++u) tl.store(r, u, res[u]);
+    }
+  }
+  if constexpr (CHAIN) {
+    // the vlen % N elements behind the last whole vector are the last ticket
+    if (bx == p.chain.nvec_tiles) {
+      const bool mine = threadIdx.x < vlen % N;
+      const size_t e = (vlen / N) * N + threadIdx.x;
+      T val = T();
+      if (mine) val = tree_elem_value<T, OP, SLOTS, HALVES>(p, in_bytes, e);
+      chain_gate(p.chain, bx, vec_bytes, (vlen % N) * sizeof(T), (unsigned)TL::BYTES);
+      if (mine) st_elem<T>(p.out[j0] + out_bytes + e * sizeof(T), val);
+    }
+  } else {
+    // the head elements and the vlen % N elements behind the last whole vector
+    if (p.seg.tile0 == 0 && blockIdx.x == 0 && threadIdx.x < head + vlen % N) {
+      const size_t e = threadIdx.x < head ? threadIdx.x : (vlen / N) * N + threadIdx.x;
+      tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e);
+    }
+  }
+}
+
+
+struct ChainArgs { const ChainScratch *scratch; size_t displ_bytes; };
+
+template <typename T, int OP, int SLOTS, int MODE, int HALVES = 1>
+int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream, ChainArgs chain) {
+  using S = TreeShape<T, OP, SLOTS, MODE>;
+  const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
+  const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES);
+  TreeParams q = p;
+  q.div = make_divisor(p.P);
+  q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0};
+  if (chain.scratch) {
+    if (nseg != 1) return set_error(ALAMD_ERR_INVALID_ARG, "a chained combine has one segment");
+    constexpr size_t N = 16 / sizeof(T);
+    const size_t tile_bytes = Tile<S::U, S::THREADS>::BYTES;
+    const size_t nvec = (max_len / N * 16 + tile_bytes - 1) / tile_bytes;
+    const size_t tickets = nvec + (max_len % N ? 1 : 0);
+    if (nvec > chain.scratch->max_tiles || tickets > 0x7fffffffull)
+      return set_error(ALAMD_ERR_INVALID_ARG, "in-place block of %zu elements needs %zu tile flags, the scratch holds %zu",
+                       max_len, nvec, chain.scratch->max_tiles);
+    int rc = chain_clear(*chain.scratch, nvec, stream);
+    if (rc) return rc;
+    q.chain = ChainParams{chain.scratch->ticket, chain.scratch->flags, chain.scratch->error, chain.displ_bytes,
+                          (unsigned)nvec};
+    q.seg.tile0 = 0;
+    q.seg.seg0 = 0;
+    q.seg.mapped = 0;
+    // only the most general variants are built for chained launches
+    if constexpr (MODE == TREE_PREFOLD || (HALVES == 2 && MODE == TREE_PARTIAL)) {
+      hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE, false, HALVES, true>), dim3((unsigned)tickets, 1, 1),
+                         dim3(S::THREADS, 1, 1), 0, stream, q);
+      ALAMD_HIP(hipGetLastError());
+      return ALAMD_OK;
+    } else {
+      return set_error(ALAMD_ERR_INVALID_ARG, "tree combine: no chained variant of this mode");
+    }
+  }
+  for (unsigned sg = 0; sg < nseg; ++sg) {
+    size_t off, len, out_bytes;
+    int j0, nj;
+    seg_range(p.seg, sg, off, len);
+    const size_t in_bytes = p.seg.in_blocked ? off * sizeof(T) : 0;
+    tree_out_select(p, sg, off * sizeof(T), in_bytes, j0, nj, out_bytes);
+    q.seg.seg_head[sg] = (unsigned char)head_count(sizeof(T), p.out[j0] + out_bytes, p.a[0] + in_bytes, len);
+    if (q.seg.seg_head[sg]) q.seg.any_head = 1;
+  }
+  void (*kern)(const TreeParams) =
+      q.seg.any_head ? tree_vec_kernel<T, OP, SLOTS, MODE, true, HALVES> : tree_vec_kernel<T, OP, SLOTS, MODE, false, HALVES>;
+  plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
+    q.seg.tile0 = t0;
+    q.seg.seg0 = s0;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(S::THREADS, 1, 1), 0, stream, q);
+  });
+  ALAMD_HIP(hipGetLastError());
+  return ALAMD_OK;
+}
+
+template <typename T, int OP, int SLOTS>
+int launch_tree_slots(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream, ChainArgs chain) {
+  bool prefold = false;
+  for (int j = 0; j < SLOTS; ++j) prefold = prefold || p.b[j] != nullptr;
+  // a chained launch takes the most general variant whatever the slots hold: fewer kernels to build
+  if (prefold || chain.scratch) return launch_tree_mode<T, OP, SLOTS, TREE_PREFOLD>(p, nseg, max_len, stream, chain);
+  if (p.nvalid == SLOTS) return launch_tree_mode<T, OP, SLOTS, TREE_FULL>(p, nseg, max_len, stream, chain);
+  return launch_tree_mode<T, OP, SLOTS, TREE_PARTIAL>(p, nseg, max_len, stream, chain);
+}
+
+// 33 to 64 slots: two halves of 32.
+template <typename T, int OP>
+int launch_tree_two_halves(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream, ChainArgs chain) {
+  for (int j = 0; j < 64; ++j)
+    if (p.b[j] != nullptr) return set_error(ALAMD_ERR_INVALID_ARG, "tree combine: pre-fold beyond 32 slots");
+  if (p.nvalid == 64 && !chain.scratch) return launch_tree_mode<T, OP, 32, TREE_FULL, 2>(p, nseg, max_len, stream, chain);
+  return launch_tree_mode<T, OP, 32, TREE_PARTIAL, 2>(p, nseg, max_len, stream, chain);
+}
+
+// The launches of one element type.
+template <typename T>
+int launch_tree_of(const TreeParams &p, int slots, unsigned nseg, size_t max_len, int op, hipStream_t stream,
+                   const ChainScratch *scratch, size_t displ_bytes) {
+  const ChainArgs chain = {scratch, displ_bytes};
+  return dispatch_fp_op<T>(op, [&](auto tt, auto ot) -> int {
+    using TT = typename decltype(tt)::type;
+    constexpr int OP = decltype(ot)::value;
+    switch (slots) {
+    case 2: return launch_tree_slots<TT, OP, 2>(p, nseg, max_len, stream, chain);
+    case 4: return launch_tree_slots<TT, OP, 4>(p, nseg, max_len, stream, chain);
+    case 8: return launch_tree_slots<TT, OP, 8>(p, nseg, max_len, stream, chain);
+    case 16: return launch_tree_slots<TT, OP, 16>(p, nseg, max_len, stream, chain);
+    case 32: return launch_tree_slots<TT, OP, 32>(p, nseg, max_len, stream, chain);
+    case 64: return launch_tree_two_halves<TT, OP>(p, nseg, max_len, stream, chain);
+    default: return set_error(ALAMD_ERR_INVALID_ARG, "tree combine: bad slot count %d", slots);
+    }
+  });
+}
+
+}  // namespace
+}  // namespace alamd

@@ -268,6 +268,41 @@ def test_reduce_scatterv(al, dtype, order):
                               "in-place reduce_scatterv %s P=%d rank %d" % (order, P, b))
 
 
+@pytest.mark.parametrize("dtype,order", [("f32", "rank_asc"), ("f32", "tree_halv"), ("bf16", "pairwise_desc"),
+                                         ("f64", "tree_dbl"), ("f16", "tree_binomial"), ("u8", "rank_asc"),
+                                         ("i64", "rank_asc"), ("f32", "ring")])
+def test_reduce_scatterv_in_place_block_overlapping_its_own_input(al, dtype, order):
+    """In place, a block that starts fewer elements into its own buffer than it is long is read and
+    overwritten by the same launch at a displacement (any counts are legal:
+    include/aluminum/ht/reduce_scatterv.hpp:40-87).  Displacements of one element, of less than a tile,
+    of several tiles and a half; lengths with and without a tail; everything behind a rank's result
+    stays as it was."""
+    import torch
+    shapes = [(3, [1, 1_000_003, 5]), (2, [1, 10_000_000]), (4, [3, 200_001, 17, 70_000]),
+              (5, [4097, 9 * 4096 + 5, 0, 150_000, 31]), (3, [100_000, 150_000, 400_000]),
+              (2, [16, 1 << 20]), (6, [7, 7, 7, 300_000, 1, 2_000_000])]
+    if order in ("tree_halv", "tree_dbl", "tree_binomial"):
+        shapes.append((40, [2] + [50_000 + 13 * k for k in range(39)]))
+    for P, counts in shapes:
+        total = sum(counts)
+        sends = make_inputs(P, total, dtype, "sum")
+        want = oracle.reduce_scatterv(sends, counts, dtype, "sum", order)
+        bufs = [to_dev(a) for a in sends]
+        al.reduce_scatterv(bufs, bufs, counts, "sum", order=order, dtype=dtype)
+        torch.cuda.synchronize()
+        for b in range(P):
+            got = to_host(bufs[b], sends[0].dtype)
+            assert_bits_equal(got[:counts[b]], want[b], dtype, "in place %s %s counts %s rank %d" % (dtype, order, counts[:4], b))
+            assert got[counts[b]:].tobytes() == sends[b][counts[b]:].tobytes(), "rank %d: bytes behind the result changed" % b
+        # some ranks in place, the others not
+        bufs = [to_dev(a) for a in sends]
+        recvs = [bufs[b] if b % 2 else dev_empty(max(counts[b], 1), sends[0].dtype) for b in range(P)]
+        al.reduce_scatterv(recvs, bufs, counts, "sum", order=order, dtype=dtype)
+        torch.cuda.synchronize()
+        for b in range(P):
+            assert_bits_equal(to_host(recvs[b], sends[0].dtype)[:counts[b]], want[b], dtype, "mixed in place rank %d" % b)
+
+
 @pytest.mark.parametrize("dtype", ("u8", "i16", "f32", "f64"))
 def test_allgatherv(al, dtype):
     import torch
