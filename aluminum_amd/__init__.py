@@ -11,7 +11,8 @@ is present, calls raise.
 from . import capi  # noqa: F401
 from .capi import (  # noqa: F401
     AlError, DTYPES, OPS, ORDERS, DISTS, RING_MODES, FLAG_MODES,
-    load, lib_path, combine, reduce_scatter, allgather, reduce_scatterv, allgatherv, ring_allreduce,
+    load, lib_path, combine, reduce_scatter, allgather, reduce_scatterv, reduce_scatterv_noalloc, allgatherv,
+    ring_allreduce,
     ring_reduce_scatter, ring_allgather, halo_pack, halo_unpack, halo_face_elems,
     fill, narrow_f32, widen_f32, copy, Flag, torch_dtype, dtype_size, check_op,
 )

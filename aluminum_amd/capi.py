@@ -62,6 +62,7 @@ def load():
     L.alamd_reduce_scatter.argtypes = [pvp, pvp, i, sz, i, i, i, vp]
     L.alamd_allgather.argtypes = [pvp, pvp, i, sz, i, vp]
     L.alamd_reduce_scatterv.argtypes = [pvp, pvp, i, C.POINTER(sz), i, i, i, vp]
+    L.alamd_reduce_scatterv_noalloc.argtypes = [pvp, pvp, i, C.POINTER(sz), i, i, i, vp]
     L.alamd_allgatherv.argtypes = [pvp, pvp, i, C.POINTER(sz), C.POINTER(sz), i, vp]
     L.alamd_ring_allreduce.argtypes = [pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_reduce_scatter.argtypes = [pvp, i, sz, i, i, sz, i, vp]
@@ -183,6 +184,14 @@ def reduce_scatterv(recvs, sends, counts, op, order="rank_asc", dtype=None, stre
     P = len(sends)
     _check(load().alamd_reduce_scatterv(_table(recvs), _table(sends), P, (C.c_size_t * P)(*counts), _dt(dtype),
                                         _op(op), _order(order), _stream(stream)))
+
+
+def reduce_scatterv_noalloc(recvs, sends, counts, op, order="rank_asc", dtype=None, stream=None):
+    """alamd_reduce_scatterv_noalloc: the same call with its scratch in a fixed device array."""
+    dtype = dtype or _infer_dtype(sends[0])
+    P = len(sends)
+    _check(load().alamd_reduce_scatterv_noalloc(_table(recvs), _table(sends), P, (C.c_size_t * P)(*counts),
+                                                _dt(dtype), _op(op), _order(order), _stream(stream)))
 
 
 def allgatherv(recvs, sends, counts, displs, dtype=None, stream=None):

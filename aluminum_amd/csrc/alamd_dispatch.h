@@ -308,6 +308,9 @@ int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, i
 // Clears the ticket counter, the error word and the first `tiles` flags on `stream` (a kernel, not a
 // memset, so that the call may be captured into a graph).
 int chain_clear(const ChainScratch &cs, size_t tiles, hipStream_t stream);
+// Looks up, for the current device, the address of the scratch array that
+// alamd_reduce_scatterv_noalloc uses (once per device).
+int chain_static_init();
 
 // A result that goes to several buffers is folded into one of them and then
 // spread (one write stream per workgroup) when that is faster than writing

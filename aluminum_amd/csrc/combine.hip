@@ -155,6 +155,32 @@ int chain_scratch_for(hipStream_t stream, size_t tiles, ChainScratch &out) {
   return ALAMD_OK;
 }
 
+// The scratch of alamd_reduce_scatterv_noalloc: part of the code object, so every device the library
+// runs on holds its own copy at its own address until the process ends.  In host code the array's
+// name is only a handle for hipGetSymbolAddress; the address it yields for the current device is what
+// kernels and the clearing launch are given.
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[ALAMD_NOALLOC_SCRATCH_BYTES];
+namespace {
+
+std::mutex g_static_mutex;
+unsigned char *g_static_ptr[64];
+
+int static_chain_scratch(ChainScratch &out) {
+  int dev = 0;
+  ALAMD_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return set_error(ALAMD_ERR_HIP, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (!g_static_ptr[dev]) {
+    unsigned char *ptr = nullptr;
+    ALAMD_HIP(hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)));
+    if (!ptr) return set_error(ALAMD_ERR_HIP, "hipGetSymbolAddress returned a null address");
+    g_static_ptr[dev] = ptr;
+  }
+  out = scratch_at(g_static_ptr[dev], ALAMD_NOALLOC_SCRATCH_BYTES);
+  return ALAMD_OK;
+}
+
 constexpr int kGatherU = 8, kGatherThreads = 128;
 
 // Slices to several destinations: the seg_len[q] bytes of source q go to byte
@@ -249,6 +275,11 @@ int check_common(int P, size_t count, int dtype) {
 }
 
 }  // namespace
+
+int chain_static_init() {
+  ChainScratch cs;
+  return static_chain_scratch(cs);
+}
 
 int chain_clear(const ChainScratch &cs, size_t tiles, hipStream_t stream) {
   if (tiles > cs.max_tiles) return set_error(ALAMD_ERR_INVALID_ARG, "chain scratch too small");
@@ -592,8 +623,8 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
   return launch_gather(recvs, sends, P, offs, lens, as_stream(stream));
 }
 
-int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, const size_t *counts, int dtype,
-                          int op, int order, void *stream) {
+static int reduce_scatterv_impl(void *const *recvs, const void *const *sends, int P, const size_t *counts,
+                               int dtype, int op, int order, void *stream, const ChainScratch *fixed) {
   int rc = check_common(P, 0, dtype);
   if (rc) return rc;
   if ((rc = check_type_op(dtype, op))) return rc;
@@ -648,7 +679,20 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, c
     lay.start_stride = order_has_start(order) ? 1 : 0;
     return launch_order(out_tab, sends, P, lay, dtype, op, order, as_stream(stream));
   }
-  return reduce_scatterv_in_place(recvs, sends, P, counts, displ, dtype, op, order, as_stream(stream), nullptr);
+  return reduce_scatterv_in_place(recvs, sends, P, counts, displ, dtype, op, order, as_stream(stream), fixed);
+}
+
+int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, const size_t *counts, int dtype,
+                          int op, int order, void *stream) {
+  return reduce_scatterv_impl(recvs, sends, P, counts, dtype, op, order, stream, nullptr);
+}
+
+int alamd_reduce_scatterv_noalloc(void *const *recvs, const void *const *sends, int P, const size_t *counts,
+                                  int dtype, int op, int order, void *stream) {
+  ChainScratch cs;
+  const int rc = static_chain_scratch(cs);
+  if (rc) return rc;
+  return reduce_scatterv_impl(recvs, sends, P, counts, dtype, op, order, stream, &cs);
 }
 
 int alamd_allgatherv(void *const *recvs, const void *const *sends, int P, const size_t *counts,

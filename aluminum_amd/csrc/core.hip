@@ -8,6 +8,8 @@
 
 namespace alamd {
 
+int chain_static_init();  // combine.hip
+
 namespace {
 thread_local char g_err[512] = "";
 std::mutex g_dev_mutex;
@@ -94,7 +96,8 @@ int alamd_init(void) {
   if (std::string(prop.gcnArchName).rfind("gfx950", 0) != 0)
     return alamd::set_error(ALAMD_ERR_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only",
                             dev, prop.gcnArchName);
-  return alamd::device_cus() > 0 ? ALAMD_OK : ALAMD_ERR_HIP;
+  if (alamd::device_cus() <= 0) return ALAMD_ERR_HIP;
+  return alamd::chain_static_init();
 }
 
 }  // extern "C"

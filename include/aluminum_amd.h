@@ -155,11 +155,36 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P,
  * counts[b] elements, the fold of elements [displ_b, displ_b + counts[b]) of
  * every sends[r], displ_b = counts[0] + ... + counts[b-1], with start = b for
  * the orders that have one.  In-place form (recvs[b] == sends[b]) puts the
- * result at the start of the buffer.  Replaces MPI_Ireduce_scatter on the
- * host copy (include/aluminum/ht/reduce_scatterv.hpp:40-87). */
+ * result at the start of the buffer; any counts are accepted, as by the
+ * reference.  A block that is in place and starts fewer elements into its own
+ * buffer than it is long is read and overwritten at a displacement: in up to
+ * 32 launches no longer than the displacement, else in one launch whose
+ * workgroups order themselves through a ticket counter and one flag per tile
+ * in device scratch memory (allocated per stream on first need and kept).
+ * Replaces MPI_Ireduce_scatter on the host copy
+ * (include/aluminum/ht/reduce_scatterv.hpp:40-87). */
 int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P,
                           const size_t *counts, int dtype, int op, int order,
                           void *stream);
+
+/* alamd_reduce_scatterv for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  Same arguments, same
+ * results, and no hipMalloc, hipFree or other allocating call is made: the
+ * ticket counter and tile flags that an in-place block needs when it overlaps
+ * its own input (see alamd_reduce_scatterv) live in a fixed array of
+ * ALAMD_NOALLOC_SCRATCH_BYTES that is part of the library's code object (every
+ * device the library runs on holds its copy until the process ends).  Limit:
+ * such a block may be at most ALAMD_NOALLOC_MAX_BLOCK_BYTES long
+ * (ALAMD_ERR_INVALID_ARG beyond that; blocks that do not overlap their own
+ * input, and separate receive buffers, have no limit).  All calls on one device
+ * share the array: calls that overlap in time on one device (different
+ * streams, different threads) race; keep them on one stream. */
+#define ALAMD_NOALLOC_SCRATCH_BYTES ((size_t)1 << 20)
+#define ALAMD_NOALLOC_MAX_BLOCK_BYTES (((ALAMD_NOALLOC_SCRATCH_BYTES - 256) / 4) * 4096)
+int alamd_reduce_scatterv_noalloc(void *const *recvs, const void *const *sends, int P,
+                                  const size_t *counts, int dtype, int op, int order,
+                                  void *stream);
 
 /* Allgatherv: recvs[r][displs[q] + i] = sends[q][i], i < counts[q].
  * In-place form: sends[q] == recvs[q] + displs[q] elements

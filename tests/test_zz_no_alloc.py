@@ -1,0 +1,64 @@
+"""alamd_reduce_scatterv_noalloc against alamd_reduce_scatterv, through the C ABI: the same bits,
+on two calls in a row (the second smaller, so what the first left in the fixed scratch array must
+not matter), also after other work has used the device; the stated limit is an error."""
+import numpy as np
+import pytest
+
+import oracle
+from util import assert_bits_equal, dev_empty, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+# (P, counts): in-place blocks that overlap their own input at a small displacement (one chained
+# launch each), at a displacement of a few runs, and blocks that do not overlap at all
+SHAPES = [(3, [1, 3_000_017, 5]), (2, [1, 40_003]), (4, [3, 900_001, 0, 20_000]), (3, [70_000, 100_000, 9]),
+          (2, [64, 64])]
+
+
+def both_ways(al, P, counts, dtype, op, order, seed):
+    import torch
+    total = sum(counts)
+    dist = "fullrange" if dtype[0] in "iu" else "uniform_pm1"
+    sends = [oracle.fill(total, dtype, dist, seed + r) for r in range(P)]
+    np_dt = sends[0].dtype
+    ref = [to_dev(a) for a in sends]
+    al.reduce_scatterv(ref, ref, counts, op, order=order, dtype=dtype)
+    got = [to_dev(a) for a in sends]
+    al.reduce_scatterv_noalloc(got, got, counts, op, order=order, dtype=dtype)
+    torch.cuda.synchronize()
+    want = oracle.reduce_scatterv(sends, counts, dtype, op, order)
+    for b in range(P):
+        g, r = to_host(got[b], np_dt), to_host(ref[b], np_dt)
+        assert_bits_equal(g[:counts[b]], r[:counts[b]], dtype, "noalloc vs alamd_reduce_scatterv, rank %d" % b)
+        assert_bits_equal(g[:counts[b]], want[b], dtype, "noalloc vs oracle, rank %d" % b)
+        assert g[counts[b]:].tobytes() == sends[b][counts[b]:].tobytes(), "bytes behind the result changed"
+    # separate receive buffers take no scratch at all
+    recvs = [dev_empty(max(c, 1), np_dt) for c in counts]
+    al.reduce_scatterv_noalloc(recvs, [to_dev(a) for a in sends], counts, op, order=order, dtype=dtype)
+    torch.cuda.synchronize()
+    for b in range(P):
+        assert_bits_equal(to_host(recvs[b], np_dt)[:counts[b]], want[b], dtype, "noalloc, separate buffers, rank %d" % b)
+
+
+@pytest.mark.parametrize("dtype,op,order", [("f32", "sum", "rank_asc"), ("bf16", "sum", "tree_halv"),
+                                            ("i16", "max", "rank_asc"), ("f64", "avg", "pairwise_desc")])
+def test_noalloc_two_calls_in_a_row(al, dtype, op, order):
+    for k, (P, counts) in enumerate(SHAPES):  # every call after the first is smaller or of another shape
+        both_ways(al, P, counts, dtype, op, order, 500 + 10 * k)
+
+
+def test_noalloc_limit_is_an_error(al):
+    import torch
+    # an in-place block that overlaps its own input and is longer than the fixed array covers
+    limit = ((1 << 20) - 256) // 4 * 4096
+    counts = [1, limit + 4096]
+    bufs = [torch.zeros(sum(counts), dtype=torch.uint8, device="cuda") for _ in range(2)]
+    with pytest.raises(al.AlError, match="beyond the .* bytes the fixed scratch covers") as e:
+        al.reduce_scatterv_noalloc(bufs, bufs, counts, "bor", dtype="u8")
+    assert e.value.code == 1
+    torch.cuda.synchronize()
+    # the same block through separate receive buffers has no limit
+    recvs = [torch.zeros(c, dtype=torch.uint8, device="cuda") for c in counts]
+    al.reduce_scatterv_noalloc(recvs, bufs, counts, "bor", dtype="u8")
+    torch.cuda.synchronize()
+    assert int(recvs[1].max()) == 0
