@@ -15,9 +15,23 @@
  * One GPU holds all P logical ranks.  A `World` owns the P communicators; a
  * collective is launched when the last of the P logical ranks has made its
  * call (calls may come from one thread in any rank order, or from P threads).
- * Every call only enqueues work and returns; results are stream-ordered on
- * the communicator's stream (docs/index.rst:33-40).  Errors are thrown as
- * Al::al_exception from the calling thread.
+ * Every call only enqueues work and returns (docs/index.rst:33-40).  Errors
+ * are thrown as Al::al_exception from the calling thread.
+ *
+ * Stream order.  The collective starts after everything that was enqueued on
+ * rank r's stream before rank r's call (the dependency is taken at the call),
+ * and everything enqueued on a rank's stream after the LAST of the P calls
+ * runs after the collective.  Work enqueued on a rank's stream between that
+ * rank's call and the last call is not ordered against the collective: it
+ * must not write the rank's send buffer or touch its receive buffer.  With P
+ * processes that window does not exist; with P logical ranks in one process
+ * it does, because the combine cannot be enqueued before every contribution
+ * is known, and a stream cannot be made to wait for work that is enqueued
+ * later without risking a deadlock on a shared hardware queue.  Callers that
+ * drive the ranks from P threads can close the window with
+ * World::set_calls_wait_for_launch(true): a call then returns when the
+ * collective has been launched, so whatever the thread enqueues next is
+ * ordered behind it.
  *
  * Needs the HIP host API (hip/hip_runtime_api.h) and libaluminum_amd.so.
  */
@@ -231,6 +245,7 @@ struct OpCompletion {
 struct Request {
   std::shared_ptr<OpCompletion> done;
   hipStream_t orig_stream = nullptr;
+  std::string error;  // set when the launch of the operation failed: Test and Wait rethrow it
 };
 
 enum class OpKind { allreduce, reduce, reduce_scatter, allgather, reduce_scatterv, allgatherv };
@@ -241,6 +256,8 @@ struct Posting {
   void *recv = nullptr;
   hipStream_t stream = nullptr;
   std::shared_ptr<Request> req;  // non-blocking: the caller's request, completed at launch
+  hipEvent_t ready = nullptr;    // recorded on `stream` at the call, unless an earlier rank of this
+                                 // operation has the same stream (then that rank's event stands for both)
   bool posted = false;
 };
 
@@ -256,6 +273,8 @@ struct PendingOp {
   int nposted = 0;
   std::vector<size_t> counts, displs;  // the *v collectives
   std::vector<Posting> ranks;
+  bool launched = false;  // set (with `failure` on error) when the last rank has called
+  std::string failure;
 };
 
 /** Non-blocking operations up to this many bytes per rank run on the caller's stream: their
@@ -280,6 +299,8 @@ class World {
     events_ = std::make_shared<EventPool>();
   }
   ~World() {
+    for (Mail &m : mail_)
+      for (hipEvent_t e : m.notified) events_->give(e);
     (void)hipStreamSynchronize(internal_stream_);
     (void)hipEventDestroy(sync_event_);
     (void)hipStreamDestroy(internal_stream_);
@@ -290,6 +311,26 @@ class World {
   int size() const { return static_cast<int>(comms_.size()); }
   Communicator &comm(int r) { return *comms_.at(static_cast<size_t>(r)); }
 
+  /** For callers that drive the logical ranks from P threads: a collective call returns only when
+   *  the collective has been launched (when all P ranks have called), so that work the thread enqueues
+   *  next on its stream is ordered behind it.  Must stay off when one thread makes the calls of several
+   *  ranks: the first call would wait for ever. */
+  void set_calls_wait_for_launch(bool on) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    calls_wait_ = on;
+  }
+
+  /* ---- one-sided extension between logical ranks (include/aluminum/mpi_cuda/rma_self.hpp:37-71 for
+   *      a rank and itself; rma_ipc.hpp:152-328 between ranks, whose handle exchange and notification
+   *      messages become a table and events here, because every rank lives in this address space) ---- */
+
+  /** Deposits `mine` for `peer` and returns what `peer` deposited for `me`. */
+  void *attach(int me, int peer, void *mine);
+  /** `me`'s stream has reached this point: the next rma_wait(peer, me) is ordered behind it. */
+  void rma_notify(int me, int peer);
+  /** Orders `me`'s stream behind the matching rma_notify of `peer`. */
+  void rma_wait(int me, int peer);
+
   /** Registers rank's part of its next collective; launches every collective
    *  that has all P parts, in order. */
   void post(Communicator &c, OpKind kind, int dtype, const void *send, void *recv, size_t count,
@@ -298,37 +339,86 @@ class World {
 
  private:
   void launch(PendingOp &p);
+  /** The stream an operation runs on: blocking operations on rank 0's stream, non-blocking ones on
+   *  the internal stream between the two synchronisations of ht_impl.hpp:866-888 - unless they are
+   *  small: moving to another stream and back costs about 20 us of event calls, more than a kernel
+   *  of a few microseconds could ever overlap with, so those run on rank 0's stream as well and only
+   *  leave a completion event behind. */
+  hipStream_t target_of(bool nonblocking, int dtype, size_t count, const std::vector<size_t> &counts) {
+    size_t per_rank = count;
+    for (size_t c : counts) per_rank += c;
+    const bool on_internal = nonblocking && per_rank * alamd_dtype_size(dtype) > kInlineNonblockingBytes;
+    return on_internal ? internal_stream_ : comms_[0]->get_stream();
+  }
   hipStream_t gather_streams(PendingOp &p, hipStream_t target);
   void release_streams(PendingOp &p, hipStream_t ran_on);
 
   std::vector<std::unique_ptr<Communicator>> comms_;
-  std::deque<PendingOp> pending_;
+  std::deque<std::shared_ptr<PendingOp>> pending_;
   std::mutex mutex_;
+  std::condition_variable launched_cv_;
+  bool calls_wait_ = false;
+  struct Mail {
+    std::deque<hipEvent_t> notified;  // recorded by the sender, not yet waited for
+    int waiting = 0;                  // waits the receiver made before the sender notified
+    std::deque<void *> attached;      // buffers the sender has deposited for the receiver
+  };
+  std::vector<Mail> mail_;  // [from * P + to]
+  Mail &mail(int from, int to) {
+    if (mail_.empty()) mail_.resize(comms_.size() * comms_.size());
+    return mail_[static_cast<size_t>(from) * comms_.size() + static_cast<size_t>(to)];
+  }
+  void check_peer(int peer) const {
+    if (peer < 0 || peer >= size()) AL_AMD_THROW("Invalid peer rank");
+  }
   hipStream_t internal_stream_ = nullptr;
+  hipStream_t last_target_ = nullptr;  // where the latest operation ran
+  bool any_launched_ = false;
   hipEvent_t sync_event_ = nullptr;
   std::shared_ptr<EventPool> events_;
 };
 
 struct Poster {
+  static uint64_t peek_seq(const Communicator &c) { return c.next_seq_; }
   static uint64_t take_seq(Communicator &c) { return c.next_seq_++; }
 };
 
 inline void World::post(Communicator &c, OpKind kind, int dtype, const void *send, void *recv, size_t count,
                         ReductionOperator op, CombineAlgorithm algo, int root, std::shared_ptr<Request> *req,
                         const std::vector<size_t> *counts, const std::vector<size_t> *displs) {
-  std::lock_guard<std::mutex> lock(mutex_);
+  std::unique_lock<std::mutex> lock(mutex_);
   const int P = size();
   static const std::vector<size_t> none;
   const std::vector<size_t> &cv = counts ? *counts : none, &dv = displs ? *displs : none;
   if ((counts && cv.size() != static_cast<size_t>(P)) || (displs && dv.size() != static_cast<size_t>(P)))
     AL_AMD_THROW("Vector of counts or displacements is not communicator-sized");
-  const uint64_t seq = Poster::take_seq(c);
-  PendingOp *slot = nullptr;
+  // Every check comes before the rank's sequence number is taken: a call that throws leaves the
+  // communicator where it was, and the operations behind it are not held up.
+  const uint64_t seq = Poster::peek_seq(c);
+  std::shared_ptr<PendingOp> slot;
   for (auto &p : pending_)
-    if (p.seq == seq) slot = &p;
+    if (p->seq == seq) slot = p;
+  if (slot && (slot->kind != kind || slot->dtype != dtype || slot->count != count || slot->op != op ||
+               slot->algo != algo || slot->root != root || slot->nonblocking != (req != nullptr) ||
+               slot->counts != cv || slot->displs != dv))
+    AL_AMD_THROW("Logical ranks disagree on the arguments of a collective");
+  // The dependency on the rank's stream is taken now, not when the last rank calls: the collective
+  // waits for what was enqueued before this call, and for nothing that is enqueued after it.
+  hipEvent_t ready = nullptr;
+  bool shared = false;
+  if (slot)
+    for (const Posting &other : slot->ranks) shared = shared || (other.posted && other.stream == c.get_stream());
+  if (!shared && c.get_stream() != target_of(req != nullptr, dtype, count, cv)) {
+    ready = events_->take();
+    const hipError_t e = hipEventRecord(ready, c.get_stream());
+    if (e != hipSuccess) {
+      events_->give(ready);
+      AL_AMD_THROW(std::string("GPU error: ") + hipGetErrorString(e));
+    }
+  }
   if (!slot) {
-    pending_.emplace_back();
-    slot = &pending_.back();
+    slot = std::make_shared<PendingOp>();
+    pending_.push_back(slot);
     slot->seq = seq;
     slot->kind = kind;
     slot->dtype = dtype;
@@ -340,15 +430,13 @@ inline void World::post(Communicator &c, OpKind kind, int dtype, const void *sen
     slot->counts = cv;
     slot->displs = dv;
     slot->ranks.resize(static_cast<size_t>(P));
-  } else if (slot->kind != kind || slot->dtype != dtype || slot->count != count || slot->op != op ||
-             slot->algo != algo || slot->root != root || slot->nonblocking != (req != nullptr) ||
-             slot->counts != cv || slot->displs != dv) {
-    AL_AMD_THROW("Logical ranks disagree on the arguments of a collective");
   }
+  Poster::take_seq(c);
   Posting &me = slot->ranks[static_cast<size_t>(c.rank())];
   me.send = send;
   me.recv = recv;
   me.stream = c.get_stream();
+  me.ready = ready;
   if (req) {
     // handed out now, "not launched yet" until the last logical rank has called
     *req = std::make_shared<Request>();
@@ -358,22 +446,102 @@ inline void World::post(Communicator &c, OpKind kind, int dtype, const void *sen
   me.posted = true;
   slot->nposted++;
   // launch in sequence order only: an operation never overtakes an earlier one
-  while (!pending_.empty() && pending_.front().nposted == P) {
-    PendingOp done = std::move(pending_.front());
+  std::string my_failure;
+  while (!pending_.empty() && pending_.front()->nposted == P) {
+    std::shared_ptr<PendingOp> done = pending_.front();
     pending_.pop_front();
-    launch(done);
+    try {
+      launch(*done);
+    } catch (const std::exception &e) {
+      // the ranks that have already returned learn of it through their requests (Test / Wait), or,
+      // when calls wait for the launch, through the exception their own call throws
+      done->failure = e.what();
+      for (Posting &r : done->ranks)
+        if (r.req) r.req->error = done->failure;
+    }
+    for (Posting &r : done->ranks)
+      if (r.ready) {
+        events_->give(r.ready);
+        r.ready = nullptr;
+      }
+    done->launched = true;
+    if (done == slot) my_failure = done->failure;
+    else if (!done->failure.empty() && my_failure.empty() && !calls_wait_) my_failure = done->failure;
   }
+  launched_cv_.notify_all();
+  if (calls_wait_ && !slot->launched) {
+    launched_cv_.wait(lock, [&] { return slot->launched; });
+    my_failure = slot->failure;
+  }
+  if (!my_failure.empty()) throw al_exception(my_failure, __FILE__, __LINE__);
 }
 
-/** Makes `target` wait for the prior work of every rank's stream; returns it. */
+inline void *World::attach(int me, int peer, void *mine) {
+  check_peer(peer);
+  if (peer == me) return mine;  // ConnectionSelf::attach_remote_buffer
+  std::unique_lock<std::mutex> lock(mutex_);
+  mail(me, peer).attached.push_back(mine);
+  Mail &in = mail(peer, me);
+  if (in.attached.empty()) {
+    if (!calls_wait_)
+      AL_AMD_THROW("AttachRemoteBuffer: the peer has not attached its buffer yet. All logical ranks share one "
+                   "address space, so a peer's pointer can be given to Put as it is; the exchange itself needs "
+                   "one thread per rank and World::set_calls_wait_for_launch(true)");
+    launched_cv_.wait(lock, [&] { return !in.attached.empty(); });
+  }
+  void *theirs = in.attached.front();
+  in.attached.pop_front();
+  launched_cv_.notify_all();
+  return theirs;
+}
+
+inline void World::rma_notify(int me, int peer) {
+  check_peer(peer);
+  const hipStream_t mine = comm(me).get_stream(), theirs = comm(peer).get_stream();
+  if (mine == theirs) return;  // one stream: its own order is the notification (ConnectionSelf::notify)
+  std::lock_guard<std::mutex> lock(mutex_);
+  hipEvent_t ev = events_->take();
+  const hipError_t e = hipEventRecord(ev, mine);
+  if (e != hipSuccess) {
+    events_->give(ev);
+    AL_AMD_THROW(std::string("GPU error: ") + hipGetErrorString(e));
+  }
+  Mail &m = mail(me, peer);
+  if (m.waiting > 0) {
+    // the receiver has already asked: from here on its stream is behind this point
+    --m.waiting;
+    const hipError_t w = hipStreamWaitEvent(theirs, ev, 0);
+    events_->give(ev);
+    if (w != hipSuccess) AL_AMD_THROW(std::string("GPU error: ") + hipGetErrorString(w));
+  } else {
+    m.notified.push_back(ev);
+  }
+  launched_cv_.notify_all();
+}
+
+inline void World::rma_wait(int me, int peer) {
+  check_peer(peer);
+  const hipStream_t mine = comm(me).get_stream(), theirs = comm(peer).get_stream();
+  if (mine == theirs) return;  // ConnectionSelf::wait
+  std::unique_lock<std::mutex> lock(mutex_);
+  Mail &m = mail(peer, me);
+  if (m.notified.empty() && calls_wait_) launched_cv_.wait(lock, [&] { return !m.notified.empty(); });
+  if (m.notified.empty()) {
+    ++m.waiting;  // the notification orders the stream when it comes (see the note on stream order above)
+    return;
+  }
+  hipEvent_t ev = m.notified.front();
+  m.notified.pop_front();
+  const hipError_t w = hipStreamWaitEvent(mine, ev, 0);
+  events_->give(ev);
+  if (w != hipSuccess) AL_AMD_THROW(std::string("GPU error: ") + hipGetErrorString(w));
+}
+
+/** Makes `target` wait for what each rank's stream held when that rank made its call; returns it. */
 inline hipStream_t World::gather_streams(PendingOp &p, hipStream_t target) {
-  for (size_t i = 0; i < p.ranks.size(); ++i) {
-    const hipStream_t s = p.ranks[i].stream;
-    bool seen = s == target;
-    for (size_t k = 0; k < i && !seen; ++k) seen = p.ranks[k].stream == s;
-    if (seen) continue;  // logical ranks often share a stream: one dependency per distinct stream
-    AL_AMD_CHECK_HIP(hipEventRecord(sync_event_, s));
-    AL_AMD_CHECK_HIP(hipStreamWaitEvent(target, sync_event_, 0));
+  for (Posting &r : p.ranks) {
+    // one event per distinct stream; a rank on the target stream itself needs none (stream order)
+    if (r.ready && r.stream != target) AL_AMD_CHECK_HIP(hipStreamWaitEvent(target, r.ready, 0));
   }
   return target;
 }
@@ -406,16 +574,15 @@ inline void World::release_streams(PendingOp &p, hipStream_t ran_on) {
 
 inline void World::launch(PendingOp &p) {
   const int P = size();
-  // Blocking operations run on rank 0's stream, non-blocking ones on the internal stream
-  // between the two synchronisations of ht_impl.hpp:866-888 - unless they are small: moving
-  // to another stream and back costs about 20 us of event calls, more than a kernel of a few
-  // microseconds could ever overlap with, so those run on rank 0's stream as well and only
-  // leave a completion event behind.
   const size_t es = alamd_dtype_size(p.dtype);
-  size_t per_rank = p.count;
-  for (size_t c : p.counts) per_rank += c;
-  const bool on_internal = p.nonblocking && per_rank * es > kInlineNonblockingBytes;
-  hipStream_t target = on_internal ? internal_stream_ : p.ranks[0].stream;
+  hipStream_t target = target_of(p.nonblocking, p.dtype, p.count, p.counts);
+  // Operations are launched in sequence order; one that runs on another stream than the one before
+  // it waits for that one, so that it sees its results whatever the ranks' events were taken before.
+  if (last_target_ != nullptr && last_target_ != target) {
+    AL_AMD_CHECK_HIP(hipEventRecord(sync_event_, last_target_));
+    AL_AMD_CHECK_HIP(hipStreamWaitEvent(target, sync_event_, 0));
+  }
+  last_target_ = target;
   gather_streams(p, target);
   std::vector<const void *> sends(static_cast<size_t>(P));
   std::vector<void *> recvs(static_cast<size_t>(P));
@@ -659,6 +826,38 @@ class HipCombineBackend {
     NonblockingAllgatherv(mine, recvbuf, std::move(counts), std::move(displs), comm, req, algo);
   }
 
+  /* ---- one-sided extension (MPICUDABackend, include/aluminum/mpi_cuda_impl.hpp:70-104) ---- */
+
+  /** Returns the address at which `peer`'s buffer is reachable: the buffer that `peer` passes to
+   *  its own matching call.  For peer == comm.rank() that is local_buf itself
+   *  (rma_self.hpp:44-46). */
+  template <typename T> static T *AttachRemoteBuffer(T *local_buf, int peer, comm_type &comm) {
+    return static_cast<T *>(comm.world().attach(comm.rank(), peer, local_buf));
+  }
+  /** Nothing is mapped, so nothing is unmapped (rma_self.hpp:47). */
+  template <typename T> static void DetachRemoteBuffer(T *, int, comm_type &) {}
+  static void Notify(int peer, comm_type &comm) { comm.world().rma_notify(comm.rank(), peer); }
+  static void Wait(int peer, comm_type &comm) { comm.world().rma_wait(comm.rank(), peer); }
+  /** An exchange of notifications (rma_ipc.hpp:254-262). */
+  static void Sync(int peer, comm_type &comm) {
+    Notify(peer, comm);
+    Wait(peer, comm);
+  }
+  static void Sync(const int *peers, int num_peers, comm_type &comm) {
+    for (int i = 0; i < num_peers; ++i) Notify(peers[i], comm);
+    for (int i = 0; i < num_peers; ++i) Wait(peers[i], comm);
+  }
+  /** count elements from srcbuf to destbuf (a buffer of rank `dest`), on the communicator's stream
+   *  (rma_self.hpp:57-70: an asynchronous copy; errors as there). */
+  template <typename T>
+  static void Put(const T *srcbuf, int dest, T *destbuf, size_t count, comm_type &comm) {
+    if (dest < 0 || dest >= comm.size()) AL_AMD_THROW("Invalid peer rank");
+    if (count == 0) return;
+    if (srcbuf == nullptr) AL_AMD_THROW("Source buffer is null");
+    if (destbuf == nullptr) AL_AMD_THROW("Destination buffer is null");
+    AL_AMD_CHECK(alamd_copy(destbuf, srcbuf, count * sizeof(T), comm.get_stream()));
+  }
+
   /** sendbuf holds count elements, recvbuf receives size()*count; in place the
    *  caller's slice is already at recvbuf + rank*count
    *  (include/aluminum/ht/allgather.hpp:48-81). */
@@ -875,11 +1074,64 @@ void NonblockingAllgatherv(T *buffer, std::vector<size_t> counts, std::vector<si
   Backend::template NonblockingAllgatherv<T>(buffer, std::move(counts), std::move(displs), comm, req, algo);
 }
 
+/* ---- one-sided extension (include/Al.hpp:1916-2001) ------------------------ */
+namespace ext {
+template <typename Backend, typename T>
+T *AttachRemoteBuffer(T *local_buf, int peer, typename Backend::comm_type &comm) {
+  return Backend::template AttachRemoteBuffer<T>(local_buf, peer, comm);
+}
+template <typename Backend, typename T>
+void DetachRemoteBuffer(T *remote_buf, int peer, typename Backend::comm_type &comm) {
+  Backend::template DetachRemoteBuffer<T>(remote_buf, peer, comm);
+}
+template <typename Backend> void Notify(int peer, typename Backend::comm_type &comm) { Backend::Notify(peer, comm); }
+template <typename Backend> void Wait(int peer, typename Backend::comm_type &comm) { Backend::Wait(peer, comm); }
+template <typename Backend> void Sync(int peer, typename Backend::comm_type &comm) { Backend::Sync(peer, comm); }
+template <typename Backend> void Sync(const int *peers, int num_peers, typename Backend::comm_type &comm) {
+  Backend::Sync(peers, num_peers, comm);
+}
+template <typename Backend, typename T>
+void Put(const T *srcbuf, int dest, T *destbuf, size_t count, typename Backend::comm_type &comm) {
+  Backend::template Put<T>(srcbuf, dest, destbuf, count, comm);
+}
+}  // namespace ext
+
+namespace amd {
+/** Halo faces of a 3-D grid, x fastest (interior dims, `halo` cells on every side): the contiguous
+ *  buffers that ext::Put moves in a halo exchange (test/test_rma_halo_exchange.cpp:171-197 puts
+ *  buffers that are already contiguous; the strided faces are this engine's addition).  Faces:
+ *  0 -x, 1 +x, 2 -y, 3 +y, 4 -z, 5 +z; bit f of face_mask selects face f.  pack fills bufs[f] from
+ *  the interior boundary slab, unpack writes bufs[f] into the ghost slab; both run on the
+ *  communicator's stream. */
+template <typename T>
+void halo_pack(T *const bufs[6], const T *grid, const size_t dims[3], size_t halo, unsigned face_mask,
+               Communicator &comm) {
+  void *tab[6];
+  for (int f = 0; f < 6; ++f) tab[f] = bufs[f];
+  AL_AMD_CHECK(alamd_halo_pack(tab, grid, dims, halo, sizeof(T), face_mask, comm.get_stream()));
+}
+template <typename T>
+void halo_unpack(T *grid, const T *const bufs[6], const size_t dims[3], size_t halo, unsigned face_mask,
+                 Communicator &comm) {
+  const void *tab[6];
+  for (int f = 0; f < 6; ++f) tab[f] = bufs[f];
+  AL_AMD_CHECK(alamd_halo_unpack(grid, tab, dims, halo, sizeof(T), face_mask, comm.get_stream()));
+}
+inline size_t halo_face_elems(const size_t dims[3], size_t halo, int face) {
+  return alamd_halo_face_elems(dims, halo, face);
+}
+}  // namespace amd
+
 /** Host-only completion test; resets the request when complete
  *  (include/aluminum/ht_impl.hpp:1113-1126). */
 template <typename Backend> bool Test(typename Backend::req_type &req);
 template <> inline bool Test<HipCombineBackend>(HipCombineBackend::req_type &req) {
   if (req == HipCombineBackend::null_req) return true;
+  if (!req->error.empty()) {
+    const std::string why = req->error;
+    req = HipCombineBackend::null_req;
+    throw al_exception("The operation could not be launched: " + why, __FILE__, __LINE__);
+  }
   if (!req->done) return false;  // not launched yet: some logical rank has not made its call
   const hipError_t e = hipEventQuery(req->done->event);
   if (e == hipSuccess) {
@@ -895,6 +1147,11 @@ template <> inline bool Test<HipCombineBackend>(HipCombineBackend::req_type &req
 template <typename Backend> void Wait(typename Backend::req_type &req);
 template <> inline void Wait<HipCombineBackend>(HipCombineBackend::req_type &req) {
   if (req == HipCombineBackend::null_req) return;
+  if (!req->error.empty()) {
+    const std::string why = req->error;
+    req = HipCombineBackend::null_req;
+    throw al_exception("The operation could not be launched: " + why, __FILE__, __LINE__);
+  }
   if (!req->done) AL_AMD_THROW("Wait on an operation that not every logical rank has started");
   if (req->orig_stream != req->done->ran_on && req->done->first_wait(req->orig_stream))
     AL_AMD_CHECK_HIP(hipStreamWaitEvent(req->orig_stream, req->done->event, 0));
@@ -957,6 +1214,8 @@ class GPUStatusFlag {
 class ProgressEngine {
  public:
   ProgressEngine() : thread_([this] { run(); }) {}
+  /** Waits until every enqueued step has been retired, i.e. until every stream given to enqueue()
+   *  has passed its step: destroy the engine only when those streams can make progress. */
   ~ProgressEngine() {
     {
       std::lock_guard<std::mutex> lock(mutex_);
@@ -985,6 +1244,17 @@ class ProgressEngine {
     std::lock_guard<std::mutex> lock(mutex_);
     return states_.size();
   }
+  /** Rethrows, once, the first exception a host step has thrown since the last call.  The stream of
+   *  a step that threw is released all the same, so nothing hangs behind it. */
+  void check() {
+    std::exception_ptr e;
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      e = failed_;
+      failed_ = nullptr;
+    }
+    if (e) std::rethrow_exception(e);
+  }
 
  private:
   struct State {
@@ -1003,9 +1273,19 @@ class ProgressEngine {
         State *st = states_[i].get();
         if (!st->ran && st->start.query()) {
           lock.unlock();
-          st->fn();          // phase 2, outside the lock: enqueue() may be called meanwhile
-          st->go.signal();   // phase 3
+          std::exception_ptr failed;
+          try {
+            st->fn();        // phase 2, outside the lock: enqueue() may be called meanwhile
+          } catch (...) {
+            failed = std::current_exception();
+          }
+          try {
+            st->go.signal();  // phase 3, whatever fn did: the stream must not stay blocked
+          } catch (...) {
+            if (!failed) failed = std::current_exception();
+          }
           lock.lock();
+          if (failed && !failed_) failed_ = failed;
           st->ran = true;
           progressed = true;
         }
@@ -1026,6 +1306,7 @@ class ProgressEngine {
   std::mutex mutex_;
   std::condition_variable wake_;
   std::deque<std::unique_ptr<State>> states_;
+  std::exception_ptr failed_;
   bool stop_ = false;
   std::thread thread_;  // last: started when everything above exists
 };

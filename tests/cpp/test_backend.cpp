@@ -87,6 +87,232 @@ static void test_threads_and_streams() {
   for (auto &s : streams) HIPCHK(hipStreamDestroy(s));
 }
 
+
+// ---- one-sided extension and halo faces ----------------------------------------
+
+struct HaloGrid {
+  size_t dims[3], h, side[3], cells;
+  std::vector<double> host;
+  std::unique_ptr<DevBuf<double>> dev;
+  HaloGrid(size_t nx, size_t ny, size_t nz, size_t halo, unsigned seed) : h(halo) {
+    dims[0] = nx; dims[1] = ny; dims[2] = nz;
+    for (int d = 0; d < 3; ++d) side[d] = dims[d] + 2 * h;
+    cells = side[0] * side[1] * side[2];
+    host = gen<double>(cells, ALO_DIST_UNIFORM_01, seed);
+    dev.reset(new DevBuf<double>(cells));
+    dev->up(host);
+  }
+  size_t face_elems(int f) const { return alo_halo_face_elems(dims[0], dims[1], dims[2], h, f); }
+};
+
+// pack -> ext::Put to the rank itself -> unpack, against the oracle's index maps
+static void test_halo_loopback(hipStream_t stream) {
+  HaloGrid g(37, 20, 9, 2, 4000u);
+  Al::amd::World world(1, stream);
+  auto &comm = world.comm(0);
+  std::vector<std::unique_ptr<DevBuf<double>>> send, recv;
+  double *sp[6], *rp[6];
+  for (int f = 0; f < 6; ++f) {
+    EXPECT(Al::amd::halo_face_elems(g.dims, g.h, f) == g.face_elems(f), "face %d size", f);
+    send.emplace_back(new DevBuf<double>(g.face_elems(f)));
+    recv.emplace_back(new DevBuf<double>(g.face_elems(f)));
+    sp[f] = send[f]->p;
+    // the address at which the peer's (here: the rank's own) receive buffer is reachable
+    rp[f] = Al::ext::AttachRemoteBuffer<Backend>(recv[f]->p, 0, comm);
+    EXPECT(rp[f] == recv[f]->p, "a rank reaches its own buffer at its own address");
+  }
+  Al::amd::halo_pack<double>(sp, g.dev->p, g.dims, g.h, 0x3f, comm);
+  for (int f = 0; f < 6; ++f) Al::ext::Put<Backend>(static_cast<const double *>(sp[f]), 0, rp[f], g.face_elems(f), comm);
+  Al::ext::Sync<Backend>(0, comm);
+  const double *crp[6];
+  for (int f = 0; f < 6; ++f) crp[f] = rp[f];
+  Al::amd::halo_unpack<double>(g.dev->p, crp, g.dims, g.h, 0x3f, comm);
+  HIPCHK(hipStreamSynchronize(stream));
+  std::vector<double> want = g.host;
+  for (int f = 0; f < 6; ++f) {
+    std::vector<double> face(g.face_elems(f));
+    alo_halo_pack(face.data(), g.host.data(), g.dims[0], g.dims[1], g.dims[2], g.h, f, sizeof(double));
+    EXPECT(same_bits(send[f]->down(), face), "packed face %d", f);
+    alo_halo_unpack(want.data(), face.data(), g.dims[0], g.dims[1], g.dims[2], g.h, f, sizeof(double));
+  }
+  EXPECT(same_bits(g.dev->down(), want), "grid after the loop-back halo exchange");
+  for (int f = 0; f < 6; ++f) Al::ext::DetachRemoteBuffer<Backend>(rp[f], 0, comm);
+  bool threw = false;
+  try { Al::ext::Put<Backend>(static_cast<const double *>(nullptr), 0, rp[0], 4, comm); } catch (const Al::al_exception &e) {
+    threw = std::string(e.what()).find("Source buffer is null") != std::string::npos;
+  }
+  EXPECT(threw, "Put from a null buffer must throw");
+  threw = false;
+  try { Al::ext::Notify<Backend>(3, comm); } catch (const Al::al_exception &) { threw = true; }
+  EXPECT(threw, "a peer outside the communicator must throw");
+}
+
+// Two logical ranks on two streams exchange their x faces (rank 0's +x neighbour is rank 1 and the
+// other way round), with Put / Notify / Wait; wait_first: the receivers ask before the senders notify.
+static void test_halo_two_ranks(bool wait_first) {
+  hipStream_t s[2];
+  for (auto &x : s) HIPCHK(hipStreamCreateWithFlags(&x, hipStreamNonBlocking));
+  {
+    Al::amd::World world(std::vector<hipStream_t>{s[0], s[1]});
+    HaloGrid g0(16, 11, 13, 3, 4100u), g1(16, 11, 13, 3, 4200u);
+    HaloGrid *g[2] = {&g0, &g1};
+    const int out_face[2] = {1, 0};  // rank 0 sends its +x face, rank 1 its -x face
+    const int in_face[2] = {1, 0};   // ... and receives into the ghost slab of the same side
+    const size_t n = g0.face_elems(0);
+    DevBuf<double> send0(n), send1(n), recv0(n), recv1(n);
+    double *send[2] = {send0.p, send1.p}, *recv[2] = {recv0.p, recv1.p};
+    Al::amd::GPUWait gate;
+    gate.wait(s[1], 1u << 24);  // rank 1's stream is late: nothing of its exchange has run when rank 0 asks
+    if (wait_first)
+      for (int r = 0; r < 2; ++r) Al::ext::Wait<Backend>(1 - r, world.comm(r));
+    for (int r = 0; r < 2; ++r) {
+      double *bufs[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+      bufs[out_face[r]] = send[r];
+      Al::amd::halo_pack<double>(bufs, g[r]->dev->p, g[r]->dims, g[r]->h, 1u << out_face[r], world.comm(r));
+      // all ranks share one address space: the peer's receive buffer is used as it is
+      Al::ext::Put<Backend>(static_cast<const double *>(send[r]), 1 - r, recv[1 - r], n, world.comm(r));
+      Al::ext::Notify<Backend>(1 - r, world.comm(r));
+    }
+    for (int r = 0; r < 2; ++r) {
+      if (!wait_first) Al::ext::Wait<Backend>(1 - r, world.comm(r));
+      const double *bufs[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+      bufs[in_face[r]] = recv[r];
+      Al::amd::halo_unpack<double>(g[r]->dev->p, bufs, g[r]->dims, g[r]->h, 1u << in_face[r], world.comm(r));
+    }
+    gate.signal();
+    for (auto &x : s) HIPCHK(hipStreamSynchronize(x));
+    EXPECT(!gate.timed_out(), "gate must not have expired");
+    for (int r = 0; r < 2; ++r) {
+      std::vector<double> face(n), want = g[r]->host;
+      alo_halo_pack(face.data(), g[1 - r]->host.data(), g0.dims[0], g0.dims[1], g0.dims[2], g0.h, out_face[1 - r], sizeof(double));
+      alo_halo_unpack(want.data(), face.data(), g0.dims[0], g0.dims[1], g0.dims[2], g0.h, in_face[r], sizeof(double));
+      EXPECT(same_bits(g[r]->dev->down(), want), "rank %d ghost cells after the exchange (%s)", r,
+             wait_first ? "wait before notify" : "notify before wait");
+    }
+  }
+  for (auto &x : s) HIPCHK(hipStreamDestroy(x));
+}
+
+// Every rank on its own stream, each stream held back by a gate the host opens late and in
+// reverse order: the collective must wait for what every stream held at its rank's call, and the
+// copies enqueued after the last call must see the result.
+static void test_stream_order(bool threaded) {
+  const int P = 4;
+  const size_t n = 30000;
+  std::vector<hipStream_t> streams(P);
+  for (auto &s : streams) HIPCHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  {
+    Al::amd::World world(streams);
+    world.set_calls_wait_for_launch(threaded);
+    std::vector<std::vector<float>> in;
+    std::vector<std::unique_ptr<DevBuf<float>>> buf;
+    std::vector<float *> pinned_in(P), pinned_out(P);
+    std::vector<std::unique_ptr<Al::amd::GPUWait>> gates;
+    for (int r = 0; r < P; ++r) {
+      in.push_back(gen<float>(n, ALO_DIST_UNIFORM_PM1, 90u + (unsigned)r));
+      buf.emplace_back(new DevBuf<float>(n));
+      HIPCHK(hipMemset(buf[r]->p, 0, n * sizeof(float)));
+      HIPCHK(hipHostMalloc(reinterpret_cast<void **>(&pinned_in[r]), n * sizeof(float), hipHostMallocDefault));
+      HIPCHK(hipHostMalloc(reinterpret_cast<void **>(&pinned_out[r]), n * sizeof(float), hipHostMallocDefault));
+      std::memcpy(pinned_in[r], in[r].data(), n * sizeof(float));
+      std::memset(pinned_out[r], 0, n * sizeof(float));
+      gates.emplace_back(new Al::amd::GPUWait);
+    }
+    auto rank_work = [&](int r) {
+      gates[r]->wait(streams[r], 1u << 24);
+      HIPCHK(hipMemcpyAsync(buf[r]->p, pinned_in[r], n * sizeof(float), hipMemcpyHostToDevice, streams[r]));  // producer
+      Al::Allreduce<Backend>(buf[r]->p, n, Op::sum, world.comm(r), Algo::rank_order);
+    };
+    auto consumer = [&](int r) {
+      HIPCHK(hipMemcpyAsync(pinned_out[r], buf[r]->p, n * sizeof(float), hipMemcpyDeviceToHost, streams[r]));
+    };
+    if (threaded) {
+      // each thread enqueues its consumer as soon as its call returns
+      std::vector<std::thread> th;
+      for (int r = 0; r < P; ++r) th.emplace_back([&, r] { rank_work(r); consumer(r); });
+      for (auto &t : th) t.join();
+    } else {
+      for (int r = 0; r < P; ++r) rank_work(r);
+      for (int r = 0; r < P; ++r) consumer(r);  // after the last call
+    }
+    for (int r = P - 1; r >= 0; --r) {
+      std::this_thread::sleep_for(std::chrono::milliseconds(3));
+      gates[r]->signal();
+    }
+    for (auto &s : streams) HIPCHK(hipStreamSynchronize(s));
+    std::vector<float> want(n);
+    std::vector<const void *> ptrs;
+    for (auto &b : in) ptrs.push_back(b.data());
+    alo_combine(want.data(), ptrs.data(), P, n, ALO_F32, ALO_SUM, ALO_ORDER_RANK_ASC, 0);
+    for (int r = 0; r < P; ++r) {
+      EXPECT(!gates[r]->timed_out(), "gate %d must not have expired", r);
+      EXPECT(std::memcmp(pinned_out[r], want.data(), n * sizeof(float)) == 0, "%s: rank %d's consumer saw the result",
+             threaded ? "threads" : "one thread", r);
+      HIPCHK(hipHostFree(pinned_in[r]));
+      HIPCHK(hipHostFree(pinned_out[r]));
+    }
+  }
+  for (auto &s : streams) HIPCHK(hipStreamDestroy(s));
+}
+
+// A call that throws leaves its communicator where it was; a launch that fails is reported to the
+// ranks that have already returned.
+static void test_error_recovery(hipStream_t stream) {
+  const size_t n = 64;
+  DevBuf<float> a(n), b(n);
+  const auto ha = gen<float>(n, ALO_DIST_UNIFORM_PM1, 7u), hb = gen<float>(n, ALO_DIST_UNIFORM_PM1, 8u);
+  a.up(ha);
+  b.up(hb);
+  Al::amd::World world(2, stream);
+  Al::Allreduce<Backend>(a.p, n, Op::sum, world.comm(0), Algo::rank_order);
+  bool threw = false;
+  try { Al::Allreduce<Backend>(b.p, n / 2, Op::sum, world.comm(1), Algo::rank_order); } catch (const Al::al_exception &) { threw = true; }
+  EXPECT(threw, "mismatched count must throw");
+  Al::Allreduce<Backend>(b.p, n, Op::sum, world.comm(1), Algo::rank_order);  // the same rank, now as agreed
+  HIPCHK(hipStreamSynchronize(stream));
+  std::vector<float> want(n);
+  const void *ptrs[2] = {ha.data(), hb.data()};
+  alo_combine(want.data(), ptrs, 2, n, ALO_F32, ALO_SUM, ALO_ORDER_RANK_ASC, 0);
+  EXPECT(same_bits(a.down(), want) && same_bits(b.down(), want), "the collective completed after the failed call");
+  // a launch that fails: rank 1's receive buffer overlaps rank 0's send buffer partially
+  DevBuf<float> big(3 * n);
+  Backend::req_type r0, r1;
+  Al::NonblockingAllreduce<Backend>(static_cast<const float *>(big.p), big.p + 2 * n, n, Op::sum, world.comm(0), r0, Algo::rank_order);
+  threw = false;
+  try {
+    Al::NonblockingAllreduce<Backend>(static_cast<const float *>(big.p + n), big.p + n / 2, n, Op::sum, world.comm(1), r1, Algo::rank_order);
+  } catch (const Al::al_exception &) { threw = true; }
+  EXPECT(threw, "overlapping buffers must throw from the call that launches");
+  threw = false;
+  try { (void)Al::Test<Backend>(r0); } catch (const Al::al_exception &e) {
+    threw = std::string(e.what()).find("could not be launched") != std::string::npos;
+  }
+  EXPECT(threw, "the rank that had already returned learns of the failure from its request");
+  EXPECT(r0 == Backend::null_req, "a failed request is released");
+  // and the world goes on
+  Al::Allreduce<Backend>(a.p, n, Op::max, world.comm(0), Algo::rank_order);
+  Al::Allreduce<Backend>(b.p, n, Op::max, world.comm(1), Algo::rank_order);
+  HIPCHK(hipStreamSynchronize(stream));
+  EXPECT(same_bits(a.down(), want), "max of equal values after the failed launch");
+}
+
+// A host step that throws must not leave its stream blocked.
+static void test_progress_engine_exception(hipStream_t stream) {
+  DevBuf<int> x(1);
+  HIPCHK(hipMemsetAsync(x.p, 0, sizeof(int), stream));
+  Al::amd::ProgressEngine pe;
+  pe.enqueue(stream, [] { throw std::runtime_error("host step failed"); });
+  HIPCHK(hipMemsetAsync(x.p, 1, sizeof(int), stream));
+  HIPCHK(hipStreamSynchronize(stream));  // returns: the step's wait was signalled all the same
+  EXPECT(x.down()[0] == 0x01010101, "work behind the failed host step ran");
+  for (int spin = 0; spin < 2000 && pe.pending(); ++spin) std::this_thread::sleep_for(std::chrono::milliseconds(1));
+  EXPECT(pe.pending() == 0, "the failed step was retired");
+  bool threw = false;
+  try { pe.check(); } catch (const std::runtime_error &e) { threw = std::string(e.what()) == "host step failed"; }
+  EXPECT(threw, "check() rethrows what the host step threw");
+  pe.check();  // once only
+}
+
 static void test_flags(hipStream_t stream) {
   Al::amd::GPUStatusFlag done;
   EXPECT(done.query(), "status flag starts complete");
@@ -193,7 +419,14 @@ int main() {
       test_v_variants<double>(P, inplace, stream);
     }
   test_errors(stream);
+  test_error_recovery(stream);
   test_threads_and_streams();
+  test_stream_order(false);
+  test_stream_order(true);
+  test_halo_loopback(stream);
+  test_halo_two_ranks(false);
+  test_halo_two_ranks(true);
+  test_progress_engine_exception(stream);
   test_flags(stream);
   test_progress_engine(stream);
 
