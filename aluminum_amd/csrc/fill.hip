@@ -1,6 +1,7 @@
 // Test and bench support: the counter-based input generator, the exposed
 // 16-bit float conversions, and a plain streaming copy.
 #include "alamd_common.h"
+#include "aluminum_amd_support.h"
 #include "alamd_tile.h"
 
 namespace alamd {

@@ -44,10 +44,36 @@ WORKLOADS = {
 }
 P = 8
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
-# the same counter's reading for the 1 GiB copy kernel (profiles/fold_vec_kernel_f32_sum_P8_c2.md).
-MEASURED_TRAFFIC = {"c2_f32_sum": 2416032085}
-KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false, 8, false>"}
+# The committed rocprofv3 summary of the primary workload: HBM bytes per call from --pmc FETCH_SIZE /
+# WRITE_SIZE, each scaled by the same counter's reading for the 1 GiB copy kernel.
+TRAFFIC_PROFILE = {"c2_f32_sum": "profiles/fold_vec_kernel_f32_sum_P8_c2.md"}
+KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false /*operand roles*/, 8 /*ranks*/, "
+                             "false /*no leading elements*/, false /*not chained*/>"}
+
+# Everything BASELINE.json configures, beside the primary workload: C2 prod and bf16, the same over
+# buffers no earlier call has touched, C4 (integer / bitwise / logical), C3 (ring, both modes), C5 (halo
+# faces), the stream flags, and the layouts an Allreduce / Reduce_scatter / Allgather reaches the kernels in.
+DEFAULT_ALSO = ("c2_f32_sum_rotating,c2_f32_prod,c2_bf16_sum,c2_bf16_sum_rotating,c4_i32_max,c4_i64_bxor,"
+                "c4_u8_lxor,c3_ring_stepwise,c3_ring_fused,c5_halo,flags,c2_f32_allreduce,"
+                "c2_f32_allreduce_rotating,c2_f32_reduce_scatter,c2_f32_reduce_scatter_rotating,"
+                "c2_f32_allgather,c2_f32_allgather_rotating")
+
+
+def measured_traffic(workload):
+    """(bytes per call, where the figure comes from) out of the committed profile summary, or (None, why)."""
+    import hashlib
+    import re
+    rel = TRAFFIC_PROFILE.get(workload)
+    if not rel:
+        return None, "no counter profile committed for this workload"
+    try:
+        text = open(os.path.join(ROOT, rel)).read()
+    except OSError:
+        return None, "%s is missing" % rel
+    m = re.search(r"=> (\d+) B per launch, (\d+) B per call", text)
+    if not m:
+        return None, "%s holds no 'B per call' line" % rel
+    return int(m.group(2)), "%s (sha1 %s)" % (rel, hashlib.sha1(text.encode()).hexdigest()[:12])
 
 
 def run_combine_workload(al, torch, name, steps, warmup, check=True):
@@ -400,10 +426,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2_f32_sum",
                     choices=sorted(WORKLOADS) + ["c3_ring_stepwise", "c3_ring_fused", "c5_halo", "flags"] + LAYOUTS)
-    ap.add_argument("--also", default="c2_bf16_sum,c2_f32_sum_rotating,c2_f32_allreduce,c2_f32_allreduce_rotating,"
-                                      "c2_f32_reduce_scatter,c2_f32_reduce_scatter_rotating,c2_f32_allgather,"
-                                      "c2_f32_allgather_rotating,c3_ring_fused",
+    ap.add_argument("--also", default=DEFAULT_ALSO,
                     help="comma-separated extra workloads reported under 'also' ('' for none)")
+    ap.add_argument("--batch", default="",
+                    help="run these workloads one after the other and print {name: record} (what 'also' runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--raw", action="store_true", help="print only the workload's own measurement record")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -425,33 +451,55 @@ def main():
         print("bench.py: " + al.load().alamd_last_error().decode(), file=sys.stderr)
         sys.exit(1)
 
+    def run_one(name, steps, warmup):
+        if name.startswith("c3_ring_"):
+            res = run_ring_workload(al, torch, name[len("c3_ring_"):], steps, warmup)
+        elif name == "c5_halo":
+            res = run_halo_workload(al, torch, steps, warmup)
+        elif name == "flags":
+            res = run_flag_workload()
+        elif name in LAYOUTS:
+            res = run_layout_workload(al, torch, name, steps, warmup)
+        else:
+            res = run_combine_workload(al, torch, name, steps, warmup)
+        if "gbps_kernel" in res:
+            res["frac"] = res["gbps_kernel"] / HBM_PEAK_GBPS  # of the 8 TB/s HBM peak, from the kernel's own time
+        return res
+
     if args.calibrate_copy:
         print(json.dumps(run_copy_calibration(al, torch, args.steps, args.warmup)))
         return
-    if args.workload.startswith("c3_ring_"):
-        main_res = run_ring_workload(al, torch, args.workload[len("c3_ring_"):], args.steps, args.warmup)
-    elif args.workload == "c5_halo":
-        main_res = run_halo_workload(al, torch, args.steps, args.warmup)
-    elif args.workload == "flags":
-        main_res = run_flag_workload()
-    elif args.workload in LAYOUTS:
-        main_res = run_layout_workload(al, torch, args.workload, args.steps, args.warmup)
-    else:
-        main_res = run_combine_workload(al, torch, args.workload, args.steps, args.warmup)
+    if args.batch:
+        # one process for all of them; each starts from an empty device
+        out = {}
+        for name in [w for w in args.batch.split(",") if w]:
+            try:
+                out[name] = run_one(name, args.steps, args.warmup)
+            except Exception as e:  # one workload must not take the others down
+                out[name] = {"workload": name, "error": str(e)[:300]}
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+        print(json.dumps(out))
+        return
+    main_res = run_one(args.workload, args.steps, args.warmup)
     if args.raw or args.workload not in WORKLOADS:
         print(json.dumps(main_res))
         return
-    # secondary workloads run in a fresh process each (same command, one workload), so that every
-    # figure is taken with its buffers allocated on an empty device, like the primary one
+    # the secondary workloads run in a fresh process, one after the other, each with its buffers
+    # allocated on an empty device like the primary one
     also = {}
-    for name in [w for w in args.also.split(",") if w and w != args.workload]:
+    names = [w for w in args.also.split(",") if w and w != args.workload]
+    if names:
         torch.cuda.empty_cache()
-        p = subprocess.run([sys.executable, os.path.abspath(__file__), "--workload", name, "--also", "",
+        p = subprocess.run([sys.executable, os.path.abspath(__file__), "--batch", ",".join(names), "--also", "",
                             "--no-cpu-baseline", "--steps", str(max(5, args.steps // 2)),
-                            "--warmup", str(max(2, args.warmup // 2)), "--raw"],
-                           capture_output=True, text=True, timeout=600)
+                            "--warmup", str(max(2, args.warmup // 2))],
+                           capture_output=True, text=True, timeout=900)
         line = [l for l in p.stdout.splitlines() if l.startswith("{")]
-        also[name] = json.loads(line[-1]) if p.returncode == 0 and line else {"error": p.stderr[-300:]}
+        also = json.loads(line[-1]) if p.returncode == 0 and line else {"error": p.stderr[-300:]}
+    traffic, traffic_source = measured_traffic(args.workload)
+    untouched = {k: also[k]["frac"] for k in ("c2_f32_sum_rotating", "c2_bf16_sum_rotating")
+                 if isinstance(also.get(k), dict) and "frac" in also[k]}
 
     out = {
         "metric": METRIC, "value": main_res["gbps_wall"], "unit": "GB/s", "n_gpus": 1,
@@ -467,10 +515,15 @@ def main():
         "parity_vs_oracle": main_res.get("parity_vs_oracle"),
         "roofline": {"bound": "hbm", "achieved": main_res["gbps_kernel"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": main_res["gbps_kernel"] / HBM_PEAK_GBPS,
-                     # measured HBM bytes (fetched + written) per call, and per launch of the kernel
-                     "traffic": MEASURED_TRAFFIC.get(args.workload),
-                     "traffic_per_launch": (MEASURED_TRAFFIC[args.workload] // main_res["launches_per_step"]
-                                            if args.workload in MEASURED_TRAFFIC else None),
+                     # the same kernel over four rotating buffer sets: nothing a call reads or writes was
+                     # touched by the three calls before it, so the 256 MiB memory-side cache cannot help
+                     "frac_untouched": untouched.get("c2_f32_sum_rotating"),
+                     "frac_untouched_bf16": untouched.get("c2_bf16_sum_rotating"),
+                     # HBM bytes (fetched + written) per call and per launch, read from the committed
+                     # counter profile, not measured by this run
+                     "traffic": traffic,
+                     "traffic_per_launch": traffic // main_res["launches_per_step"] if traffic else None,
+                     "traffic_source": traffic_source,
                      "kernel": KERNEL_NAME.get(args.workload, "alamd::fold_vec_kernel"),
                      "kernel_ms": main_res["kernel_ms"],
                      # one call is cut into launches of at most 4096 tiles of 16 KiB per stream

@@ -16,6 +16,10 @@
  * class (include/aluminum/ht_impl.hpp:125-1111).  The header-only C++ shim
  * include/aluminum_amd/Al.hpp maps that class interface onto the functions
  * below, turning error codes into Al::al_exception.
+ *
+ * Entry points that replace nothing in the reference and exist for tests and
+ * benchmarks only (input generator, the 16-bit float conversions on their own)
+ * are declared in aluminum_amd_support.h, not here.
  */
 #ifndef ALUMINUM_AMD_H
 #define ALUMINUM_AMD_H
@@ -282,29 +286,15 @@ int32_t alamd_flag_query(alamd_flag *flag);
 /* 1 if a bounded kernel wait on this flag has expired since creation. */
 int alamd_flag_timed_out(alamd_flag *flag);
 
-/* ---- test and bench support -------------------------------------------- */
+/* ---- plain copy ---------------------------------------------------------- */
 
-/* Input distributions of the counter-based generator. */
-typedef enum {
-  ALAMD_DIST_UNIFORM_PM1 = 0, ALAMD_DIST_UNIFORM_09_11 = 1, ALAMD_DIST_UNIFORM_01 = 2,
-  ALAMD_DIST_FULLRANGE = 3, ALAMD_DIST_BOOL01 = 4, ALAMD_DIST_NORMAL = 5,
-  ALAMD_DIST_SMALLINT = 6
-} alamd_dist;
-
-/* dst[i] = value of element (idx0 + i) of stream `seed` under `dist`: a pure
- * integer hash followed by correctly rounded fp64 operations, so a host
- * implementation of the same formula yields the same bits.  (Stands in for
- * gen_data, test/test_utils.hpp:157-256, whose libstdc++ distributions are
- * not reproducible on a device.) */
-int alamd_fill(void *dst, size_t count, int dtype, int dist, uint64_t seed,
-               uint64_t idx0, void *stream);
-/* The library's own fp32 -> fp16 / bf16 narrowing and the exact widening,
- * as used inside the combine kernels (exposed so that all 2^32 inputs can be
- * checked). */
-int alamd_narrow_f32(void *dst16, const float *src, size_t count, int dtype, void *stream);
-int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void *stream);
-/* dst[i] = src[i] for `bytes` bytes with the same load / store path as the
- * combine kernels: the practical 1-read + 1-write bandwidth ceiling. */
+/* dst[i] = src[i] for `bytes` bytes on `stream`, with the load / store path of
+ * the combine kernels (any alignment; the ranges must not overlap).  This is
+ * what a Put between two logical ranks of one GPU is
+ * (ConnectionSelf::put, include/aluminum/mpi_cuda/rma_self.hpp:57-70, there a
+ * cudaMemcpyAsync), and the copy that precedes an out-of-place ring allreduce;
+ * it is also the practical 1-read + 1-write bandwidth ceiling that counter
+ * readings of the other kernels are scaled by. */
 int alamd_copy(void *dst, const void *src, size_t bytes, void *stream);
 
 #ifdef __cplusplus

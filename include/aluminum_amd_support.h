@@ -1,0 +1,41 @@
+/*
+ * aluminum_amd - test and benchmark support of the C-ABI library.
+ *
+ * Nothing declared here replaces an interface of the reference and nothing
+ * here is needed to use the combine engine: these entry points let tests and
+ * benchmarks produce seeded inputs in device memory and check the library's
+ * 16-bit float conversions on their own.  The boundary proper is
+ * aluminum_amd.h.
+ */
+#ifndef ALUMINUM_AMD_SUPPORT_H
+#define ALUMINUM_AMD_SUPPORT_H
+
+#include "aluminum_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Input distributions of the counter-based generator. */
+typedef enum {
+  ALAMD_DIST_UNIFORM_PM1 = 0, ALAMD_DIST_UNIFORM_09_11 = 1, ALAMD_DIST_UNIFORM_01 = 2,
+  ALAMD_DIST_FULLRANGE = 3, ALAMD_DIST_BOOL01 = 4, ALAMD_DIST_NORMAL = 5,
+  ALAMD_DIST_SMALLINT = 6
+} alamd_dist;
+
+/* dst[i] = value of element (idx0 + i) of stream `seed` under `dist`: a pure
+ * integer hash followed by correctly rounded fp64 operations, so a host
+ * implementation of the same formula yields the same bits.  (Stands in for
+ * gen_data, test/test_utils.hpp:157-256, whose libstdc++ distributions are
+ * not reproducible on a device.) */
+int alamd_fill(void *dst, size_t count, int dtype, int dist, uint64_t seed,
+               uint64_t idx0, void *stream);
+/* The library's own fp32 -> fp16 / bf16 narrowing and the exact widening,
+ * as used inside the combine kernels (exposed so that all 2^32 inputs can be
+ * checked). */
+int alamd_narrow_f32(void *dst16, const float *src, size_t count, int dtype, void *stream);
+int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void *stream);
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -21,6 +21,7 @@
 #include <vector>
 
 #include "aluminum_amd/Al.hpp"
+#include "aluminum_amd_support.h"
 
 using Backend = Al::HipCombineBackend;
 using Algo = Al::amd::CombineAlgorithm;

@@ -10,8 +10,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "aluminum_amd.h")
 
 
+SUPPORT_HEADER = os.path.join(ROOT, "include", "aluminum_amd_support.h")
+
+
 def declared_functions():
-    text = open(HEADER).read()
+    text = open(HEADER).read() + open(SUPPORT_HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(alamd_[a-z0-9_]+)\s*\(", text)))
 

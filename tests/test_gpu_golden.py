@@ -108,7 +108,7 @@ MPI_PROGRAM = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__fil
 
 @pytest.mark.skipif(not (os.path.exists(MPIEXEC) and os.path.exists(MPI_PROGRAM)),
                     reason="needs mpiexec and the built oracle/mpi_baseline")
-@pytest.mark.parametrize("P", (2, 3, 5, 8))
+@pytest.mark.parametrize("P", (2, 3, 4, 5, 8))
 def test_live_mpi_allreduce_against_the_gpu(al, P):
     """MPI_Allreduce(MPI_SUM, MPI_FLOAT) run now, on this machine's host cores, over generated inputs
     (uniform[-1,1), seed 1000+rank), against the GPU's combine of the same inputs: equal checksums."""
