@@ -286,15 +286,39 @@ def run_halo_workload(al, torch, steps, warmup):
     face_bytes = bufs[0].numel() * 8
     res = {"workload": "c5_halo", "dtype": "f64", "grid": [side] * 3, "halo": h, "face_bytes": face_bytes,
            "parity_vs_oracle": bool(ok)}
-    wall, kms = timed(torch, lambda: al.halo_pack(bufs, grid, dims, h), steps, warmup)
+    # the timed calls go straight to the C ABI with their arguments built once: a launch of a few
+    # microseconds must not be timed through ten microseconds of Python
+    import ctypes as C
+    L = al.load()
+    tab = (C.c_void_p * 6)(*[bufs[f].data_ptr() for f in range(6)])
+    cdims = (C.c_size_t * 3)(*dims)
+    gp = C.c_void_p(grid.data_ptr())
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def pack(mask):
+        assert L.alamd_halo_pack(tab, gp, cdims, h, 8, mask, st) == 0
+
+    def unpack(mask):
+        assert L.alamd_halo_unpack(gp, tab, cdims, h, 8, mask, st) == 0
+
+    wall, kms = timed(torch, lambda: pack(0x3f), steps, warmup)
     res["pack_all_us"], res["pack_all_gbps"] = kms * 1e3, 2 * 6 * face_bytes / (kms * 1e-3) * 1e-9
-    wall2, kms2 = timed(torch, lambda: al.halo_unpack(grid, bufs, dims, h), steps, warmup)
+    wall2, kms2 = timed(torch, lambda: unpack(0x3f), steps, warmup)
     res["unpack_all_us"], res["unpack_all_gbps"] = kms2 * 1e3, 2 * 6 * face_bytes / (kms2 * 1e-3) * 1e-9
+    # what the six-face launches really move (one 128-byte line per 16-byte run of an x face, 1.26 lines
+    # per row when both x faces go together; ghost runs written as 32-byte pieces): from the counter
+    # profile profiles/halo_kernel_f64_c5.md
+    res["pack_all_hbm_bytes"], res["unpack_all_hbm_bytes"] = 84213504, 59270144
+    res["pack_all_hbm_gbps"] = res["pack_all_hbm_bytes"] / (kms * 1e-3) * 1e-9
+    res["unpack_all_hbm_gbps"] = res["unpack_all_hbm_bytes"] / (kms2 * 1e-3) * 1e-9
     for f, name in enumerate(("-x", "+x", "-y", "+y", "-z", "+z")):
-        _, k1 = timed(torch, lambda: al.halo_pack({f: bufs[f]}, grid, dims, h), steps, warmup)
-        _, k2 = timed(torch, lambda: al.halo_unpack(grid, {f: bufs[f]}, dims, h), steps, warmup)
+        _, k1 = timed(torch, lambda: pack(1 << f), steps, warmup)
+        _, k2 = timed(torch, lambda: unpack(1 << f), steps, warmup)
         res["face" + name] = {"pack_us": k1 * 1e3, "pack_gbps": 2 * face_bytes / (k1 * 1e-3) * 1e-9,
                               "unpack_us": k2 * 1e3, "unpack_gbps": 2 * face_bytes / (k2 * 1e-3) * 1e-9}
+    _, k1 = timed(torch, lambda: pack(3), steps, warmup)
+    _, k2 = timed(torch, lambda: unpack(3), steps, warmup)
+    res["faces-x+x"] = {"pack_us": k1 * 1e3, "unpack_us": k2 * 1e3}
     alg = 4 * 6 * face_bytes
     res.update({"algorithmic_bytes": alg, "ms_per_step": (wall + wall2) * 1e3, "kernel_ms": kms + kms2,
                 "gbps_wall": alg / (wall + wall2) * 1e-9, "gbps_kernel": alg / ((kms + kms2) * 1e-3) * 1e-9})
