@@ -308,7 +308,7 @@ def run_halo_workload(al, torch, steps, warmup):
     # what the six-face launches really move (one 128-byte line per 16-byte run of an x face, 1.26 lines
     # per row when both x faces go together; ghost runs written as 32-byte pieces): from the counter
     # profile profiles/halo_kernel_f64_c5.md
-    res["pack_all_hbm_bytes"], res["unpack_all_hbm_bytes"] = 84213504, 59270144
+    res["pack_all_hbm_bytes"], res["unpack_all_hbm_bytes"] = 84243968, 59262464
     res["pack_all_hbm_gbps"] = res["pack_all_hbm_bytes"] / (kms * 1e-3) * 1e-9
     res["unpack_all_hbm_gbps"] = res["unpack_all_hbm_bytes"] / (kms2 * 1e-3) * 1e-9
     for f, name in enumerate(("-x", "+x", "-y", "+y", "-z", "+z")):

@@ -1227,9 +1227,26 @@ class ProgressEngine {
   ProgressEngine(const ProgressEngine &) = delete;
   ProgressEngine &operator=(const ProgressEngine &) = delete;
 
+  /** When the stream is let go on: once the host step has completed
+   *  (HostTransferCollectiveSignalAtEndState, ht/base_state.hpp:86-117), or as soon as it has been
+   *  started, for a rank whose device data the step no longer needs (the root under
+   *  HostTransferCollectiveSignalRootEarlyState, :124-163; the other ranks under
+   *  HostTransferCollectiveSignalNonRootEarlyState, :170-209). */
+  enum class SignalWhen { at_end, after_start };
+  static SignalWhen root_early(bool is_root) { return is_root ? SignalWhen::after_start : SignalWhen::at_end; }
+  static SignalWhen non_root_early(bool is_root) { return is_root ? SignalWhen::at_end : SignalWhen::after_start; }
+
+  /** A host step that runs to its end in one call. */
   void enqueue(hipStream_t stream, std::function<void()> fn) {
+    enqueue(stream, std::move(fn), [] { return true; }, SignalWhen::at_end);
+  }
+  /** A host step in two parts, like the reference's start_mpi_op() / poll_mpi(): `start` begins it and
+   *  returns, `poll` is called until it returns true (other steps make progress in between). */
+  void enqueue(hipStream_t stream, std::function<void()> start, std::function<bool()> poll, SignalWhen when) {
     auto st = std::make_unique<State>();
-    st->fn = std::move(fn);
+    st->fn = std::move(start);
+    st->poll = std::move(poll);
+    st->when = when;
     st->start.record(stream);
     st->go.wait(stream);
     st->end.record(stream);
@@ -1261,7 +1278,9 @@ class ProgressEngine {
     GPUStatusFlag start, end;
     GPUWait go;
     std::function<void()> fn;
-    bool ran = false;
+    std::function<bool()> poll;
+    SignalWhen when = SignalWhen::at_end;
+    bool started = false, signalled = false, ran = false;
   };
   void run() {
     std::unique_lock<std::mutex> lock(mutex_);
@@ -1271,23 +1290,31 @@ class ProgressEngine {
       bool progressed = false;
       for (size_t i = 0; i < states_.size();) {
         State *st = states_[i].get();
-        if (!st->ran && st->start.query()) {
+        if (!st->ran && (st->started || st->start.query())) {
           lock.unlock();
           std::exception_ptr failed;
+          bool done = false;
           try {
-            st->fn();        // phase 2, outside the lock: enqueue() may be called meanwhile
+            if (!st->started) st->fn();  // phase 2, outside the lock: enqueue() may be called meanwhile
+            st->started = true;
+            done = st->poll();
           } catch (...) {
             failed = std::current_exception();
+            done = true;  // a step that throws is over
           }
-          try {
-            st->go.signal();  // phase 3, whatever fn did: the stream must not stay blocked
-          } catch (...) {
-            if (!failed) failed = std::current_exception();
+          if (!st->signalled && (done || st->when == SignalWhen::after_start)) {
+            try {
+              st->go.signal();  // phase 3, whatever the step did: the stream must not stay blocked
+            } catch (...) {
+              if (!failed) failed = std::current_exception();
+            }
+            st->signalled = true;
           }
           lock.lock();
           if (failed && !failed_) failed_ = failed;
-          st->ran = true;
-          progressed = true;
+          st->started = true;
+          st->ran = done;
+          progressed = progressed || done;
         }
         if (st->ran && st->end.query()) {  // phase 4: the wait has been consumed
           states_.erase(states_.begin() + static_cast<long>(i));

@@ -296,6 +296,33 @@ static void test_error_recovery(hipStream_t stream) {
   EXPECT(same_bits(a.down(), want), "max of equal values after the failed launch");
 }
 
+// The early-signal policies: the stream goes on as soon as the host step has started, the step
+// itself completes later (ht/base_state.hpp:124-209).
+static void test_progress_engine_early_signal(hipStream_t stream) {
+  using PE = Al::amd::ProgressEngine;
+  EXPECT(PE::root_early(true) == PE::SignalWhen::after_start && PE::root_early(false) == PE::SignalWhen::at_end &&
+             PE::non_root_early(false) == PE::SignalWhen::after_start && PE::non_root_early(true) == PE::SignalWhen::at_end,
+         "who is let go early under the two rooted policies");
+  DevBuf<int> x(1);
+  HIPCHK(hipMemsetAsync(x.p, 0, sizeof(int), stream));
+  std::atomic<bool> release{false};
+  std::atomic<int> polls{0};
+  PE pe;
+  pe.enqueue(stream, [] {}, [&] { ++polls; return release.load(); }, PE::SignalWhen::after_start);
+  HIPCHK(hipMemsetAsync(x.p, 1, sizeof(int), stream));
+  HIPCHK(hipStreamSynchronize(stream));  // returns although the step has not completed
+  EXPECT(x.down()[0] == 0x01010101, "the stream went on after the step had started");
+  EXPECT(pe.pending() == 1, "the step itself is still in progress");
+  // an at-end step behind it on the same engine makes progress while the first one is polled
+  int ran = 0;
+  pe.enqueue(stream, [&] { ran = 1; });
+  HIPCHK(hipStreamSynchronize(stream));
+  EXPECT(ran == 1, "a later step ran while the early-signalled one was still polling");
+  release = true;
+  for (int spin = 0; spin < 2000 && pe.pending(); ++spin) std::this_thread::sleep_for(std::chrono::milliseconds(1));
+  EXPECT(pe.pending() == 0 && polls.load() > 1, "the step was polled to its end and retired");
+}
+
 // A host step that throws must not leave its stream blocked.
 static void test_progress_engine_exception(hipStream_t stream) {
   DevBuf<int> x(1);
@@ -426,6 +453,7 @@ int main() {
   test_halo_loopback(stream);
   test_halo_two_ranks(false);
   test_halo_two_ranks(true);
+  test_progress_engine_early_signal(stream);
   test_progress_engine_exception(stream);
   test_flags(stream);
   test_progress_engine(stream);
