@@ -134,7 +134,11 @@ int alamd_init(void);
  * must not overlap one partially.  `start` is the rank s of the orders that
  * have one and must be 0 otherwise.  Here and in every entry point below a
  * buffer must be aligned to its element type (ALAMD_ERR_INVALID_ARG if not);
- * no wider alignment is needed. */
+ * no wider alignment is needed.
+ * Outside every parity claim: which operand a float min / max keeps when NaN
+ * or +-0 operands meet under an order with more than two operands (the
+ * reference's own result there differs from rank to rank; the two-operand step
+ * is the MPI library's and is checked), and the payload bits of a NaN result. */
 int alamd_combine(void *const *outs, int nout, const void *const *ins, int P,
                   size_t count, int dtype, int op, int order, int start,
                   void *stream);

@@ -18,8 +18,8 @@ OPS = ["allreduce", "reduce", "reduce_scatter", "allgather", "reduce_scatterv", 
 DATATYPES = ["char", "schar", "uchar", "short", "ushort", "int", "uint", "long", "ulong", "longlong", "ulonglong",
              "float", "double", "half", "bfloat16"]
 FLOATS = ("float", "double", "half", "bfloat16")
-INT_REDUCTIONS = ["sum", "prod", "min", "max", "lor", "land", "lxor", "bor", "band", "bxor"]
-FP_REDUCTIONS = ["sum", "prod", "min", "max"]
+INT_REDUCTIONS = ["sum", "prod", "min", "max", "lor", "land", "lxor", "bor", "band", "bxor", "avg"]
+FP_REDUCTIONS = ["sum", "prod", "min", "max", "avg"]
 ALGORITHMS = {
     "allreduce": ["automatic", "rank_order", "tree_doubling", "tree_halving", "tree_binomial", "ring", "ring_fused"],
     "reduce": ["automatic", "rank_order", "tree_doubling", "tree_halving", "tree_binomial"],
@@ -42,7 +42,7 @@ def main():
     t0, fails = time.time(), 0
     for k in range(args.runs):
         op, dt = rng.choice(OPS), rng.choice(DATATYPES)
-        ranks = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16, 24, 32])
+        ranks = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16, 24, 32, 33, 40, 48, 63, 64])
         cmd = [exe, "--op", op, "--datatype", dt,
                "--reduction-op", rng.choice(FP_REDUCTIONS if dt in FLOATS else INT_REDUCTIONS),
                "--algorithm", rng.choice(ALGORITHMS[op]), "--ranks", str(ranks), "--root", str(rng.randrange(ranks)),
