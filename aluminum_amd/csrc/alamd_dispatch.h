@@ -168,7 +168,10 @@ __device__ __forceinline__ void chain_gate(const ChainParams &c, unsigned self, 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's loads have returned
   __syncthreads();                                  // ... and every other wave's of the workgroup
   if (threadIdx.x == 0) {
-    if (self < c.nvec_tiles) __hip_atomic_store(&c.flags[self], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    // Nothing this workgroup wrote has to become visible with the flag, and a waiting workgroup reads nothing
+    // that this one wrote: the flag only says "my loads are done".  Relaxed accesses that go past the caches
+    // are therefore enough; release / acquire would add a write-back and an invalidation of the L2 per tile.
+    if (self < c.nvec_tiles) __hip_atomic_store(&c.flags[self], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     // tiles t that read output bytes [w0, w0 + wlen): displ + t*TB < w0 + wlen and displ + (t+1)*TB > w0
     const long long tb = (long long)tile_bytes;
     const long long a0 = (long long)w0 - (long long)c.displ_bytes, a1 = a0 + (long long)wlen;
@@ -179,7 +182,7 @@ __device__ __forceinline__ void chain_gate(const ChainParams &c, unsigned self, 
       if (hi > (long long)c.nvec_tiles - 1) hi = (long long)c.nvec_tiles - 1;
       for (long long t = lo; t <= hi; ++t) {
         unsigned spins = 0;
-        while (__hip_atomic_load(&c.flags[t], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
+        while (__hip_atomic_load(&c.flags[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == 0u) {
           __builtin_amdgcn_s_sleep(2);
           if (++spins > kChainMaxSpins) {
             __hip_atomic_store(c.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -437,11 +437,16 @@ int reduce_scatterv_in_place(void *const *recvs, const void *const *sends, int P
     if (counts[b] == 0) continue;
     const bool inplace = recvs[b] == sends[b];
     const bool overlapped = inplace && displ[b] != 0 && displ[b] < counts[b];
-    // A few runs no longer than the displacement, each launched after the one before it, never read
-    // what an unfinished launch writes and run at the full rate (a chained launch reaches about a third
-    // of it: 1.9 to 2.5 TB/s at P = 8); more than kMaxRuns of them would be launch-bound.
+    // One or two runs no longer than the displacement, each launched after the one before it, never read
+    // what an unfinished launch writes; beyond that one chained launch (85 to 100 % of the ordinary rate at
+    // P = 8) beats a train of launches.  With the fixed scratch too small for the block, up to kMaxRuns
+    // plain launches stand in.
     constexpr size_t kMaxRuns = 32;
-    const bool chained = overlapped && (counts[b] + displ[b] - 1) / displ[b] > kMaxRuns;
+    const size_t runs = overlapped ? (counts[b] + displ[b] - 1) / displ[b] : 1;
+    bool chained = runs > 2;
+    if (chained && fixed && runs <= kMaxRuns &&
+        (counts[b] * es + kChainMinTileBytes - 1) / kChainMinTileBytes > fixed->max_tiles)
+      chained = false;
     const size_t run = overlapped && !chained ? displ[b] : counts[b];
     int rc = ALAMD_OK;
     for (size_t done = 0; done < counts[b] && rc == ALAMD_OK; done += run) {

@@ -202,8 +202,13 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
       q.seg.seg0 = 0;
       q.seg.mapped = 0;
       void (*ck)(const FoldParams) = nullptr;
-      if constexpr (FP_MINMAX) ck = roles ? fold_vec_kernel<T, OP, true, 0, false, true> : fold_vec_kernel<T, OP, false, 0, false, true>;
-      else ck = fold_vec_kernel<T, OP, false, 0, false, true>;
+      if (p.P == 8) {  // all eight streams in flight at once, as in the ordinary launches
+        if constexpr (FP_MINMAX) ck = roles ? fold_vec_kernel<T, OP, true, 8, false, true> : fold_vec_kernel<T, OP, false, 8, false, true>;
+        else ck = fold_vec_kernel<T, OP, false, 8, false, true>;
+      } else {
+        if constexpr (FP_MINMAX) ck = roles ? fold_vec_kernel<T, OP, true, 0, false, true> : fold_vec_kernel<T, OP, false, 0, false, true>;
+        else ck = fold_vec_kernel<T, OP, false, 0, false, true>;
+      }
       hipLaunchKernelGGL(ck, dim3((unsigned)tickets, 1, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
       ALAMD_HIP(hipGetLastError());
       return ALAMD_OK;

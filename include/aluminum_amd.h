@@ -165,10 +165,11 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P,
  * the orders that have one.  In-place form (recvs[b] == sends[b]) puts the
  * result at the start of the buffer; any counts are accepted, as by the
  * reference.  A block that is in place and starts fewer elements into its own
- * buffer than it is long is read and overwritten at a displacement: in up to
- * 32 launches no longer than the displacement, else in one launch whose
- * workgroups order themselves through a ticket counter and one flag per tile
- * in device scratch memory (allocated per stream on first need and kept).
+ * buffer than it is long is read and overwritten at a displacement: in two
+ * launches no longer than the displacement where they suffice, else in one
+ * launch whose workgroups order themselves through a ticket counter and one
+ * flag per tile in device scratch memory (allocated per stream on first need
+ * and kept).
  * Replaces MPI_Ireduce_scatter on the host copy
  * (include/aluminum/ht/reduce_scatterv.hpp:40-87). */
 int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P,
@@ -183,8 +184,9 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P,
  * its own input (see alamd_reduce_scatterv) live in a fixed array of
  * ALAMD_NOALLOC_SCRATCH_BYTES that is part of the library's code object (every
  * device the library runs on holds its copy until the process ends).  Limit:
- * such a block may be at most ALAMD_NOALLOC_MAX_BLOCK_BYTES long
- * (ALAMD_ERR_INVALID_ARG beyond that; blocks that do not overlap their own
+ * such a block may be at most ALAMD_NOALLOC_MAX_BLOCK_BYTES long unless it
+ * starts at least a 32nd of its length into its buffer (then up to 32 plain
+ * launches do; ALAMD_ERR_INVALID_ARG otherwise; blocks that do not overlap their own
  * input, and separate receive buffers, have no limit).  All calls on one device
  * share the array: calls that overlap in time on one device (different
  * streams, different threads) race; keep them on one stream. */

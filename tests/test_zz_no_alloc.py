@@ -62,3 +62,13 @@ def test_noalloc_limit_is_an_error(al):
     al.reduce_scatterv_noalloc(recvs, bufs, counts, "bor", dtype="u8")
     torch.cuda.synchronize()
     assert int(recvs[1].max()) == 0
+    del recvs, bufs
+    # as long a block that starts a 16th of its length into its buffer: plain launches stand in for the chain
+    counts = [(limit + 4096) // 16, limit + 4096]
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    bufs = [torch.randint(0, 256, (sum(counts),), dtype=torch.uint8, device="cuda", generator=gen) for _ in range(2)]
+    want = [bufs[0][:counts[0]] | bufs[1][:counts[0]], bufs[0][counts[0]:] | bufs[1][counts[0]:]]
+    al.reduce_scatterv_noalloc(bufs, bufs, counts, "bor", dtype="u8")
+    torch.cuda.synchronize()
+    for b in range(2):
+        assert torch.equal(bufs[b][:counts[b]], want[b]), "long in-place block, rank %d" % b
