@@ -256,8 +256,8 @@ struct Posting {
   void *recv = nullptr;
   hipStream_t stream = nullptr;
   std::shared_ptr<Request> req;  // non-blocking: the caller's request, completed at launch
-  hipEvent_t ready = nullptr;    // recorded on `stream` at the call, unless an earlier rank of this
-                                 // operation has the same stream (then that rank's event stands for both)
+  hipEvent_t ready = nullptr;    // recorded on `stream` at the call; of the ranks of one operation that
+                                 // share a stream, the one that called last holds their common event
   bool posted = false;
 };
 
@@ -404,12 +404,17 @@ inline void World::post(Communicator &c, OpKind kind, int dtype, const void *sen
     AL_AMD_THROW("Logical ranks disagree on the arguments of a collective");
   // The dependency on the rank's stream is taken now, not when the last rank calls: the collective
   // waits for what was enqueued before this call, and for nothing that is enqueued after it.
+  // Ranks that share a stream share one event, recorded again at each of their calls, so that it
+  // stands for the latest of them.
   hipEvent_t ready = nullptr;
-  bool shared = false;
-  if (slot)
-    for (const Posting &other : slot->ranks) shared = shared || (other.posted && other.stream == c.get_stream());
-  if (!shared && c.get_stream() != target_of(req != nullptr, dtype, count, cv)) {
-    ready = events_->take();
+  if (c.get_stream() != target_of(req != nullptr, dtype, count, cv)) {
+    if (slot)
+      for (Posting &other : slot->ranks)
+        if (other.posted && other.stream == c.get_stream() && other.ready) {
+          ready = other.ready;
+          other.ready = nullptr;
+        }
+    if (!ready) ready = events_->take();
     const hipError_t e = hipEventRecord(ready, c.get_stream());
     if (e != hipSuccess) {
       events_->give(ready);
@@ -483,10 +488,12 @@ inline void *World::attach(int me, int peer, void *mine) {
   mail(me, peer).attached.push_back(mine);
   Mail &in = mail(peer, me);
   if (in.attached.empty()) {
-    if (!calls_wait_)
+    if (!calls_wait_) {
+      mail(me, peer).attached.pop_back();  // a call that throws leaves nothing behind
       AL_AMD_THROW("AttachRemoteBuffer: the peer has not attached its buffer yet. All logical ranks share one "
                    "address space, so a peer's pointer can be given to Put as it is; the exchange itself needs "
                    "one thread per rank and World::set_calls_wait_for_launch(true)");
+    }
     launched_cv_.wait(lock, [&] { return !in.attached.empty(); });
   }
   void *theirs = in.attached.front();

@@ -255,6 +255,52 @@ static void test_stream_order(bool threaded) {
   for (auto &s : streams) HIPCHK(hipStreamDestroy(s));
 }
 
+// Every rank on one stream, a non-blocking operation large enough for the internal stream, each rank's
+// producer enqueued just before its call: the operation has to wait for the last producer, not the first.
+static void test_stream_order_shared_stream() {
+  const int P = 3;
+  const size_t n = (6u << 20) / sizeof(float);
+  hipStream_t s;
+  HIPCHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  {
+    Al::amd::World world(P, s);
+    std::vector<std::vector<float>> in;
+    std::vector<std::unique_ptr<DevBuf<float>>> buf;
+    std::vector<float *> pinned_in(P);
+    float *pinned_out = nullptr;
+    HIPCHK(hipHostMalloc(reinterpret_cast<void **>(&pinned_out), n * sizeof(float), hipHostMallocDefault));
+    for (int r = 0; r < P; ++r) {
+      in.push_back(gen<float>(n, ALO_DIST_UNIFORM_PM1, 190u + (unsigned)r));
+      buf.emplace_back(new DevBuf<float>(n));
+      HIPCHK(hipMemset(buf[r]->p, 0, n * sizeof(float)));
+      HIPCHK(hipHostMalloc(reinterpret_cast<void **>(&pinned_in[r]), n * sizeof(float), hipHostMallocDefault));
+      std::memcpy(pinned_in[r], in[r].data(), n * sizeof(float));
+    }
+    Al::amd::GPUWait gate;
+    gate.wait(s, 1u << 24);
+    std::vector<Backend::req_type> reqs(P);
+    for (int r = 0; r < P; ++r) {
+      HIPCHK(hipMemcpyAsync(buf[r]->p, pinned_in[r], n * sizeof(float), hipMemcpyHostToDevice, s));  // producer
+      Al::NonblockingAllreduce<Backend>(buf[r]->p, n, Op::sum, world.comm(r), reqs[r], Algo::rank_order);
+    }
+    std::this_thread::sleep_for(std::chrono::milliseconds(3));
+    gate.signal();
+    for (int r = 0; r < P; ++r) Al::Wait<Backend>(reqs[r]);
+    HIPCHK(hipMemcpyAsync(pinned_out, buf[P - 1]->p, n * sizeof(float), hipMemcpyDeviceToHost, s));
+    HIPCHK(hipStreamSynchronize(s));
+    std::vector<float> want(n);
+    std::vector<const void *> ptrs;
+    for (auto &b : in) ptrs.push_back(b.data());
+    alo_combine(want.data(), ptrs.data(), P, n, ALO_F32, ALO_SUM, ALO_ORDER_RANK_ASC, 0);
+    EXPECT(!gate.timed_out(), "the gate must not have expired");
+    EXPECT(std::memcmp(pinned_out, want.data(), n * sizeof(float)) == 0,
+           "one stream for every rank: the operation waited for the last rank's producer");
+    for (int r = 0; r < P; ++r) HIPCHK(hipHostFree(pinned_in[r]));
+    HIPCHK(hipHostFree(pinned_out));
+  }
+  HIPCHK(hipStreamDestroy(s));
+}
+
 // A call that throws leaves its communicator where it was; a launch that fails is reported to the
 // ranks that have already returned.
 static void test_error_recovery(hipStream_t stream) {
@@ -450,6 +496,7 @@ int main() {
   test_threads_and_streams();
   test_stream_order(false);
   test_stream_order(true);
+  test_stream_order_shared_stream();
   test_halo_loopback(stream);
   test_halo_two_ranks(false);
   test_halo_two_ranks(true);
