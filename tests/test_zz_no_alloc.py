@@ -72,3 +72,41 @@ def test_noalloc_limit_is_an_error(al):
     torch.cuda.synchronize()
     for b in range(2):
         assert torch.equal(bufs[b][:counts[b]], want[b]), "long in-place block, rank %d" % b
+
+
+def test_noalloc_in_a_hip_graph(al):
+    """What the entry point is for: an in-place Reduce_scatterv whose block overlaps its own input,
+    captured into a HIP graph (no allocation may happen under capture; the scratch is cleared by a
+    kernel).  Every replay, with fresh inputs and eager work in between, gives the oracle's bits."""
+    import torch
+    P, counts = 3, [1, 2_000_003, 7]
+    total = sum(counts)
+    src = [dev_empty(total, np.float32) for _ in range(P)]
+    work = [dev_empty(total, np.float32) for _ in range(P)]
+
+    def run():
+        for r in range(P):
+            al.copy(work[r], src[r])
+        al.reduce_scatterv_noalloc(work, work, counts, "sum", order="tree_halv", dtype="f32")
+
+    for t in src:
+        t.zero_()
+    run()  # eager warm-up outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        run()
+    for rep in range(3):
+        fresh = [oracle.fill(total, "f32", "uniform_pm1", 700 + 10 * rep + r) for r in range(P)]
+        for t, a in zip(src, fresh):
+            t.copy_(torch.from_numpy(a))  # eager work between the replays
+        for t in work:
+            t.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        want = oracle.reduce_scatterv(fresh, counts, "f32", "sum", "tree_halv")
+        for b in range(P):
+            got = to_host(work[b], np.float32)
+            assert_bits_equal(got[:counts[b]], want[b], "f32", "graph replay %d rank %d" % (rep, b))
+            assert got[counts[b]:].tobytes() == fresh[b][counts[b]:].tobytes(), "bytes behind the result changed"
