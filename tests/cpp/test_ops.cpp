@@ -70,6 +70,7 @@ template <typename T> int run(const Options &o, Op rop, Algo algo) {
     }
   HIPCHK(hipStreamDestroy(stream));
   std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks, g_fail);
+  std::fflush(stdout);  // before the runtime libraries are torn down
   return g_fail ? 1 : 0;
 }
 
