@@ -56,7 +56,7 @@ KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false /*o
 DEFAULT_ALSO = ("c2_f32_sum_rotating,c2_f32_prod,c2_bf16_sum,c2_bf16_sum_rotating,c4_i32_max,c4_i64_bxor,"
                 "c4_u8_lxor,c3_ring_stepwise,c3_ring_fused,c5_halo,flags,c2_f32_allreduce,"
                 "c2_f32_allreduce_rotating,c2_f32_reduce_scatter,c2_f32_reduce_scatter_rotating,"
-                "c2_f32_allgather,c2_f32_allgather_rotating")
+                "c2_f32_allgather,c2_f32_allgather_rotating,c2_f32_reduce_scatterv_in_place")
 
 
 def measured_traffic(workload):
@@ -180,6 +180,7 @@ def run_ring_workload(al, torch, mode, steps, warmup):
 
 
 LAYOUTS = [w + r for w in ("c2_f32_allreduce", "c2_f32_allgather", "c2_f32_reduce_scatter") for r in ("", "_rotating")]
+LAYOUTS.append("c2_f32_reduce_scatterv_in_place")
 
 
 def run_layout_workload(al, torch, name, steps, warmup):
@@ -191,6 +192,9 @@ def run_layout_workload(al, torch, name, steps, warmup):
     c2_f32_reduce_scatter - eight send buffers of 2^26 elements, block b folded into receive buffer b of
     2^23 elements (order pairwise_desc from the receiving rank: what MPI_Reduce_scatter_block yields above
     512 KiB).
+    c2_f32_reduce_scatterv_in_place - eight buffers of 2^26 elements, counts (1, 2^26 - 1, 0, ...), in place:
+    rank 1's block of 2^26 - 1 elements is read one element behind where its result is written, the worst
+    case of the chained launch (every tile waits for its neighbour's loads).
     With the suffix _rotating the calls go round four sets of buffers, so that nothing a call reads or
     writes was touched by the three calls before it (no help from the 256 MiB memory-side cache)."""
     import oracle
@@ -247,6 +251,21 @@ def run_layout_workload(al, torch, name, steps, warmup):
                     want = oracle.fill(m, "f32", "uniform_pm1", 1000 + q, count - m)
                     got = recvs[j][(q + 1) * count - m:(q + 1) * count].cpu().numpy()
                     ok = ok and got.tobytes() == want.tobytes()
+        elif base == "c2_f32_reduce_scatterv_in_place":
+            count = 1 << 26
+            counts = [1, count - 1] + [0] * (P - 2)
+            bufs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
+            for r in range(P):
+                al.fill(bufs[r], "uniform_pm1", 1000 + r)
+            fn = lambda bufs=bufs, counts=counts: al.reduce_scatterv(bufs, bufs, counts, "sum",
+                                                                     order="pairwise_desc", dtype="f32")
+            alg = (P + 1) * count * 4
+            launches = 3  # the one-element block, the clearing of the tile flags, the chained fold
+            fn()  # later calls fold what this one left: the same traffic, other values
+            torch.cuda.synchronize()
+            for lo in (0, count - 1 - m):
+                want = oracle.combine_generated(P, m, "f32", "sum", "pairwise_desc", 1, "uniform_pm1", 1000, 1 + lo)
+                ok = ok and bufs[1][lo:lo + m].cpu().numpy().tobytes() == want.tobytes()
         else:
             raise SystemExit("unknown workload %s" % name)
         fns.append(fn)
