@@ -64,6 +64,8 @@ def load():
     L.alamd_reduce_scatterv.argtypes = [pvp, pvp, i, C.POINTER(sz), i, i, i, vp]
     L.alamd_reduce_scatterv_noalloc.argtypes = [pvp, pvp, i, C.POINTER(sz), i, i, i, vp]
     L.alamd_allgatherv.argtypes = [pvp, pvp, i, C.POINTER(sz), C.POINTER(sz), i, vp]
+    L.alamd_reduce_scatterv_wait_expired.argtypes = []
+    L.alamd_set_chain_poll_limit.argtypes = [C.c_uint]
     L.alamd_ring_allreduce.argtypes = [pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_reduce_scatter.argtypes = [pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_allgather.argtypes = [pvp, i, sz, i, sz, vp]
@@ -192,6 +194,16 @@ def reduce_scatterv_noalloc(recvs, sends, counts, op, order="rank_asc", dtype=No
     P = len(sends)
     _check(load().alamd_reduce_scatterv_noalloc(_table(recvs), _table(sends), P, (C.c_size_t * P)(*counts),
                                                 _dt(dtype), _op(op), _order(order), _stream(stream)))
+
+
+def reduce_scatterv_wait_expired():
+    """True, once, if a wait inside a chained in-place Reduce_scatterv launch has given up since the last call."""
+    return bool(load().alamd_reduce_scatterv_wait_expired())
+
+
+def set_chain_poll_limit(polls):
+    """Polls after which such a wait gives up (0: the default); for tests of that path."""
+    _check(load().alamd_set_chain_poll_limit(polls))
 
 
 def allgatherv(recvs, sends, counts, displs, dtype=None, stream=None):

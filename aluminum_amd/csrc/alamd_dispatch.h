@@ -144,15 +144,17 @@ __host__ __device__ inline void out_select(const SegParams &s, int P, unsigned s
 //    the same way.
 // The counter and the flags are scratch memory in HBM, cleared on the stream
 // before the launch.  A wait is bounded: if it expires (it cannot, unless the
-// device loses a workgroup) the error word is set and the workgroup goes on.
+// device loses a workgroup) the error word, which the host can read, is set and
+// the workgroup goes on.
 struct ChainParams {
   unsigned *ticket;                 // next tile; null: not a chained launch
   unsigned *flags;                  // flags[t] != 0: tile t has loaded its inputs
   unsigned *error;                  // set to 1 by a wait that expired
   unsigned long long displ_bytes;   // the overlapping input starts this far behind the output
   unsigned nvec_tiles;              // whole-vector tiles (the tail is ticket nvec_tiles)
+  unsigned max_polls;               // polls of one flag before a wait gives up
 };
-constexpr unsigned kChainMaxSpins = 1u << 24;
+constexpr unsigned kChainDefaultPolls = 1u << 24;
 
 __device__ __forceinline__ unsigned chain_take_tile(const ChainParams &c) {
   __shared__ unsigned s_tile;
@@ -184,8 +186,8 @@ __device__ __forceinline__ void chain_gate(const ChainParams &c, unsigned self, 
         unsigned spins = 0;
         while (__hip_atomic_load(&c.flags[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == 0u) {
           __builtin_amdgcn_s_sleep(2);
-          if (++spins > kChainMaxSpins) {
-            __hip_atomic_store(c.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (++spins >= c.max_polls) {
+            __hip_atomic_store(c.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             break;
           }
         }
@@ -303,7 +305,7 @@ void plan_launches(SegParams &seg, unsigned nseg, size_t max_len, size_t tile_el
 
 // chain: null for an ordinary launch; else the scratch of a chained launch (one segment, one output,
 // every tile in one launch; displ_bytes and nvec_tiles are filled in here).
-struct ChainScratch { unsigned *ticket, *flags, *error; size_t max_tiles; };
+struct ChainScratch { unsigned *ticket, *flags, *error; size_t max_tiles; unsigned max_polls; };
 int launch_fold(const FoldParams &p, unsigned nseg, size_t max_len, int dtype, int op, bool acc_is_in,
                 hipStream_t stream, const ChainScratch *chain = nullptr, size_t displ_bytes = 0);
 int launch_tree(const TreeParams &p, int slots, unsigned nseg, size_t max_len, int dtype, int op,

@@ -1,6 +1,7 @@
 // Host side of the combine entry points: argument checks, the mapping of a
 // named order onto one of the two kernel families, the Reduce_scatter and
 // Allgather layouts.
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <string>
@@ -122,6 +123,38 @@ ChainPool &chain_pool() {
   return *pool;
 }
 
+// Where a wait that gave up leaves its mark: one word of pinned host memory for the whole process,
+// allocated by alamd_init (or by the first chained launch that may allocate), so that the host can
+// read it without touching the device.  Until it exists the mark goes to the scratch's own word.
+std::mutex g_expired_mutex;
+unsigned *g_expired_host = nullptr, *g_expired_dev = nullptr;
+std::atomic<unsigned> g_chain_polls{kChainDefaultPolls};
+
+int expired_word_init() {
+  std::lock_guard<std::mutex> lock(g_expired_mutex);
+  if (g_expired_host) return ALAMD_OK;
+  void *host = nullptr, *dev = nullptr;
+  ALAMD_HIP(hipHostMalloc(&host, 256, hipHostMallocMapped | hipHostMallocCoherent | hipHostMallocPortable));
+  *static_cast<volatile unsigned *>(host) = 0u;
+  ALAMD_HIP(hipHostGetDevicePointer(&dev, host, 0));
+  g_expired_dev = static_cast<unsigned *>(dev);
+  g_expired_host = static_cast<unsigned *>(host);
+  return ALAMD_OK;
+}
+
+// 1 (once) if a chained launch has given up a wait since the last call.
+bool take_expired() {
+  std::lock_guard<std::mutex> lock(g_expired_mutex);
+  if (!g_expired_host) return false;
+  return __atomic_exchange_n(g_expired_host, 0u, __ATOMIC_SEQ_CST) != 0u;
+}
+
+void finish_scratch(ChainScratch &cs) {
+  std::lock_guard<std::mutex> lock(g_expired_mutex);
+  if (g_expired_dev) cs.error = g_expired_dev;
+  cs.max_polls = g_chain_polls.load();
+}
+
 ChainScratch scratch_at(void *base, size_t bytes) {
   ChainScratch cs;
   char *b = static_cast<char *>(base);
@@ -129,18 +162,21 @@ ChainScratch scratch_at(void *base, size_t bytes) {
   cs.error = reinterpret_cast<unsigned *>(b + 4);
   cs.flags = reinterpret_cast<unsigned *>(b + kChainHeaderBytes);
   cs.max_tiles = (bytes - kChainHeaderBytes) / sizeof(unsigned);
+  cs.max_polls = kChainDefaultPolls;
   return cs;
 }
 
 int chain_scratch_for(hipStream_t stream, size_t tiles, ChainScratch &out) {
   int dev = 0;
   ALAMD_HIP(hipGetDevice(&dev));
+  if (int rc = expired_word_init()) return rc;
   ChainPool &pool = chain_pool();
   std::lock_guard<std::mutex> lock(pool.mutex);
   auto key = std::make_pair(dev, stream);
   auto it = pool.live.find(key);
   if (it != pool.live.end() && it->second.max_tiles >= tiles) {
     out = it->second;
+    finish_scratch(out);
     return ALAMD_OK;
   }
   size_t cap = (size_t)1 << 16;
@@ -152,6 +188,7 @@ int chain_scratch_for(hipStream_t stream, size_t tiles, ChainScratch &out) {
   if (it != pool.live.end()) pool.retired.push_back(it->second.ticket);
   out = scratch_at(mem, bytes);
   pool.live[key] = out;
+  finish_scratch(out);
   return ALAMD_OK;
 }
 
@@ -178,6 +215,7 @@ int static_chain_scratch(ChainScratch &out) {
     g_static_ptr[dev] = ptr;
   }
   out = scratch_at(g_static_ptr[dev], ALAMD_NOALLOC_SCRATCH_BYTES);
+  finish_scratch(out);
   return ALAMD_OK;
 }
 
@@ -277,6 +315,7 @@ int check_common(int P, size_t count, int dtype) {
 }  // namespace
 
 int chain_static_init() {
+  if (int rc = expired_word_init()) return rc;
   ChainScratch cs;
   return static_chain_scratch(cs);
 }
@@ -630,6 +669,9 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P, size_t 
 
 static int reduce_scatterv_impl(void *const *recvs, const void *const *sends, int P, const size_t *counts,
                                int dtype, int op, int order, void *stream, const ChainScratch *fixed) {
+  if (take_expired())
+    return set_error(ALAMD_ERR_TIMEOUT, "an earlier in-place Reduce_scatterv gave up waiting for a tile of its chained "
+                                        "launch: its result is not valid (this call has done nothing)");
   int rc = check_common(P, 0, dtype);
   if (rc) return rc;
   if ((rc = check_type_op(dtype, op))) return rc;
@@ -698,6 +740,13 @@ int alamd_reduce_scatterv_noalloc(void *const *recvs, const void *const *sends, 
   const int rc = static_chain_scratch(cs);
   if (rc) return rc;
   return reduce_scatterv_impl(recvs, sends, P, counts, dtype, op, order, stream, &cs);
+}
+
+int alamd_reduce_scatterv_wait_expired(void) { return take_expired() ? 1 : 0; }
+
+int alamd_set_chain_poll_limit(unsigned polls) {
+  g_chain_polls.store(polls ? polls : kChainDefaultPolls);
+  return ALAMD_OK;
 }
 
 int alamd_allgatherv(void *const *recvs, const void *const *sends, int P, const size_t *counts,

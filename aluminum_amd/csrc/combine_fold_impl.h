@@ -184,7 +184,7 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
     const size_t tile_elems = Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES / sizeof(T);
     FoldParams q = p;
     q.div = make_divisor(p.P);
-    q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0};
+    q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0, 0};
     if (chain) {
       // one segment, one output, every tile in one launch, tiles handed out by the ticket counter
       if (nseg != 1) return set_error(ALAMD_ERR_INVALID_ARG, "a chained fold has one segment");
@@ -197,7 +197,7 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
                          max_len, nvec, chain->max_tiles);
       int rc = chain_clear(*chain, nvec, stream);
       if (rc) return rc;
-      q.chain = ChainParams{chain->ticket, chain->flags, chain->error, displ_bytes, (unsigned)nvec};
+      q.chain = ChainParams{chain->ticket, chain->flags, chain->error, displ_bytes, (unsigned)nvec, chain->max_polls};
       q.seg.tile0 = 0;
       q.seg.seg0 = 0;
       q.seg.mapped = 0;

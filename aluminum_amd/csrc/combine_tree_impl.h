@@ -188,7 +188,7 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES);
   TreeParams q = p;
   q.div = make_divisor(p.P);
-  q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0};
+  q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0, 0};
   if (chain.scratch) {
     if (nseg != 1) return set_error(ALAMD_ERR_INVALID_ARG, "a chained combine has one segment");
     constexpr size_t N = 16 / sizeof(T);
@@ -201,7 +201,7 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
     int rc = chain_clear(*chain.scratch, nvec, stream);
     if (rc) return rc;
     q.chain = ChainParams{chain.scratch->ticket, chain.scratch->flags, chain.scratch->error, chain.displ_bytes,
-                          (unsigned)nvec};
+                          (unsigned)nvec, chain.scratch->max_polls};
     q.seg.tile0 = 0;
     q.seg.seg0 = 0;
     q.seg.mapped = 0;

@@ -176,6 +176,16 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P,
                           const size_t *counts, int dtype, int op, int order,
                           void *stream);
 
+/* The waits inside a chained in-place launch (see alamd_reduce_scatterv) are
+ * bounded, so that a device that loses a workgroup cannot hang the stream; a
+ * wait that gives up lets its workgroup go on, and the block's result is then
+ * not valid.  This returns 1, once, if that has happened since the last call
+ * (meaningful once the streams concerned have been synchronised); the next
+ * alamd_reduce_scatterv / _noalloc call reports it too, with
+ * ALAMD_ERR_TIMEOUT, and does nothing else.  No counterpart in the reference,
+ * whose collectives wait without bound. */
+int alamd_reduce_scatterv_wait_expired(void);
+
 /* alamd_reduce_scatterv for callers that cannot allocate device memory: code
  * under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc.  It has no counterpart in the reference.  Same arguments, same

@@ -35,6 +35,10 @@ int alamd_fill(void *dst, size_t count, int dtype, int dist, uint64_t seed,
  * checked). */
 int alamd_narrow_f32(void *dst16, const float *src, size_t count, int dtype, void *stream);
 int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void *stream);
+/* Polls after which a wait inside a chained in-place Reduce_scatterv launch
+ * gives up (0 restores the default, 2^24): lets a test make waits expire
+ * without anything being wrong with the device. */
+int alamd_set_chain_poll_limit(unsigned polls);
 #ifdef __cplusplus
 }
 #endif

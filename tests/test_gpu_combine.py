@@ -502,3 +502,36 @@ def test_collectives_in_a_hip_graph(al):
                               "replay %d reduce_scatterv rank %d" % (rep, r))
             assert_bits_equal(to_host(ag_out[r], np.float32), want_ag, "f32", "replay %d allgatherv rank %d" % (rep, r))
             assert_bits_equal(to_host(ring[r], np.float32), want_ring, "f32", "replay %d ring rank %d" % (rep, r))
+
+
+def test_reduce_scatterv_chained_wait_that_gives_up_is_reported(al):
+    """The waits inside a chained in-place launch are bounded.  With the bound set to a single poll
+    (a hook for this test; nothing is wrong with the device and every kernel ends normally) some tile
+    finds its neighbour's loads not yet done and gives up: the result of that call is not valid, the
+    query says so once, and so does the next Reduce_scatterv, after which everything works again."""
+    import torch
+    P, counts = 4, [1, 6_000_000, 3, 0]
+    sends = make_inputs(P, sum(counts), "f32", "sum")
+    want = oracle.reduce_scatterv(sends, counts, "f32", "sum", "rank_asc")
+    assert not al.reduce_scatterv_wait_expired()
+    try:
+        al.set_chain_poll_limit(1)
+        bufs = [to_dev(a) for a in sends]
+        al.reduce_scatterv(bufs, bufs, counts, "sum", order="rank_asc", dtype="f32")
+        torch.cuda.synchronize()
+        assert al.reduce_scatterv_wait_expired(), "no wait gave up although one poll was all they had"
+        assert not al.reduce_scatterv_wait_expired(), "reported once only"
+        bufs = [to_dev(a) for a in sends]
+        al.reduce_scatterv(bufs, bufs, counts, "sum", order="rank_asc", dtype="f32")
+        torch.cuda.synchronize()
+    finally:
+        al.set_chain_poll_limit(0)
+    bufs = [to_dev(a) for a in sends]
+    with pytest.raises(al.AlError, match="gave up waiting") as e:  # the second call's waits gave up as well
+        al.reduce_scatterv(bufs, bufs, counts, "sum", order="rank_asc", dtype="f32")
+    assert e.value.code == 7
+    al.reduce_scatterv(bufs, bufs, counts, "sum", order="rank_asc", dtype="f32")
+    torch.cuda.synchronize()
+    assert not al.reduce_scatterv_wait_expired()
+    for b in range(P):
+        assert_bits_equal(to_host(bufs[b], np.float32)[:counts[b]], want[b], "f32", "after the report, rank %d" % b)
