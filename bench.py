@@ -50,7 +50,7 @@ TRAFFIC_PROFILE = {"c2_f32_sum": "profiles/fold_vec_kernel_f32_sum_P8_c2.md"}
 KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false /*operand roles*/, 8 /*ranks*/, "
                              "false /*no leading elements*/, false /*not chained*/>"}
 
-# Everything BASELINE.json configures, beside the primary workload: C2 prod and bf16, the same over
+# Every configuration of the headline benchmark beside the primary workload: C2 prod and bf16, the same over
 # buffers no earlier call has touched, C4 (integer / bitwise / logical), C3 (ring, both modes), C5 (halo
 # faces), the stream flags, and the layouts an Allreduce / Reduce_scatter / Allgather reaches the kernels in.
 DEFAULT_ALSO = ("c2_f32_sum_rotating,c2_f32_prod,c2_bf16_sum,c2_bf16_sum_rotating,c4_i32_max,c4_i64_bxor,"
