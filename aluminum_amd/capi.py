@@ -66,6 +66,9 @@ def load():
     L.alamd_allgatherv.argtypes = [pvp, pvp, i, C.POINTER(sz), C.POINTER(sz), i, vp]
     L.alamd_reduce_scatterv_wait_expired.argtypes = []
     L.alamd_set_chain_poll_limit.argtypes = [C.c_uint]
+    L.alamd_tune.argtypes = [C.c_char_p, sz]
+    L.alamd_tuned.argtypes = [C.c_char_p]
+    L.alamd_tuned.restype = sz
     L.alamd_ring_allreduce.argtypes = [pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_reduce_scatter.argtypes = [pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_allgather.argtypes = [pvp, i, sz, i, sz, vp]
@@ -204,6 +207,15 @@ def reduce_scatterv_wait_expired():
 def set_chain_poll_limit(polls):
     """Polls after which such a wait gives up (0: the default); for tests of that path."""
     _check(load().alamd_set_chain_poll_limit(polls))
+
+
+def tune(name, value):
+    """Sets one of the launch planners' sizes (0: its default); speed only, never results."""
+    _check(load().alamd_tune(name.encode(), value))
+
+
+def tuned(name):
+    return int(load().alamd_tuned(name.encode()))
 
 
 def allgatherv(recvs, sends, counts, displs, dtype=None, stream=None):

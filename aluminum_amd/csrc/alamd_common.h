@@ -30,6 +30,20 @@ void clear_error();
 // error (message set).
 int device_cus();
 
+// The sizes the launch planners work with (what each one means, and the measurements behind its default,
+// stands where it is used).  Defaults suit an MI355X; alamd_tune() changes them for comparisons.
+struct Tunables {
+  size_t launch_bytes = (size_t)800 << 20;          // bytes one fold / tree launch moves
+  size_t two_step_min_bytes = (size_t)16 << 20;     // fold + spread instead of one kernel: from this size ...
+  size_t two_step_min_outputs = 3;                  // ... and this many outputs up
+  size_t two_step_piece_bytes = (size_t)128 << 20;  // piece of the result the two steps alternate over
+  size_t ring_piece_bytes = (size_t)256 << 20;      // the same for the fused ring allreduce
+  size_t spread_launch_bytes = (size_t)288 << 20;   // bytes one spread launch moves
+  size_t spread_hbm_chunk_tiles = 1024, spread_hbm_launch_chunks = 2;      // slices read from HBM
+  size_t spread_cache_chunk_tiles = 512, spread_cache_launch_chunks = 16;  // a result just written
+};
+Tunables &tunables();
+
 // Checks (dtype, op) as alamd_check_op does, setting the error message.
 int check_type_op(int dtype, int op);
 

@@ -327,20 +327,20 @@ int chain_static_init();
 // 77 / 84, 40 MiB 119 / 103, 64 MiB 196 / 162, 128 MiB 394 / 318 (the two steps
 // take the same time either way).  At 256 MiB: two outputs 437 / 455, four
 // 544 / 529.
-constexpr size_t kTwoStepMinBytes = (size_t)16 << 20;
-constexpr int kTwoStepMinOutputs = 3;
+// (Tunables::two_step_min_bytes, two_step_min_outputs)
 // The two steps alternate over pieces of the result of this many bytes, so that
 // the spread reads what the fold has just written from the 256 MiB memory-side
 // cache instead of HBM (P = 8, 1 GiB per rank, buffers no earlier call has
 // touched: 80 % of peak with pieces of 64 to 256 MiB, 75 % with the whole
 // result folded first; no difference up to 256 MiB per rank, which stay one piece).
-constexpr size_t kTwoStepPieceBytes = (size_t)128 << 20;
+// (Tunables::two_step_piece_bytes)
 // The fused ring allreduce does the same over pieces of this many bytes in all
-// (8 MiB of each of eight segments: one fold launch of 4096 workgroups, one
-// spread launch).  P = 8, untouched buffers, 256 MiB / 1 GiB per rank: 81.6 % /
-// 81.3 % of peak; 80 % / 80 % with pieces of 32 MiB or 256 MiB, 75 % with 16 or
-// 48 MiB, 80 % / 77 % with the whole result folded first.
-constexpr size_t kRingPieceBytes = (size_t)64 << 20;
+// (32 MiB of each of eight segments: what the memory-side cache holds).  P = 8,
+// bf16, untouched buffers, 256 MiB / 1 GiB per rank, default and alternatives
+// taking turns in one process: 256 MiB pieces 79.6 % / 79.6 % of peak, 64 MiB
+// 78.5 % / 77.8 %, 128 MiB - / 79.1 %, 512 MiB and the whole result folded
+// first - / 71.5 % (at 256 MiB per rank the whole result is one piece).
+// (Tunables::ring_piece_bytes)
 
 // Copies [src, src + bytes) to each of dests[0..ndest) (none overlapping the
 // source, any alignment).

@@ -37,14 +37,14 @@ constexpr unsigned kRsrcFlags = 0x00020000u;
 // The rule below picks 16384, 8192, 8192, 4096, 4096 and 2048 for these.
 constexpr size_t kLaunchBytes = (size_t)800 << 20;
 // Tiles (of `tile_bytes` per stream) in one launch of a kernel that reads `nin` streams and
-// writes one: the largest power of two that keeps the launch within kLaunchBytes.
+// writes one: the largest power of two that keeps the launch within launch_bytes.
 inline size_t floor_pow2(size_t v) {
   size_t t = 1;
   while (t * 2 <= v) t *= 2;
   return t;
 }
-inline size_t launch_tiles(int nin, size_t tile_bytes) {
-  const size_t t = floor_pow2(kLaunchBytes / ((size_t)(nin + 1) * tile_bytes));
+inline size_t launch_tiles(int nin, size_t tile_bytes, size_t launch_bytes = kLaunchBytes) {
+  const size_t t = floor_pow2(launch_bytes / ((size_t)(nin + 1) * tile_bytes));
   return t < 8 ? 8 : t;
 }
 

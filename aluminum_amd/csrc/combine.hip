@@ -258,8 +258,13 @@ constexpr int kGatherU = 8, kGatherThreads = 128;
 //    81.5 %, 1024/8 81.5 % / 80 %, 1024/2 79.6 % / 78.8 %, whole piece in one
 //    launch 80.4 % / 80.5 %; repeated: 512/16 86 %, 1024/2 83 %.
 struct SpreadShape { unsigned chunk_tiles, launch_chunks; bool group_sources; };
-constexpr SpreadShape kSpreadFromHbm = {1024, 2, true}, kSpreadFromCache = {512, 16, false};
-constexpr size_t kSpreadLaunchBytes = (size_t)288 << 20;  // two 16 MiB chunks read, eight times that written
+inline SpreadShape spread_from_hbm() {
+  return {(unsigned)tunables().spread_hbm_chunk_tiles, (unsigned)tunables().spread_hbm_launch_chunks, true};
+}
+inline SpreadShape spread_from_cache() {
+  return {(unsigned)tunables().spread_cache_chunk_tiles, (unsigned)tunables().spread_cache_launch_chunks, false};
+}
+// Tunables::spread_launch_bytes: two 16 MiB chunks read, eight times that written
 __global__ void __launch_bounds__(kGatherThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
 spread_kernel(FoldParams p, unsigned tpc, unsigned tile0, unsigned src0, unsigned src_end, unsigned nsrc_x) {
   using TL = Tile<kGatherU, kGatherThreads>;
@@ -340,16 +345,16 @@ int launch_spread_once(const FoldParams &fp, int nsrc, SpreadShape shape, hipStr
   const size_t tiles = (max_len + tile - 1) / tile;
   // always a multiple of 8 (see spread_kernel); workgroups past the last tile exit at once
   const size_t tpc = tiles < shape.chunk_tiles ? (tiles + 7) & ~(size_t)7 : shape.chunk_tiles;
-  // A launch moves about kSpreadLaunchBytes: with two or three destinations more chunks per launch
+  // A launch moves about spread_launch_bytes: with two or three destinations more chunks per launch
   // (untouched 128 MiB slices to two buffers 69 % -> 75 % of peak, 85 MiB slices to three 71 % -> 73 %;
   // four destinations ran 2 points better with the two chunks they have), and of many short sources
   // only some side by side along blockIdx.y (32 slices of 2 MiB to 32 buffers 64 % -> 69 %, 16 slices
   // of 8 MiB 77 % -> 81 %).  Compared in one process, both libraries loaded.
   size_t launch_chunks = shape.launch_chunks;
   const size_t per_chunk = tpc * tile * (size_t)(fp.P + 1);
-  if (launch_chunks * per_chunk < kSpreadLaunchBytes / 2) launch_chunks = kSpreadLaunchBytes / per_chunk;
+  if (launch_chunks * per_chunk < tunables().spread_launch_bytes / 2) launch_chunks = tunables().spread_launch_bytes / per_chunk;
   const size_t per_launch = tpc * launch_chunks;
-  size_t side = shape.group_sources ? kSpreadLaunchBytes / (tiles * tile * (size_t)(fp.P + 1)) : (size_t)nsrc;
+  size_t side = shape.group_sources ? tunables().spread_launch_bytes / (tiles * tile * (size_t)(fp.P + 1)) : (size_t)nsrc;
   if (side < 1) side = 1;
   // sources of one group: as many as keep the group's chunk within 8 MiB
   size_t in_x = shape.group_sources ? ((size_t)8 << 20) / (tpc * tile) : 1;
@@ -383,8 +388,8 @@ int launch_spread_once(const FoldParams &fp, int nsrc, SpreadShape shape, hipStr
 // one, 83 % together; 8 MiB slices: 85 us together, 98 us one by one; 1 MiB: 15 us against 43 us).
 // Otherwise the sources are what a fold has just written, and all of them share the launches.
 int launch_spread_table(const FoldParams &fp, int nsrc, bool from_hbm, hipStream_t stream) {
-  if (!from_hbm) return launch_spread_once(fp, nsrc, kSpreadFromCache, stream);
-  const size_t big = (size_t)kSpreadFromHbm.chunk_tiles * Tile<kGatherU, kGatherThreads>::BYTES;
+  if (!from_hbm) return launch_spread_once(fp, nsrc, spread_from_cache(), stream);
+  const size_t big = (size_t)spread_from_hbm().chunk_tiles * Tile<kGatherU, kGatherThreads>::BYTES;
   FoldParams rest = fp;
   for (int q = 0; q < nsrc && nsrc > 1; ++q) {
     if (fp.seg.seg_len[q] < big) continue;
@@ -392,7 +397,7 @@ int launch_spread_table(const FoldParams &fp, int nsrc, bool from_hbm, hipStream
     one.in[0] = fp.in[q];
     one.seg.seg_off[0] = fp.seg.seg_off[q];
     one.seg.seg_len[0] = fp.seg.seg_len[q];
-    const int rc = launch_spread_once(one, 1, kSpreadFromHbm, stream);
+    const int rc = launch_spread_once(one, 1, spread_from_hbm(), stream);
     if (rc) return rc;
     rest.seg.seg_len[q] = 0;
   }
@@ -419,7 +424,7 @@ int launch_spread_table(const FoldParams &fp, int nsrc, bool from_hbm, hipStream
       run.seg.seg_len[n] = fp.seg.seg_len[q];
       ++n;
     }
-    const int rc = launch_spread_once(run, n, kSpreadFromHbm, stream);
+    const int rc = launch_spread_once(run, n, spread_from_hbm(), stream);
     if (rc) return rc;
     i0 += n;
   }
@@ -565,7 +570,7 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   lay.max_len = count;
   lay.start0 = start;
   lay.start_stride = 0;
-  if (nout < kTwoStepMinOutputs || bytes < kTwoStepMinBytes)
+  if ((size_t)nout < tunables().two_step_min_outputs || bytes < tunables().two_step_min_bytes)
     return launch_order(out_tab, ins, P, lay, dtype, op, order, as_stream(stream));
   // Several outputs of a large result: a workgroup that wrote its tile to every
   // output would interleave nout write streams (measured 69 % of peak).  Instead
@@ -573,7 +578,7 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   // In place (outs[j] == ins[j]) this is safe: a piece of the inputs is
   // overwritten by a launch that follows the fold of that piece on the same
   // stream, and no other piece reads it.
-  const size_t piece = bytes > 2 * kTwoStepPieceBytes ? kTwoStepPieceBytes / es : count;
+  const size_t piece = bytes > 2 * tunables().two_step_piece_bytes ? tunables().two_step_piece_bytes / es : count;
   for (size_t e0 = 0, n; e0 < count; e0 += n) {
     n = count - e0 < piece + piece / 2 ? count - e0 : piece;  // no short last piece
     Layout pl = lay;

@@ -240,7 +240,7 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
       if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, PN{}) : pick(No{}, PN{});
       else kern = pick(No{}, PN{});
     }
-    const size_t per_launch = launch_tiles(p.P, Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES);
+    const size_t per_launch = launch_tiles(p.P, Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES, tunables().launch_bytes);
     plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
       q.seg.tile0 = t0;
       q.seg.seg0 = s0;

@@ -185,7 +185,7 @@ template <typename T, int OP, int SLOTS, int MODE, int HALVES = 1>
 int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream, ChainArgs chain) {
   using S = TreeShape<T, OP, SLOTS, MODE>;
   const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
-  const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES);
+  const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES, tunables().launch_bytes);
   TreeParams q = p;
   q.div = make_divisor(p.P);
   q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0, 0};

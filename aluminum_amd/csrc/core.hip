@@ -27,6 +27,27 @@ int set_error(int code, const char *fmt, ...) {
 
 void clear_error() { g_err[0] = 0; }
 
+Tunables &tunables() {
+  static Tunables t;
+  return t;
+}
+
+namespace {
+struct TunableName { const char *name; size_t Tunables::*field; };
+const TunableName kTunableNames[] = {
+    {"launch_bytes", &Tunables::launch_bytes},
+    {"two_step_min_bytes", &Tunables::two_step_min_bytes},
+    {"two_step_min_outputs", &Tunables::two_step_min_outputs},
+    {"two_step_piece_bytes", &Tunables::two_step_piece_bytes},
+    {"ring_piece_bytes", &Tunables::ring_piece_bytes},
+    {"spread_launch_bytes", &Tunables::spread_launch_bytes},
+    {"spread_hbm_chunk_tiles", &Tunables::spread_hbm_chunk_tiles},
+    {"spread_hbm_launch_chunks", &Tunables::spread_hbm_launch_chunks},
+    {"spread_cache_chunk_tiles", &Tunables::spread_cache_chunk_tiles},
+    {"spread_cache_launch_chunks", &Tunables::spread_cache_launch_chunks},
+};
+}  // namespace
+
 int device_cus() {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
@@ -84,6 +105,24 @@ size_t alamd_dtype_size(int dtype) {
   case ALAMD_I64: case ALAMD_U64: case ALAMD_F64: return 8;
   default: return 0;
   }
+}
+
+int alamd_tune(const char *name, size_t value) {
+  if (!name) return alamd::set_error(ALAMD_ERR_INVALID_ARG, "null name");
+  const alamd::Tunables defaults;
+  for (const auto &t : alamd::kTunableNames)
+    if (std::string(name) == t.name) {
+      alamd::tunables().*(t.field) = value ? value : defaults.*(t.field);
+      return ALAMD_OK;
+    }
+  return alamd::set_error(ALAMD_ERR_INVALID_ARG, "no launch-planner size is called %s", name);
+}
+
+size_t alamd_tuned(const char *name) {
+  if (name)
+    for (const auto &t : alamd::kTunableNames)
+      if (std::string(name) == t.name) return alamd::tunables().*(t.field);
+  return 0;
 }
 
 int alamd_check_op(int dtype, int op) { return alamd::check_type_op(dtype, op); }

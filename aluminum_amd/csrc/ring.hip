@@ -190,7 +190,7 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   const size_t max_len = fp.seg.seg_base + (fp.seg.seg_rem ? 1 : 0);
   if (max_len == 0) return ALAMD_OK;
   const size_t es = alamd_dtype_size(dtype);
-  if (!all || P < kTwoStepMinOutputs || count * es < kTwoStepMinBytes)
+  if (!all || (size_t)P < tunables().two_step_min_outputs || count * es < tunables().two_step_min_bytes)
     return launch_fold(fp, (unsigned)P, max_len, dtype, op, true, stream);
   // Large allreduce.  Writing each result tile to all P buffers from the fold
   // kernel interleaves P write streams; instead every segment is folded into
@@ -202,11 +202,11 @@ int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool a
   };
   auto seg_len = [&](int s) { return fp.seg.seg_base + ((size_t)s < fp.seg.seg_rem ? 1 : 0); };
   // piece by piece: fold the same range of every segment (P reads + 1 write), then spread it
-  // (one fold launch's worth of tiles over all segments: one fold launch and one spread launch per piece)
+  // (the fold's launches over the piece, then one pass of spread launches)
   const size_t tile_elems = Tile<8, 128>::BYTES / es;
-  // (64 MiB from P = 8 up, where that is what one fold launch covers; more below: 128 MiB at P = 3 and 4)
-  size_t piece_bytes = launch_tiles(P, Tile<8, 128>::BYTES) * Tile<8, 128>::BYTES;
-  if (piece_bytes < kRingPieceBytes) piece_bytes = kRingPieceBytes;
+  // (never less than one fold launch covers)
+  size_t piece_bytes = launch_tiles(P, Tile<8, 128>::BYTES, tunables().launch_bytes) * Tile<8, 128>::BYTES;
+  if (piece_bytes < tunables().ring_piece_bytes) piece_bytes = tunables().ring_piece_bytes;
   size_t piece = piece_bytes / (size_t)P / es / tile_elems * tile_elems;
   if (piece == 0) piece = tile_elems;
   for (size_t e0 = 0, pn; e0 < max_len; e0 += pn) {
