@@ -112,35 +112,55 @@ fold_vec_kernel(const FoldParams p) {
           acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[k][u]) : step_vec<T, OP>(x[k][u], acc[u]);
       }
     } else {
-      constexpr int B = 4;  // streams in flight between uses
+      // Run-time rank count: the streams are taken in batches of a compile-time size - the pointers
+      // of a batch, then all its loads, then all its steps, no branch in between - so that up to
+      // seven ranks have every stream in flight at once, like the P = 8 body above.  (With one
+      // branch per stream the compiler fetched each stream's pointer, waited for it and only then
+      // issued that stream's loads: 1.5 % slower at P = 12 and 16, and for 16-bit and 8-bit types
+      // at P = 4.  A compile-time P = 4 body gains another 0.5 to 1 %, not worth its kernels.)
       int idx = s;
-      {
-        const auto r = TL::rsrc(p.in[idx] + vin + tb, nrec);
+      auto batch = [&](auto rc, auto first_c) {
+        constexpr int R = decltype(rc)::value;
+        constexpr bool FIRST = decltype(first_c)::value;  // the batch starts the fold
+        const char *src[R];
 #pragma unroll
-        for (int u = 0; u < U; ++u) acc[u] = tl.load(r, u);
-      }
-      for (int k = 1; k < P; k += B) {
-        u32x4 x[B][U];
-        int id = idx;
+        for (int b = 0; b < R; ++b) {
+          if (!(FIRST && b == 0)) idx = next_rank(idx, p.dir, P);
+          src[b] = p.in[idx];
+        }
+        u32x4 x[R][U];
 #pragma unroll
-        for (int b = 0; b < B; ++b) {
-          if (k + b < P) {
-            id = next_rank(id, p.dir, P);
-            const auto r = TL::rsrc(p.in[id] + vin + tb, nrec);
+        for (int b = 0; b < R; ++b) {
+          const auto r = TL::rsrc(src[b] + vin + tb, nrec);
 #pragma unroll
-            for (int u = 0; u < U; ++u) x[b][u] = tl.load(r, u);
-          }
+          for (int u = 0; u < U; ++u) x[b][u] = tl.load(r, u);
+        }
+        if constexpr (FIRST) {
+#pragma unroll
+          for (int u = 0; u < U; ++u) acc[u] = x[0][u];
         }
 #pragma unroll
-        for (int b = 0; b < B; ++b) {
-          if (k + b < P) {
+        for (int b = FIRST ? 1 : 0; b < R; ++b) {
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-              acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[b][u]) : step_vec<T, OP>(x[b][u], acc[u]);
-          }
+          for (int u = 0; u < U; ++u)
+            acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[b][u]) : step_vec<T, OP>(x[b][u], acc[u]);
         }
-        idx = id;
+      };
+      using Yes = std::true_type;
+      using No = std::false_type;
+      // up to seven streams in one batch; beyond that a first batch that leaves a multiple of six
+      constexpr int B = 6;
+      int left = P;
+      switch (P <= 7 ? P : (P - 1) % B + 1) {
+      case 7: batch(std::integral_constant<int, 7>{}, Yes{}); left -= 7; break;
+      case 6: batch(std::integral_constant<int, 6>{}, Yes{}); left -= 6; break;
+      case 5: batch(std::integral_constant<int, 5>{}, Yes{}); left -= 5; break;
+      case 4: batch(std::integral_constant<int, 4>{}, Yes{}); left -= 4; break;
+      case 3: batch(std::integral_constant<int, 3>{}, Yes{}); left -= 3; break;
+      case 2: batch(std::integral_constant<int, 2>{}, Yes{}); left -= 2; break;
+      default: batch(std::integral_constant<int, 1>{}, Yes{}); left -= 1; break;
       }
+      for (; left >= B; left -= B) batch(std::integral_constant<int, B>{}, No{});
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) acc[u] = finish_vec<T, OP>(acc[u], p.div);

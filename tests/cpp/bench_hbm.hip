@@ -12,6 +12,7 @@
 //   copy     one read, one written
 //   mix8     eight read, one written (the shape of the P = 8 fold)
 //   mix8ip   eight read, the result written over the stream read last
+//   mix2, mix3, mix4, mix6   the folds of fewer ranks
 //
 // usage: bench_hbm [pattern ...] [--mib N per stream, default 256] [--sets S, default 4] [--reps R, default 12]
 // Prints one JSON line per pattern.  A bench / profiling aid; not part of the library.
@@ -107,6 +108,8 @@ int main(int argc, char **argv) {
       {"read8", 8, 0, false, probe_kernel<8, false>}, {"read1", 1, 0, false, probe_kernel<1, false>},
       {"write1", 0, 1, false, probe_kernel<0, true>}, {"copy", 1, 1, false, probe_kernel<1, true>},
       {"mix8", 8, 1, false, probe_kernel<8, true>},   {"mix8ip", 8, 1, true, probe_kernel<8, true>},
+      {"mix2", 2, 1, false, probe_kernel<2, true>},   {"mix3", 3, 1, false, probe_kernel<3, true>},
+      {"mix4", 4, 1, false, probe_kernel<4, true>},   {"mix6", 6, 1, false, probe_kernel<6, true>},
   };
   const size_t bytes = mib << 20;
   if (bytes % TL::BYTES != 0 || sets < 1 || reps < 1) { std::printf("bad sizes\n"); return 2; }
