@@ -86,6 +86,7 @@ struct SegParams {
   int out_mode;     // OUT_ALL / OUT_SEG / OUT_OWNER
   int owner_shift;  // OUT_OWNER: output index is (segment + owner_shift) mod P
   int nout;         // OUT_ALL: number of outputs written
+  int simple;       // 1: one segment from element 0, one output, no head (the kernels then skip the lookups)
   int ragged;       // 1: segments are given by the two tables below
   unsigned long long seg_off[ALAMD_MAX_RANKS];
   unsigned long long seg_len[ALAMD_MAX_RANKS];
@@ -104,6 +105,9 @@ inline SegParams make_seg(size_t seg_base, size_t seg_rem, int in_blocked, int o
 }
 
 // The segment a workgroup works on: launches walk positions, which the host may have sorted by length.
+// (These lookups are a chain of dependent scalar loads, one branch per mode.  Reading every table
+// whatever the mode and choosing afterwards shortens the chain but ran 2 to 3 % slower for a
+// Reduce_scatter; the launches that need no lookup at all skip them instead: SegParams::simple.)
 __device__ __forceinline__ unsigned seg_of(const SegParams &s, unsigned pos) {
   return s.mapped ? s.order[pos] : pos;
 }

@@ -70,15 +70,19 @@ fold_vec_kernel(const FoldParams p) {
   using TL = Tile<U, THREADS>;
   const TL tl;
   const int P = PT ? PT : p.P;
-  const unsigned seg = seg_of(p.seg, blockIdx.y + p.seg.seg0);
-  size_t off, len;
-  seg_range(p.seg, seg, off, len);
-  const size_t off_bytes = off * sizeof(T);
-  const size_t in_bytes = p.seg.in_blocked ? off_bytes : 0;
-  const int s = (p.start0 + (int)seg * p.start_stride) % P;
-  int j0, nj;
-  size_t out_bytes;
-  out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
+  // The general case looks its segment up in several tables, one dependent scalar load after the
+  // other; a launch over one whole segment into one output needs none of that.
+  unsigned seg = 0;
+  size_t off = 0, len = p.seg.seg_base, in_bytes = 0, out_bytes = 0;
+  int s = p.start0, j0 = 0, nj = 1;
+  if (!p.seg.simple) {
+    seg = seg_of(p.seg, blockIdx.y + p.seg.seg0);
+    seg_range(p.seg, seg, off, len);
+    const size_t off_bytes = off * sizeof(T);
+    in_bytes = p.seg.in_blocked ? off_bytes : 0;
+    s = (p.start0 + (int)seg * p.start_stride) % P;
+    out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
+  }
 
   const size_t head = HEAD ? p.seg.seg_head[seg] : 0;
   const size_t vlen = len - head;
@@ -205,6 +209,7 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
     FoldParams q = p;
     q.div = make_divisor(p.P);
     q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0, 0};
+    q.seg.simple = 0;
     if (chain) {
       // one segment, one output, every tile in one launch, tiles handed out by the ticket counter
       if (nseg != 1) return set_error(ALAMD_ERR_INVALID_ARG, "a chained fold has one segment");
@@ -243,6 +248,8 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
                                                      p.in[first] + (p.seg.in_blocked ? off * sizeof(T) : 0), len);
       if (q.seg.seg_head[sg]) q.seg.any_head = 1;
     }
+    q.seg.simple = nseg == 1 && !q.seg.ragged && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1 &&
+                   !q.seg.any_head && p.start0 >= 0 && p.start0 < p.P;
     auto pick = [&](auto acc_is_in_t, auto pt_t) -> void (*)(const FoldParams) {
       constexpr bool A = decltype(acc_is_in_t)::value;
       constexpr int PT = decltype(pt_t)::value;

@@ -83,14 +83,17 @@ tree_vec_kernel(const TreeParams p) {
   static_assert(HALVES == 1 || MODE != TREE_PREFOLD, "a pre-fold never meets more than 32 slots");
   using TL = Tile<U, THREADS>;
   const TL tl;
-  const unsigned seg = seg_of(p.seg, blockIdx.y + p.seg.seg0);
-  size_t off, len;
-  seg_range(p.seg, seg, off, len);
-  const size_t off_bytes = off * sizeof(T);
-  const size_t in_bytes = p.seg.in_blocked ? off_bytes : 0;
-  int j0, nj;
-  size_t out_bytes;
-  tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
+  // (a launch over one whole segment into one output skips the lookups: see the fold kernel)
+  unsigned seg = 0;
+  size_t off = 0, len = p.seg.seg_base, in_bytes = 0, out_bytes = 0;
+  int j0 = 0, nj = 1;
+  if (!p.seg.simple) {
+    seg = seg_of(p.seg, blockIdx.y + p.seg.seg0);
+    seg_range(p.seg, seg, off, len);
+    const size_t off_bytes = off * sizeof(T);
+    in_bytes = p.seg.in_blocked ? off_bytes : 0;
+    tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
+  }
 
   const size_t head = HEAD ? p.seg.seg_head[seg] : 0;
   const size_t vlen = len - head;
@@ -189,6 +192,7 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   TreeParams q = p;
   q.div = make_divisor(p.P);
   q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0, 0};
+  q.seg.simple = 0;
   if (chain.scratch) {
     if (nseg != 1) return set_error(ALAMD_ERR_INVALID_ARG, "a chained combine has one segment");
     constexpr size_t N = 16 / sizeof(T);
@@ -224,6 +228,8 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
     q.seg.seg_head[sg] = (unsigned char)head_count(sizeof(T), p.out[j0] + out_bytes, p.a[0] + in_bytes, len);
     if (q.seg.seg_head[sg]) q.seg.any_head = 1;
   }
+  q.seg.simple = nseg == 1 && !q.seg.ragged && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1 &&
+                 !q.seg.any_head;
   void (*kern)(const TreeParams) =
       q.seg.any_head ? tree_vec_kernel<T, OP, SLOTS, MODE, true, HALVES> : tree_vec_kernel<T, OP, SLOTS, MODE, false, HALVES>;
   plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
