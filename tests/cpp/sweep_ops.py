@@ -40,6 +40,7 @@ def main():
         sys.exit("tests/cpp/test_ops is not built (make -C tests/cpp)")
     rng = random.Random(args.seed)
     t0, fails = time.time(), 0
+    last = t0
     for k in range(args.runs):
         op, dt = rng.choice(OPS), rng.choice(DATATYPES)
         ranks = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16, 24, 32, 33, 40, 48, 63, 64])
@@ -57,7 +58,8 @@ def main():
             fails += 1
             print("FAIL rc=%d: %s\n%s\n%s" % (p.returncode, " ".join(cmd[1:]), p.stdout[-600:], p.stderr[-300:]),
                   flush=True)
-        if k % 25 == 24:
+        if k % 25 == 24 or time.time() - last > 30:  # a line at least every half minute
+            last = time.time()
             print("%d runs, %d failed, %.0f s" % (k + 1, fails, time.time() - t0), flush=True)
     print("TOTAL %d runs, %d failed" % (args.runs, fails))
     sys.exit(1 if fails else 0)
