@@ -411,6 +411,47 @@ def c1_gpu_checksum(al, torch):
     return "%016x" % oracle.checksum(out.cpu().numpy())
 
 
+def c1_gpu_time(al, torch):
+    """The same configuration as an Allreduce on the GPU (the result in all four ranks' buffers):
+    microseconds per call, one call at a time (each followed by a synchronisation), 200 in a row, and
+    200 replayed from a HIP graph."""
+    n, ranks = 1 << 20, 4
+    ins = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(ranks)]
+    outs = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(ranks)]
+    for r in range(ranks):
+        al.fill(ins[r], "uniform_pm1", 1000 + r)
+    call = lambda: al.combine(outs, ins, "sum", order="tree_dbl")
+    for _ in range(10):
+        call()
+    torch.cuda.synchronize()
+    one = []
+    for _ in range(100):
+        t0 = time.perf_counter()
+        call()
+        torch.cuda.synchronize()
+        one.append(time.perf_counter() - t0)
+    t0 = time.perf_counter()
+    for _ in range(200):
+        call()
+    torch.cuda.synchronize()
+    row = (time.perf_counter() - t0) / 200
+    # the same call captured in a HIP graph and replayed: no binding or argument checking in between
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(20):
+            call()
+    g.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        g.replay()
+    torch.cuda.synchronize()
+    replay = (time.perf_counter() - t0) / 200
+    return {"one_call_and_wait_us": sorted(one)[len(one) // 2] * 1e6, "in_a_row_us": row * 1e6,
+            "in_a_graph_us": replay * 1e6,
+            "note": "in_a_row is bound by the Python binding that makes the calls, in_a_graph by the device"}
+
+
 def cpu_model():
     try:
         with open("/proc/cpuinfo") as f:
@@ -437,12 +478,14 @@ def cpu_baseline(al=None, torch=None):
                 if al is not None and "checksum" in r:
                     # the bits MPI_Allreduce produced on the host against the GPU's for the same inputs
                     same = c1_gpu_checksum(al, torch) == r["checksum"]
+                gpu_us = c1_gpu_time(al, torch) if al is not None else None
                 return {"value": r["gbps_median"], "unit": "GB/s", "cores": 4, "kind": "port",
                         "sample": "MPI_Allreduce(MPI_SUM, MPI_FLOAT) on a dup'd communicator, the call "
                                   "Al::Allreduce<MPIBackend> forwards to; 4 MPICH ranks on this host, "
                                   "2^20 elements per rank, uniform[-1,1] seed 1000+rank, 10 warm-up + 3000 "
                                   "timed (about 10 s), median of max-over-ranks; GB/s over (P+1)*n*4 bytes",
                         "median_ms": r["median_ms"], "min_ms": r["min_ms"], "gpu_result_identical": same,
+                        "gpu_same_configuration": gpu_us,
                         "host_cpus": os.cpu_count(), "cpu_model": cpu_model(), "same_workload_port": c2_port_sample()}
         except Exception:
             pass
