@@ -353,9 +353,12 @@ int launch_spread_once(const FoldParams &fp, int nsrc, SpreadShape shape, hipStr
   size_t launch_chunks = shape.launch_chunks;
   const size_t per_chunk = tpc * tile * (size_t)(fp.P + 1);
   if (launch_chunks * per_chunk < tunables().spread_launch_bytes / 2) launch_chunks = tunables().spread_launch_bytes / per_chunk;
+  const size_t all_chunks = (tiles + tpc - 1) / tpc;
+  if (launch_chunks > all_chunks) launch_chunks = all_chunks;  // whatever the settings ask for
   const size_t per_launch = tpc * launch_chunks;
   size_t side = shape.group_sources ? tunables().spread_launch_bytes / (tiles * tile * (size_t)(fp.P + 1)) : (size_t)nsrc;
   if (side < 1) side = 1;
+  if (side > (size_t)nsrc) side = (size_t)nsrc;
   // sources of one group: as many as keep the group's chunk within 8 MiB
   size_t in_x = shape.group_sources ? ((size_t)8 << 20) / (tpc * tile) : 1;
   if (in_x < 1) in_x = 1;

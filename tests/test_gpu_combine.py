@@ -535,3 +535,58 @@ def test_reduce_scatterv_chained_wait_that_gives_up_is_reported(al):
     assert not al.reduce_scatterv_wait_expired()
     for b in range(P):
         assert_bits_equal(to_host(bufs[b], np.float32)[:counts[b]], want[b], "f32", "after the report, rank %d" % b)
+
+
+SETTINGS = [
+    {},  # the defaults
+    {"launch_bytes": 1 << 20, "two_step_min_bytes": 4096, "two_step_piece_bytes": 64 << 10,
+     "ring_piece_bytes": 128 << 10, "spread_launch_bytes": 1 << 20, "spread_hbm_chunk_tiles": 8,
+     "spread_hbm_launch_chunks": 1, "spread_cache_chunk_tiles": 8, "spread_cache_launch_chunks": 1},
+    {"launch_bytes": 1 << 40, "two_step_min_outputs": 99, "spread_hbm_chunk_tiles": 24, "spread_hbm_launch_chunks": 3,
+     "spread_launch_bytes": 1 << 40, "ring_piece_bytes": 1 << 40},
+    {"two_step_min_bytes": 1, "two_step_min_outputs": 2, "two_step_piece_bytes": 1 << 20,
+     "spread_cache_chunk_tiles": 16, "spread_cache_launch_chunks": 2, "launch_bytes": 3 << 20},
+]
+
+
+@pytest.mark.parametrize("k", range(len(SETTINGS)))
+def test_results_do_not_depend_on_the_launch_planners_sizes(al, k):
+    """The sizes the launch planners cut their work by (bytes per launch, the thresholds and pieces of
+    the two-step calls, the spread's chunks) only decide how the same work is spread over launches:
+    extreme settings give the bits of the defaults, i.e. the oracle's."""
+    import torch
+    P, n = 5, 1_300_007
+    ins_h = make_inputs(P, n, "f32", "sum")
+    try:
+        for name, value in SETTINGS[k].items():
+            al.tune(name, value)
+            assert al.tuned(name) == value
+        ins = [to_dev(a) for a in ins_h]
+        outs = [dev_empty(n, np.float32) for _ in range(P)]
+        al.combine(outs, ins, "sum", order="tree_dbl")
+        one = dev_empty(n, np.float32)
+        al.combine([one], ins, "sum", order="rank_asc")
+        counts = [n // P + (1 if q < n % P else 0) for q in range(P)]
+        displs = [sum(counts[:q]) for q in range(P)]
+        rs = [dev_empty(c, np.float32) for c in counts]
+        al.reduce_scatterv(rs, ins, counts, "sum", order="pairwise_desc")
+        ag = [dev_empty(n, np.float32) for _ in range(P)]
+        al.allgatherv(ag, rs, counts, displs)
+        ring = [to_dev(a) for a in ins_h]
+        al.ring_allreduce(ring, "sum", mode="fused")
+        torch.cuda.synchronize()
+    finally:
+        for name in SETTINGS[k]:
+            al.tune(name, 0)
+    want_tree = oracle.combine(ins_h, "f32", "sum", "tree_dbl")
+    want_fold = oracle.combine(ins_h, "f32", "sum", "rank_asc")
+    want_rs = oracle.reduce_scatterv(ins_h, counts, "f32", "sum", "pairwise_desc")
+    want_ring = oracle.ring_allreduce(ins_h, "f32", "sum", (4 << 20) // 4)[0]
+    assert_bits_equal(to_host(one, np.float32), want_fold, "f32", "fold, settings %d" % k)
+    for r in range(P):
+        assert_bits_equal(to_host(outs[r], np.float32), want_tree, "f32", "allreduce rank %d, settings %d" % (r, k))
+        assert_bits_equal(to_host(rs[r], np.float32), want_rs[r], "f32", "reduce_scatterv rank %d, settings %d" % (r, k))
+        assert_bits_equal(to_host(ag[r], np.float32), np.concatenate(want_rs), "f32", "allgatherv rank %d, settings %d" % (r, k))
+        assert_bits_equal(to_host(ring[r], np.float32), want_ring, "f32", "fused ring rank %d, settings %d" % (r, k))
+    with pytest.raises(al.AlError):
+        al.tune("no_such_size", 1)
