@@ -152,12 +152,17 @@ fold_vec_kernel(const FoldParams p) {
       };
       using Yes = std::true_type;
       using No = std::false_type;
-      // up to seven streams in one batch; beyond that a first batch that leaves a multiple of six
-      constexpr int B = 6;
+      // Up to seven streams in one batch; beyond that a first batch that leaves a multiple of six.
+      // For 8- and 16-bit types, whose arithmetic needs registers as well, the kernel then no longer
+      // fits two waves per SIMD.  Batches of five and four, which do, ran 1 to 3 % slower all the
+      // same - except in a chained launch, where the second wave hides the waits for the
+      // neighbouring tile (bf16, a block one element into its buffer: 5.2 TB/s against 4.5).
+      constexpr bool kTwoWaves = CHAIN && sizeof(T) <= 2;
+      constexpr int B0 = kTwoWaves ? 5 : 7, B = kTwoWaves ? 4 : 6;
       int left = P;
-      switch (P <= 7 ? P : (P - 1) % B + 1) {
-      case 7: batch(std::integral_constant<int, 7>{}, Yes{}); left -= 7; break;
-      case 6: batch(std::integral_constant<int, 6>{}, Yes{}); left -= 6; break;
+      switch (P <= B0 ? P : (P - 1) % B + 1) {
+      case 7: if constexpr (B0 >= 7) { batch(std::integral_constant<int, 7>{}, Yes{}); left -= 7; } break;
+      case 6: if constexpr (B0 >= 6) { batch(std::integral_constant<int, 6>{}, Yes{}); left -= 6; } break;
       case 5: batch(std::integral_constant<int, 5>{}, Yes{}); left -= 5; break;
       case 4: batch(std::integral_constant<int, 4>{}, Yes{}); left -= 4; break;
       case 3: batch(std::integral_constant<int, 3>{}, Yes{}); left -= 3; break;
@@ -227,13 +232,11 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
       q.seg.seg0 = 0;
       q.seg.mapped = 0;
       void (*ck)(const FoldParams) = nullptr;
-      if (p.P == 8) {  // all eight streams in flight at once, as in the ordinary launches
-        if constexpr (FP_MINMAX) ck = roles ? fold_vec_kernel<T, OP, true, 8, false, true> : fold_vec_kernel<T, OP, false, 8, false, true>;
-        else ck = fold_vec_kernel<T, OP, false, 8, false, true>;
-      } else {
-        if constexpr (FP_MINMAX) ck = roles ? fold_vec_kernel<T, OP, true, 0, false, true> : fold_vec_kernel<T, OP, false, 0, false, true>;
-        else ck = fold_vec_kernel<T, OP, false, 0, false, true>;
-      }
+      // Always the run-time-P body: with the gate in it the P = 8 body no longer fits two waves per SIMD,
+      // and a second wave is what hides a tile's wait for its neighbour (a block one element into its
+      // buffer: 3 to 11 % faster than with the P = 8 body; from a few MiB in, 3 % slower).
+      if constexpr (FP_MINMAX) ck = roles ? fold_vec_kernel<T, OP, true, 0, false, true> : fold_vec_kernel<T, OP, false, 0, false, true>;
+      else ck = fold_vec_kernel<T, OP, false, 0, false, true>;
       hipLaunchKernelGGL(ck, dim3((unsigned)tickets, 1, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
       ALAMD_HIP(hipGetLastError());
       return ALAMD_OK;
