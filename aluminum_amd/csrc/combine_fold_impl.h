@@ -251,7 +251,7 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
                                                      p.in[first] + (p.seg.in_blocked ? off * sizeof(T) : 0), len);
       if (q.seg.seg_head[sg]) q.seg.any_head = 1;
     }
-    q.seg.simple = nseg == 1 && !q.seg.ragged && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1 &&
+    q.seg.simple = nseg == 1 && !q.seg.ragged && q.seg.seg_rem == 0 && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1 &&
                    !q.seg.any_head && p.start0 >= 0 && p.start0 < p.P;
     auto pick = [&](auto acc_is_in_t, auto pt_t) -> void (*)(const FoldParams) {
       constexpr bool A = decltype(acc_is_in_t)::value;
