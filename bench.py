@@ -50,10 +50,10 @@ TRAFFIC_PROFILE = {"c2_f32_sum": "profiles/fold_vec_kernel_f32_sum_P8_c2.md"}
 KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false /*operand roles*/, 8 /*ranks*/, "
                              "false /*no leading elements*/, false /*not chained*/>"}
 
-# Every configuration of the headline benchmark beside the primary workload: C2 prod and bf16, the same over
+# Every configuration of the headline benchmark beside the primary workload: C2 in the tree order, prod and bf16, the same over
 # buffers no earlier call has touched, C4 (integer / bitwise / logical), C3 (ring, both modes), C5 (halo
 # faces), the stream flags, and the layouts an Allreduce / Reduce_scatter / Allgather reaches the kernels in.
-DEFAULT_ALSO = ("c2_f32_sum_rotating,c2_f32_prod,c2_bf16_sum,c2_bf16_sum_rotating,c4_i32_max,c4_i64_bxor,"
+DEFAULT_ALSO = ("c2_f32_sum_rotating,c2_f32_sum_tree,c2_f32_prod,c2_bf16_sum,c2_bf16_sum_rotating,c4_i32_max,c4_i64_bxor,"
                 "c4_u8_lxor,c3_ring_stepwise,c3_ring_fused,c5_halo,flags,c2_f32_allreduce,"
                 "c2_f32_allreduce_rotating,c2_f32_reduce_scatter,c2_f32_reduce_scatter_rotating,"
                 "c2_f32_allgather,c2_f32_allgather_rotating,c2_f32_reduce_scatterv_in_place")
