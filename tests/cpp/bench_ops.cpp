@@ -8,11 +8,16 @@
 // rank of a trial reports the same time.
 //
 // usage: bench_ops [--op allreduce|reduce|reduce_scatter|allgather] [--datatype float|double|int|...]
-//                  [--reduction-op sum|prod|min|max|...] [--algo automatic|rank_order|tree_doubling|
+//                  [--reduction-op sum|prod|min|max|...] [--algorithm automatic|rank_order|tree_doubling|
 //                  tree_halving|tree_binomial|pairwise|ring|ring_fused] [--ranks P] [--root R]
-//                  [--inplace] [--nonblocking] [--min-size N] [--max-size N] [--num-iters N] [--num-warmup N]
+//                  [--inplace] [--nonblocking] [--min-size N] [--max-size N] [--size N] [--num-iters N]
+//                  [--num-warmup N] [--summarize] [--save-to-file FILE] [--no-print-table] [--backend hip]
+// (--summarize: per size "Size Mean Median Stdev Min Max" over the timed trials, benchmark_ops.cpp:211-224;
+// --save-to-file / --no-print-table: where the table of rows goes, :225-230.)
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -32,6 +37,36 @@ struct Options {
   int ranks = 8, root = 0;
   bool inplace = false, nonblocking = false;
   size_t min_size = 1, max_size = (size_t)1 << 22, iters = 100, warmup = 10;
+  bool summarize = false, print_table = true;
+  std::string save_to;
+};
+
+// The rows of one run: trial times in seconds by message size.
+struct Results {
+  std::string prefix;  // "Backend Type Operation Algo NonBlocking InPlace Root CommSize "
+  int ranks = 0;
+  std::map<size_t, std::vector<double>> times;
+  void write(std::FILE *f) const {
+    std::fprintf(f, "Backend Type Operation Algo NonBlocking InPlace Root CommSize Size CommRank Time\n");
+    for (const auto &kv : times)
+      for (int r = 0; r < ranks; ++r)
+        for (double t : kv.second) std::fprintf(f, "%s%zu %d %.9g\n", prefix.c_str(), kv.first, r, t);
+  }
+  void summary(std::FILE *f) const {
+    std::fprintf(f, "Size\t\tMean\t\tMedian\t\tStdev\t\tMin\t\tMax\n");
+    for (const auto &kv : times) {
+      std::vector<double> v = kv.second;
+      if (v.empty()) continue;
+      std::sort(v.begin(), v.end());
+      double mean = 0, sq = 0;
+      for (double t : v) mean += t;
+      mean /= (double)v.size();
+      for (double t : v) sq += (t - mean) * (t - mean);
+      const double stdev = v.size() > 1 ? std::sqrt(sq / (double)(v.size() - 1)) : 0.0;
+      std::fprintf(f, "%zu\t\t%.9g\t%.9g\t%.9g\t%.9g\t%.9g\n", kv.first, mean, v[v.size() / 2], stdev, v.front(),
+                   v.back());
+    }
+  }
 };
 
 template <typename T> int run(const Options &o, Al::ReductionOperator rop, Algo algo, const char *tname) {
@@ -42,7 +77,10 @@ template <typename T> int run(const Options &o, Al::ReductionOperator rop, Algo 
   HIPCHK(hipEventCreate(&e1));
   const int P = o.ranks;
   const int dt = Al::amd::TypeMap<T>::value;
-  std::printf("Backend Type Operation Algo NonBlocking InPlace Root CommSize Size CommRank Time\n");
+  Results res;
+  res.ranks = P;
+  res.prefix = Backend::Name() + " " + tname + " " + o.op + " " + o.algo + " " + (o.nonblocking ? "1" : "0") + " " +
+               (o.inplace ? "1" : "0") + " " + std::to_string(o.root) + " " + std::to_string(P) + " ";
   for (size_t size = o.min_size; size <= o.max_size; size *= 2) {
     const size_t in_elems = o.op == "reduce_scatter" ? size * (size_t)P : size;
     const size_t out_elems = o.op == "allgather" ? size * (size_t)P : size;
@@ -93,12 +131,17 @@ template <typename T> int run(const Options &o, Al::ReductionOperator rop, Algo 
       HIPCHK(hipEventElapsedTime(&ms, e0, e1));
       if (trial >= o.warmup) times.push_back(ms * 1e-3);
     }
-    for (int r = 0; r < P; ++r)
-      for (double t : times)
-        std::printf("%s %s %s %s %d %d %d %d %zu %d %.9g\n", Backend::Name().c_str(), tname, o.op.c_str(),
-                    o.algo.c_str(), o.nonblocking ? 1 : 0, o.inplace ? 1 : 0, o.root, P, size, r, t);
+    res.times[size] = times;
     for (int r = 0; r < P; ++r) { HIPCHK(hipFree(in[r])); HIPCHK(hipFree(out[r])); }
   }
+  if (o.summarize) res.summary(stdout);
+  if (!o.save_to.empty()) {
+    std::FILE *f = std::fopen(o.save_to.c_str(), "w");
+    if (!f) { std::fprintf(stderr, "Error opening %s\n", o.save_to.c_str()); return 2; }
+    res.write(f);
+    std::fclose(f);
+  }
+  if (o.print_table) res.write(stdout);
   HIPCHK(hipEventDestroy(e0));
   HIPCHK(hipEventDestroy(e1));
   HIPCHK(hipStreamDestroy(stream));
@@ -113,7 +156,13 @@ int main(int argc, char **argv) {
     if (a == "--op") o.op = next();
     else if (a == "--datatype") o.datatype = next();
     else if (a == "--reduction-op") o.redop = next();
-    else if (a == "--algo") o.algo = next();
+    else if (a == "--algo" || a == "--algorithm") o.algo = next();
+    else if (a == "--size") o.min_size = o.max_size = std::strtoull(next().c_str(), nullptr, 10);
+    else if (a == "--summarize") o.summarize = true;
+    else if (a == "--save-to-file") o.save_to = next();
+    else if (a == "--no-print-table") o.print_table = false;
+    else if (a == "--backend") { if (next() != "hip") { std::fprintf(stderr, "this program benchmarks the hip backend only\n"); return 2; } }
+    else if (a == "--help") { std::printf("see the usage comment at the top of tests/cpp/bench_ops.cpp\n"); return 0; }
     else if (a == "--ranks") o.ranks = std::atoi(next().c_str());
     else if (a == "--root") o.root = std::atoi(next().c_str());
     else if (a == "--inplace") o.inplace = true;

@@ -57,6 +57,21 @@ def test_benchmark_sweep_rows():
     bad = subprocess.run([exe, "--op", "allreduce", "--reduction-op", "bxor", "--max-size", "4"], capture_output=True,
                          text=True, timeout=60)
     assert bad.returncode == 1 and "Reduction operator not supported" in bad.stderr
+    # the summary and the file output of the reference's benchmark (benchmark/benchmark_ops.cpp:211-230)
+    import tempfile
+    with tempfile.TemporaryDirectory() as d:
+        out = os.path.join(d, "rows.txt")
+        q = subprocess.run([exe, "--backend", "hip", "--op", "reduce_scatter", "--algorithm", "pairwise", "--ranks", "3",
+                            "--size", "1000", "--num-iters", "5", "--num-warmup", "1", "--summarize", "--save-to-file",
+                            out, "--no-print-table"], capture_output=True, text=True, timeout=120)
+        assert q.returncode == 0, q.stderr
+        shown = q.stdout.strip().splitlines()
+        assert shown[0].split() == ["Size", "Mean", "Median", "Stdev", "Min", "Max"] and len(shown) == 2
+        size, mean, median, stdev, lo, hi = shown[1].split()
+        assert size == "1000" and 0 < float(lo) <= float(median) <= float(hi) and float(stdev) >= 0
+        saved = open(out).read().strip().splitlines()
+        assert saved[0] == lines[0] and len(saved) == 1 + 3 * 5
+        assert all(r.split()[3] == "pairwise" and r.split()[8] == "1000" for r in saved[1:])
 
 
 OPS_EXE = os.path.join(ROOT, "tests", "cpp", "test_ops")
