@@ -471,19 +471,61 @@ int launch_gather(void *const *recvs, const void *const *sends, int P, const siz
 
 namespace {
 
-// The in-place part of Reduce_scatterv: one fold per block, in ascending block order; block b's
-// result overwrites the start of rank b's buffer, which only blocks <= b read.  A block that is in
-// place and starts displ elements into its own buffer with 0 < displ < count reads its own rank's
-// elements displ + i while it writes element i of the same buffer; it runs as a chained launch (see
-// ChainParams), with scratch from `fixed` if given, else from the pool of the stream.
+// The in-place part of Reduce_scatterv, in ascending block order.  Block b's result overwrites
+// elements [0, counts[b]) of rank b's buffer, which block k reads (from every rank's buffer) if
+// displ[k] < counts[b]; only blocks k <= b can.  Consecutive blocks among which no such pair
+// exists share one launch (with equal counts: block 0, then all the others, like Reduce_scatter);
+// a block that overlaps its own input - in place and 0 < displ < count: it reads its rank's
+// elements displ + i while it writes element i of the same buffer - goes alone, as a chained launch
+// (see ChainParams), with scratch from `fixed` if given, else from the pool of the stream.
 int reduce_scatterv_in_place(void *const *recvs, const void *const *sends, int P, const size_t *counts,
                              const size_t *displ, int dtype, int op, int order, hipStream_t stream,
                              const ChainScratch *fixed) {
   const size_t es = alamd_dtype_size(dtype);
-  for (int b = 0; b < P; ++b) {
-    if (counts[b] == 0) continue;
-    const bool inplace = recvs[b] == sends[b];
-    const bool overlapped = inplace && displ[b] != 0 && displ[b] < counts[b];
+  auto overlaps_itself = [&](int k) {
+    return recvs[k] == sends[k] && displ[k] != 0 && displ[k] < counts[k];
+  };
+  for (int b = 0; b < P;) {
+    if (counts[b] == 0) { ++b; continue; }
+    const bool overlapped = overlaps_itself(b);
+    if (!overlapped) {
+      // the blocks that can go with block b
+      int members[ALAMD_MAX_RANKS], n = 0, j = b + 1;
+      members[n++] = b;
+      for (; j < P; ++j) {
+        if (counts[j] == 0) continue;
+        if (overlaps_itself(j)) break;
+        bool safe = true;
+        if (recvs[j] == sends[j])
+          for (int m = 0; m < n; ++m) safe = safe && displ[members[m]] >= counts[j];
+        if (!safe) break;
+        members[n++] = j;
+      }
+      if (n > 1) {
+        Layout lay;
+        lay.nseg = (unsigned)P;
+        lay.seg = make_seg(0, 0, 1, OUT_SEG, 1);
+        lay.seg.ragged = 1;
+        void *out_tab[ALAMD_MAX_RANKS] = {nullptr};
+        size_t longest = 0;
+        for (int m = 0; m < n; ++m) {
+          const int k = members[m];
+          lay.seg.seg_off[k] = displ[k];
+          lay.seg.seg_len[k] = counts[k];
+          out_tab[k] = recvs[k];
+          if (counts[k] > longest) longest = counts[k];
+        }
+        for (int k = 0; k < P; ++k)
+          if (!out_tab[k]) out_tab[k] = recvs[k] ? recvs[k] : const_cast<void *>(sends[0]);  // never written: length 0
+        lay.max_len = longest;
+        lay.start0 = 0;
+        lay.start_stride = order_has_start(order) ? 1 : 0;
+        const int rc = launch_order(out_tab, sends, P, lay, dtype, op, order, stream);
+        if (rc) return rc;
+        b = j;
+        continue;
+      }
+    }
     // One or two runs no longer than the displacement, each launched after the one before it, never read
     // what an unfinished launch writes; beyond that one chained launch (85 to 100 % of the ordinary rate at
     // P = 8) beats a train of launches.  With the fixed scratch too small for the block, up to kMaxRuns
@@ -526,6 +568,7 @@ int reduce_scatterv_in_place(void *const *recvs, const void *const *sends, int P
       }
     }
     if (rc) return rc;
+    ++b;
   }
   return ALAMD_OK;
 }

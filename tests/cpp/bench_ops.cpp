@@ -7,7 +7,7 @@
 // time in seconds).  All logical ranks share one GPU and one launch, so every
 // rank of a trial reports the same time.
 //
-// usage: bench_ops [--op allreduce|reduce|reduce_scatter|allgather] [--datatype float|double|int|...]
+// usage: bench_ops [--op allreduce|reduce|reduce_scatter|allgather|reduce_scatterv|allgatherv] [--datatype float|double|int|...]
 //                  [--reduction-op sum|prod|min|max|...] [--algorithm automatic|rank_order|tree_doubling|
 //                  tree_halving|tree_binomial|pairwise|ring|ring_fused] [--ranks P] [--root R]
 //                  [--inplace] [--nonblocking] [--min-size N] [--max-size N] [--size N] [--num-iters N]
@@ -82,8 +82,8 @@ template <typename T> int run(const Options &o, Al::ReductionOperator rop, Algo 
   res.prefix = Backend::Name() + " " + tname + " " + o.op + " " + o.algo + " " + (o.nonblocking ? "1" : "0") + " " +
                (o.inplace ? "1" : "0") + " " + std::to_string(o.root) + " " + std::to_string(P) + " ";
   for (size_t size = o.min_size; size <= o.max_size; size *= 2) {
-    const size_t in_elems = o.op == "reduce_scatter" ? size * (size_t)P : size;
-    const size_t out_elems = o.op == "allgather" ? size * (size_t)P : size;
+    const size_t in_elems = o.op == "reduce_scatter" || o.op == "reduce_scatterv" ? size * (size_t)P : size;
+    const size_t out_elems = o.op == "allgather" || o.op == "allgatherv" ? size * (size_t)P : size;
     const size_t buf_elems = in_elems > out_elems ? in_elems : out_elems;
     std::vector<T *> in(P), out(P);
     for (int r = 0; r < P; ++r) {
@@ -116,6 +116,21 @@ template <typename T> int run(const Options &o, Al::ReductionOperator rop, Algo 
           else if (o.nonblocking) Al::NonblockingReduce_scatter<Backend>(send, recv, size, rop, comm, reqs[r], algo);
           else if (o.inplace) Al::Reduce_scatter<Backend>(buf, size, rop, comm, algo);
           else Al::Reduce_scatter<Backend>(send, recv, size, rop, comm, algo);
+        } else if (o.op == "reduce_scatterv") {
+          // every rank contributes the same count, as in the reference's benchmark
+          const std::vector<size_t> counts((size_t)P, size);
+          if (o.nonblocking && o.inplace) Al::NonblockingReduce_scatterv<Backend>(buf, counts, rop, comm, reqs[r], algo);
+          else if (o.nonblocking) Al::NonblockingReduce_scatterv<Backend>(send, recv, counts, rop, comm, reqs[r], algo);
+          else if (o.inplace) Al::Reduce_scatterv<Backend>(buf, counts, rop, comm, algo);
+          else Al::Reduce_scatterv<Backend>(send, recv, counts, rop, comm, algo);
+        } else if (o.op == "allgatherv") {
+          const std::vector<size_t> counts((size_t)P, size);
+          std::vector<size_t> displs((size_t)P);
+          for (int q = 0; q < P; ++q) displs[(size_t)q] = (size_t)q * size;
+          if (o.nonblocking && o.inplace) Al::NonblockingAllgatherv<Backend>(recv, counts, displs, comm, reqs[r], algo);
+          else if (o.nonblocking) Al::NonblockingAllgatherv<Backend>(send, recv, counts, displs, comm, reqs[r], algo);
+          else if (o.inplace) Al::Allgatherv<Backend>(recv, counts, displs, comm, algo);
+          else Al::Allgatherv<Backend>(send, recv, counts, displs, comm, algo);
         } else {
           if (o.nonblocking && o.inplace) Al::NonblockingAllgather<Backend>(recv, size, comm, reqs[r], algo);
           else if (o.nonblocking) Al::NonblockingAllgather<Backend>(send, recv, size, comm, reqs[r], algo);
@@ -183,7 +198,8 @@ int main(int argc, char **argv) {
       {"tree_halving", Algo::tree_halving}, {"tree_binomial", Algo::tree_binomial}, {"pairwise", Algo::pairwise},
       {"ring", Algo::ring}, {"ring_fused", Algo::ring_fused}};
   if (!rops.count(o.redop) || !algos.count(o.algo) || o.min_size == 0 ||
-      (o.op != "allreduce" && o.op != "reduce" && o.op != "reduce_scatter" && o.op != "allgather")) {
+      (o.op != "allreduce" && o.op != "reduce" && o.op != "reduce_scatter" && o.op != "allgather" &&
+       o.op != "reduce_scatterv" && o.op != "allgatherv")) {
     std::fprintf(stderr, "bad --op / --reduction-op / --algo / --min-size\n");
     return 2;
   }

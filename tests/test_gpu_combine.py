@@ -590,3 +590,39 @@ def test_results_do_not_depend_on_the_launch_planners_sizes(al, k):
         assert_bits_equal(to_host(ring[r], np.float32), want_ring, "f32", "fused ring rank %d, settings %d" % (r, k))
     with pytest.raises(al.AlError):
         al.tune("no_such_size", 1)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_reduce_scatterv_in_place_random_counts(al, seed):
+    """In place, with random counts (zeros, a few elements, thousands), some ranks in place and some
+    not: blocks that do not read what another writes share a launch, the others follow in order, the
+    ones that overlap their own input are chained.  Every result against the oracle, and the bytes
+    behind each result unchanged."""
+    import torch
+    rng = np.random.default_rng(1234 + seed)
+    for _ in range(5):
+        P = int(rng.choice([2, 3, 5, 8, 13, 33, 64]))
+        kind = rng.integers(0, 3)
+        if kind == 0:
+            counts = [int(c) for c in rng.integers(0, 3000, P)]
+        elif kind == 1:
+            counts = [int(rng.choice([0, 1, 7, 500, 20000])) for _ in range(P)]
+        else:  # ascending, so that late blocks are longer than early displacements
+            counts = sorted(int(c) for c in rng.integers(1, 30000, P))
+        if sum(counts) == 0:
+            counts[0] = 5
+        dtype, op = [("f32", "sum"), ("i32", "bxor"), ("bf16", "max")][int(rng.integers(0, 3))]
+        order = ["rank_asc", "pairwise_desc", "tree_halv"][int(rng.integers(0, 3))]
+        sends = make_inputs(P, sum(counts), dtype, op, seed=int(rng.integers(1, 1 << 20)))
+        want = oracle.reduce_scatterv(sends, counts, dtype, op, order)
+        bufs = [to_dev(a) for a in sends]
+        in_place = [bool(rng.integers(0, 4)) for _ in range(P)]
+        recvs = [bufs[b] if in_place[b] else dev_empty(max(counts[b], 1), sends[0].dtype) for b in range(P)]
+        al.reduce_scatterv(recvs, bufs, counts, op, order=order, dtype=dtype)
+        torch.cuda.synchronize()
+        for b in range(P):
+            got = to_host(recvs[b], sends[0].dtype)
+            assert_bits_equal(got[:counts[b]], want[b], dtype, "P=%d counts %s... %s %s %s rank %d" % (
+                P, counts[:6], dtype, op, order, b))
+            if in_place[b]:
+                assert got[counts[b]:].tobytes() == sends[b][counts[b]:].tobytes(), "rank %d: bytes behind the result changed" % b
