@@ -343,8 +343,10 @@ int launch_spread_once(const FoldParams &fp, int nsrc, SpreadShape shape, hipStr
   if (max_len == 0 || fp.P <= 0) return ALAMD_OK;
   const size_t tile = Tile<kGatherU, kGatherThreads>::BYTES;
   const size_t tiles = (max_len + tile - 1) / tile;
-  // always a multiple of 8 (see spread_kernel); workgroups past the last tile exit at once
-  const size_t tpc = tiles < shape.chunk_tiles ? (tiles + 7) & ~(size_t)7 : shape.chunk_tiles;
+  // a multiple of 8 (see spread_kernel; workgroups past the last tile exit at once) - except for
+  // slices of fewer than 8 tiles, where the idle workgroups would cost more than the sharing of an L2
+  // gains (64 slices of 4 KB to 64 buffers: 50 us with seven idle workgroups beside every busy one)
+  const size_t tpc = tiles >= shape.chunk_tiles ? shape.chunk_tiles : (tiles < 8 ? tiles : (tiles + 7) & ~(size_t)7);
   // A launch moves about spread_launch_bytes: with two or three destinations more chunks per launch
   // (untouched 128 MiB slices to two buffers 69 % -> 75 % of peak, 85 MiB slices to three 71 % -> 73 %;
   // four destinations ran 2 points better with the two chunks they have), and of many short sources
