@@ -70,6 +70,7 @@ def load():
     L.alamd_tuned.argtypes = [C.c_char_p]
     L.alamd_tuned.restype = sz
     L.alamd_ring_allreduce.argtypes = [pvp, i, sz, i, i, sz, i, vp]
+    L.alamd_ring_allreduce_from.argtypes = [pvp, pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_reduce_scatter.argtypes = [pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_allgather.argtypes = [pvp, i, sz, i, sz, vp]
     L.alamd_ring_segment.argtypes = [sz, i, i, C.POINTER(sz), C.POINTER(sz)]
@@ -226,9 +227,14 @@ def allgatherv(recvs, sends, counts, displs, dtype=None, stream=None):
 
 
 def ring_allreduce(bufs, op, chunk_bytes=4 << 20, mode="stepwise", dtype=None, count=None,
-                   stream=None):
+                   stream=None, sends=None):
+    """In place on bufs, or (sends given) from sends into bufs."""
     dtype = dtype or _infer_dtype(bufs[0])
     count = bufs[0].numel() if count is None else count
+    if sends is not None:
+        _check(load().alamd_ring_allreduce_from(_table(bufs), _table(sends), len(bufs), count, _dt(dtype), _op(op),
+                                                chunk_bytes, RING_MODES[mode], _stream(stream)))
+        return
     _check(load().alamd_ring_allreduce(_table(bufs), len(bufs), count, _dt(dtype), _op(op),
                                        chunk_bytes, RING_MODES[mode], _stream(stream)))
 

@@ -175,10 +175,12 @@ int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, bool last, h
   });
 }
 
-int fused_fold(void *const *bufs, int P, size_t count, int dtype, int op, bool all, hipStream_t stream) {
+// ins[r] is bufs[r] itself (in place) or a buffer that overlaps none of bufs.
+int fused_fold(void *const *bufs, const void *const *ins, int P, size_t count, int dtype, int op, bool all,
+               hipStream_t stream) {
   FoldParams fp;
   for (int r = 0; r < ALAMD_MAX_RANKS; ++r) {
-    fp.in[r] = r < P ? static_cast<const char *>(bufs[r]) : nullptr;
+    fp.in[r] = r < P ? static_cast<const char *>(ins[r]) : nullptr;
     fp.out[r] = r < P ? static_cast<char *>(bufs[r]) : nullptr;
   }
   fp.P = P;
@@ -264,7 +266,7 @@ int alamd_ring_reduce_scatter(void *const *bufs, int P, size_t count, int dtype,
   if (mode != ALAMD_RING_STEPWISE && mode != ALAMD_RING_FUSED)
     return set_error(ALAMD_ERR_INVALID_ALGO, "Invalid algorithm");
   if (count == 0 || P == 1) return ALAMD_OK;
-  if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, P, count, dtype, op, false, as_stream(stream));
+  if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, bufs, P, count, dtype, op, false, as_stream(stream));
   for (int t = 0; t < P - 1; ++t) {
     pl.rp.t = t;
     if ((rc = launch_step(pl, dtype, op, true, t == P - 2, as_stream(stream)))) return rc;
@@ -294,10 +296,44 @@ int alamd_ring_allreduce(void *const *bufs, int P, size_t count, int dtype, int 
   if (mode != ALAMD_RING_STEPWISE && mode != ALAMD_RING_FUSED)
     return set_error(ALAMD_ERR_INVALID_ALGO, "Invalid algorithm");
   if (count == 0 || P == 1) return ALAMD_OK;
-  if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, P, count, dtype, op, true, as_stream(stream));
+  if (mode == ALAMD_RING_FUSED) return fused_fold(bufs, bufs, P, count, dtype, op, true, as_stream(stream));
   rc = alamd_ring_reduce_scatter(bufs, P, count, dtype, op, chunk_bytes, mode, stream);
   if (rc) return rc;
   return alamd_ring_allgather(bufs, P, count, dtype, chunk_bytes, stream);
+}
+
+int alamd_ring_allreduce_from(void *const *recvs, const void *const *sends, int P, size_t count, int dtype, int op,
+                              size_t chunk_bytes, int mode, void *stream) {
+  RingPlan pl;
+  int rc = make_plan(pl, recvs, P, count, dtype, chunk_bytes);
+  if (rc) return rc;
+  if ((rc = check_type_op(dtype, op))) return rc;
+  if (mode != ALAMD_RING_STEPWISE && mode != ALAMD_RING_FUSED)
+    return set_error(ALAMD_ERR_INVALID_ALGO, "Invalid algorithm");
+  if (!sends) return set_error(ALAMD_ERR_INVALID_ARG, "null pointer table");
+  if (count == 0) return ALAMD_OK;
+  const size_t bytes = count * pl.es;
+  bool in_place = true;
+  for (int r = 0; r < P; ++r) {
+    if (!sends[r]) return set_error(ALAMD_ERR_INVALID_ARG, "send buffer %d is null", r);
+    if (!aligned_to(sends[r], pl.es))
+      return set_error(ALAMD_ERR_INVALID_ARG, "send buffer %d is not aligned to its element type", r);
+    in_place = in_place && sends[r] == recvs[r];
+    for (int k = 0; k < P; ++k) {
+      if (k == r && sends[r] == recvs[k]) continue;  // this rank in place
+      const uintptr_t x = reinterpret_cast<uintptr_t>(sends[r]), y = reinterpret_cast<uintptr_t>(recvs[k]);
+      if (x < y + bytes && y < x + bytes)
+        return set_error(ALAMD_ERR_OVERLAP, "receive buffer %d overlaps send buffer %d", k, r);
+    }
+  }
+  if (in_place) return alamd_ring_allreduce(recvs, P, count, dtype, op, chunk_bytes, mode, stream);
+  // the fused form reads the contributions where they are; the step-by-step form moves them first,
+  // as a rank of a ring would copy its send buffer before the first step
+  if (mode == ALAMD_RING_FUSED && P > 1)
+    return fused_fold(recvs, sends, P, count, dtype, op, true, as_stream(stream));
+  for (int r = 0; r < P; ++r)
+    if (sends[r] != recvs[r] && (rc = alamd_copy(recvs[r], sends[r], bytes, stream))) return rc;
+  return alamd_ring_allreduce(recvs, P, count, dtype, op, chunk_bytes, mode, stream);
 }
 
 }  // extern "C"

@@ -236,6 +236,14 @@ typedef enum {
  * carries no implementation of it. */
 int alamd_ring_allreduce(void *const *bufs, int P, size_t count, int dtype,
                          int op, size_t chunk_bytes, int mode, void *stream);
+/* The same allreduce with the contributions read from sends[r] (each identical
+ * to recvs[r] or overlapping no receive buffer), as Al::Allreduce's form with
+ * separate send and receive buffers (include/Al.hpp:118-152).  The fused mode
+ * reads them where they are; the step-by-step mode copies each into its
+ * receive buffer first. */
+int alamd_ring_allreduce_from(void *const *recvs, const void *const *sends, int P,
+                              size_t count, int dtype, int op, size_t chunk_bytes,
+                              int mode, void *stream);
 int alamd_ring_reduce_scatter(void *const *bufs, int P, size_t count, int dtype,
                               int op, size_t chunk_bytes, int mode, void *stream);
 int alamd_ring_allgather(void *const *bufs, int P, size_t count, int dtype,

@@ -621,14 +621,9 @@ inline void World::launch(PendingOp &p) {
       void *out = recvs[static_cast<size_t>(p.root)];
       rc = alamd_combine(&out, 1, sends.data(), P, p.count, p.dtype, op, order, 0, target);
     } else if (ring) {
-      // the ring works in place on each rank's receive buffer
-      for (int r = 0; r < P && rc == ALAMD_OK; ++r)
-        if (sends[static_cast<size_t>(r)] != recvs[static_cast<size_t>(r)])
-          rc = alamd_copy(recvs[static_cast<size_t>(r)], sends[static_cast<size_t>(r)], p.count * es, target);
-      if (rc == ALAMD_OK)
-        rc = alamd_ring_allreduce(recvs.data(), P, p.count, p.dtype, op, ring_chunk_bytes(es),
-                                  p.algo == CombineAlgorithm::ring ? ALAMD_RING_STEPWISE : ALAMD_RING_FUSED,
-                                  target);
+      rc = alamd_ring_allreduce_from(recvs.data(), sends.data(), P, p.count, p.dtype, op, ring_chunk_bytes(es),
+                                     p.algo == CombineAlgorithm::ring ? ALAMD_RING_STEPWISE : ALAMD_RING_FUSED,
+                                     target);
     } else {
       rc = alamd_combine(recvs.data(), P, sends.data(), P, p.count, p.dtype, op, order, 0, target);
     }

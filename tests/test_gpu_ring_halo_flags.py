@@ -87,6 +87,35 @@ def test_ring_ragged_segments_and_offsets(al, dtype, op, mode):
             assert_bits_equal(to_host(bufs[r], host[0].dtype), want[r], dtype, "%s P=%d rank %d" % (mode, P, r))
 
 
+@pytest.mark.parametrize("dtype,op", [("bf16", "sum"), ("f32", "prod"), ("i16", "min"), ("f64", "avg")])
+@pytest.mark.parametrize("mode", ("stepwise", "fused"))
+def test_ring_allreduce_from_separate_send_buffers(al, dtype, op, mode):
+    """Al::Allreduce's form with a send and a receive buffer per rank: the same bits as in place, the
+    send buffers untouched; also with some ranks in place and the others not, and at a size that
+    takes the fused form's fold-then-spread path."""
+    import torch
+    es = oracle.dtype_size(dtype)
+    for P, n in ((1, 10), (2, 4099), (5, 70_001), (8, (18 << 20) // es + 5)):
+        bufs = ring_inputs(P, n, dtype, op)
+        want = oracle.ring_allreduce(bufs, dtype, op, 512)
+        for in_place in ([False] * P, [r % 2 == 0 for r in range(P)]):
+            sends = [to_dev(b) for b in bufs]
+            recvs = [sends[r] if in_place[r] else dev_empty(n, bufs[0].dtype) for r in range(P)]
+            al.ring_allreduce(recvs, op, chunk_bytes=512 * es, mode=mode, dtype=dtype, count=n, sends=sends)
+            torch.cuda.synchronize()
+            for r in range(P):
+                assert_bits_equal(to_host(recvs[r], bufs[0].dtype), want[r], dtype,
+                                  "ring %s from send buffers, P=%d n=%d rank %d" % (mode, P, n, r))
+                if not in_place[r]:
+                    assert to_host(sends[r], bufs[0].dtype).tobytes() == bufs[r].tobytes(), "send buffer %d changed" % r
+    # a receive buffer that overlaps another rank's send buffer is refused
+    a = to_dev(oracle.fill(200, dtype, "fullrange" if dtype == "i16" else "uniform_pm1", 1))
+    b = dev_empty(100, a.cpu().numpy().dtype if False else bufs[0].dtype)
+    with pytest.raises(al.AlError) as e:
+        al.ring_allreduce([a[:100], b], op, mode=mode, dtype=dtype, count=100, sends=[b, a[50:150]])
+    assert e.value.code == 5
+
+
 def test_ring_errors(al):
     bufs = [to_dev(np.zeros(64, np.float32)) for _ in range(4)]
     with pytest.raises(al.AlError):
