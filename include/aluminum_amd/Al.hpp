@@ -277,10 +277,11 @@ struct PendingOp {
   std::string failure;
 };
 
-/** Non-blocking operations up to this many bytes per rank run on the caller's stream: their
- *  kernels take less time (about 15 us at this size for 8 ranks) than the 25 us it costs to
- *  move an operation to the internal stream and back. */
-constexpr size_t kInlineNonblockingBytes = static_cast<size_t>(4) << 20;
+/** Non-blocking operations that move up to this many bytes in all run on the caller's stream: their
+ *  kernels take less time (about 40 us at this size) than the 50 to 55 us that the two dependencies
+ *  between streams cost which move an operation to the internal stream and back (measured with 8 ranks
+ *  and 64 MiB each: blocking 95 / 168 us for a reduce / allreduce, non-blocking 150 / 226 us). */
+constexpr size_t kInlineNonblockingMovedBytes = static_cast<size_t>(256) << 20;
 
 /** The P logical ranks that live in one GPU's memory. */
 class World {
@@ -341,13 +342,25 @@ class World {
   void launch(PendingOp &p);
   /** The stream an operation runs on: blocking operations on rank 0's stream, non-blocking ones on
    *  the internal stream between the two synchronisations of ht_impl.hpp:866-888 - unless they are
-   *  small: moving to another stream and back costs about 20 us of event calls, more than a kernel
-   *  of a few microseconds could ever overlap with, so those run on rank 0's stream as well and only
-   *  leave a completion event behind. */
-  hipStream_t target_of(bool nonblocking, int dtype, size_t count, const std::vector<size_t> &counts) {
-    size_t per_rank = count;
-    for (size_t c : counts) per_rank += c;
-    const bool on_internal = nonblocking && per_rank * alamd_dtype_size(dtype) > kInlineNonblockingBytes;
+   *  small: moving to another stream and back costs 50 us and more of dependencies between streams, more
+   *  than their kernels could ever overlap with, so those run on rank 0's stream as well and only leave
+   *  a completion event behind. */
+  hipStream_t target_of(bool nonblocking, OpKind kind, int dtype, size_t count, const std::vector<size_t> &counts) {
+    if (!nonblocking) return comms_[0]->get_stream();
+    // bytes read and written by the kernels of the operation
+    const size_t P = comms_.size();
+    size_t total = 0;
+    for (size_t c : counts) total += c;
+    size_t elems = 0;
+    switch (kind) {
+    case OpKind::allreduce: elems = 2 * P * count; break;
+    case OpKind::reduce: elems = (P + 1) * count; break;
+    case OpKind::reduce_scatter: elems = (P + 1) * P * count; break;
+    case OpKind::allgather: elems = (P + 1) * P * count; break;
+    case OpKind::reduce_scatterv: elems = (P + 1) * total; break;
+    case OpKind::allgatherv: elems = (P + 1) * total; break;
+    }
+    const bool on_internal = elems * alamd_dtype_size(dtype) > kInlineNonblockingMovedBytes;
     return on_internal ? internal_stream_ : comms_[0]->get_stream();
   }
   hipStream_t gather_streams(PendingOp &p, hipStream_t target);
@@ -407,7 +420,7 @@ inline void World::post(Communicator &c, OpKind kind, int dtype, const void *sen
   // Ranks that share a stream share one event, recorded again at each of their calls, so that it
   // stands for the latest of them.
   hipEvent_t ready = nullptr;
-  if (c.get_stream() != target_of(req != nullptr, dtype, count, cv)) {
+  if (c.get_stream() != target_of(req != nullptr, kind, dtype, count, cv)) {
     if (slot)
       for (Posting &other : slot->ranks)
         if (other.posted && other.stream == c.get_stream() && other.ready) {
@@ -582,7 +595,7 @@ inline void World::release_streams(PendingOp &p, hipStream_t ran_on) {
 inline void World::launch(PendingOp &p) {
   const int P = size();
   const size_t es = alamd_dtype_size(p.dtype);
-  hipStream_t target = target_of(p.nonblocking, p.dtype, p.count, p.counts);
+  hipStream_t target = target_of(p.nonblocking, p.kind, p.dtype, p.count, p.counts);
   // Operations are launched in sequence order; one that runs on another stream than the one before
   // it waits for that one, so that it sees its results whatever the ranks' events were taken before.
   if (last_target_ != nullptr && last_target_ != target) {

@@ -259,7 +259,7 @@ static void test_stream_order(bool threaded) {
 // producer enqueued just before its call: the operation has to wait for the last producer, not the first.
 static void test_stream_order_shared_stream() {
   const int P = 3;
-  const size_t n = (6u << 20) / sizeof(float);
+  const size_t n = (48u << 20) / sizeof(float);  // 2 * P * n * 4 bytes moved: beyond what runs on the caller's stream
   hipStream_t s;
   HIPCHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
   {

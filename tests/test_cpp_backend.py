@@ -100,9 +100,9 @@ OPS_SWEEPS = [
     "--op allgather --datatype short --inplace --nonblocking --odd-sizes --max-size 65536 --ranks 8",
     "--op reduce_scatterv --datatype double --nonblocking --odd-sizes --max-size 16384 --ranks 5",
     "--op allgatherv --datatype char --inplace --nonblocking --odd-sizes --max-size 16384 --ranks 8",
-    # above 4 MiB per rank non-blocking operations take the internal stream
-    "--op allreduce --datatype double --nonblocking --odd-sizes --min-size 524288 --max-size 2097152 --ranks 4",
-    "--op reduce_scatter --datatype float --nonblocking --inplace --min-size 1048576 --max-size 2097152 --ranks 3",
+    # non-blocking operations that move more than 256 MiB in all take the internal stream
+    "--op allreduce --datatype double --nonblocking --odd-sizes --min-size 1048576 --max-size 4194304 --ranks 8",
+    "--op reduce_scatter --datatype float --nonblocking --inplace --min-size 1048576 --max-size 2097152 --ranks 8",
 ]
 
 
