@@ -34,7 +34,8 @@ int device_cus();
 // stands where it is used).  Defaults suit an MI355X; alamd_tune() changes them for comparisons.
 struct Tunables {
   size_t launch_bytes = (size_t)800 << 20;          // bytes one fold / tree launch moves
-  size_t two_step_min_bytes = (size_t)16 << 20;     // fold + spread instead of one kernel: from this size ...
+  size_t two_step_min_total_bytes = (size_t)128 << 20;  // fold + spread instead of one kernel: from this many
+                                                        // bytes written in all (outputs x bytes each) ...
   size_t two_step_min_outputs = 3;                  // ... and this many outputs up
   size_t two_step_piece_bytes = (size_t)128 << 20;  // piece of the result the two steps alternate over
   size_t ring_piece_bytes = (size_t)256 << 20;      // the same for the fused ring allreduce

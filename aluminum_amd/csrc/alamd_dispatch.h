@@ -323,15 +323,19 @@ int chain_static_init();
 
 // A result that goes to several buffers is folded into one of them and then
 // spread (one write stream per workgroup) when that is faster than writing
-// every tile to all of them from the fold kernel: from three outputs and 16 MiB
-// up.  Measured at P = 8, eight outputs, us per call in one kernel / in two
-// steps, on buffers that no earlier call has touched: 8 MiB 25 / 24, 16 MiB
-// 50 / 44, 32 MiB 99 / 85, 64 MiB 197 / 165, 128 MiB 393 / 328 (4 MiB: 12 / 15);
-// on the same buffers again and again: 8 MiB 20 / 24, 16 MiB 40 / 44, 32 MiB
-// 77 / 84, 40 MiB 119 / 103, 64 MiB 196 / 162, 128 MiB 394 / 318 (the two steps
-// take the same time either way).  At 256 MiB: two outputs 437 / 455, four
-// 544 / 529.
-// (Tunables::two_step_min_bytes, two_step_min_outputs)
+// every tile to all of them from the fold kernel: from three outputs up, once
+// outputs x bytes reaches 128 MiB (the more outputs, the earlier the interleaved
+// write streams of the single kernel cost more than a second launch).  us per
+// call in one kernel / in two steps, on buffers that no earlier call has touched:
+//   3 outputs: 16 MiB 18 / 22, 32 MiB 36 / 39, 64 MiB 72 / 72, 128 MiB 140 / 142
+//   4 outputs: 16 MiB 24 / 27, 32 MiB 49 / 48, 64 MiB 95 / 91, 128 MiB 190 / 183
+//   5 outputs: 16 MiB 29 / 33, 32 MiB 61 / 59, 64 MiB 120 / 112
+//   8 outputs: 8 MiB 22 / 22, 16 MiB 52 / 46, 32 MiB 101 / 88, 64 MiB 196 / 170
+//   16 outputs: 4 MiB 21 / 25, 8 MiB 50 / 44, 16 MiB 100 / 84
+//   33 outputs: 2 MiB 30 / 32, 4 MiB 67 / 58, 8 MiB 120 / 103
+// (on the same buffers again and again the single kernel holds out up to twice
+// these sizes: 8 outputs 16 MiB 41 / 46, 32 MiB 84 / 88, 64 MiB 197 / 170).
+// (Tunables::two_step_min_total_bytes, two_step_min_outputs)
 // The two steps alternate over pieces of the result of this many bytes, so that
 // the spread reads what the fold has just written from the 256 MiB memory-side
 // cache instead of HBM (P = 8, 1 GiB per rank, buffers no earlier call has

@@ -618,7 +618,7 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
   lay.max_len = count;
   lay.start0 = start;
   lay.start_stride = 0;
-  if ((size_t)nout < tunables().two_step_min_outputs || bytes < tunables().two_step_min_bytes)
+  if ((size_t)nout < tunables().two_step_min_outputs || bytes * (size_t)nout < tunables().two_step_min_total_bytes)
     return launch_order(out_tab, ins, P, lay, dtype, op, order, as_stream(stream));
   // Several outputs of a large result: a workgroup that wrote its tile to every
   // output would interleave nout write streams (measured 69 % of peak).  Instead

@@ -36,7 +36,7 @@ namespace {
 struct TunableName { const char *name; size_t Tunables::*field; };
 const TunableName kTunableNames[] = {
     {"launch_bytes", &Tunables::launch_bytes},
-    {"two_step_min_bytes", &Tunables::two_step_min_bytes},
+    {"two_step_min_total_bytes", &Tunables::two_step_min_total_bytes},
     {"two_step_min_outputs", &Tunables::two_step_min_outputs},
     {"two_step_piece_bytes", &Tunables::two_step_piece_bytes},
     {"ring_piece_bytes", &Tunables::ring_piece_bytes},

@@ -192,7 +192,7 @@ int fused_fold(void *const *bufs, const void *const *ins, int P, size_t count, i
   const size_t max_len = fp.seg.seg_base + (fp.seg.seg_rem ? 1 : 0);
   if (max_len == 0) return ALAMD_OK;
   const size_t es = alamd_dtype_size(dtype);
-  if (!all || (size_t)P < tunables().two_step_min_outputs || count * es < tunables().two_step_min_bytes)
+  if (!all || (size_t)P < tunables().two_step_min_outputs || count * es * (size_t)P < tunables().two_step_min_total_bytes)
     return launch_fold(fp, (unsigned)P, max_len, dtype, op, true, stream);
   // Large allreduce.  Writing each result tile to all P buffers from the fold
   // kernel interleaves P write streams; instead every segment is folded into

@@ -37,7 +37,7 @@ int alamd_narrow_f32(void *dst16, const float *src, size_t count, int dtype, voi
 int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void *stream);
 /* The sizes the launch planners cut their work by, for comparisons on a given
  * machine (not thread-safe against running calls; value 0 restores the
- * default): launch_bytes, two_step_min_bytes, two_step_min_outputs,
+ * default): launch_bytes, two_step_min_total_bytes, two_step_min_outputs,
  * two_step_piece_bytes, ring_piece_bytes, spread_launch_bytes,
  * spread_hbm_chunk_tiles, spread_hbm_launch_chunks, spread_cache_chunk_tiles,
  * spread_cache_launch_chunks.  Results never depend on them, only speed. */

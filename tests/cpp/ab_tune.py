@@ -79,7 +79,10 @@ def main():
         ("fold P=4, 256 MiB per rank, one output", lambda: combine(4, 256, 1), "launch_bytes", [400 * M, 1600 * M, HUGE]),
         ("allreduce P=8, 64 MiB per rank, eight outputs", lambda: combine(8, 64, 8), "two_step_min_outputs", [99]),
         ("allreduce P=8, 16 MiB per rank, eight outputs", lambda: combine(8, 16, 8), "two_step_min_outputs", [99]),
-        ("allreduce P=8, 8 MiB per rank, eight outputs", lambda: combine(8, 8, 8), "two_step_min_bytes", [4 * M]),
+        ("allreduce P=8, 8 MiB per rank, eight outputs", lambda: combine(8, 8, 8), "two_step_min_total_bytes", [32 * M]),
+        ("allreduce P=4, 16 MiB per rank, four outputs", lambda: combine(4, 16, 4), "two_step_min_total_bytes", [32 * M]),
+        ("allreduce P=4, 64 MiB per rank, four outputs", lambda: combine(4, 64, 4), "two_step_min_total_bytes", [HUGE]),
+        ("allreduce P=16, 8 MiB per rank, sixteen outputs", lambda: combine(16, 8, 16), "two_step_min_total_bytes", [HUGE]),
         ("allreduce P=8, 1 GiB per rank, eight outputs", lambda: combine(8, 1024, 8), "two_step_piece_bytes", [32 * M, 64 * M, 256 * M, 512 * M, HUGE]),
         ("allreduce P=8, 512 MiB per rank, eight outputs", lambda: combine(8, 512, 8), "two_step_piece_bytes", [64 * M, 256 * M, HUGE]),
         ("allreduce P=8, 256 MiB per rank: the spread of a result just written", lambda: combine(8, 256, 8),

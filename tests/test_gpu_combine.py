@@ -539,12 +539,12 @@ def test_reduce_scatterv_chained_wait_that_gives_up_is_reported(al):
 
 SETTINGS = [
     {},  # the defaults
-    {"launch_bytes": 1 << 20, "two_step_min_bytes": 4096, "two_step_piece_bytes": 64 << 10,
+    {"launch_bytes": 1 << 20, "two_step_min_total_bytes": 4096, "two_step_piece_bytes": 64 << 10,
      "ring_piece_bytes": 128 << 10, "spread_launch_bytes": 1 << 20, "spread_hbm_chunk_tiles": 8,
      "spread_hbm_launch_chunks": 1, "spread_cache_chunk_tiles": 8, "spread_cache_launch_chunks": 1},
     {"launch_bytes": 1 << 40, "two_step_min_outputs": 99, "spread_hbm_chunk_tiles": 24, "spread_hbm_launch_chunks": 3,
      "spread_launch_bytes": 1 << 40, "ring_piece_bytes": 1 << 40},
-    {"two_step_min_bytes": 1, "two_step_min_outputs": 2, "two_step_piece_bytes": 1 << 20,
+    {"two_step_min_total_bytes": 1, "two_step_min_outputs": 2, "two_step_piece_bytes": 1 << 20,
      "spread_cache_chunk_tiles": 16, "spread_cache_launch_chunks": 2, "launch_bytes": 3 << 20},
 ]
 
