@@ -12,6 +12,7 @@
 //                  tree_halving|tree_binomial|pairwise|ring|ring_fused] [--ranks P] [--root R]
 //                  [--inplace] [--nonblocking] [--min-size N] [--max-size N] [--size N] [--num-iters N]
 //                  [--num-warmup N] [--summarize] [--save-to-file FILE] [--no-print-table] [--backend hip]
+//                  [--stream-per-rank]
 // (--summarize: per size "Size Mean Median Stdev Min Max" over the timed trials, benchmark_ops.cpp:211-224;
 // --save-to-file / --no-print-table: where the table of rows goes, :225-230.)
 #include <hip/hip_runtime_api.h>
@@ -37,7 +38,7 @@ struct Options {
   int ranks = 8, root = 0;
   bool inplace = false, nonblocking = false;
   size_t min_size = 1, max_size = (size_t)1 << 22, iters = 100, warmup = 10;
-  bool summarize = false, print_table = true;
+  bool summarize = false, print_table = true, stream_per_rank = false;
   std::string save_to;
 };
 
@@ -94,8 +95,14 @@ template <typename T> int run(const Options &o, Al::ReductionOperator rop, Algo 
         return 2;
       }
     }
-    Al::amd::World world(P, stream);
+    // every logical rank on one stream, or each on its own (the time is still taken on rank 0's, where
+    // a blocking operation runs; the others are made to wait for it)
+    std::vector<hipStream_t> streams((size_t)P, stream);
+    if (o.stream_per_rank)
+      for (int r = 1; r < P; ++r) HIPCHK(hipStreamCreateWithFlags(&streams[(size_t)r], hipStreamNonBlocking));
     std::vector<double> times;
+    {
+    Al::amd::World world(streams);
     for (size_t trial = 0; trial < o.warmup + o.iters; ++trial) {
       std::vector<Backend::req_type> reqs(P);
       HIPCHK(hipStreamSynchronize(stream));  // stands in for the barrier before each trial
@@ -146,6 +153,10 @@ template <typename T> int run(const Options &o, Al::ReductionOperator rop, Algo 
       HIPCHK(hipEventElapsedTime(&ms, e0, e1));
       if (trial >= o.warmup) times.push_back(ms * 1e-3);
     }
+    for (int r = 1; r < P; ++r) HIPCHK(hipStreamSynchronize(streams[(size_t)r]));
+    }
+    if (o.stream_per_rank)
+      for (int r = 1; r < P; ++r) HIPCHK(hipStreamDestroy(streams[(size_t)r]));
     res.times[size] = times;
     for (int r = 0; r < P; ++r) { HIPCHK(hipFree(in[r])); HIPCHK(hipFree(out[r])); }
   }
@@ -176,6 +187,7 @@ int main(int argc, char **argv) {
     else if (a == "--summarize") o.summarize = true;
     else if (a == "--save-to-file") o.save_to = next();
     else if (a == "--no-print-table") o.print_table = false;
+    else if (a == "--stream-per-rank") o.stream_per_rank = true;
     else if (a == "--backend") { if (next() != "hip") { std::fprintf(stderr, "this program benchmarks the hip backend only\n"); return 2; } }
     else if (a == "--help") { std::printf("see the usage comment at the top of tests/cpp/bench_ops.cpp\n"); return 0; }
     else if (a == "--ranks") o.ranks = std::atoi(next().c_str());
