@@ -92,9 +92,9 @@ def main():
         ("allgather P=8, 32 MiB slices", lambda: allgather(8, 32), "spread_hbm_chunk_tiles", [512, 2048]),
         ("allgather P=8, 128 MiB slices", lambda: allgather(8, 128), "spread_hbm_launch_chunks", [1, 8, HUGE]),
         ("allgather P=8, 32 MiB slices: bytes per launch", lambda: allgather(8, 32), "spread_launch_bytes", [72 * M, 1152 * M]),
-        ("fused ring allreduce bf16 P=8, 256 MiB per rank", lambda: ring(8, 256), "ring_piece_bytes", [16 * M, 256 * M, HUGE]),
-        ("fused ring allreduce bf16 P=8, 1 GiB per rank", lambda: ring(8, 1024), "ring_piece_bytes", [128 * M, 256 * M, 512 * M, HUGE]),
-        ("fused ring allreduce bf16 P=4, 256 MiB per rank", lambda: ring(4, 256), "ring_piece_bytes", [256 * M, HUGE]),
+        ("fused ring allreduce bf16 P=8, 256 MiB per rank", lambda: ring(8, 256), "ring_piece_bytes", [16 * M, 64 * M, HUGE]),
+        ("fused ring allreduce bf16 P=8, 1 GiB per rank", lambda: ring(8, 1024), "ring_piece_bytes", [64 * M, 128 * M, 512 * M, HUGE]),
+        ("fused ring allreduce bf16 P=4, 256 MiB per rank", lambda: ring(4, 256), "ring_piece_bytes", [64 * M, HUGE]),
     ]
     for label, make, name, alts in cases:
         if args.only and args.only not in name and args.only not in label:
