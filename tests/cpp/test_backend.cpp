@@ -193,6 +193,98 @@ static void test_halo_two_ranks(bool wait_first) {
   for (auto &x : s) HIPCHK(hipStreamDestroy(x));
 }
 
+// A token goes round the ring of logical ranks and back, one thread and one stream per rank, with
+// AttachRemoteBuffer / Put / Notify / Wait as the reference's ring test drives them
+// (test/test_rma_ring.cpp:38-108): rank 0 starts, every other rank waits for its left neighbour,
+// puts to its right one and notifies it; then the same from the last rank leftwards.  Stricter than
+// there: every buffer starts from a sentinel, so a rank holds the token only if the puts brought it.
+struct ThreadBarrier {
+  std::mutex m;
+  std::condition_variable cv;
+  int n, waiting = 0;
+  unsigned long generation = 0;
+  explicit ThreadBarrier(int n_) : n(n_) {}
+  void arrive_and_wait() {
+    std::unique_lock<std::mutex> lock(m);
+    const unsigned long g = generation;
+    if (++waiting == n) {
+      waiting = 0;
+      ++generation;
+      cv.notify_all();
+    } else {
+      cv.wait(lock, [&] { return generation != g; });
+    }
+  }
+};
+
+static void test_rma_token_ring(int P) {
+  std::vector<hipStream_t> streams(static_cast<size_t>(P));
+  for (auto &s : streams) HIPCHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  {
+    Al::amd::World world(streams);
+    world.set_calls_wait_for_launch(true);
+    std::vector<size_t> sizes = {0};
+    for (size_t n = 1; n <= (size_t(1) << 18); n *= 4) {
+      sizes.push_back(n);
+      if (n > 1) sizes.push_back(n + 1);
+    }
+    ThreadBarrier barrier(P);
+    std::vector<std::unique_ptr<DevBuf<float>>> buf(static_cast<size_t>(P));
+    std::vector<std::thread> th;
+    for (int rank = 0; rank < P; ++rank)
+      th.emplace_back([&, rank] {
+        auto &comm = world.comm(rank);
+        const hipStream_t stream = streams[static_cast<size_t>(rank)];
+        const int rhs = (rank + 1) % P, lhs = (rank - 1 + P) % P;
+        for (size_t n : sizes) {
+          const std::vector<float> token = gen<float>(n, ALO_DIST_UNIFORM_PM1, 7000u + static_cast<unsigned>(n));
+          buf[static_cast<size_t>(rank)].reset(new DevBuf<float>(n));
+          float *mine = buf[static_cast<size_t>(rank)]->p;
+          float *rhs_buf, *lhs_buf;
+          if (rank % 2) {
+            rhs_buf = Al::ext::AttachRemoteBuffer<Backend>(mine, rhs, comm);
+            lhs_buf = Al::ext::AttachRemoteBuffer<Backend>(mine, lhs, comm);
+          } else {
+            lhs_buf = Al::ext::AttachRemoteBuffer<Backend>(mine, lhs, comm);
+            rhs_buf = Al::ext::AttachRemoteBuffer<Backend>(mine, rhs, comm);
+          }
+          barrier.arrive_and_wait();
+          if (rank == 0) {
+            EXPECT(lhs_buf == buf[static_cast<size_t>(lhs)]->p && rhs_buf == buf[static_cast<size_t>(rhs)]->p,
+                   "rank 0 reaches its neighbours' buffers (%d ranks, %zu elements)", P, n);
+          }
+          for (int pass = 0; pass < 2; ++pass) {
+            const int first = pass == 0 ? 0 : P - 1, to = pass == 0 ? rhs : lhs, from = pass == 0 ? lhs : rhs;
+            float *to_buf = pass == 0 ? rhs_buf : lhs_buf;
+            if (n) HIPCHK(hipMemsetAsync(mine, 0xff, n * sizeof(float), stream));
+            HIPCHK(hipStreamSynchronize(stream));
+            barrier.arrive_and_wait();  // every sentinel is in place before the first put
+            if (rank != first)
+              Al::ext::Wait<Backend>(from, comm);
+            else if (n)
+              HIPCHK(hipMemcpyAsync(mine, token.data(), n * sizeof(float), hipMemcpyHostToDevice, stream));
+            Al::ext::Put<Backend>(static_cast<const float *>(mine), to, to_buf, n, comm);
+            Al::ext::Notify<Backend>(to, comm);
+            if (rank == first) Al::ext::Wait<Backend>(from, comm);
+            HIPCHK(hipStreamSynchronize(stream));
+            barrier.arrive_and_wait();
+            if (rank == 0)  // one thread checks, the others stand at the next barrier
+              for (int r = 0; r < P; ++r)
+                EXPECT(same_bits(buf[static_cast<size_t>(r)]->down(), token),
+                       "token at rank %d after the pass %s (%d ranks, %zu elements)", r,
+                       pass == 0 ? "rightwards" : "leftwards", P, n);
+            barrier.arrive_and_wait();
+          }
+          Al::ext::DetachRemoteBuffer<Backend>(rhs_buf, rhs, comm);
+          Al::ext::DetachRemoteBuffer<Backend>(lhs_buf, lhs, comm);
+          barrier.arrive_and_wait();  // nobody frees a buffer a neighbour still reads
+        }
+      });
+    for (auto &t : th) t.join();
+  }
+  for (auto &s : streams) HIPCHK(hipStreamDestroy(s));
+}
+
 // Every rank on its own stream, each stream held back by a gate the host opens late and in
 // reverse order: the collective must wait for what every stream held at its rank's call, and the
 // copies enqueued after the last call must see the result.
@@ -500,6 +592,7 @@ int main() {
   test_halo_loopback(stream);
   test_halo_two_ranks(false);
   test_halo_two_ranks(true);
+  for (int P : {1, 2, 3, 5, 8}) test_rma_token_ring(P);
   test_progress_engine_early_signal(stream);
   test_progress_engine_exception(stream);
   test_flags(stream);
