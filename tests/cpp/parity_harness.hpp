@@ -24,9 +24,10 @@ using Backend = Al::HipCombineBackend;
 using Algo = Al::amd::CombineAlgorithm;
 using Op = Al::ReductionOperator;
 
-static int g_fail = 0, g_checks = 0;  // one translation unit per program
+static std::atomic<int> g_fail{0}, g_checks{0};  // one translation unit per program
+static thread_local int t_fail = 0;               // the calling thread's share of g_fail
 #define HIPCHK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { std::printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__); std::exit(2); } } while (0)
-#define EXPECT(cond, ...) do { ++g_checks; if (!(cond)) { ++g_fail; std::printf("FAIL line %d: ", __LINE__); std::printf(__VA_ARGS__); std::printf("\n"); } } while (0)
+#define EXPECT(cond, ...) do { ++g_checks; if (!(cond)) { ++g_fail; ++t_fail; std::printf("FAIL line %d: ", __LINE__); std::printf(__VA_ARGS__); std::printf("\n"); } } while (0)
 
 template <typename T> struct DevBuf {
   T *p = nullptr;

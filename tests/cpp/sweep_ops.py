@@ -2,7 +2,7 @@
 reference's test driver (test/run_tests.py: collective x datatype x in place x
 non-blocking x sizes), with logical ranks in place of MPI processes.
 
-    python tests/cpp/sweep_ops.py [--seed S] [--runs N] [--max-size M]
+    python tests/cpp/sweep_ops.py [--seed S] [--runs N] [--max-size M] [--threads SHARE]
 
 Every run is one test_ops process; it compares with the CPU oracle bit for bit.
 Exit status 1 if any run fails."""
@@ -34,6 +34,8 @@ def main():
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--runs", type=int, default=200)
     ap.add_argument("--max-size", type=int, default=262144)
+    ap.add_argument("--threads", type=float, default=0.0,
+                    help="share of runs that drive the sweep from 2 to 4 threads at once (test_ops --threads)")
     args = ap.parse_args()
     exe = os.path.join(HERE, "test_ops")
     if not os.path.exists(exe):
@@ -53,6 +55,8 @@ def main():
             cmd.append("--inplace")
         if rng.random() < 0.5:
             cmd.append("--nonblocking")
+        if args.threads > 0 and rng.random() < args.threads:
+            cmd += ["--threads", str(rng.choice([2, 3, 4]))]
         p = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
         if p.returncode != 0 or "PASSED" not in p.stdout:
             fails += 1

@@ -601,7 +601,7 @@ int main() {
   HIPCHK(hipStreamDestroy(stream));
   Al::Finalize();
   EXPECT(!Al::Initialized(), "not initialised after Finalize");
-  std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks, g_fail);
+  std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks.load(), g_fail.load());
   std::fflush(stdout);  // before the runtime libraries are torn down
   return g_fail ? 1 : 0;
 }

@@ -10,7 +10,7 @@
 //                 [--backend hip] [--inplace] [--nonblocking] [--reduction-op sum|prod|min|max|lor|land|lxor|bor|band|bxor]
 //                 [--algorithm automatic|rank_order|tree_doubling|tree_halving|tree_binomial|pairwise|ring|ring_fused]
 //                 [--root R] [--size N | --min-size N --max-size N] [--odd-sizes] [--datatype float|...]
-//                 [--trials N] [--ranks P]
+//                 [--trials N] [--ranks P] [--threads N]
 #include <map>
 
 #include "parity_harness.hpp"
@@ -18,7 +18,7 @@
 struct Options {
   std::string op, backend = "hip", redop = "sum", algorithm = "automatic", datatype = "float";
   bool inplace = false, nonblocking = false, odd_sizes = false, have_size = false;
-  int root = 0, ranks = 4;
+  int root = 0, ranks = 4, threads = 0;
   size_t size = 0, min_size = 1, max_size = (size_t)1 << 22, trials = 1;
 };
 
@@ -49,14 +49,14 @@ template <typename T> int dist_for(Op op) {
   return ALO_DIST_FULLRANGE;
 }
 
-template <typename T> int run(const Options &o, Op rop, Algo algo) {
+template <typename T> void sweep(const Options &o, Op rop, Algo algo, int thread) {
   hipStream_t stream;
   HIPCHK(hipStreamCreate(&stream));
   const int P = o.ranks;
   const int dist = dist_for<T>(rop);
   for (size_t trial = 0; trial < o.trials; ++trial)
     for (size_t size : get_sizes(o)) {
-      const int before = g_fail;
+      const int before = t_fail;
       if (o.op == "allreduce") test_allreduce<T>(P, size, rop, algo, dist, o.inplace, o.nonblocking, stream);
       else if (o.op == "reduce") test_reduce<T>(P, size, rop, o.root, stream, o.nonblocking ? 1 : 0, o.inplace, dist, algo);
       else if (o.op == "reduce_scatter") test_reduce_scatter<T>(P, size, rop, algo, o.inplace, stream, o.nonblocking, dist);
@@ -64,12 +64,33 @@ template <typename T> int run(const Options &o, Op rop, Algo algo) {
       else if (o.op == "reduce_scatterv")
         test_v_variants<T>(P, o.inplace, stream, o.nonblocking, size, size / 4 + 1, rop, true, false, dist);
       else test_v_variants<T>(P, o.inplace, stream, o.nonblocking, size, size / 4 + 1, rop, false, true, dist);
-      std::printf("%s %s %s %s nonblocking=%d inplace=%d root=%d ranks=%d size=%zu: %s\n", o.op.c_str(),
-                  o.datatype.c_str(), o.redop.c_str(), o.algorithm.c_str(), o.nonblocking, o.inplace, o.root, P, size,
-                  g_fail == before ? "ok" : "MISMATCH");
+      std::printf("%s %s %s %s nonblocking=%d inplace=%d root=%d ranks=%d%s size=%zu: %s\n", o.op.c_str(),
+                  o.datatype.c_str(), o.redop.c_str(), o.algorithm.c_str(), o.nonblocking, o.inplace, o.root, P,
+                  thread < 0 ? "" : (" thread=" + std::to_string(thread)).c_str(), size,
+                  t_fail == before ? "ok" : "MISMATCH");
     }
   HIPCHK(hipStreamDestroy(stream));
-  std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks, g_fail);
+}
+
+// --threads N: N threads run the sweep at the same time, each with communicators and a stream of
+// its own (test/test_ops.cpp:267-273,373-391); without it the calling thread runs it.
+template <typename T> int run(const Options &o, Op rop, Algo algo) {
+  if (o.threads <= 0) {
+    sweep<T>(o, rop, algo, -1);
+  } else {
+    std::vector<std::thread> th;
+    for (int i = 0; i < o.threads; ++i)
+      th.emplace_back([&, i] {
+        try {
+          sweep<T>(o, rop, algo, i);
+        } catch (const std::exception &e) {
+          std::printf("thread %d: exception: %s\n", i, e.what());
+          ++g_fail;
+        }
+      });
+    for (auto &t : th) t.join();
+  }
+  std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks.load(), g_fail.load());
   std::fflush(stdout);  // before the runtime libraries are torn down
   return g_fail ? 1 : 0;
 }
@@ -96,6 +117,7 @@ int main(int argc, char **argv) {
     else if (a == "--datatype") o.datatype = next();
     else if (a == "--trials") o.trials = std::strtoull(next().c_str(), nullptr, 10);
     else if (a == "--ranks") o.ranks = std::atoi(next().c_str());
+    else if (a == "--threads") o.threads = std::atoi(next().c_str());
     else if (a == "--help") { std::printf("see the head of tests/cpp/test_ops.cpp\n"); return 0; }
     else { std::fprintf(stderr, "unknown option %s\n", a.c_str()); return 2; }
   }

@@ -103,6 +103,12 @@ OPS_SWEEPS = [
     # non-blocking operations that move more than 256 MiB in all take the internal stream
     "--op allreduce --datatype double --nonblocking --odd-sizes --min-size 1048576 --max-size 4194304 --ranks 8",
     "--op reduce_scatter --datatype float --nonblocking --inplace --min-size 1048576 --max-size 2097152 --ranks 8",
+    # several threads at once, each with communicators and a stream of its own (test/test_ops.cpp:373-391)
+    "--op allreduce --datatype float --threads 4 --odd-sizes --max-size 262144 --ranks 4",
+    "--op allreduce --datatype bfloat16 --threads 3 --nonblocking --algorithm ring --max-size 65536 --ranks 8",
+    "--op reduce_scatterv --datatype float --threads 4 --inplace --odd-sizes --max-size 1048576 --ranks 8",
+    "--op allgatherv --datatype int --threads 4 --nonblocking --odd-sizes --max-size 65536 --ranks 5",
+    "--op allreduce --datatype double --threads 2 --nonblocking --min-size 2097152 --max-size 4194304 --ranks 8",
 ]
 
 
