@@ -173,3 +173,29 @@ def test_halo_grid_beyond_4_gib(al):
         slab = before[tuple(take)]
         assert torch.equal(bufs[f], slab.contiguous().view(-1)), "face %d" % f
         assert torch.equal(g3[tuple(put)], slab), "ghost slab of face %d" % f
+
+
+def test_eight_buffers_of_16_gib(al):
+    """Half of the 288 GB: eight 16 GiB inputs and one output, bitwise xor.  Slices against the oracle,
+    and a whole-buffer property: folding the result with seven inputs again gives back the eighth."""
+    import torch
+    P, n = 8, (1 << 34) + 4099
+    free, _ = torch.cuda.mem_get_info()
+    if free < (P + 2) * n + (4 << 30):
+        pytest.skip("needs %d GiB of free device memory" % (((P + 2) * n >> 30) + 4))
+    ins = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(P)]
+    for r in range(P):
+        al.fill(ins[r], "fullrange", 900 + r, dtype="u8")
+    out = torch.empty(n, dtype=torch.uint8, device="cuda")
+    al.combine([out], ins, "bxor", dtype="u8")
+    torch.cuda.synchronize()
+    for lo in (0, (1 << 32) - SLICE // 2, (1 << 33) + 12345, n - SLICE):
+        want = oracle.combine_generated(P, SLICE, "u8", "bxor", "rank_asc", 0, "fullrange", 900, lo)
+        assert out[lo:lo + SLICE].cpu().numpy().tobytes() == want.tobytes(), "slice at %d" % lo
+    back = torch.empty(n, dtype=torch.uint8, device="cuda")
+    al.combine([back], [out] + ins[1:], "bxor", dtype="u8")
+    torch.cuda.synchronize()
+    same = torch.equal(back, ins[0])
+    del ins, out, back
+    torch.cuda.empty_cache()  # give the 160 GiB back: other processes of the test run allocate too
+    assert same
