@@ -46,11 +46,19 @@ def main():
     for k in range(args.runs):
         op, dt = rng.choice(OPS), rng.choice(DATATYPES)
         ranks = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16, 24, 32, 33, 40, 48, 63, 64])
+        max_size = rng.choice([4096, 65536, args.max_size])
+        # what the run holds in memory (and checks on the host) grows with ranks^2 x size for every
+        # collective but allreduce and reduce: keep it to a few GB, or one draw takes minutes
+        elem = {"char": 1, "schar": 1, "uchar": 1, "short": 2, "ushort": 2, "half": 2, "bfloat16": 2, "int": 4,
+                "uint": 4, "float": 4}.get(dt, 8)
+        held = ranks * (ranks if op not in ("allreduce", "reduce") else 2) * elem * 2
+        while max_size > 4096 and held * max_size > (8 << 30):
+            max_size //= 2
         cmd = [exe, "--op", op, "--datatype", dt,
                "--reduction-op", rng.choice(FP_REDUCTIONS if dt in FLOATS else INT_REDUCTIONS),
                "--algorithm", rng.choice(ALGORITHMS[op]), "--ranks", str(ranks), "--root", str(rng.randrange(ranks)),
                "--odd-sizes", "--min-size", str(rng.choice([0, 1, 3, 64])),
-               "--max-size", str(rng.choice([4096, 65536, args.max_size]))]
+               "--max-size", str(max_size)]
         if rng.random() < 0.5:
             cmd.append("--inplace")
         if rng.random() < 0.5:
