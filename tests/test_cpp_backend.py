@@ -19,6 +19,17 @@ def test_front_end_compiles_with_the_host_compiler():
     assert os.path.exists(EXE)
 
 
+def test_launch_planner_covers_every_tile_once():
+    """plan_launches (alamd_dispatch.h) on random segment tables, on the host: every tile of every
+    segment in exactly one launch, grids within the device's limits."""
+    exe = os.path.join(ROOT, "tests", "cpp", "test_planner")
+    if not os.path.exists(exe):
+        subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp"), "test_planner"], check=True,
+                       stdout=subprocess.DEVNULL)
+    p = subprocess.run([exe, "1200"], capture_output=True, text=True, timeout=280)
+    assert p.returncode == 0 and "PASSED" in p.stdout, p.stdout[-2000:] + p.stderr[-1000:]
+
+
 def test_front_end_names_the_reference_interface():
     text = open(os.path.join(ROOT, "include", "aluminum_amd", "Al.hpp")).read()
     for name in ("comm_type", "req_type", "null_req", "allreduce_algo_type", "reduce_scatter_algo_type",
