@@ -33,18 +33,20 @@ Tunables &tunables() {
 }
 
 namespace {
-struct TunableName { const char *name; size_t Tunables::*field; };
+// least: the pieces of a two-step call at least 64 KiB (smaller ones would turn one call into millions
+// of launches; less than one element, into a loop that never ends)
+struct TunableName { const char *name; size_t Tunables::*field; size_t least; };
 const TunableName kTunableNames[] = {
-    {"launch_bytes", &Tunables::launch_bytes},
-    {"two_step_min_total_bytes", &Tunables::two_step_min_total_bytes},
-    {"two_step_min_outputs", &Tunables::two_step_min_outputs},
-    {"two_step_piece_bytes", &Tunables::two_step_piece_bytes},
-    {"ring_piece_bytes", &Tunables::ring_piece_bytes},
-    {"spread_launch_bytes", &Tunables::spread_launch_bytes},
-    {"spread_hbm_chunk_tiles", &Tunables::spread_hbm_chunk_tiles},
-    {"spread_hbm_launch_chunks", &Tunables::spread_hbm_launch_chunks},
-    {"spread_cache_chunk_tiles", &Tunables::spread_cache_chunk_tiles},
-    {"spread_cache_launch_chunks", &Tunables::spread_cache_launch_chunks},
+    {"launch_bytes", &Tunables::launch_bytes, 1},
+    {"two_step_min_total_bytes", &Tunables::two_step_min_total_bytes, 1},
+    {"two_step_min_outputs", &Tunables::two_step_min_outputs, 1},
+    {"two_step_piece_bytes", &Tunables::two_step_piece_bytes, (size_t)64 << 10},
+    {"ring_piece_bytes", &Tunables::ring_piece_bytes, (size_t)64 << 10},
+    {"spread_launch_bytes", &Tunables::spread_launch_bytes, 1},
+    {"spread_hbm_chunk_tiles", &Tunables::spread_hbm_chunk_tiles, 1},
+    {"spread_hbm_launch_chunks", &Tunables::spread_hbm_launch_chunks, 1},
+    {"spread_cache_chunk_tiles", &Tunables::spread_cache_chunk_tiles, 1},
+    {"spread_cache_launch_chunks", &Tunables::spread_cache_launch_chunks, 1},
 };
 }  // namespace
 
@@ -112,6 +114,8 @@ int alamd_tune(const char *name, size_t value) {
   const alamd::Tunables defaults;
   for (const auto &t : alamd::kTunableNames)
     if (std::string(name) == t.name) {
+      if (value != 0 && value < t.least)
+        return alamd::set_error(ALAMD_ERR_INVALID_ARG, "%s must be at least %zu (0 restores the default)", name, t.least);
       alamd::tunables().*(t.field) = value ? value : defaults.*(t.field);
       return ALAMD_OK;
     }

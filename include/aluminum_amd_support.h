@@ -40,7 +40,8 @@ int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void
  * default): launch_bytes, two_step_min_total_bytes, two_step_min_outputs,
  * two_step_piece_bytes, ring_piece_bytes, spread_launch_bytes,
  * spread_hbm_chunk_tiles, spread_hbm_launch_chunks, spread_cache_chunk_tiles,
- * spread_cache_launch_chunks.  Results never depend on them, only speed. */
+ * spread_cache_launch_chunks.  Piece sizes below 64 KiB are refused.
+ * Results never depend on them, only speed. */
 int alamd_tune(const char *name, size_t value);
 size_t alamd_tuned(const char *name);
 /* Polls after which a wait inside a chained in-place Reduce_scatterv launch

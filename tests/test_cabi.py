@@ -99,6 +99,21 @@ def test_argument_checks_need_no_gpu():
     assert L.alamd_version() >= 1
 
 
+def test_launch_planner_sizes_are_checked():
+    """alamd_tune: unknown names and piece sizes that would never finish a call are errors; 0 restores a default."""
+    import aluminum_amd as al
+    default = al.tuned("ring_piece_bytes")
+    assert default == 256 << 20 and al.tuned("no such size") == 0
+    al.tune("ring_piece_bytes", 1 << 20)
+    assert al.tuned("ring_piece_bytes") == 1 << 20
+    al.tune("ring_piece_bytes", 0)
+    assert al.tuned("ring_piece_bytes") == default
+    for name, value in (("two_step_piece_bytes", 4), ("ring_piece_bytes", 1000), ("no such size", 1 << 20)):
+        with pytest.raises(al.AlError):
+            al.tune(name, value)
+    assert al.tuned("two_step_piece_bytes") == 128 << 20
+
+
 def test_graft_entry_has_build_and_smoke():
     import importlib
     g = importlib.import_module("__graft_entry__")
