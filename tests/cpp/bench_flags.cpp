@@ -3,6 +3,9 @@
 //   enqueue   host cost of enqueueing one wait / one flag write
 //   resume    host signal -> the stream gets past the wait and writes the
 //             next flag -> the host sees it
+//   completion  a flag written by the stream against a runtime event, as
+//             benchmark_events.cpp compares them: cost of recording on an
+//             idle stream, and how long until the host's query sees it
 // Prints one JSON line.  usage: bench_flags [iterations]
 #include <hip/hip_runtime_api.h>
 
@@ -55,6 +58,45 @@ static int run_mode(int mode, const char *name, int iters, hipStream_t stream, b
   return 0;
 }
 
+// record on an idle stream, then poll from the host: the status flag (alamd_stream_write_flag +
+// alamd_flag_query) against hipEventRecord + hipEventQuery
+static int run_completion(int mode, const char *name, int iters, hipStream_t stream) {
+  alamd_flag *flag;
+  CHK(alamd_flag_create(&flag, 0));
+  hipEvent_t ev;
+  HIPCHK(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+  std::vector<double> rec_flag, seen_flag, rec_ev, seen_ev;
+  for (int it = 0; it < iters + 20; ++it) {
+    CHK(alamd_flag_signal(flag, 0));
+    auto t0 = clk::now();
+    CHK(alamd_stream_write_flag(stream, flag, 1, mode));
+    auto t1 = clk::now();
+    while (alamd_flag_query(flag) != 1) {
+      if (us(t1, clk::now()) > 5e6) { std::printf("timeout in completion %s\n", name); return 3; }
+    }
+    auto t2 = clk::now();
+    HIPCHK(hipStreamSynchronize(stream));
+    auto t3 = clk::now();
+    HIPCHK(hipEventRecord(ev, stream));
+    auto t4 = clk::now();
+    while (hipEventQuery(ev) == hipErrorNotReady) {
+      if (us(t4, clk::now()) > 5e6) { std::printf("timeout in completion %s\n", name); return 3; }
+    }
+    auto t5 = clk::now();
+    HIPCHK(hipStreamSynchronize(stream));
+    if (it >= 20) {
+      rec_flag.push_back(us(t0, t1)); seen_flag.push_back(us(t1, t2));
+      rec_ev.push_back(us(t3, t4)); seen_ev.push_back(us(t4, t5));
+    }
+  }
+  std::printf(", \"completion_%s\": {\"flag_record_us\": %.3f, \"flag_seen_after_us\": %.3f, "
+              "\"hip_event_record_us\": %.3f, \"hip_event_seen_after_us\": %.3f}",
+              name, median(rec_flag), median(seen_flag), median(rec_ev), median(seen_ev));
+  HIPCHK(hipEventDestroy(ev));
+  CHK(alamd_flag_destroy(flag));
+  return 0;
+}
+
 int main(int argc, char **argv) {
   const int iters = argc > 1 ? std::atoi(argv[1]) : 2000;
   HIPCHK(hipSetDevice(0));
@@ -69,6 +111,9 @@ int main(int argc, char **argv) {
     rc = run_mode(ALAMD_FLAG_MEMOP, "memop", iters, stream, true);
     if (rc) return rc;
   }
+  rc = run_completion(ALAMD_FLAG_KERNEL, "kernel", iters, stream);
+  if (rc) return rc;
+  if (memops && (rc = run_completion(ALAMD_FLAG_MEMOP, "memop", iters, stream))) return rc;
   std::printf("}\n");
   HIPCHK(hipStreamDestroy(stream));
   return 0;
