@@ -421,14 +421,43 @@ int alo_schedule(int P, int order, int start, int *pairs, int *result) {
     return np;
   }
   case ALO_ORDER_TREE_BINOMIAL:
-    /* binomial reduce to rank 0: at distance d every rank that is a multiple
-     * of 2d folds in the partial of rank+d, if that rank exists */
+    /* binomial reduce to rank `start`, over ranks counted from it with wrap:
+     * at distance d every relative rank that is a multiple of 2d folds in the
+     * partial of relative rank + d, if that rank exists */
     for (int d = 1; d < P; d *= 2)
       for (int i = 0; i + d < P; i += 2 * d) {
-        pairs[2 * np] = i; pairs[2 * np + 1] = i + d; np++;
+        pairs[2 * np] = (i + start) % P; pairs[2 * np + 1] = (i + d + start) % P; np++;
       }
-    *result = 0;
+    *result = start;
     return np;
+  case ALO_ORDER_TREE_RSG: {
+    /* Reduce-scatter by recursive halving of the data at distance 1, 2, 4, ...
+     * followed by a gather.  Non-power-of-two P: the odd ranks among the first
+     * 2*rem send to the even rank below them, which keeps the result.  The
+     * survivors then pair at distance d = 1, 2, 4, ...; of a pair, the one
+     * whose bit d equals that bit of `start` keeps the result.  `start` is the
+     * survivor that ends up owning the block the element lies in (see
+     * alo_rsg_owner); only survivors that agree with it below bit d still
+     * hold a partial of that block. */
+    int pof2 = floor_pow2(P), rem = P - pof2;
+    if (start >= pof2) return -1;
+    int *L = (int *)malloc(sizeof(int) * (size_t)pof2);
+    if (!L) return -1;
+    for (int j = 0; j < rem; j++) {
+      pairs[2 * np] = 2 * j; pairs[2 * np + 1] = 2 * j + 1; np++;
+      L[j] = 2 * j;
+    }
+    for (int j = rem; j < pof2; j++) L[j] = j + rem;
+    for (int d = 1; d < pof2; d *= 2)
+      for (int i = 0; i < pof2; i++) {
+        if ((i & d) || ((i ^ start) & (d - 1))) continue; /* i: lower of a pair of holders */
+        int keep = (start & d) ? (i | d) : i, other = (start & d) ? i : (i | d);
+        pairs[2 * np] = L[keep]; pairs[2 * np + 1] = L[other]; np++;
+      }
+    *result = L[start];
+    free(L);
+    return np;
+  }
   case ALO_ORDER_TREE_DBL:
   case ALO_ORDER_TREE_HALV: {
     /* Non-power-of-two P: the first 2*rem ranks fold pairwise (even rank
@@ -447,19 +476,40 @@ int alo_schedule(int P, int order, int start, int *pairs, int *result) {
         for (int i = 0; i + d < pof2; i += 2 * d) {
           pairs[2 * np] = L[i]; pairs[2 * np + 1] = L[i + d]; np++;
         }
+      *result = L[0];
     } else {
+      /* the result is for rank `start`: survivor o holds it in the end, and at
+       * every distance the half that o lies in keeps its own data (inoutvec)
+       * and folds in what the other half sends */
+      int o = start < 2 * rem ? start / 2 : start - rem;
       for (int d = pof2 / 2; d >= 1; d /= 2)
-        for (int i = 0; i < d; i++) {
-          pairs[2 * np] = L[i]; pairs[2 * np + 1] = L[i + d]; np++;
+        for (int i = 0; i < pof2; i++) {
+          if ((i & d) != (o & d) || ((i ^ o) & ~(2 * d - 1))) continue; /* i: a holder on o's side */
+          pairs[2 * np] = L[i]; pairs[2 * np + 1] = L[i ^ d]; np++;
         }
+      *result = L[o];
     }
-    *result = L[0];
     free(L);
     return np;
   }
   default:
     return -1;
   }
+}
+
+/* TREE_RSG: the n elements are cut into pof2 blocks of n / pof2 (the last one
+ * takes the remainder); block k ends up on survivor bit_reverse(k): the first
+ * exchange, at distance 1, already halves the data, the lower half staying with
+ * the survivors whose lowest bit is clear. */
+int alo_rsg_blocks(int P) { return floor_pow2(P); }
+void alo_rsg_block(int P, size_t n, int k, size_t *lo, size_t *hi, int *owner) {
+  int pof2 = floor_pow2(P), bits = 0, o = 0;
+  size_t b = n / (size_t)pof2;
+  while ((1 << bits) < pof2) bits++;
+  for (int j = 0; j < bits; j++) if (k & (1 << j)) o |= 1 << (bits - 1 - j);
+  *lo = (size_t)k * b;
+  *hi = k == pof2 - 1 ? n : (size_t)(k + 1) * b;
+  *owner = o;
 }
 
 /* Run a schedule over P tiles held in `slots` (each `len` elements). */
@@ -476,37 +526,44 @@ static int combine_impl(void *out, const void *const *in, int P, size_t n,
   int rc = alo_check_op(dtype, op);
   if (rc) return rc;
   int *pairs = (int *)malloc(sizeof(int) * 2 * (size_t)(P > 1 ? P : 1));
-  int result = 0;
   if (!pairs) return 3;
-  int np = alo_schedule(P, order, start, pairs, &result);
-  if (np < 0) { free(pairs); return 4; }
-  const size_t ntiles = (n + ALO_TILE - 1) / ALO_TILE;
   int fail = 0;
+  /* one schedule for the whole range, except under TREE_RSG: one per block */
+  const int nblocks = order == ALO_ORDER_TREE_RSG ? alo_rsg_blocks(P) : 1;
+  if (order == ALO_ORDER_TREE_RSG && start != 0) { free(pairs); return 4; }
+  for (int k = 0; k < nblocks && !fail; k++) {
+    size_t b_lo = 0, b_hi = n;
+    int owner = start, result = 0;
+    if (order == ALO_ORDER_TREE_RSG) alo_rsg_block(P, n, k, &b_lo, &b_hi, &owner);
+    int np = alo_schedule(P, order, owner, pairs, &result);
+    if (np < 0) { free(pairs); return 4; }
+    const size_t bn = b_hi - b_lo, ntiles = (bn + ALO_TILE - 1) / ALO_TILE;
 #pragma omp parallel
-  {
-    char *tiles = (char *)malloc((size_t)P * ALO_TILE * es);
-    char **slots = (char **)malloc(sizeof(char *) * (size_t)P);
-    if (!tiles || !slots) {
+    {
+      char *tiles = (char *)malloc((size_t)P * ALO_TILE * es);
+      char **slots = (char **)malloc(sizeof(char *) * (size_t)P);
+      if (!tiles || !slots) {
 #pragma omp atomic write
-      fail = 1;
-    } else {
-      for (int r = 0; r < P; r++) slots[r] = tiles + (size_t)r * ALO_TILE * es;
+        fail = 1;
+      } else {
+        for (int r = 0; r < P; r++) slots[r] = tiles + (size_t)r * ALO_TILE * es;
 #pragma omp for schedule(static)
-      for (size_t t = 0; t < ntiles; t++) {
-        size_t lo = t * ALO_TILE, len = n - lo < ALO_TILE ? n - lo : ALO_TILE;
-        for (int r = 0; r < P; r++) {
-          if (generated)
-            fill_range(slots[r], len, dtype, dist, seed_base + (uint64_t)r, idx0 + lo);
-          else
-            memcpy(slots[r], (const char *)in[r] + lo * es, len * es);
+        for (size_t t = 0; t < ntiles; t++) {
+          size_t lo = b_lo + t * ALO_TILE, len = b_hi - lo < ALO_TILE ? b_hi - lo : ALO_TILE;
+          for (int r = 0; r < P; r++) {
+            if (generated)
+              fill_range(slots[r], len, dtype, dist, seed_base + (uint64_t)r, idx0 + lo);
+            else
+              memcpy(slots[r], (const char *)in[r] + lo * es, len * es);
+          }
+          run_schedule(slots, pairs, np, len, dtype, op);
+          if (op == ALO_AVG) divide_serial(slots[result], len, dtype, P);
+          memcpy((char *)out + lo * es, slots[result], len * es);
         }
-        run_schedule(slots, pairs, np, len, dtype, op);
-        if (op == ALO_AVG) divide_serial(slots[result], len, dtype, P);
-        memcpy((char *)out + lo * es, slots[result], len * es);
       }
+      free(tiles);
+      free(slots);
     }
-    free(tiles);
-    free(slots);
   }
   free(pairs);
   return fail ? 3 : 0;
@@ -524,6 +581,12 @@ int alo_combine_generated(void *out, int P, size_t n, int dtype, int op,
                       seed_base, idx0);
 }
 
+/* The `start` a Reduce_scatter passes for the block that rank b receives: the
+ * orders whose result is "for" a rank take b, the others have no such notion. */
+int alo_order_start(int order, int b) {
+  return order == ALO_ORDER_PAIRWISE_DESC || order == ALO_ORDER_RING || order == ALO_ORDER_TREE_HALV ? b : 0;
+}
+
 int alo_reduce_scatter(void *const *recv, const void *const *send, int P,
                        size_t count, int dtype, int op, int order) {
   const size_t es = alo_dtype_size(dtype);
@@ -533,7 +596,7 @@ int alo_reduce_scatter(void *const *recv, const void *const *send, int P,
   if (!blk) return 3;
   for (int b = 0; b < P && rc == 0; b++) {
     for (int r = 0; r < P; r++) blk[r] = (const char *)send[r] + (size_t)b * count * es;
-    rc = alo_combine(recv[b], blk, P, count, dtype, op, order, b);
+    rc = alo_combine(recv[b], blk, P, count, dtype, op, order, alo_order_start(order, b));
   }
   free(blk);
   return rc;
@@ -561,7 +624,7 @@ int alo_reduce_scatterv(void *const *recv, const void *const *send, int P,
   size_t displ = 0;
   for (int b = 0; b < P && rc == 0; b++) {
     for (int r = 0; r < P; r++) blk[r] = (const char *)send[r] + displ * es;
-    if (counts[b]) rc = alo_combine(recv[b], blk, P, counts[b], dtype, op, order, b);
+    if (counts[b]) rc = alo_combine(recv[b], blk, P, counts[b], dtype, op, order, alo_order_start(order, b));
     displ += counts[b];
   }
   free(blk);

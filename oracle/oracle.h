@@ -25,10 +25,16 @@
  *     with (invec, inoutvec) argument order.
  *
  * Pin status (what checks each function against something other than itself):
- *   alo_step (int / f32 / f64), the TREE_DBL / TREE_HALV / PAIRWISE_DESC
- *     schedules: MPICH 3.3.2 golden vectors in tests/golden (MPI_Allreduce,
- *     MPI_Reduce_scatter_block; the exact calls the reference makes), numpy
- *     closed forms for the order-free integer ops.
+ *   alo_step (int / f32 / f64), the TREE_BINOMIAL / TREE_RSG / TREE_DBL /
+ *     TREE_HALV / PAIRWISE_DESC schedules: MPICH 3.3.2 golden vectors in
+ *     tests/golden (MPI_Allreduce, MPI_Reduce to the first, second and last
+ *     rank, MPI_Reduce_scatter_block, MPI_Reduce_scatter with uneven counts;
+ *     the exact calls the reference makes; 2 to 16 ranks; fp32 / fp64 and, as
+ *     user-defined operations on MPI_SHORT the way the reference registers
+ *     them, fp16 / bf16), numpy closed forms for the order-free integer ops.
+ *     The vectors with NaN, signed zeros and infinities planted in every
+ *     operand position (3, 4 and 8 ranks) pin which operand of every pair is
+ *     the inoutvec, i.e. which one a tie or a NaN lets through.
  *   alo_step (f16 / bf16): numpy float16 and torch bfloat16 arithmetic
  *     (library round-to-nearest-even narrowing), exhaustive over all 2^16
  *     values for widening, sampled + edge cases for narrowing.
@@ -45,10 +51,6 @@
  *     unpinned".
  *   Halo pack/unpack: numpy slicing of the same grid.
  *   NaN payload bits are outside every parity claim (tests compare NaN-ness).
- *   Float min/max with NaN or +-0 operands under an order with more than two
- *   operands: "parity unpinned" - the reference's own result there depends on
- *   the calling rank, so no single reference value exists; the two-operand
- *   step itself is pinned by the golden vectors.
  */
 #ifndef ALO_ORACLE_H
 #define ALO_ORACLE_H
@@ -72,16 +74,26 @@ enum {
   ALO_BOR, ALO_BAND, ALO_BXOR, ALO_AVG
 };
 
-/* Named combine orders. */
+/* Named combine orders.  `s` is the `start` argument of the calls below. */
 enum {
   ALO_ORDER_RANK_ASC = 0,      /* ((x0 . x1) . x2) ...                        */
-  ALO_ORDER_TREE_DBL = 1,      /* pairwise tree, distance 1,2,4,...           */
-  ALO_ORDER_TREE_HALV = 2,     /* pairwise tree, distance P/2,...,1           */
+  ALO_ORDER_TREE_DBL = 1,      /* pairwise tree, distance 1,2,4,...; the lower
+                                  rank of a pair keeps the result            */
+  ALO_ORDER_TREE_HALV = 2,     /* pairwise tree, distance P/2,...,1, for rank
+                                  s: of a pair, the rank on s's side keeps
+                                  the result (recursive-halving
+                                  reduce-scatter, block of rank s)           */
   ALO_ORDER_PAIRWISE_DESC = 3, /* ((x_s . x_{s-1}) . x_{s-2}) ... with wrap   */
   ALO_ORDER_RING = 4,          /* ((x_s . x_{s+1}) . x_{s+2}) ... with wrap,
                                   the running partial is the `in` operand    */
-  ALO_ORDER_TREE_BINOMIAL = 5  /* binomial tree to rank 0; equals TREE_DBL
-                                  when P is a power of two                   */
+  ALO_ORDER_TREE_BINOMIAL = 5, /* binomial tree to rank s over the ranks
+                                  counted from s with wrap (rooted reduce)   */
+  ALO_ORDER_TREE_RSG = 6       /* reduce-scatter + gather (MPI_Reduce and
+                                  MPI_Allreduce of long messages): the tree
+                                  of TREE_DBL, but which rank of a pair keeps
+                                  the result depends on the element's block;
+                                  s must be 0 (in alo_schedule: the block's
+                                  owner among the survivors)                 */
 };
 
 /* Input distributions of the counter-based generator. */
@@ -133,6 +145,13 @@ int alo_divide(void *x, size_t n, int dtype, int ranks);
  * (inout_slot, in_slot) pairs, executed in sequence; the result ends in
  * slot *result.  Returns the number of pairs, or -1 on bad arguments. */
 int alo_schedule(int P, int order, int start, int *pairs, int *result);
+
+/* TREE_RSG: the blocks the n elements are cut into, and the survivor that
+ * ends up owning block k (what alo_schedule takes as `start`). */
+int alo_rsg_blocks(int P);
+void alo_rsg_block(int P, size_t n, int k, size_t *lo, size_t *hi, int *owner);
+/* The `start` a Reduce_scatter passes for the block that rank b receives. */
+int alo_order_start(int order, int b);
 
 /* out[i] = fold of in[0..P-1][i] in the named order.  `out` must not alias
  * an input. */

@@ -5,7 +5,9 @@
  * straight to the MPI library (include/aluminum/mpi/allreduce.hpp:38-44,
  * include/aluminum/mpi/reduce_scatter.hpp:40-46), so the values it produces
  * are those of MPI_Allreduce / MPI_Reduce_scatter_block in the MPI it was
- * built with.  This program makes exactly those calls against the image's
+ * built with; Al::Reduce and Al::Reduce_scatterv likewise end in MPI_Reduce and
+ * MPI_Reduce_scatter (include/aluminum/mpi/reduce.hpp:41-49,
+ * include/aluminum/ht/reduce.hpp:72-82, ht/reduce_scatterv.hpp:75-79).  This program makes exactly those calls against the image's
  * MPICH and prints one JSON document (inputs and outputs as hex strings) that
  * is committed next to it as a fixture.  It runs nothing from the reference.
  *
@@ -36,6 +38,7 @@ static MPI_Datatype mpi_type(int dt) {
   case ALO_U32: return MPI_UNSIGNED;
   case ALO_I64: return MPI_LONG;
   case ALO_U64: return MPI_UNSIGNED_LONG;
+  case ALO_F16: case ALO_BF16: return MPI_SHORT;
   case ALO_F32: return MPI_FLOAT;
   case ALO_F64: return MPI_DOUBLE;
   default: return MPI_DATATYPE_NULL;
@@ -47,6 +50,42 @@ static MPI_Op mpi_op(int op) {
   t[0] = MPI_SUM; t[1] = MPI_PROD; t[2] = MPI_MIN; t[3] = MPI_MAX; t[4] = MPI_LOR;
   t[5] = MPI_LAND; t[6] = MPI_LXOR; t[7] = MPI_BOR; t[8] = MPI_BAND; t[9] = MPI_BXOR;
   return t[op];
+}
+
+/* The reference's own reduction functions for fp16 / bf16 (src/mpi_impl.cpp:61-145) are registered
+ * as commutative user-defined operations on MPI_SHORT (src/mpi_impl.cpp:190-204,
+ * include/aluminum/mpi/utils.hpp:59-67).  The same is done here with the oracle's step as the
+ * function body: these cases pin the ORDER in which the MPI library applies a user-defined
+ * commutative operation, not the step's arithmetic (which other tests pin). */
+static int user_dt, user_op;
+static void user_fn(void *in, void *inout, int *len, MPI_Datatype *type) {
+  (void)type;
+  alo_step(inout, in, (size_t)*len, user_dt, user_op);
+}
+static MPI_Op user_mpi_op = MPI_OP_NULL;
+static int is_half(int dt) { return dt == ALO_F16 || dt == ALO_BF16; }
+
+/* The operation to pass to MPI for (dt, op). */
+static MPI_Op op_for(int dt, int op) {
+  if (!is_half(dt)) return mpi_op(op);
+  user_dt = dt;
+  user_op = op;
+  if (user_mpi_op == MPI_OP_NULL) MPI_Op_create(&user_fn, 1, &user_mpi_op);
+  return user_mpi_op;
+}
+
+/* 1 if `mine` is nonzero on every rank. */
+static int on_all(int mine) {
+  int all = 0;
+  MPI_Allreduce(&mine, &all, 1, MPI_INT, MPI_LAND, MPI_COMM_WORLD);
+  return all;
+}
+
+/* The host-transfer backend makes the non-blocking, in-place form of every call
+ * (include/aluminum/ht/allreduce.hpp:76-79, ht/reduce.hpp:72-82, ht/reduce_scatter.hpp:71-74,
+ * ht/reduce_scatterv.hpp:76-79); every case records whether that form returned the same bytes. */
+static void emit_nb(int same) {
+  if (rank_ == 0) printf(", \"nonblocking_in_place_same\": %s", same ? "true" : "false");
 }
 
 static void print_hex(const unsigned char *p, size_t nbytes) {
@@ -101,7 +140,10 @@ static void tail(void) {
 /* Special values planted over the start of a float buffer (P = 2 only):
  * element i of rank 0 meets element i of rank 1.  NaN against numbers on
  * either side, signed-zero ties both ways, infinities, denormals. */
+static void plant_specials_many(void *buf, size_t n, int dt);
+
 static void plant_specials(void *buf, size_t n, int dt) {
+  if (P_ != 2) { plant_specials_many(buf, n, dt); return; }
   static const unsigned r0[] = {0x7fc00000u, 0xbf800000u, 0x7fc00000u, 0x00000000u, 0x80000000u,
                                 0x7f800000u, 0xff800000u, 0x00000001u, 0x80000001u, 0x3f800000u,
                                 0x7f7fffffu, 0x00800000u, 0x00000000u, 0x80000000u, 0x7f800000u,
@@ -120,6 +162,26 @@ static void plant_specials(void *buf, size_t n, int dt) {
   }
 }
 
+/* More than two ranks: every element of every rank is drawn from a pool of
+ * special values (and two ordinary ones) by a fixed rule, so that NaNs, zeros
+ * of both signs and infinities meet in every position of the combine order. */
+static void plant_specials_many(void *buf, size_t n, int dt) {
+  static const unsigned pool[] = {0x7fc00000u, 0xbf800000u, 0x00000000u, 0x80000000u, 0x7f800000u,
+                                  0xff800000u, 0x00000001u, 0x80000001u, 0x3f800000u, 0x7f7fffffu,
+                                  0x00800000u, 0x00400000u, 0x3e99999au};
+  const size_t cnt = sizeof(pool) / sizeof(pool[0]);
+  for (size_t i = 0; i < n; i++) {
+    unsigned long long h = alo_mix64(77, (unsigned long long)i * 64u + (unsigned long long)rank_);
+    unsigned u = pool[(size_t)(h % cnt)];
+    if (i % 4 == 0 && (h >> 32) % 3 == 0) u = 0x80000000u;      /* plenty of zero ties */
+    else if (i % 4 == 0) u = 0x00000000u;
+    float f;
+    memcpy(&f, &u, 4);
+    if (dt == ALO_F32) ((float *)buf)[i] = f;
+    else ((double *)buf)[i] = (double)f;
+  }
+}
+
 static void case_allreduce(int dt, int op, size_t n, int dist, int specials,
                            const char *note) {
   const unsigned long long seed = 1000;
@@ -127,12 +189,20 @@ static void case_allreduce(int dt, int op, size_t n, int dist, int specials,
   void *in = malloc(n * es), *out = malloc(n * es);
   alo_fill(in, n, dt, dist, seed + (unsigned long long)rank_, 0);
   if (specials) plant_specials(in, n, dt);
-  MPI_Allreduce(in, out, (int)n, mpi_type(dt), mpi_op(op), MPI_COMM_WORLD);
+  MPI_Allreduce(in, out, (int)n, mpi_type(dt), op_for(dt, op), MPI_COMM_WORLD);
+  void *nb = malloc(n * es);
+  MPI_Request req;
+  memcpy(nb, in, n * es);
+  MPI_Iallreduce(MPI_IN_PLACE, nb, (int)n, mpi_type(dt), op_for(dt, op), MPI_COMM_WORLD, &req);
+  MPI_Wait(&req, MPI_STATUS_IGNORE);
+  int same = on_all(memcmp(nb, out, n * es) == 0);
   head("allreduce", dt, op, n, dist, seed, note);
-  emit_list("in", in, n * es);
+  emit_nb(same);
+  /* inputs are repeated for short messages and planted values; the others are the generator's */
+  if (!is_half(dt) && (specials || n * es <= 2048)) emit_list("in", in, n * es);
   emit_list("out", out, n * es);
   tail();
-  free(in); free(out);
+  free(in); free(out); free(nb);
 }
 
 /* count = elements per rank; send buffer holds P*count. */
@@ -142,10 +212,18 @@ static void case_reduce_scatter(int dt, int op, size_t count, int dist, int full
   size_t es = alo_dtype_size(dt), n = count * (size_t)P_;
   void *in = malloc(n * es), *out = malloc(count * es);
   alo_fill(in, n, dt, dist, seed + (unsigned long long)rank_, 0);
-  MPI_Reduce_scatter_block(in, out, (int)count, mpi_type(dt), mpi_op(op), MPI_COMM_WORLD);
+  MPI_Reduce_scatter_block(in, out, (int)count, mpi_type(dt), op_for(dt, op), MPI_COMM_WORLD);
+  void *nb = malloc(n * es);
+  MPI_Request req;
+  memcpy(nb, in, n * es);
+  MPI_Ireduce_scatter_block(MPI_IN_PLACE, nb, (int)count, mpi_type(dt), op_for(dt, op), MPI_COMM_WORLD, &req);
+  MPI_Wait(&req, MPI_STATUS_IGNORE);
+  int same = on_all(memcmp(nb, out, count * es) == 0);
+  free(nb);
   head("reduce_scatter", dt, op, count, dist, seed, note);
+  emit_nb(same);
   if (full) {
-    emit_list("in", in, n * es);
+    if (!is_half(dt)) emit_list("in", in, n * es);
     emit_list("out", out, count * es);
   } else {
     emit_sums("out_checksum", out, count * es);
@@ -164,15 +242,92 @@ static void case_reduce_scatterv(int dt, int op, int dist, const char *note) {
   void *in = malloc(n * es), *out = malloc(16 * es);
   memset(out, 0, 16 * es);
   alo_fill(in, n, dt, dist, seed + (unsigned long long)rank_, 0);
-  MPI_Reduce_scatter(in, out, counts, mpi_type(dt), mpi_op(op), MPI_COMM_WORLD);
+  MPI_Reduce_scatter(in, out, counts, mpi_type(dt), op_for(dt, op), MPI_COMM_WORLD);
+  void *nb = malloc((n ? n : 1) * es);
+  MPI_Request req;
+  memcpy(nb, in, n * es);
+  MPI_Ireduce_scatter(MPI_IN_PLACE, nb, counts, mpi_type(dt), op_for(dt, op), MPI_COMM_WORLD, &req);
+  MPI_Wait(&req, MPI_STATUS_IGNORE);
+  int same = on_all(memcmp(nb, out, (size_t)counts[rank_] * es) == 0);
+  free(nb);
   head("reduce_scatterv", dt, op, n, dist, seed, note);
+  emit_nb(same);
   if (rank_ == 0) {
     printf(", \"counts\": [");
     for (int b = 0; b < P_; b++) printf("%s%d", b ? ", " : "", counts[b]);
     printf("]");
   }
-  emit_list("in", in, n * es);
+  if (!is_half(dt)) emit_list("in", in, n * es);
   emit_list("out", out, 16 * es); /* first counts[rank] elements are significant */
+  tail();
+  free(in); free(out); free(counts);
+}
+
+/* MPI_Reduce to `root`; only the root's output is significant. */
+static void case_reduce(int dt, int op, size_t n, int dist, int root, int specials, const char *note) {
+  const unsigned long long seed = 1000;
+  size_t es = alo_dtype_size(dt);
+  void *in = malloc(n * es), *out = malloc(n * es);
+  memset(out, 0, n * es);
+  alo_fill(in, n, dt, dist, seed + (unsigned long long)rank_, 0);
+  if (specials) plant_specials(in, n, dt);
+  MPI_Reduce(in, out, (int)n, mpi_type(dt), op_for(dt, op), root, MPI_COMM_WORLD);
+  void *nb = malloc(n * es);
+  MPI_Request req;
+  memcpy(nb, in, n * es);
+  if (rank_ == root) MPI_Ireduce(MPI_IN_PLACE, nb, (int)n, mpi_type(dt), op_for(dt, op), root, MPI_COMM_WORLD, &req);
+  else MPI_Ireduce(nb, NULL, (int)n, mpi_type(dt), op_for(dt, op), root, MPI_COMM_WORLD, &req);
+  MPI_Wait(&req, MPI_STATUS_IGNORE);
+  int same = on_all(rank_ != root || memcmp(nb, out, n * es) == 0);
+  free(nb);
+  if (root != 0) { /* bring the root's result to rank 0, which prints */
+    if (rank_ == root) MPI_Send(out, (int)(n * es), MPI_BYTE, 0, 7, MPI_COMM_WORLD);
+    if (rank_ == 0) MPI_Recv(out, (int)(n * es), MPI_BYTE, root, 7, MPI_COMM_WORLD, MPI_STATUS_IGNORE);
+  }
+  head("reduce", dt, op, n, dist, seed, note);
+  if (rank_ == 0) printf(", \"root\": %d", root);
+  emit_nb(same);
+  if (n <= 1024) {
+    /* inputs other than the planted ones are the generator's and not repeated here */
+    if (specials) emit_list("in", in, n * es);
+    if (rank_ == 0) { printf(", \"out\": "); print_hex((unsigned char *)out, n * es); }
+  } else if (rank_ == 0) {
+    printf(", \"out_checksum\": \"%016llx\", \"out_head\": ", (unsigned long long)alo_checksum(out, n * es));
+    print_hex((unsigned char *)out, 8 * es);
+  }
+  tail();
+  free(in); free(out);
+}
+
+/* MPI_Reduce_scatter with uneven counts whose total reaches 512 KiB (the size
+ * from which the block variant changes algorithm): rank b receives
+ * base + 1000*((b*5) % 4) + b elements, rank 1 none.  Outputs as checksums. */
+static void case_reduce_scatterv_long(int dt, int op, int dist, const char *note) {
+  const unsigned long long seed = 1000;
+  size_t es = alo_dtype_size(dt), n = 0;
+  int *counts = (int *)malloc(sizeof(int) * (size_t)P_);
+  const int base = (int)((size_t)(1u << 20) / (size_t)P_ / es);
+  for (int b = 0; b < P_; b++) { counts[b] = b == 1 ? 0 : base + 1000 * ((b * 5) % 4) + b; n += (size_t)counts[b]; }
+  void *in = malloc(n * es), *out = malloc(((size_t)base + 4096) * es);
+  memset(out, 0, ((size_t)base + 4096) * es);
+  alo_fill(in, n, dt, dist, seed + (unsigned long long)rank_, 0);
+  MPI_Reduce_scatter(in, out, counts, mpi_type(dt), op_for(dt, op), MPI_COMM_WORLD);
+  void *nb = malloc(n * es);
+  MPI_Request req;
+  memcpy(nb, in, n * es);
+  MPI_Ireduce_scatter(MPI_IN_PLACE, nb, counts, mpi_type(dt), op_for(dt, op), MPI_COMM_WORLD, &req);
+  MPI_Wait(&req, MPI_STATUS_IGNORE);
+  int same = on_all(memcmp(nb, out, (size_t)counts[rank_] * es) == 0);
+  free(nb);
+  head("reduce_scatterv", dt, op, n, dist, seed, note);
+  emit_nb(same);
+  if (rank_ == 0) {
+    printf(", \"counts\": [");
+    for (int b = 0; b < P_; b++) printf("%s%d", b ? ", " : "", counts[b]);
+    printf("]");
+  }
+  emit_sums("out_checksum", out, (size_t)counts[rank_] * es);
+  emit_list("out_head", out, 8 * es);
   tail();
   free(in); free(out); free(counts);
 }
@@ -207,11 +362,59 @@ int main(int argc, char **argv) {
       for (int op = ALO_SUM; op <= ALO_MAX; op++)
         case_allreduce(fdt[d], op, 48, ALO_DIST_UNIFORM_PM1, 1, "specials");
     }
+    if (P_ == 3 || P_ == 4 || P_ == 8) { /* special values under a whole order; every rank's output is kept */
+      for (int op = ALO_SUM; op <= ALO_MAX; op++) {
+        case_allreduce(fdt[d], op, 96, ALO_DIST_UNIFORM_PM1, 1, "specials");
+        case_allreduce(fdt[d], op, nlong, ALO_DIST_UNIFORM_PM1, 1, "specials");
+      }
+    }
+    /* rooted reduce: first, second and last rank as root, below and above 2048 bytes */
+    const int roots[3] = {0, 1, P_ - 1};
+    for (int k = 0; k < 3; k++) {
+      if (k == 2 && roots[k] <= 1) break;
+      case_reduce(fdt[d], ALO_SUM, 16, ALO_DIST_UNIFORM_PM1, roots[k], 0, "short message");
+      case_reduce(fdt[d], ALO_SUM, nlong, ALO_DIST_UNIFORM_PM1, roots[k], 0, "long message");
+      case_reduce(fdt[d], ALO_PROD, 16, ALO_DIST_UNIFORM_09_11, roots[k], 0, "short message");
+      case_reduce(fdt[d], ALO_PROD, nlong, ALO_DIST_UNIFORM_09_11, roots[k], 0, "long message");
+      if (big) case_reduce(fdt[d], ALO_SUM, (size_t)(1u << 18) + 3, ALO_DIST_UNIFORM_PM1, roots[k], 0, "1 MiB and more");
+      if ((P_ == 3 || P_ == 4 || P_ == 8) && (d == 0 || k == 1))
+        for (int op = ALO_MIN; op <= ALO_MAX; op++) {
+          case_reduce(fdt[d], op, 96, ALO_DIST_UNIFORM_PM1, roots[k], 1, "specials");
+          case_reduce(fdt[d], op, nlong, ALO_DIST_UNIFORM_PM1, roots[k], 1, "specials");
+        }
+    }
     case_reduce_scatter(fdt[d], ALO_SUM, 8, ALO_DIST_UNIFORM_PM1, 1, "short message");
     case_reduce_scatterv(fdt[d], ALO_SUM, ALO_DIST_UNIFORM_PM1, "uneven counts");
-    if (big) /* >= 512 KiB in total selects the pairwise exchange */
+    if (big) { /* >= 512 KiB in total selects the pairwise exchange */
       case_reduce_scatter(fdt[d], ALO_SUM, (size_t)(1u << 20) / (size_t)P_ / alo_dtype_size(fdt[d]) + 64,
                           ALO_DIST_UNIFORM_PM1, 0, "long message");
+      case_reduce_scatterv_long(fdt[d], ALO_SUM, ALO_DIST_UNIFORM_PM1, "uneven counts, long message");
+    }
+  }
+
+  /* fp16 / bf16 through user-defined commutative operations on MPI_SHORT, as the reference
+   * registers them: which order does the library apply such an operation in?  Inputs are the
+   * generator's and are not repeated here. */
+  const int hdt[2] = {ALO_F16, ALO_BF16};
+  for (int d = 0; d < 2; d++) {
+    const size_t nlong = 2048 / 2 + 8;
+    case_allreduce(hdt[d], ALO_SUM, 16, ALO_DIST_UNIFORM_PM1, 0, "short message");
+    case_allreduce(hdt[d], ALO_SUM, nlong, ALO_DIST_UNIFORM_PM1, 0, "long message");
+    case_allreduce(hdt[d], ALO_PROD, nlong, ALO_DIST_UNIFORM_09_11, 0, "long message");
+    const int roots[3] = {0, 1, P_ - 1};
+    for (int k = 0; k < 3; k++) {
+      if (k == 2 && roots[k] <= 1) break;
+      case_reduce(hdt[d], ALO_SUM, 16, ALO_DIST_UNIFORM_PM1, roots[k], 0, "short message");
+      case_reduce(hdt[d], ALO_SUM, nlong, ALO_DIST_UNIFORM_PM1, roots[k], 0, "long message");
+      if (big) case_reduce(hdt[d], ALO_SUM, (size_t)(1u << 19) + 3, ALO_DIST_UNIFORM_PM1, roots[k], 0, "1 MiB and more");
+    }
+    case_reduce_scatter(hdt[d], ALO_SUM, 8, ALO_DIST_UNIFORM_PM1, 1, "short message");
+    case_reduce_scatterv(hdt[d], ALO_SUM, ALO_DIST_UNIFORM_PM1, "uneven counts");
+    if (big) {
+      case_reduce_scatter(hdt[d], ALO_SUM, (size_t)(1u << 20) / (size_t)P_ / 2 + 64, ALO_DIST_UNIFORM_PM1, 0,
+                          "long message");
+      case_reduce_scatterv_long(hdt[d], ALO_SUM, ALO_DIST_UNIFORM_PM1, "uneven counts, long message");
+    }
   }
 
   /* integer types: every op, full-range bits (logical ops see arbitrary
@@ -227,6 +430,8 @@ int main(int argc, char **argv) {
       }
     case_reduce_scatter(ALO_I32, ALO_SUM, 8, ALO_DIST_FULLRANGE, 1, "");
     case_reduce_scatter(ALO_U64, ALO_BXOR, 8, ALO_DIST_FULLRANGE, 1, "");
+    case_reduce(ALO_I32, ALO_SUM, 12, ALO_DIST_FULLRANGE, P_ - 1, 0, "");
+    case_reduce(ALO_U8, ALO_LXOR, 12, ALO_DIST_FULLRANGE, 1, 0, "");
   }
 
   if (rank_ == 0) printf("\n]}\n");

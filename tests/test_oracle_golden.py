@@ -1,11 +1,15 @@
 """The CPU oracle against the MPICH golden vectors in tests/golden.
 
-The vectors were produced by MPI_Allreduce / MPI_Reduce_scatter_block of MPICH
-3.3.2, the calls the reference's MPI backend forwards to
-(include/aluminum/mpi/allreduce.hpp:38-44, mpi/reduce_scatter.hpp:40-46).
-They pin the two-operand step of every native type (including NaN, signed
-zeros, infinities and denormals), and which named order the reference's
-result follows for which collective and message size."""
+The vectors were produced by MPI_Allreduce / MPI_Reduce / MPI_Reduce_scatter_block /
+MPI_Reduce_scatter of MPICH 3.3.2, the calls the reference's MPI backend forwards to
+(include/aluminum/mpi/allreduce.hpp:38-44, mpi/reduce.hpp:41-49, mpi/reduce_scatter.hpp:40-46)
+and whose non-blocking in-place forms its host-transfer backend makes
+(include/aluminum/ht/allreduce.hpp:76-79, ht/reduce.hpp:72-82, ht/reduce_scatter.hpp:71-74,
+ht/reduce_scatterv.hpp:76-79).  They pin the two-operand step of every native type (including
+NaN, signed zeros, infinities and denormals), which named order the reference's result follows
+for which collective, root, message size and kind of operation, and - through the cases with
+special values planted in every operand position - which operand of every pair of the order is
+the one a tie or a NaN lets through."""
 import glob
 import gzip
 import json
@@ -15,9 +19,11 @@ import numpy as np
 import pytest
 
 import oracle
-from util import assert_bits_equal
+from util import assert_bits_equal, mpich_order
 
-GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "mpich_P*.json.gz")))
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "mpich_P*.json.gz")),
+                key=lambda p: int(os.path.basename(p)[7:-8]))
+IDS = [os.path.basename(p)[:-8] for p in GOLDEN]
 
 
 def load(path):
@@ -29,41 +35,77 @@ def arr(hexstr, dtype):
     return np.frombuffer(bytes.fromhex(hexstr), dtype=oracle.NP_CARRIER[dtype]).copy()
 
 
+def inputs_of(c, P, n):
+    """The P input buffers of a case: the committed ones, or the generator's where the fixture
+    does not repeat them."""
+    if "in" in c:
+        return [arr(h, c["dtype"]) for h in c["in"]]
+    return [oracle.fill(n, c["dtype"], c["dist"], c["seed_base"] + r) for r in range(P)]
+
+
 def test_fixtures_present():
-    assert len(GOLDEN) == 6
+    assert [load(p)["P"] for p in GOLDEN] == [2, 3, 4, 5, 7, 8, 16]
     for p in GOLDEN:
-        assert "MPICH Version" in load(p)["mpi"]
+        doc = load(p)
+        assert "MPICH Version" in doc["mpi"]
+        # the non-blocking in-place form, which the host-transfer backend calls, returned the
+        # same bytes as the blocking one in every case
+        assert all(c["nonblocking_in_place_same"] for c in doc["cases"])
 
 
-@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-8] for p in GOLDEN])
+@pytest.mark.parametrize("path", GOLDEN, ids=IDS)
 def test_allreduce_vectors(path):
     doc = load(path)
     P = doc["P"]
-    seen = 0
+    seen = halves = 0
     for c in doc["cases"]:
         if c["coll"] != "allreduce":
             continue
         dt, op, n = c["dtype"], c["op"], c["n"]
-        ins = [arr(h, dt) for h in c["in"]]
+        ins = inputs_of(c, P, n)
         outs = [arr(h, dt) for h in c["out"]]
         assert len(ins) == P and ins[0].size == n
-        if c["note"] != "specials":
+        if "in" in c and c["note"] != "specials":
             # the committed inputs are what the generator makes
             for r in range(P):
                 assert oracle.fill(n, dt, c["dist"], c["seed_base"] + r).tobytes() == ins[r].tobytes()
-        # MPICH 3.3.2 on one host: binomial tree up to 2048 bytes, else the
-        # pre-fold + distance-doubling tree
-        order = "tree_binomial" if n * ins[0].itemsize <= 2048 else "tree_dbl"
+        order, start = mpich_order("allreduce", dt, n, P)
         want = outs[0]
-        got = oracle.combine(ins, dt, op, order)
-        assert_bits_equal(got, want, dt, "P=%d %s %s n=%d %s" % (P, dt, op, n, c["note"]))
+        got = oracle.combine(ins, dt, op, order, start)
+        assert_bits_equal(got, want, dt, "P=%d %s %s n=%d %s (%s)" % (P, dt, op, n, c["note"], order))
         for r in range(1, P):  # every rank received the same bits
-            assert_bits_equal(outs[r], want, dt, "rank %d" % r)
+            assert outs[r].tobytes() == want.tobytes(), "rank %d" % r
         seen += 1
-    assert seen >= 12
+        halves += dt in ("f16", "bf16")
+    assert seen >= 12 and halves >= 6
 
 
-@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-8] for p in GOLDEN])
+@pytest.mark.parametrize("path", GOLDEN, ids=IDS)
+def test_reduce_vectors(path):
+    """MPI_Reduce to the first, second and last rank, below and above 2048 bytes, and at 1 MiB."""
+    doc = load(path)
+    P = doc["P"]
+    seen, roots, orders = 0, set(), set()
+    for c in doc["cases"]:
+        if c["coll"] != "reduce":
+            continue
+        dt, op, n, root = c["dtype"], c["op"], c["n"], c["root"]
+        order, start = mpich_order("reduce", dt, n, P, root)
+        what = "P=%d %s %s n=%d root %d %s (%s)" % (P, dt, op, n, root, c["note"], order)
+        if "out" in c:
+            got = oracle.combine(inputs_of(c, P, n), dt, op, order, start)
+            assert_bits_equal(got, arr(c["out"], dt), dt, what)
+        else:
+            got = oracle.combine_generated(P, n, dt, op, order, start, c["dist"], c["seed_base"])
+            assert "%016x" % oracle.checksum(got) == c["out_checksum"], what
+            assert_bits_equal(got[:8], arr(c["out_head"], dt), dt, what)
+        seen += 1
+        roots.add(root)
+        orders.add(order)
+    assert seen >= 30 and roots == {0, 1, P - 1} and orders == {"tree_binomial", "tree_rsg"}
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=IDS)
 def test_reduce_scatter_vectors(path):
     doc = load(path)
     P = doc["P"]
@@ -72,51 +114,88 @@ def test_reduce_scatter_vectors(path):
         if c["coll"] != "reduce_scatter":
             continue
         dt, op, count = c["dtype"], c["op"], c["n"]
-        if "in" in c:
-            ins = [arr(h, dt) for h in c["in"]]
+        order, _ = mpich_order("reduce_scatter", dt, count, P)
+        if "out" in c:
+            assert order == "tree_halv"  # short: recursive halving
+            ins = inputs_of(c, P, P * count)
             outs = [arr(h, dt) for h in c["out"]]
-            got = oracle.reduce_scatter(ins, dt, op, "tree_halv")  # short: recursive halving
+            got = oracle.reduce_scatter(ins, dt, op, order)
             for r in range(P):
-                assert_bits_equal(got[r], outs[r], dt, "reduce_scatter short P=%d rank %d" % (P, r))
+                assert_bits_equal(got[r], outs[r], dt, "reduce_scatter short P=%d %s rank %d" % (P, dt, r))
         else:
             # long: pairwise exchange, rank r folds x_r, x_{r-1}, ... ; outputs kept as checksums
+            assert order == "pairwise_desc"
             for r in range(P):
-                got = oracle.combine_generated(P, count, dt, op, "pairwise_desc", r, c["dist"],
+                got = oracle.combine_generated(P, count, dt, op, order, r, c["dist"],
                                                c["seed_base"], r * count)
-                assert "%016x" % oracle.checksum(got) == c["out_checksum"][r], (P, r)
+                assert "%016x" % oracle.checksum(got) == c["out_checksum"][r], (P, dt, r)
                 assert_bits_equal(got[:8], arr(c["out_head"][r], dt), dt, "head")
         seen += 1
-    assert seen >= 4
+    assert seen >= 8
 
 
-@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-8] for p in GOLDEN])
+@pytest.mark.parametrize("path", GOLDEN, ids=IDS)
 def test_reduce_scatterv_vectors(path):
-    """MPI_Reduce_scatter with uneven counts (one of them zero): distance-halving tree."""
+    """MPI_Reduce_scatter with uneven counts (one of them zero), below and above 512 KiB in all."""
     doc = load(path)
     P = doc["P"]
     cases = [c for c in doc["cases"] if c["coll"] == "reduce_scatterv"]
-    assert len(cases) == 2
+    assert len(cases) == 8
     for c in cases:
-        dt, counts = c["dtype"], c["counts"]
-        ins = [arr(h, dt) for h in c["in"]]
-        outs = [arr(h, dt) for h in c["out"]]
-        assert ins[0].size == sum(counts)
-        got = oracle.reduce_scatterv(ins, counts, dt, c["op"], "tree_halv")
-        for b in range(P):
-            assert_bits_equal(got[b], outs[b][:counts[b]], dt, "reduce_scatterv P=%d rank %d" % (P, b))
+        dt, counts, total = c["dtype"], c["counts"], c["n"]
+        assert total == sum(counts)
+        order, _ = mpich_order("reduce_scatterv", dt, 0, P, total=total)
+        if "out" in c:
+            assert order == "tree_halv"
+            ins = inputs_of(c, P, total)
+            outs = [arr(h, dt) for h in c["out"]]
+            got = oracle.reduce_scatterv(ins, counts, dt, c["op"], order)
+            for b in range(P):
+                assert_bits_equal(got[b], outs[b][:counts[b]], dt, "reduce_scatterv P=%d rank %d" % (P, b))
+        else:
+            assert order == "pairwise_desc"
+            displ = 0
+            for b in range(P):
+                got = oracle.combine_generated(P, counts[b], dt, c["op"], order, b, c["dist"], c["seed_base"], displ)
+                assert "%016x" % oracle.checksum(got) == c["out_checksum"][b], (P, dt, b)
+                if counts[b]:
+                    assert_bits_equal(got[:8], arr(c["out_head"][b], dt), dt, "head")
+                displ += counts[b]
 
 
 def test_orders_are_distinguishable():
-    """The vectors really separate the orders: a wrong order fails them."""
-    doc = load([p for p in GOLDEN if p.endswith("P8.json.gz")][0])
+    """The vectors really separate the orders: a wrong order, or a wrong root, fails them."""
+    doc = load([p for p in GOLDEN if p.endswith("P5.json.gz")][0])
     c = [c for c in doc["cases"] if c["coll"] == "allreduce" and c["dtype"] == "f32" and c["op"] == "sum"
          and c["note"] == "long message"][0]
-    ins = [arr(h, "f32") for h in c["in"]]
+    ins = inputs_of(c, 5, c["n"])
     want = arr(c["out"][0], "f32")
     match = {o: int((oracle.combine(ins, "f32", "sum", o).view(np.uint32) == want.view(np.uint32)).sum())
-             for o in ("rank_asc", "tree_dbl", "tree_halv", "ring")}
-    assert match["tree_dbl"] == want.size
-    assert match["rank_asc"] < 0.8 * want.size and match["tree_halv"] < 0.8 * want.size
+             for o in ("rank_asc", "tree_dbl", "tree_rsg", "tree_halv", "ring", "tree_binomial")}
+    assert match["tree_rsg"] == want.size == match["tree_dbl"]  # the same tree; operand roles differ
+    assert all(match[o] < 0.8 * want.size for o in ("rank_asc", "tree_halv", "ring", "tree_binomial"))
+    c = [c for c in doc["cases"] if c["coll"] == "reduce" and c["dtype"] == "f32" and c["op"] == "sum"
+         and c["note"] == "short message" and c["root"] == 4][0]
+    ins = inputs_of(c, 5, c["n"])
+    want = arr(c["out"], "f32")
+    assert oracle.combine(ins, "f32", "sum", "tree_binomial", 4).tobytes() == want.tobytes()
+    assert oracle.combine(ins, "f32", "sum", "tree_binomial", 0).tobytes() != want.tobytes()
+
+
+def test_specials_separate_the_operand_roles():
+    """With NaNs and zeros of both signs in every position, min / max tell which operand of a pair is
+    the inoutvec: the doubling tree with fixed roles gets the sums right and the minima wrong."""
+    doc = load([p for p in GOLDEN if p.endswith("P8.json.gz")][0])
+    cases = [c for c in doc["cases"] if c["coll"] == "allreduce" and c["note"] == "specials" and c["dtype"] == "f32"
+             and c["n"] > 512]
+    assert {c["op"] for c in cases} == {"sum", "prod", "min", "max"}
+    for c in cases:
+        ins = inputs_of(c, 8, c["n"])
+        want = arr(c["out"][0], "f32")
+        assert_bits_equal(oracle.combine(ins, "f32", c["op"], "tree_rsg"), want, "f32", c["op"])
+        fixed = oracle.combine(ins, "f32", c["op"], "tree_dbl")
+        same = (fixed.view(np.uint32) == want.view(np.uint32)) | (np.isnan(fixed) & np.isnan(want))
+        assert same.all() == (c["op"] in ("sum", "prod")), c["op"]
 
 
 def test_two_operand_step_specials():

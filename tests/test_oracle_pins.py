@@ -214,7 +214,7 @@ def brute(xs, op, order, start):
             acc = st(acc, xs[(start + k) % P])  # the travelling partial is `in`
         return acc
     if order == "tree_binomial":
-        v = list(xs)
+        v = [xs[(j + start) % P] for j in range(P)]  # ranks counted from the root, with wrap
         d = 1
         while d < P:
             for i in range(0, P - d, 2 * d):
@@ -229,26 +229,140 @@ def brute(xs, op, order, start):
     def dbl(v):
         return v[0] if len(v) == 1 else st(dbl(v[len(v) // 2:]), dbl(v[:len(v) // 2]))
 
-    def halv(v):
+    def halv(v, o):
+        # the half that holds survivor o keeps its own values and folds in the other half's
         if len(v) == 1:
             return v[0]
         h = len(v) // 2
-        return halv([st(v[i + h], v[i]) for i in range(h)])
+        if o < h:
+            return halv([st(v[i + h], v[i]) for i in range(h)], o)
+        return halv([st(v[i], v[i + h]) for i in range(h)], o - h)
 
-    return dbl(L) if order == "tree_dbl" else halv(L)
+    return dbl(L) if order == "tree_dbl" else halv(L, start // 2 if start < 2 * rem else start - rem)
 
 
 @pytest.mark.parametrize("P", (1, 2, 3, 4, 5, 6, 7, 8, 11, 16))
 def test_orders_against_brute_force(P):
     n = 40
-    for op, dist in (("sum", "uniform_pm1"), ("prod", "uniform_09_11"), ("max", "uniform_pm1")):
+    for op, dist in (("sum", "uniform_pm1"), ("prod", "uniform_09_11"), ("max", "uniform_pm1"), ("min", "bool01")):
+        # {0, 1} inputs under min: ties everywhere, so the operand roles show
         ins = [oracle.fill(n, "f64", dist, 50 + r) for r in range(P)]
+        if dist == "bool01":
+            ins = [np.where(a == 0, np.where(np.arange(n) % (r + 2) == 0, -0.0, 0.0), a) for r, a in enumerate(ins)]
         for order in oracle.ORDERS:
-            starts = range(P) if order in ("pairwise_desc", "ring") else (0,)
+            if order == "tree_rsg":
+                continue  # depends on the element's position: see the simulation below
+            starts = range(P) if order in ("pairwise_desc", "ring", "tree_binomial", "tree_halv") else (0,)
             for start in starts:
                 got = oracle.combine(ins, "f64", op, order, start)
                 want = np.array([brute([float(a[i]) for a in ins], op, order, start) for i in range(n)])
                 assert got.tobytes() == want.tobytes(), (P, op, order, start)
+
+
+def simulate_reduce_scatter_gather(ins, dtype, op):
+    """P ranks exchanging messages: a reduce-scatter by recursive halving of the data at distance 1, 2,
+    4, ... (odd ranks among the first 2 * rem hand their data to the even rank below them first; what
+    a rank receives is the invec of its step, what it holds the inoutvec), then the blocks gathered from
+    their owners.  The vector that MPI_Reduce and MPI_Allreduce of a long message leave at the root."""
+    P, n = len(ins), ins[0].size
+    pof2 = 1 << (P.bit_length() - 1)
+    rem = P - pof2
+    buf = [a.copy() for a in ins]
+    real = [2 * nr if nr < rem else nr + rem for nr in range(pof2)]
+    for j in range(rem):
+        buf[2 * j] = oracle.step(buf[2 * j], buf[2 * j + 1], dtype, op)
+    cnts = [n // pof2] * pof2
+    cnts[-1] = n - (n // pof2) * (pof2 - 1)
+    disps = [sum(cnts[:k]) for k in range(pof2 + 1)]
+    lo_hi = {nr: (0, pof2) for nr in range(pof2)}  # the blocks a rank still works on
+    mask = 1
+    while mask < pof2:
+        before = [b.copy() for b in buf]
+        for nr in range(pof2):
+            lo, hi = lo_hi[nr]
+            mid = (lo + hi) // 2
+            keep = (lo, mid) if nr < (nr ^ mask) else (mid, hi)
+            a, b = disps[keep[0]], disps[keep[1]]
+            me, other = real[nr], real[nr ^ mask]
+            buf[me][a:b] = oracle.step(before[me][a:b].copy(), before[other][a:b].copy(), dtype, op)
+            lo_hi[nr] = keep
+        mask *= 2
+    out = np.empty_like(ins[0])
+    for nr in range(pof2):
+        k = lo_hi[nr][0]
+        out[disps[k]:disps[k + 1]] = buf[real[nr]][disps[k]:disps[k + 1]]
+    return out
+
+
+def simulate_recursive_halving_reduce_scatter(ins, counts, dtype, op):
+    """P ranks exchanging messages: even ranks among the first 2 * rem hand their data to the odd rank
+    above them; the survivors exchange halves of the blocks they still work on at distance pof2 / 2, ...,
+    1, keeping the half their own blocks lie in (what arrives is the invec); a survivor that stands for
+    two ranks hands the even one its block back.  Returns the block each rank ends with."""
+    P = len(ins)
+    pof2 = 1 << (P.bit_length() - 1)
+    rem = P - pof2
+    disp = [sum(counts[:b]) for b in range(P + 1)]
+    buf = [a.copy() for a in ins]
+    real = [2 * nr + 1 if nr < rem else nr + rem for nr in range(pof2)]
+    for j in range(rem):
+        buf[2 * j + 1] = oracle.step(buf[2 * j + 1], buf[2 * j], dtype, op)
+    # the ranks whose blocks survivor nr is responsible for
+    owned = [[2 * nr, 2 * nr + 1] if nr < rem else [nr + rem] for nr in range(pof2)]
+    lo_hi = {nr: (0, pof2) for nr in range(pof2)}
+    d = pof2 // 2
+    while d >= 1:
+        before = [b.copy() for b in buf]
+        for nr in range(pof2):
+            lo, hi = lo_hi[nr]
+            mid = (lo + hi) // 2
+            keep = (lo, mid) if nr < mid else (mid, hi)
+            first, last = owned[keep[0]][0], owned[keep[1] - 1][-1]
+            a, b = disp[first], disp[last + 1]
+            me, other = real[nr], real[nr ^ d]
+            buf[me][a:b] = oracle.step(before[me][a:b].copy(), before[other][a:b].copy(), dtype, op)
+            lo_hi[nr] = keep
+        d //= 2
+    out = []
+    for b in range(P):
+        nr = b // 2 if b < 2 * rem else b - rem
+        out.append(buf[real[nr]][disp[b]:disp[b + 1]].copy())
+    return out
+
+
+def specials(n, seed):
+    pool = np.array([np.nan, -1.0, 0.0, -0.0, np.inf, -np.inf, 1e-45, 1.0, 3.0e38, 0.3], np.float32)
+    idx = np.array([oracle.mix64(seed, i) % pool.size for i in range(n)])
+    return pool[idx]
+
+
+@pytest.mark.parametrize("P", (2, 3, 4, 5, 6, 7, 8, 12, 16, 33))
+def test_tree_rsg_against_a_message_passing_simulation(P):
+    for n in (P, 64, 67, 300):
+        if n < (1 << (P.bit_length() - 1)):
+            continue
+        for op in ("sum", "min", "max"):
+            ins = [specials(n, 900 + r) if op != "sum" else oracle.fill(n, "f32", "uniform_pm1", 900 + r) for r in range(P)]
+            got = oracle.combine(ins, "f32", op, "tree_rsg")
+            want = simulate_reduce_scatter_gather(ins, "f32", op)
+            assert_same(got, want, (P, n, op))
+
+
+@pytest.mark.parametrize("P", (2, 3, 4, 5, 6, 7, 8, 12, 16))
+def test_tree_halv_against_a_message_passing_simulation(P):
+    counts = [3 + (5 * b) % 4 if b != 1 else 0 for b in range(P)]
+    for op in ("sum", "min", "max"):
+        ins = [specials(sum(counts), 700 + r) if op != "sum" else oracle.fill(sum(counts), "f32", "uniform_pm1", 700 + r)
+               for r in range(P)]
+        got = oracle.reduce_scatterv(ins, counts, "f32", op, "tree_halv")
+        want = simulate_recursive_halving_reduce_scatter(ins, counts, "f32", op)
+        for b in range(P):
+            assert_same(got[b], want[b], (P, op, b))
+
+
+def assert_same(got, want, what):
+    same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+    assert same.all(), (what, np.flatnonzero(~same)[:5])
 
 
 def test_orders_agree_where_arithmetic_is_exact():
