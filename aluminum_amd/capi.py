@@ -14,7 +14,7 @@ _LIB = os.path.join(_HERE, "libaluminum_amd.so")
 DTYPES = ["i8", "u8", "i16", "u16", "i32", "u32", "i64", "u64", "f16", "bf16", "f32", "f64"]
 OPS = ["sum", "prod", "min", "max", "lor", "land", "lxor", "bor", "band", "bxor", "avg"]
 ORDERS = {"rank_asc": 0, "tree_dbl": 1, "tree_halv": 2, "pairwise_desc": 3, "ring": 4,
-          "tree_binomial": 5}
+          "tree_binomial": 5, "tree_rsg": 6}
 DISTS = {"uniform_pm1": 0, "uniform_09_11": 1, "uniform_01": 2, "fullrange": 3, "bool01": 4,
          "normal": 5, "smallint": 6}
 RING_MODES = {"stepwise": 0, "fused": 1}
@@ -58,6 +58,7 @@ def load():
     L.alamd_dtype_size.argtypes = [i]
     L.alamd_check_op.argtypes = [i, i]
     L.alamd_init.argtypes = []
+    L.alamd_reference_order.argtypes = [i, i, sz, i, i, C.POINTER(i), C.POINTER(i)]
     L.alamd_combine.argtypes = [pvp, i, pvp, i, sz, i, i, i, i, vp]
     L.alamd_reduce_scatter.argtypes = [pvp, pvp, i, sz, i, i, i, vp]
     L.alamd_allgather.argtypes = [pvp, pvp, i, sz, i, vp]
@@ -168,6 +169,18 @@ def combine(outs, ins, op, order="rank_asc", start=0, dtype=None, count=None, st
     count = ins[0].numel() if count is None else count
     _check(load().alamd_combine(_table(outs), len(outs), _table(ins), len(ins), count, _dt(dtype),
                                 _op(op), _order(order), start, _stream(stream)))
+
+
+COLLECTIVES = {"allreduce": 0, "reduce": 1, "reduce_scatter": 2}
+_ORDER_NAMES = {v: k for k, v in ORDERS.items()}
+
+
+def reference_order(collective, P, count, dtype, root=0):
+    """(order name, start) the reference's result follows for this collective (alamd_reference_order)."""
+    order, start = C.c_int(0), C.c_int(0)
+    _check(load().alamd_reference_order(COLLECTIVES[collective], P, count, _dt(dtype), root, C.byref(order),
+                                        C.byref(start)))
+    return _ORDER_NAMES[order.value], start.value
 
 
 def reduce_scatter(recvs, sends, op, order="rank_asc", dtype=None, count=None, stream=None):

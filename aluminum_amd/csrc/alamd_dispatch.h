@@ -218,6 +218,16 @@ struct FoldParams {
 // step(in = a[j], inout = b[j]) when b[j] is set (only among the first 32: a
 // pre-fold leaves at most 32 slots); slots >= nvalid are empty.
 // Level d = 1,2,4..: slot i (multiple of 2d) = step(in = slot i+d, inout = slot i).
+//
+// Operand roles (which of the two partial results of a pair is the inoutvec) only show in the bits of
+// a float min / max, where a tie or a NaN lets the invec through.  Two orders let them depend on
+// where the result goes: TREE_HALV (a recursive-halving reduce-scatter: at every level the half that
+// holds the receiving rank keeps its own data) and TREE_RSG (reduce-scatter by recursive halving of
+// the data plus gather: the same, per block of the message).  In both, the side that keeps is the same
+// for every pair of a level, so the tree with fixed roles gives the right bits once slot j reads what
+// slot j ^ w would have read, w being the slot of the survivor the result is for: the min / max
+// kernels apply that mask (role_mode), the others ignore it.
+enum { ROLE_FIXED = 0, ROLE_PER_SEGMENT = 1, ROLE_PER_BLOCK = 2 };
 struct TreeParams {
   const char *a[ALAMD_MAX_RANKS];
   const char *b[ALAMD_MAX_RANKS];
@@ -227,7 +237,33 @@ struct TreeParams {
   int nvalid;   // occupied slots
   Divisor div;  // avg: the number of ranks as a divisor
   ChainParams chain;  // set for a chained launch only
+  int role_mode;                     // ROLE_*
+  int role_rem, role_bits;           // P = 2^role_bits + role_rem
+  int role_start0, role_stride;      // ROLE_PER_SEGMENT: segment s is for rank (role_start0 + s * role_stride) mod P
+  unsigned long long role_base;      // ROLE_PER_BLOCK: element 0 of a segment is element role_base of the message,
+  unsigned long long role_count;     // which has role_count elements (0: the segment is the message)
 };
+
+__host__ __device__ inline unsigned role_bit_reverse(unsigned v, int bits) {
+  unsigned r = 0;
+  for (int b = 0; b < bits; ++b) r |= ((v >> b) & 1u) << (bits - 1 - b);
+  return r;
+}
+// ROLE_PER_SEGMENT: the slot mask of the segment whose result is for `rank` (the halving tree lists the
+// survivors in bit-reversed order).
+__host__ __device__ inline unsigned role_mask_of_rank(const TreeParams &p, int rank) {
+  const int o = rank < 2 * p.role_rem ? rank / 2 : rank - p.role_rem;
+  return role_bit_reverse((unsigned)o, p.role_bits);
+}
+// ROLE_PER_BLOCK: the message is cut into 2^role_bits blocks of count >> role_bits elements (the last
+// one takes the remainder); block k ends up on survivor bit_reverse(k).
+__host__ __device__ inline unsigned role_mask_of_elem(const TreeParams &p, size_t seg_len, size_t e) {
+  const unsigned long long n = p.role_count ? p.role_count : seg_len, blk = n >> p.role_bits;
+  const unsigned long long last = (1ull << p.role_bits) - 1;
+  unsigned long long k = blk ? (p.role_base + e) / blk : last;
+  if (k > last) k = last;
+  return role_bit_reverse((unsigned)k, p.role_bits);
+}
 
 // The launches of a kernel whose grid is (tiles, segments): `launch(tile0, ntiles, seg0, nsegs)` is
 // called for each.  About `per_launch` workgroups per launch (see launch_tiles), whatever the number of

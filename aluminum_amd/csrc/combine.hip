@@ -29,29 +29,50 @@ int bit_reverse(int v, int bits) {
   return r;
 }
 
-bool order_has_start(int order) { return order == ALAMD_ORDER_PAIRWISE_DESC || order == ALAMD_ORDER_RING; }
-bool order_is_tree(int order) {
-  return order == ALAMD_ORDER_TREE_DBL || order == ALAMD_ORDER_TREE_HALV || order == ALAMD_ORDER_TREE_BINOMIAL;
+// Orders whose `start` argument means something: the first rank of a fold, the root of the binomial
+// tree, the rank a halving tree's result is for.
+bool order_has_start(int order) {
+  return order == ALAMD_ORDER_PAIRWISE_DESC || order == ALAMD_ORDER_RING || order == ALAMD_ORDER_TREE_BINOMIAL ||
+         order == ALAMD_ORDER_TREE_HALV;
 }
-bool order_valid(int order) { return order >= ALAMD_ORDER_RANK_ASC && order <= ALAMD_ORDER_TREE_BINOMIAL; }
+// ... and of those, the ones for which a Reduce_scatter passes the receiving rank (the block's index).
+bool order_start_per_block(int order) {
+  return order == ALAMD_ORDER_PAIRWISE_DESC || order == ALAMD_ORDER_RING || order == ALAMD_ORDER_TREE_HALV;
+}
+bool order_is_tree(int order) {
+  return order == ALAMD_ORDER_TREE_DBL || order == ALAMD_ORDER_TREE_HALV || order == ALAMD_ORDER_TREE_BINOMIAL ||
+         order == ALAMD_ORDER_TREE_RSG;
+}
+bool order_valid(int order) { return order >= ALAMD_ORDER_RANK_ASC && order <= ALAMD_ORDER_TREE_RSG; }
 
-// Fills the slot tables of a tree order over the P inputs `ins`.
-int build_tree(TreeParams &tp, const void *const *ins, int P, int order) {
+// Fills the slot tables of a tree order over the P inputs `ins`.  start: the root of the binomial tree.
+int build_tree(TreeParams &tp, const void *const *ins, int P, int order, int start) {
   for (int j = 0; j < ALAMD_MAX_RANKS; ++j) { tp.a[j] = nullptr; tp.b[j] = nullptr; }
   tp.P = P;
+  tp.role_mode = ROLE_FIXED;
+  tp.role_rem = tp.role_bits = tp.role_start0 = tp.role_stride = 0;
+  tp.role_base = tp.role_count = 0;
   if (order == ALAMD_ORDER_TREE_BINOMIAL) {
-    for (int j = 0; j < P; ++j) tp.a[j] = static_cast<const char *>(ins[j]);
+    // the ranks counted from the root, with wrap
+    for (int j = 0; j < P; ++j) tp.a[j] = static_cast<const char *>(ins[(j + start) % P]);
     tp.nvalid = P;
     return ceil_pow2(P);
   }
   const int pof2 = floor_pow2(P), rem = P - pof2;
   const char *la[ALAMD_MAX_RANKS], *lb[ALAMD_MAX_RANKS];
+  // pre-fold of the first 2 * rem ranks: the slot holds step(in = la, inout = lb).  The odd rank
+  // keeps the result, except under TREE_RSG, where the even one does.
+  const int keep = order == ALAMD_ORDER_TREE_RSG ? 0 : 1;
   for (int j = 0; j < pof2; ++j) {
-    if (j < rem) { la[j] = static_cast<const char *>(ins[2 * j]); lb[j] = static_cast<const char *>(ins[2 * j + 1]); }
+    if (j < rem) { la[j] = static_cast<const char *>(ins[2 * j + 1 - keep]); lb[j] = static_cast<const char *>(ins[2 * j + keep]); }
     else { la[j] = static_cast<const char *>(ins[j + rem]); lb[j] = nullptr; }
   }
   int bits = 0;
   while ((1 << bits) < pof2) ++bits;
+  tp.role_rem = rem;
+  tp.role_bits = bits;
+  if (order == ALAMD_ORDER_TREE_HALV) tp.role_mode = ROLE_PER_SEGMENT;
+  if (order == ALAMD_ORDER_TREE_RSG) tp.role_mode = ROLE_PER_BLOCK;
   for (int k = 0; k < pof2; ++k) {
     // pairing at distance pof2/2, ..., 1 is the adjacent-pair tree over the
     // bit-reversed slot order
@@ -67,7 +88,10 @@ struct Layout {
   unsigned nseg;
   SegParams seg;
   size_t max_len;
-  int start0, start_stride;  // fold orders
+  int start0, start_stride;  // segment s is for rank (start0 + s * start_stride) mod P (orders with a start)
+  // TREE_RSG, when the launch covers part of a message only: where element 0 of a segment lies in the
+  // message, and the message's length (0: every segment is a message of its own)
+  size_t msg_base = 0, msg_count = 0;
 };
 
 // Launches the fold or tree kernels for `order` over inputs `ins`.
@@ -79,9 +103,13 @@ int launch_order(void *const *outs, const void *const *ins, int P, const Layout 
   if (P == 1 && order_is_tree(order)) order = ALAMD_ORDER_RANK_ASC;
   if (order_is_tree(order)) {
     TreeParams tp;
-    const int slots = build_tree(tp, ins, P, order);
+    const int slots = build_tree(tp, ins, P, order, order == ALAMD_ORDER_TREE_BINOMIAL ? lay.start0 % P : 0);
     for (int j = 0; j < ALAMD_MAX_RANKS; ++j) tp.out[j] = static_cast<char *>(outs[j]);
     tp.seg = lay.seg;
+    tp.role_start0 = lay.start0;
+    tp.role_stride = lay.start_stride;
+    tp.role_base = lay.msg_base;
+    tp.role_count = lay.msg_count;
     return launch_tree(tp, slots, lay.nseg, lay.max_len, dtype, op, stream, chain, displ_bytes);
   }
   FoldParams fp;
@@ -521,7 +549,7 @@ int reduce_scatterv_in_place(void *const *recvs, const void *const *sends, int P
           if (!out_tab[k]) out_tab[k] = recvs[k] ? recvs[k] : const_cast<void *>(sends[0]);  // never written: length 0
         lay.max_len = longest;
         lay.start0 = 0;
-        lay.start_stride = order_has_start(order) ? 1 : 0;
+        lay.start_stride = order_start_per_block(order) ? 1 : 0;
         const int rc = launch_order(out_tab, sends, P, lay, dtype, op, order, stream);
         if (rc) return rc;
         b = j;
@@ -550,8 +578,10 @@ int reduce_scatterv_in_place(void *const *recvs, const void *const *sends, int P
       lay.nseg = 1;
       lay.seg = make_seg(n, 0, 0, OUT_ALL, 1);
       lay.max_len = n;
-      lay.start0 = order_has_start(order) ? b : 0;
+      lay.start0 = order_start_per_block(order) ? b : 0;
       lay.start_stride = 0;
+      lay.msg_base = done;
+      lay.msg_count = counts[b];
       if (chained) {
         ChainScratch cs;
         const size_t tiles = (n * es + kChainMinTileBytes - 1) / kChainMinTileBytes;
@@ -632,6 +662,8 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P, si
     Layout pl = lay;
     pl.seg = make_seg(n, 0, 0, OUT_ALL, 1);
     pl.max_len = n;
+    pl.msg_base = e0;
+    pl.msg_count = count;
     void *first[ALAMD_MAX_RANKS] = {nullptr};
     first[0] = static_cast<char *>(outs[0]) + e0 * es;
     const void *pin[ALAMD_MAX_RANKS];
@@ -674,7 +706,7 @@ int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, si
   lay.seg = make_seg(count, 0, 1, OUT_SEG, 1);
   lay.max_len = count;
   lay.start0 = 0;
-  lay.start_stride = order_has_start(order) ? 1 : 0;
+  lay.start_stride = order_start_per_block(order) ? 1 : 0;
   if (!inplace || P == 1) {
     lay.nseg = (unsigned)P;
     return launch_order(out_tab, sends, P, lay, dtype, op, order, as_stream(stream));
@@ -691,7 +723,7 @@ int alamd_reduce_scatter(void *const *recvs, const void *const *sends, int P, si
   for (int r = 0; r < P; ++r) in_shift[r] = static_cast<const char *>(sends[r]) + blk;
   for (int b = 1; b < P; ++b) out_shift[b - 1] = recvs[b];
   lay.nseg = (unsigned)(P - 1);
-  lay.start0 = order_has_start(order) ? 1 : 0;
+  lay.start0 = order_start_per_block(order) ? 1 : 0;
   return launch_order(out_shift, in_shift, P, lay, dtype, op, order, as_stream(stream));
 }
 
@@ -776,7 +808,7 @@ static int reduce_scatterv_impl(void *const *recvs, const void *const *sends, in
     }
     lay.max_len = max_count;
     lay.start0 = 0;
-    lay.start_stride = order_has_start(order) ? 1 : 0;
+    lay.start_stride = order_start_per_block(order) ? 1 : 0;
     return launch_order(out_tab, sends, P, lay, dtype, op, order, as_stream(stream));
   }
   return reduce_scatterv_in_place(recvs, sends, P, counts, displ, dtype, op, order, as_stream(stream), fixed);

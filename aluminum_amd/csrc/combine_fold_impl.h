@@ -47,6 +47,15 @@ __device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, siz
 template <typename T, int OP> struct Shape {
   static constexpr int U = 8;
   static constexpr int THREADS = 128;
+  // P = 8 body: streams whose loads are issued before the first use (0: left to the compiler, which
+  // keeps as many in flight as the registers hold).  bf16 spends seven instructions per dword and
+  // step where the other types spend one; with everything requested up front the compiler ends up
+  // with a schedule that asks for 36 vectors, works through 27 of them and only then asks for the
+  // rest.  Two streams up front and one more requested for every one consumed is worth 0.3 to 0.5
+  // points to bf16 (6253 against 6227 GB/s, and 6250 against 6210, on buffers that are not reused)
+  // and nothing to fp32 (6144 / 6122, 6179 / 6173); three to seven streams up front, or more than
+  // two waves per SIMD with two, lose 1 to 5 points for both.
+  static constexpr int FRONT = std::is_same<T, bf16_t>::value ? 2 : 0;
 };
 
 // amdgpu_waves_per_eu(1, 2): the loads in flight are the point of this kernel;
@@ -95,7 +104,46 @@ fold_vec_kernel(const FoldParams p) {
     const size_t rem = vec_bytes - tb;
     const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
     u32x4 acc[U];
-    if constexpr (PT > 0) {
+    if constexpr (PT == 8 && Shape<T, OP>::FRONT >= 2) {
+      // FRONT streams have their loads issued before the first use; every vector consumed then frees
+      // four registers, which the same vector of the next stream not yet requested takes.
+      constexpr int FRONT = Shape<T, OP>::FRONT;
+      u32x4 x[PT][U];
+      __amdgpu_buffer_rsrc_t r[PT];
+      int idx = s;
+#pragma unroll
+      for (int k = 0; k < PT; ++k) {
+        r[k] = TL::rsrc(p.in[idx] + vin + tb, nrec);
+        idx = next_rank(idx, p.dir, PT);
+      }
+#pragma unroll
+      for (int k = 0; k < FRONT; ++k) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) x[k][u] = tl.load(r[k], u);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // a later load takes its offset from an empty asm statement that reads the step's result, so
+      // that it cannot be issued earlier
+      auto load_after = [&](__amdgpu_buffer_rsrc_t rs, int u, const u32x4 &after) {
+        unsigned vo = tl.vo;
+        asm volatile("" : "+v"(vo) : "v"(after));
+        return __builtin_amdgcn_raw_buffer_load_b128(rs, vo + (unsigned)u * 1024u, 0, kAuxLoadStream);
+      };
+#pragma unroll
+      for (int k = 1; k < PT; ++k) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const u32x4 a = k == 1 ? x[0][u] : acc[u];
+          acc[u] = ACC_IS_IN ? step_vec<T, OP>(a, x[k][u]) : step_vec<T, OP>(x[k][u], a);
+          const int nx = FRONT + k - 1;  // the stream requested next
+          if (nx < PT) x[nx < PT ? nx : 0][u] = load_after(r[nx < PT ? nx : 0], u, acc[u]);
+        }
+        // an empty asm statement per accumulator: the steps of stream k can neither sink below it nor
+        // mix with those of stream k + 1
+#pragma unroll
+        for (int u = 0; u < U; ++u) asm volatile("" : "+v"(acc[u]));
+      }
+    } else if constexpr (PT > 0) {
       u32x4 x[PT][U];
       int idx = s;
 #pragma unroll

@@ -13,8 +13,12 @@ namespace {
 
 // The tree over one element position, one element per access.  HALVES = 2: 2 * SLOTS slots, the
 // two halves reduced one after the other and combined by the tree's top level.
+// Float min / max: the kernels that honour TreeParams::role_mode.
+template <int OP> constexpr bool op_has_roles() { return OP == ALAMD_MIN || OP == ALAMD_MAX; }
+
+// w: slot j reads what slot j ^ w holds (see TreeParams).
 template <typename T, int OP, int SLOTS, int HALVES>
-__device__ __forceinline__ T tree_elem_value(const TreeParams &p, size_t in_bytes, size_t e) {
+__device__ __forceinline__ T tree_elem_value(const TreeParams &p, size_t in_bytes, size_t e, unsigned w = 0) {
   T res;
 #pragma unroll
   for (int h = 0; h < HALVES; ++h) {
@@ -24,11 +28,11 @@ __device__ __forceinline__ T tree_elem_value(const TreeParams &p, size_t in_byte
     T v[SLOTS];
 #pragma unroll
     for (int j = 0; j < SLOTS; ++j)
-      if (j < nvalid) v[j] = ld_elem<T>(p.a[base + j] + in_bytes + e * sizeof(T));
+      if (j < nvalid) v[j] = ld_elem<T>(p.a[(base + j) ^ w] + in_bytes + e * sizeof(T));
 #pragma unroll
     for (int j = 0; j < SLOTS; ++j)
-      if (j < nvalid && p.b[base + j] != nullptr)
-        v[j] = Step<T, OP>::apply(v[j], ld_elem<T>(p.b[base + j] + in_bytes + e * sizeof(T)));
+      if (j < nvalid && p.b[(base + j) ^ w] != nullptr)
+        v[j] = Step<T, OP>::apply(v[j], ld_elem<T>(p.b[(base + j) ^ w] + in_bytes + e * sizeof(T)));
 #pragma unroll
     for (int d = 1; d < SLOTS; d *= 2) {
 #pragma unroll
@@ -41,8 +45,8 @@ __device__ __forceinline__ T tree_elem_value(const TreeParams &p, size_t in_byte
 }
 template <typename T, int OP, int SLOTS, int HALVES>
 __device__ __forceinline__ void tree_elem(const TreeParams &p, size_t in_bytes, int j0, int nj,
-                                          size_t out_bytes, size_t e) {
-  const T res = tree_elem_value<T, OP, SLOTS, HALVES>(p, in_bytes, e);
+                                          size_t out_bytes, size_t e, unsigned w = 0) {
+  const T res = tree_elem_value<T, OP, SLOTS, HALVES>(p, in_bytes, e, w);
   for (int j = j0; j < j0 + nj; ++j) st_elem<T>(p.out[j] + out_bytes + e * sizeof(T), res);
 }
 
@@ -102,7 +106,30 @@ tree_vec_kernel(const TreeParams p) {
   unsigned bx = blockIdx.x;
   if constexpr (CHAIN) bx = chain_take_tile(p.chain);
   const size_t tb = ((size_t)p.seg.tile0 + bx) * TL::BYTES;
-  if (tb < vec_bytes) {
+  // float min / max: the slot mask of this tile (uniform), or, where a tile straddles two blocks of a
+  // TREE_RSG message, one mask per element
+  constexpr bool ROLES = op_has_roles<OP>();
+  unsigned w = 0;
+  bool mixed = false;
+  if constexpr (ROLES) {
+    if (p.role_mode == ROLE_PER_SEGMENT) {
+      w = role_mask_of_rank(p, (p.role_start0 + (int)seg * p.role_stride) % p.P);
+    } else if (p.role_mode == ROLE_PER_BLOCK && tb < vec_bytes) {
+      const size_t rem = vec_bytes - tb, nb = rem > TL::BYTES ? TL::BYTES : rem;
+      const size_t e0 = head + tb / sizeof(T);
+      w = role_mask_of_elem(p, len, e0);
+      mixed = role_mask_of_elem(p, len, e0 + nb / sizeof(T) - 1) != w;
+    }
+  }
+  if (ROLES && !CHAIN && mixed) {
+    // one element per access, every element under its own mask (never in a chained launch: the host
+    // refuses that combination)
+    const size_t rem = vec_bytes - tb, nb = rem > TL::BYTES ? TL::BYTES : rem;
+    const size_t e0 = head + tb / sizeof(T), ne = nb / sizeof(T);
+#pragma unroll 1
+    for (size_t k = threadIdx.x; k < ne; k += THREADS)
+      tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e0 + k, role_mask_of_elem(p, len, e0 + k));
+  } else if (tb < vec_bytes) {
     const size_t rem = vec_bytes - tb;
     const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
     u32x4 res[U];
@@ -115,7 +142,7 @@ tree_vec_kernel(const TreeParams p) {
 #pragma unroll
       for (int j = 0; j < SLOTS; ++j) {
         if (j < nvalid) {
-          const auto r = TL::rsrc(p.a[base + j] + vin + tb, nrec);
+          const auto r = TL::rsrc(p.a[ROLES ? (base + j) ^ w : base + j] + vin + tb, nrec);
 #pragma unroll
           for (int u = 0; u < U; ++u) v[j][u] = tl.load(r, u);
         }
@@ -123,20 +150,20 @@ tree_vec_kernel(const TreeParams p) {
       if constexpr (MODE == TREE_PREFOLD) {
         // pre-folded slots: the odd rank keeps step(in = even rank, inout = odd rank); all of
         // their loads are issued before the first use, like the slots' own
-        u32x4 w[SLOTS][U];
+        u32x4 pre[SLOTS][U];
 #pragma unroll
         for (int j = 0; j < SLOTS; ++j) {
-          if (j < nvalid && p.b[j] != nullptr) {
-            const auto r = TL::rsrc(p.b[j] + vin + tb, nrec);
+          if (j < nvalid && p.b[ROLES ? j ^ w : j] != nullptr) {
+            const auto r = TL::rsrc(p.b[ROLES ? j ^ w : j] + vin + tb, nrec);
 #pragma unroll
-            for (int u = 0; u < U; ++u) w[j][u] = tl.load(r, u);
+            for (int u = 0; u < U; ++u) pre[j][u] = tl.load(r, u);
           }
         }
 #pragma unroll
         for (int j = 0; j < SLOTS; ++j) {
-          if (j < nvalid && p.b[j] != nullptr) {
+          if (j < nvalid && p.b[ROLES ? j ^ w : j] != nullptr) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) v[j][u] = step_vec<T, OP>(v[j][u], w[j][u]);
+            for (int u = 0; u < U; ++u) v[j][u] = step_vec<T, OP>(v[j][u], pre[j][u]);
           }
         }
       }
@@ -168,7 +195,7 @@ tree_vec_kernel(const TreeParams p) {
       const bool mine = threadIdx.x < vlen % N;
       const size_t e = (vlen / N) * N + threadIdx.x;
       T val = T();
-      if (mine) val = tree_elem_value<T, OP, SLOTS, HALVES>(p, in_bytes, e);
+      if (mine) val = tree_elem_value<T, OP, SLOTS, HALVES>(p, in_bytes, e, ROLES && p.role_mode == ROLE_PER_BLOCK ? role_mask_of_elem(p, len, e) : w);
       chain_gate(p.chain, bx, vec_bytes, (vlen % N) * sizeof(T), (unsigned)TL::BYTES);
       if (mine) st_elem<T>(p.out[j0] + out_bytes + e * sizeof(T), val);
     }
@@ -176,7 +203,8 @@ tree_vec_kernel(const TreeParams p) {
     // the head elements and the vlen % N elements behind the last whole vector
     if (p.seg.tile0 == 0 && blockIdx.x == 0 && threadIdx.x < head + vlen % N) {
       const size_t e = threadIdx.x < head ? threadIdx.x : (vlen / N) * N + threadIdx.x;
-      tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e);
+      tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e,
+                                      ROLES && p.role_mode == ROLE_PER_BLOCK ? role_mask_of_elem(p, len, e) : w);
     }
   }
 }
@@ -195,6 +223,9 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   q.seg.simple = 0;
   if (chain.scratch) {
     if (nseg != 1) return set_error(ALAMD_ERR_INVALID_ARG, "a chained combine has one segment");
+    if (op_has_roles<OP>() && p.role_mode == ROLE_PER_BLOCK)
+      return set_error(ALAMD_ERR_INVALID_ALGO, "a float min / max under the reduce-scatter + gather order is not available "
+                       "for an in-place block that overlaps its own input");
     constexpr size_t N = 16 / sizeof(T);
     const size_t tile_bytes = Tile<S::U, S::THREADS>::BYTES;
     const size_t nvec = (max_len / N * 16 + tile_bytes - 1) / tile_bytes;

@@ -131,6 +131,43 @@ size_t alamd_tuned(const char *name) {
 
 int alamd_check_op(int dtype, int op) { return alamd::check_type_op(dtype, op); }
 
+int alamd_reference_order(int collective, int P, size_t count, int dtype, int root, int *order, int *start) {
+  if (!order || !start) return alamd::set_error(ALAMD_ERR_INVALID_ARG, "null result pointer");
+  if (P < 1 || P > ALAMD_MAX_RANKS) return alamd::set_error(ALAMD_ERR_INVALID_ARG, "number of ranks %d outside [1, %d]", P, ALAMD_MAX_RANKS);
+  const size_t es = alamd_dtype_size(dtype);
+  if (es == 0) return alamd::set_error(ALAMD_ERR_UNSUPPORTED_TYPE, "unknown dtype %d", dtype);
+  *start = 0;
+  switch (collective) {
+  case ALAMD_COLL_ALLREDUCE:
+  case ALAMD_COLL_REDUCE: {
+    if (collective == ALAMD_COLL_REDUCE && (root < 0 || root >= P))
+      return alamd::set_error(ALAMD_ERR_INVALID_ARG, "root %d outside [0, %d)", root, P);
+    // An allreduce among ranks of one host is a reduce to rank 0 followed by a broadcast.  The reduce
+    // is a binomial tree to the root, over the ranks counted from it, for short messages, for fewer
+    // elements than the largest power of two of ranks and for every operation that is not one of the
+    // library's own (fp16 and bf16 are user-defined operations to it); otherwise a reduce-scatter by
+    // recursive halving followed by a gather, which does not depend on the root.
+    size_t pof2 = 1;
+    while (2 * pof2 <= (size_t)P) pof2 *= 2;
+    const bool user_op = dtype == ALAMD_F16 || dtype == ALAMD_BF16;
+    if (user_op || count * es <= 2048 || count < pof2) {
+      *order = ALAMD_ORDER_TREE_BINOMIAL;
+      *start = collective == ALAMD_COLL_REDUCE ? root : 0;
+    } else {
+      *order = ALAMD_ORDER_TREE_RSG;
+    }
+    return ALAMD_OK;
+  }
+  case ALAMD_COLL_REDUCE_SCATTER:
+    // recursive halving below 512 KiB in all, pairwise exchange from there on (commutative operations,
+    // user-defined ones included)
+    *order = count * es < ((size_t)512 << 10) ? ALAMD_ORDER_TREE_HALV : ALAMD_ORDER_PAIRWISE_DESC;
+    return ALAMD_OK;
+  default:
+    return alamd::set_error(ALAMD_ERR_INVALID_ARG, "unknown collective %d", collective);
+  }
+}
+
 int alamd_init(void) {
   int dev = 0;
   ALAMD_HIP(hipGetDevice(&dev));

@@ -84,23 +84,46 @@ typedef enum {
  *   RANK_ASC       acc = x0; acc = step(in = x_k, inout = acc), k = 1..P-1
  *   PAIRWISE_DESC  acc = x_s; acc = step(in = x_{s-k}, inout = acc)  (wrap)
  *   RING           acc = x_s; acc = step(in = acc, inout = x_{s+k})  (wrap)
- *   TREE_BINOMIAL  distance 1,2,4..: x_i = step(in = x_{i+d}, inout = x_i)
+ *   TREE_BINOMIAL  binomial tree to rank s: with y_i = x_{(s+i) mod P},
+ *                  distance d = 1,2,4..: y_i = step(in = y_{i+d}, inout = y_i)
  *                  for every i that is a multiple of 2d with i+d < P
  *   TREE_DBL       the first 2*(P - 2^k) ranks fold pairwise
  *                  (step(in = x_{2j}, inout = x_{2j+1})), the 2^k survivors
- *                  then pair at distance 1,2,4,...
- *   TREE_HALV      the same pre-fold, survivors pair at distance 2^k/2,...,1
- * With MPICH 3.3.2 on one host the reference's MPI backend produces
- * TREE_BINOMIAL (Allreduce up to 2048 bytes), TREE_DBL (larger Allreduce),
- * TREE_HALV (Reduce_scatter below 512 KiB in total) and PAIRWISE_DESC with
- * s = receiving rank (larger Reduce_scatter). */
+ *                  then pair at distance 1,2,4,..., the lower one keeping the
+ *                  result (the inout operand)
+ *   TREE_HALV      the same pre-fold, survivors pair at distance 2^k/2,...,1;
+ *                  of a pair, the survivor on the side of rank s keeps the
+ *                  result: the order in which a recursive-halving
+ *                  reduce-scatter makes the block that rank s receives
+ *   TREE_RSG       reduce-scatter by recursive halving of the data, then
+ *                  gather: the first 2*(P - 2^k) ranks fold pairwise, the even
+ *                  one keeping the result (step(in = x_{2j+1}, inout = x_{2j}));
+ *                  the survivors pair at distance 1,2,4,... as under TREE_DBL,
+ *                  but which one of a pair keeps the result depends on where
+ *                  the element lies: the count elements are cut into 2^k blocks
+ *                  of count / 2^k (the last one takes the remainder), block b
+ *                  ends up on survivor bit_reverse(b), and at distance d the
+ *                  survivor whose bit d equals that survivor's bit d keeps.
+ *                  For sum and prod this gives the bits of TREE_DBL; it differs
+ *                  where a float min / max meets a tie (+0 / -0) or a NaN.
+ * Which of two operands is the inout one only shows in float min / max (a tie
+ * or a NaN lets the in operand through); every other result depends on the
+ * shape of the tree alone.
+ * With MPICH 3.3.2 on one host the reference's MPI and host-transfer backends
+ * produce: Allreduce and Reduce of native types - TREE_BINOMIAL with s = root
+ * (Allreduce: 0) up to 2048 bytes or when count < 2^k, TREE_RSG above, whatever
+ * the root; of fp16 / bf16, which are user-defined operations to the MPI
+ * library - TREE_BINOMIAL at every size; Reduce_scatter, with equal or unequal
+ * counts - TREE_HALV with s = receiving rank below 512 KiB in total,
+ * PAIRWISE_DESC with s = receiving rank from there on. */
 typedef enum {
   ALAMD_ORDER_RANK_ASC = 0,
   ALAMD_ORDER_TREE_DBL = 1,
   ALAMD_ORDER_TREE_HALV = 2,
   ALAMD_ORDER_PAIRWISE_DESC = 3,
   ALAMD_ORDER_RING = 4,
-  ALAMD_ORDER_TREE_BINOMIAL = 5
+  ALAMD_ORDER_TREE_BINOMIAL = 5,
+  ALAMD_ORDER_TREE_RSG = 6
 } alamd_order;
 
 /* ---- library ---------------------------------------------------------- */
@@ -122,6 +145,23 @@ int alamd_check_op(int dtype, int op);
  * src/cuda/cuda.cpp:52-78.) */
 int alamd_init(void);
 
+/* The order (and its start rank) under which the reference's result comes
+ * about for a collective over P ranks when its MPI library is MPICH 3.3.2 and
+ * all ranks share one host - what an `automatic` algorithm should pick to give
+ * the reference's bits.  The reference hands the call to MPI_(I)allreduce,
+ * MPI_(I)reduce, MPI_(I)reduce_scatter_block and MPI_(I)reduce_scatter
+ * (include/aluminum/mpi/allreduce.hpp:38-44, mpi/reduce.hpp:41-49,
+ * mpi/reduce_scatter.hpp:40-46, include/aluminum/ht/allreduce.hpp:76-79,
+ * ht/reduce.hpp:72-82, ht/reduce_scatter.hpp:71-74, ht/reduce_scatterv.hpp:76-79);
+ * the table was read off that library's results for 2 to 16 ranks.
+ * `count`: elements per rank for ALAMD_COLL_ALLREDUCE and ALAMD_COLL_REDUCE,
+ * elements in a whole send buffer for ALAMD_COLL_REDUCE_SCATTER (with equal or
+ * unequal counts).  `root` is ignored except for ALAMD_COLL_REDUCE.  *start is
+ * what alamd_combine takes; alamd_reduce_scatter(v) add the receiving rank
+ * themselves. */
+typedef enum { ALAMD_COLL_ALLREDUCE = 0, ALAMD_COLL_REDUCE = 1, ALAMD_COLL_REDUCE_SCATTER = 2 } alamd_collective;
+int alamd_reference_order(int collective, int P, size_t count, int dtype, int root, int *order, int *start);
+
 /* ---- combine: the element-wise fold of P rank contributions ----------- */
 
 /* outs[j][i] = fold over r of ins[r][i], i in [0, count), for each of the
@@ -135,17 +175,15 @@ int alamd_init(void);
  * have one and must be 0 otherwise.  Here and in every entry point below a
  * buffer must be aligned to its element type (ALAMD_ERR_INVALID_ARG if not);
  * no wider alignment is needed.
- * Outside every parity claim: which operand a float min / max keeps when NaN
- * or +-0 operands meet under an order with more than two operands (the
- * reference's own result there differs from rank to rank; the two-operand step
- * is the MPI library's and is checked), and the payload bits of a NaN result. */
+ * Outside every parity claim: the payload bits of a NaN result. */
 int alamd_combine(void *const *outs, int nout, const void *const *ins, int P,
                   size_t count, int dtype, int op, int order, int start,
                   void *stream);
 
 /* Reduce_scatter over P logical ranks: sends[r] holds P*count elements;
  * recvs[b] receives count elements, the fold of block b of every sends[r],
- * with start = b for the orders that have one.  In-place form
+ * with start = b under PAIRWISE_DESC, RING and TREE_HALV (TREE_BINOMIAL: 0;
+ * TREE_RSG: every block is a message of its own).  In-place form
  * (recvs[b] == sends[b]) puts the result at the start of the buffer.
  * Replaces MPI_Ireduce_scatter_block on the host copy
  * (include/aluminum/ht/reduce_scatter.hpp:45-74; layout docs/comm.rst:284-285). */
@@ -161,8 +199,8 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P,
 
 /* Reduce_scatterv: sends[r] holds sum(counts) elements; recvs[b] receives
  * counts[b] elements, the fold of elements [displ_b, displ_b + counts[b]) of
- * every sends[r], displ_b = counts[0] + ... + counts[b-1], with start = b for
- * the orders that have one.  In-place form (recvs[b] == sends[b]) puts the
+ * every sends[r], displ_b = counts[0] + ... + counts[b-1], with start = b as
+ * for alamd_reduce_scatter.  In-place form (recvs[b] == sends[b]) puts the
  * result at the start of the buffer; any counts are accepted, as by the
  * reference.  A block that is in place and starts fewer elements into its own
  * buffer than it is long is read and overwritten at a displacement: in two

@@ -40,6 +40,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <atomic>
 #include <cstddef>
 #include <chrono>
 #include <condition_variable>
@@ -57,8 +58,20 @@
 
 #include "aluminum_amd.h"
 
+// Two ways to use this header.  On its own it is a front end of the reference's shape: it defines
+// Al::al_exception, Al::ReductionOperator, Al::AlOperation, the trait templates and the Al::Allreduce /
+// Reduce / Reduce_scatter(v) / Allgather(v) / Test / Wait templates itself.  With AL_AMD_WITH_REFERENCE
+// defined it is one more backend inside the reference: it is included after the reference's own
+// declarations (the way include/Al.hpp:2005-2014 includes the other backends), defines none of those
+// and only adds Al::HipCombineBackend, its traits and its Test / Wait specialisations.
+#ifdef AL_AMD_WITH_REFERENCE
+#include "aluminum/base.hpp"
+#include "aluminum/traits/traits_base.hpp"
+#endif
+
 namespace Al {
 
+#ifndef AL_AMD_WITH_REFERENCE
 /** Same text layout as the reference's exception (include/aluminum/base.hpp:52-70). */
 class al_exception : public std::exception {
  public:
@@ -73,6 +86,7 @@ class al_exception : public std::exception {
   const int line;
   std::string err;
 };
+#endif
 #define AL_AMD_THROW(s) throw ::Al::al_exception((s), __FILE__, __LINE__)
 #define AL_AMD_CHECK(call)                                                   \
   do {                                                                       \
@@ -85,6 +99,7 @@ class al_exception : public std::exception {
       AL_AMD_THROW(std::string("GPU error: ") + hipGetErrorString(al_amd_e_)); \
   } while (0)
 
+#ifndef AL_AMD_WITH_REFERENCE
 /** Predefined reduction operations (include/aluminum/base.hpp:103-105). */
 enum class ReductionOperator { sum, prod, min, max, lor, land, lxor, bor, band, bxor, avg };
 
@@ -104,6 +119,15 @@ inline void Initialize(int & /*argc*/, char **& /*argv*/) {
 }
 inline void Finalize() { amd::initialized_flag() = false; }
 inline bool Initialized() { return amd::initialized_flag(); }
+#endif
+// The C ABI numbers its operators like the reference, so the front end casts.
+static_assert(static_cast<int>(ReductionOperator::sum) == ALAMD_SUM && static_cast<int>(ReductionOperator::prod) == ALAMD_PROD &&
+                  static_cast<int>(ReductionOperator::min) == ALAMD_MIN && static_cast<int>(ReductionOperator::max) == ALAMD_MAX &&
+                  static_cast<int>(ReductionOperator::lor) == ALAMD_LOR && static_cast<int>(ReductionOperator::land) == ALAMD_LAND &&
+                  static_cast<int>(ReductionOperator::lxor) == ALAMD_LXOR && static_cast<int>(ReductionOperator::bor) == ALAMD_BOR &&
+                  static_cast<int>(ReductionOperator::band) == ALAMD_BAND && static_cast<int>(ReductionOperator::bxor) == ALAMD_BXOR &&
+                  static_cast<int>(ReductionOperator::avg) == ALAMD_AVG,
+              "ReductionOperator and alamd_op must agree");
 
 namespace amd {
 
@@ -144,15 +168,17 @@ AL_AMD_TYPEMAP(__hip_bfloat16, ALAMD_BF16);
 
 /** Combine orders and ring modes a caller can ask for by name. */
 enum class CombineAlgorithm {
-  automatic,      /**< what the reference's MPI backend yields with MPICH on one
-                       host: binomial tree up to 2048 bytes, distance-doubling tree
-                       above (Allreduce / Reduce); distance-halving tree below
-                       512 KiB in total, descending pairwise fold above
-                       (Reduce_scatter) */
+  automatic,      /**< what the reference's MPI and host-transfer backends yield with MPICH
+                       3.3.2 on one host (alamd_reference_order): Allreduce and Reduce - binomial
+                       tree to the root up to 2048 bytes and for fp16 / bf16, reduce-scatter +
+                       gather above; Reduce_scatter(v) - distance-halving tree below 512 KiB in
+                       total, descending pairwise fold from there on */
   rank_order,     /**< ((x0 . x1) . x2) ... */
   tree_doubling,
   tree_halving,
-  tree_binomial,
+  tree_binomial,  /**< to the root of a Reduce, to rank 0 otherwise */
+  tree_reduce_scatter_gather,  /**< the doubling tree with the operand roles of a reduce-scatter by
+                                    recursive halving of the data followed by a gather */
   pairwise,       /**< x_r . x_{r-1} . x_{r-2} ... for the block of rank r */
   ring,           /**< ring reduce-scatter + allgather, one launch per ring step */
   ring_fused      /**< the same values with every segment folded in one pass */
@@ -243,9 +269,14 @@ struct OpCompletion {
  *  (internal::ht::HostTransferRequest, include/aluminum/ht_impl.hpp:882-888).
  *  `done` is empty until the last logical rank has made its call. */
 struct Request {
+  enum { not_launched = 0, launched = 1, failed = 2 };
+  // The thread that makes the last call of a collective launches it and publishes the outcome here:
+  // `done` or `error` first, then `state` with release order.  Test and Wait, which any rank's thread
+  // may call meanwhile, read `state` with acquire order and only then the field it names.
+  std::atomic<int> state{not_launched};
   std::shared_ptr<OpCompletion> done;
   hipStream_t orig_stream = nullptr;
-  std::string error;  // set when the launch of the operation failed: Test and Wait rethrow it
+  std::string error;  // the launch of the operation failed: Test and Wait rethrow it
 };
 
 enum class OpKind { allreduce, reduce, reduce_scatter, allgather, reduce_scatterv, allgatherv };
@@ -475,7 +506,10 @@ inline void World::post(Communicator &c, OpKind kind, int dtype, const void *sen
       // when calls wait for the launch, through the exception their own call throws
       done->failure = e.what();
       for (Posting &r : done->ranks)
-        if (r.req) r.req->error = done->failure;
+        if (r.req) {
+          r.req->error = done->failure;
+          r.req->state.store(Request::failed, std::memory_order_release);
+        }
     }
     for (Posting &r : done->ranks)
       if (r.ready) {
@@ -575,7 +609,10 @@ inline void World::release_streams(PendingOp &p, hipStream_t ran_on) {
     done->event = events_->take();
     done->ran_on = ran_on;
     AL_AMD_CHECK_HIP(hipEventRecord(done->event, ran_on));
-    for (auto &r : p.ranks) r.req->done = done;
+    for (auto &r : p.ranks) {
+      r.req->done = done;
+      r.req->state.store(Request::launched, std::memory_order_release);
+    }
     return;
   }
   bool recorded = false;
@@ -615,38 +652,44 @@ inline void World::launch(PendingOp &p) {
   switch (p.kind) {
   case OpKind::allreduce:
   case OpKind::reduce: {
-    int order = ALAMD_ORDER_RANK_ASC;
+    const bool rooted = p.kind == OpKind::reduce;
+    int order = ALAMD_ORDER_RANK_ASC, start = 0;
     bool ring = false;
     switch (p.algo) {
     case CombineAlgorithm::automatic:
-      order = p.count * es <= 2048 ? ALAMD_ORDER_TREE_BINOMIAL : ALAMD_ORDER_TREE_DBL;
+      if (alamd_reference_order(rooted ? ALAMD_COLL_REDUCE : ALAMD_COLL_ALLREDUCE, P, p.count, p.dtype, p.root, &order,
+                                &start) != ALAMD_OK)
+        AL_AMD_THROW(std::string(alamd_last_error()));
       break;
     case CombineAlgorithm::rank_order: order = ALAMD_ORDER_RANK_ASC; break;
     case CombineAlgorithm::tree_doubling: order = ALAMD_ORDER_TREE_DBL; break;
     case CombineAlgorithm::tree_halving: order = ALAMD_ORDER_TREE_HALV; break;
-    case CombineAlgorithm::tree_binomial: order = ALAMD_ORDER_TREE_BINOMIAL; break;
+    case CombineAlgorithm::tree_binomial: order = ALAMD_ORDER_TREE_BINOMIAL; start = rooted ? p.root : 0; break;
+    case CombineAlgorithm::tree_reduce_scatter_gather: order = ALAMD_ORDER_TREE_RSG; break;
     case CombineAlgorithm::ring:
     case CombineAlgorithm::ring_fused: ring = true; break;
     default: AL_AMD_THROW("Invalid algorithm");
     }
-    if (p.kind == OpKind::reduce) {
+    if (rooted) {
       if (ring) AL_AMD_THROW("Invalid algorithm");
       void *out = recvs[static_cast<size_t>(p.root)];
-      rc = alamd_combine(&out, 1, sends.data(), P, p.count, p.dtype, op, order, 0, target);
+      rc = alamd_combine(&out, 1, sends.data(), P, p.count, p.dtype, op, order, start, target);
     } else if (ring) {
       rc = alamd_ring_allreduce_from(recvs.data(), sends.data(), P, p.count, p.dtype, op, ring_chunk_bytes(es),
                                      p.algo == CombineAlgorithm::ring ? ALAMD_RING_STEPWISE : ALAMD_RING_FUSED,
                                      target);
     } else {
-      rc = alamd_combine(recvs.data(), P, sends.data(), P, p.count, p.dtype, op, order, 0, target);
+      rc = alamd_combine(recvs.data(), P, sends.data(), P, p.count, p.dtype, op, order, start, target);
     }
     break;
   }
   case OpKind::reduce_scatter: {
-    int order = ALAMD_ORDER_RANK_ASC;
+    int order = ALAMD_ORDER_RANK_ASC, start = 0;
     switch (p.algo) {
     case CombineAlgorithm::automatic:
-      order = p.count * es * static_cast<size_t>(P) < (512u << 10) ? ALAMD_ORDER_TREE_HALV : ALAMD_ORDER_PAIRWISE_DESC;
+      if (alamd_reference_order(ALAMD_COLL_REDUCE_SCATTER, P, p.count * static_cast<size_t>(P), p.dtype, 0, &order,
+                                &start) != ALAMD_OK)
+        AL_AMD_THROW(std::string(alamd_last_error()));
       break;
     case CombineAlgorithm::rank_order: order = ALAMD_ORDER_RANK_ASC; break;
     case CombineAlgorithm::tree_doubling: order = ALAMD_ORDER_TREE_DBL; break;
@@ -666,10 +709,11 @@ inline void World::launch(PendingOp &p) {
   case OpKind::reduce_scatterv: {
     size_t total = 0;
     for (size_t c : p.counts) total += c;
-    int order = ALAMD_ORDER_RANK_ASC;
+    int order = ALAMD_ORDER_RANK_ASC, start = 0;
     switch (p.algo) {
     case CombineAlgorithm::automatic:
-      order = total * es < (512u << 10) ? ALAMD_ORDER_TREE_HALV : ALAMD_ORDER_PAIRWISE_DESC;
+      if (alamd_reference_order(ALAMD_COLL_REDUCE_SCATTER, P, total, p.dtype, 0, &order, &start) != ALAMD_OK)
+        AL_AMD_THROW(std::string(alamd_last_error()));
       break;
     case CombineAlgorithm::rank_order: order = ALAMD_ORDER_RANK_ASC; break;
     case CombineAlgorithm::tree_doubling: order = ALAMD_ORDER_TREE_DBL; break;
@@ -903,12 +947,14 @@ class HipCombineBackend {
 /* ---- compile-time traits (include/aluminum/traits/traits_base.hpp:43-62, 86-92, 155-184;
  *      the host-transfer backend's answers: traits/ht_traits.hpp:41-105) ------ */
 
+#ifndef AL_AMD_WITH_REFERENCE
 enum class AlOperation {
   allgather, allgatherv, allreduce, alltoall, alltoallv, barrier, bcast, gather, gatherv, reduce,
   reduce_scatter, reduce_scatterv, scatter, scatterv, send, recv, sendrecv, multisendrecv
 };
 
 template <typename Backend> constexpr char AlBackendName[] = "unknown";
+#endif
 template <> inline constexpr char AlBackendName<HipCombineBackend>[] = "hip";
 
 namespace amd {
@@ -921,24 +967,34 @@ template <typename T, typename = void> struct HasTypeMap : std::false_type {};
 template <typename T> struct HasTypeMap<T, decltype(void(TypeMap<T>::value))> : std::true_type {};
 }  // namespace amd
 
+#ifndef AL_AMD_WITH_REFERENCE
 template <AlOperation Op, typename Backend> struct IsOpSupported : std::false_type {};
+template <typename Backend, typename T> struct IsTypeSupported : std::false_type {};
+template <typename Backend, ReductionOperator op> struct IsReductionOpSupported : std::false_type {};
+template <AlOperation Op, typename Backend> struct OpAlgoType {};
+#endif
 template <AlOperation Op>
 struct IsOpSupported<Op, HipCombineBackend> : std::integral_constant<bool, amd::implements(Op)> {};
 
-template <typename Backend, typename T> struct IsTypeSupported : std::false_type {};
 template <typename T> struct IsTypeSupported<HipCombineBackend, T> : amd::HasTypeMap<T> {};
 
 /** Every operator, avg included: the sum in the collective's order followed by one division by
  *  comm.size() in the element type's arithmetic (the reference has avg on its NCCL backend only,
  *  include/aluminum/nccl_impl.hpp:176; its MPI and host-transfer backends throw, mpi/utils.hpp:192-194). */
-template <typename Backend, ReductionOperator op> struct IsReductionOpSupported : std::false_type {};
 template <ReductionOperator op> struct IsReductionOpSupported<HipCombineBackend, op> : std::true_type {};
 
-template <AlOperation Op, typename Backend, typename = void> struct OpAlgoType {};
-template <AlOperation Op>
-struct OpAlgoType<Op, HipCombineBackend, typename std::enable_if<amd::implements(Op)>::type> {
-  using type = amd::CombineAlgorithm;
-};
+// one specialisation per collective of the engine (the shape of AL_ADD_OP_ALGO_TYPE, traits_base.hpp:180-183)
+#define AL_AMD_ALGO_TYPE(op) \
+  template <> struct OpAlgoType<AlOperation::op, HipCombineBackend> { using type = amd::CombineAlgorithm; }
+AL_AMD_ALGO_TYPE(allreduce);
+AL_AMD_ALGO_TYPE(reduce);
+AL_AMD_ALGO_TYPE(reduce_scatter);
+AL_AMD_ALGO_TYPE(reduce_scatterv);
+AL_AMD_ALGO_TYPE(allgather);
+AL_AMD_ALGO_TYPE(allgatherv);
+#undef AL_AMD_ALGO_TYPE
+
+#ifndef AL_AMD_WITH_REFERENCE
 
 /* ---- the public API templates (include/Al.hpp) ---------------------------- */
 
@@ -1110,6 +1166,7 @@ void Put(const T *srcbuf, int dest, T *destbuf, size_t count, typename Backend::
   Backend::template Put<T>(srcbuf, dest, destbuf, count, comm);
 }
 }  // namespace ext
+#endif  // AL_AMD_WITH_REFERENCE
 
 namespace amd {
 /** Halo faces of a 3-D grid, x fastest (interior dims, `halo` cells on every side): the contiguous
@@ -1142,12 +1199,13 @@ inline size_t halo_face_elems(const size_t dims[3], size_t halo, int face) {
 template <typename Backend> bool Test(typename Backend::req_type &req);
 template <> inline bool Test<HipCombineBackend>(HipCombineBackend::req_type &req) {
   if (req == HipCombineBackend::null_req) return true;
-  if (!req->error.empty()) {
+  const int state = req->state.load(std::memory_order_acquire);
+  if (state == amd::Request::failed) {
     const std::string why = req->error;
     req = HipCombineBackend::null_req;
     throw al_exception("The operation could not be launched: " + why, __FILE__, __LINE__);
   }
-  if (!req->done) return false;  // not launched yet: some logical rank has not made its call
+  if (state == amd::Request::not_launched) return false;  // some logical rank has not made its call
   const hipError_t e = hipEventQuery(req->done->event);
   if (e == hipSuccess) {
     req = HipCombineBackend::null_req;
@@ -1162,12 +1220,13 @@ template <> inline bool Test<HipCombineBackend>(HipCombineBackend::req_type &req
 template <typename Backend> void Wait(typename Backend::req_type &req);
 template <> inline void Wait<HipCombineBackend>(HipCombineBackend::req_type &req) {
   if (req == HipCombineBackend::null_req) return;
-  if (!req->error.empty()) {
+  const int state = req->state.load(std::memory_order_acquire);
+  if (state == amd::Request::failed) {
     const std::string why = req->error;
     req = HipCombineBackend::null_req;
     throw al_exception("The operation could not be launched: " + why, __FILE__, __LINE__);
   }
-  if (!req->done) AL_AMD_THROW("Wait on an operation that not every logical rank has started");
+  if (state == amd::Request::not_launched) AL_AMD_THROW("Wait on an operation that not every logical rank has started");
   if (req->orig_stream != req->done->ran_on && req->done->first_wait(req->orig_stream))
     AL_AMD_CHECK_HIP(hipStreamWaitEvent(req->orig_stream, req->done->event, 0));
   req = HipCombineBackend::null_req;

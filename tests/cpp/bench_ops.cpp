@@ -9,7 +9,7 @@
 //
 // usage: bench_ops [--op allreduce|reduce|reduce_scatter|allgather|reduce_scatterv|allgatherv] [--datatype float|double|int|...]
 //                  [--reduction-op sum|prod|min|max|...] [--algorithm automatic|rank_order|tree_doubling|
-//                  tree_halving|tree_binomial|pairwise|ring|ring_fused] [--ranks P] [--root R]
+//                  tree_halving|tree_binomial|tree_reduce_scatter_gather|pairwise|ring|ring_fused] [--ranks P] [--root R]
 //                  [--inplace] [--nonblocking] [--min-size N] [--max-size N] [--size N] [--num-iters N]
 //                  [--num-warmup N] [--summarize] [--save-to-file FILE] [--no-print-table] [--backend hip]
 //                  [--stream-per-rank]
@@ -207,7 +207,7 @@ int main(int argc, char **argv) {
       {"bxor", Al::ReductionOperator::bxor}, {"avg", Al::ReductionOperator::avg}};
   const std::map<std::string, Algo> algos = {
       {"automatic", Algo::automatic}, {"rank_order", Algo::rank_order}, {"tree_doubling", Algo::tree_doubling},
-      {"tree_halving", Algo::tree_halving}, {"tree_binomial", Algo::tree_binomial}, {"pairwise", Algo::pairwise},
+      {"tree_halving", Algo::tree_halving}, {"tree_binomial", Algo::tree_binomial}, {"tree_reduce_scatter_gather", Algo::tree_reduce_scatter_gather}, {"pairwise", Algo::pairwise},
       {"ring", Algo::ring}, {"ring_fused", Algo::ring_fused}};
   if (!rops.count(o.redop) || !algos.count(o.algo) || o.min_size == 0 ||
       (o.op != "allreduce" && o.op != "reduce" && o.op != "reduce_scatter" && o.op != "allgather" &&

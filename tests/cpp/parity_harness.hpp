@@ -12,12 +12,18 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <fstream>
+#include <map>
 #include <memory>
+#include <sstream>
 #include <string>
 #include <thread>
 #include <vector>
 
+#include <unistd.h>
+
 #include "aluminum_amd/Al.hpp"
+#include "aluminum_amd_support.h"
 #include "oracle.h"
 
 using Backend = Al::HipCombineBackend;
@@ -53,18 +59,37 @@ template <typename T> bool same_bits(const std::vector<T> &a, const std::vector<
   return a.size() == b.size() && (a.empty() || std::memcmp(a.data(), b.data(), a.size() * sizeof(T)) == 0);
 }
 
+// The oracle's order for an algorithm of the front end.  `automatic` is stated here on its own, not
+// asked of the library: what MPICH 3.3.2 does on one host (pinned by the golden vectors in tests/golden;
+// test_backend's test_automatic_against_mpich checks the front end itself against that library's bits).
 static int order_of(Algo a, size_t bytes, bool reduce_scatter, size_t total_bytes) {
   switch (a) {
   case Algo::automatic:
-    if (reduce_scatter) return total_bytes < (512u << 10) ? ALO_ORDER_TREE_HALV : ALO_ORDER_PAIRWISE_DESC;
-    return bytes <= 2048 ? ALO_ORDER_TREE_BINOMIAL : ALO_ORDER_TREE_DBL;
+    return total_bytes < (512u << 10) ? ALO_ORDER_TREE_HALV : ALO_ORDER_PAIRWISE_DESC;
   case Algo::rank_order: return ALO_ORDER_RANK_ASC;
   case Algo::tree_doubling: return ALO_ORDER_TREE_DBL;
   case Algo::tree_halving: return ALO_ORDER_TREE_HALV;
   case Algo::tree_binomial: return ALO_ORDER_TREE_BINOMIAL;
+  case Algo::tree_reduce_scatter_gather: return ALO_ORDER_TREE_RSG;
   case Algo::pairwise: return ALO_ORDER_PAIRWISE_DESC;
   default: return ALO_ORDER_RING;
   }
+  (void)bytes;
+  (void)reduce_scatter;
+}
+
+struct OrderPick { int order, start; };
+// Allreduce (root = 0) and Reduce.
+static OrderPick rooted_order(Algo a, int dt, size_t count, size_t elem_size, int P, int root) {
+  if (a == Algo::automatic) {
+    size_t pof2 = 1;
+    while (2 * pof2 <= (size_t)P) pof2 *= 2;
+    const bool user_op = dt == ALO_F16 || dt == ALO_BF16;
+    if (user_op || count * elem_size <= 2048 || count < pof2) return {ALO_ORDER_TREE_BINOMIAL, root};
+    return {ALO_ORDER_TREE_RSG, 0};
+  }
+  if (a == Algo::tree_binomial) return {ALO_ORDER_TREE_BINOMIAL, root};
+  return {order_of(a, 0, false, 0), 0};
 }
 
 template <typename T>
@@ -108,7 +133,8 @@ void test_allreduce(int P, size_t n, Op op, Algo algo, int dist, bool inplace, b
   } else {
     std::vector<const void *> ptrs;
     for (auto &b : in) ptrs.push_back(b.data());
-    alo_combine(want.data(), ptrs.data(), P, n, dt, (int)op, order_of(algo, n * sizeof(T), false, 0), 0);
+    const OrderPick pick = rooted_order(algo, dt, n, sizeof(T), P, 0);
+    alo_combine(want.data(), ptrs.data(), P, n, dt, (int)op, pick.order, pick.start);
   }
   for (int r = 0; r < P; ++r) {
     auto got = inplace ? send[r]->down() : recv[r]->down();
@@ -150,7 +176,8 @@ void test_reduce(int P, size_t n, Op op, int root, hipStream_t stream, int nonbl
   std::vector<T> want(n);
   std::vector<const void *> ptrs;
   for (auto &b : in) ptrs.push_back(b.data());
-  alo_combine(want.data(), ptrs.data(), P, n, dt, (int)op, order_of(algo, n * sizeof(T), false, 0), 0);
+  const OrderPick pick = rooted_order(algo, dt, n, sizeof(T), P, root);
+  alo_combine(want.data(), ptrs.data(), P, n, dt, (int)op, pick.order, pick.start);
   for (int r = 0; r < P; ++r) {
     // in place only the root's buffer changes; the others keep their contribution
     if (inplace) EXPECT(same_bits(send[r]->down(), r == root ? want : in[r]), "reduce in place P=%d n=%zu root=%d rank %d", P, n, root, r);

@@ -50,6 +50,141 @@ static void test_errors(hipStream_t stream) {
   Al::Wait<Backend>(none);
 }
 
+// `automatic` against MPICH's own results: tests/golden/mpich_front_end_cases.txt holds, for every
+// fixture case whose inputs are the generator's, the checksum of what MPI_Allreduce / MPI_Reduce /
+// MPI_Reduce_scatter_block / MPI_Reduce_scatter returned (2 to 16 ranks, every root tried, below and
+// above each size at which that library changes algorithm, fp32 / fp64 / fp16 / bf16 and integers).
+// The front end, left to choose its order, must return the same bytes.  No oracle in between.
+template <typename T>
+static void run_mpich_case(const std::string &coll, int P, Op op, size_t n, int dist, unsigned seed, int root,
+                           const std::vector<size_t> &counts, const std::vector<std::string> &want, hipStream_t stream) {
+  const int dt = Al::amd::TypeMap<T>::value;
+  const bool scatter = coll == "reduce_scatter" || coll == "reduce_scatterv";
+  size_t in_len = n;
+  if (coll == "reduce_scatter") in_len = n * (size_t)P;
+  if (coll == "reduce_scatterv") { in_len = 0; for (size_t c : counts) in_len += c; }
+  std::vector<std::unique_ptr<DevBuf<T>>> send, recv;
+  for (int r = 0; r < P; ++r) {
+    send.emplace_back(new DevBuf<T>(in_len));
+    recv.emplace_back(new DevBuf<T>(in_len));
+    if (alamd_fill(send[r]->p, in_len, dt, dist, seed + (unsigned)r, 0, stream) != ALAMD_OK) {
+      EXPECT(false, "alamd_fill: %s", alamd_last_error());
+      return;
+    }
+  }
+  Al::amd::World world(P, stream);
+  for (int r = 0; r < P; ++r) {
+    auto &comm = world.comm(r);
+    const T *src = send[r]->p;
+    if (coll == "allreduce") Al::Allreduce<Backend>(src, recv[r]->p, n, op, comm);
+    else if (coll == "reduce") Al::Reduce<Backend>(src, recv[r]->p, n, op, root, comm);
+    else if (coll == "reduce_scatter") Al::Reduce_scatter<Backend>(src, recv[r]->p, n, op, comm);
+    else Al::Reduce_scatterv<Backend>(src, recv[r]->p, counts, op, comm);
+  }
+  HIPCHK(hipStreamSynchronize(stream));
+  for (int r = 0; r < P; ++r) {
+    if (!scatter && r != (coll == "reduce" ? root : r)) continue;
+    const size_t len = coll == "reduce_scatterv" ? counts[(size_t)r] : n;
+    auto got = recv[r]->down();
+    char cs[32];
+    std::snprintf(cs, sizeof(cs), "%016llx", (unsigned long long)alo_checksum(got.data(), len * sizeof(T)));
+    const std::string &w = scatter ? want[(size_t)r] : want[0];
+    EXPECT(w == cs, "%s against MPICH: P=%d dt=%d op=%d n=%zu root=%d rank %d: %s, MPICH %s", coll.c_str(), P, dt, (int)op,
+           len, root, r, cs, w.c_str());
+  }
+}
+
+static void test_automatic_against_mpich(hipStream_t stream) {
+  char exe[4096];
+  const ssize_t len = readlink("/proc/self/exe", exe, sizeof(exe) - 1);
+  EXPECT(len > 0, "readlink /proc/self/exe");
+  if (len <= 0) return;
+  exe[len] = 0;
+  std::string path(exe);
+  path = path.substr(0, path.rfind('/')) + "/../golden/mpich_front_end_cases.txt";
+  std::ifstream f(path);
+  EXPECT(f.good(), "cannot open %s", path.c_str());
+  static const std::map<std::string, Op> ops = {
+      {"sum", Op::sum}, {"prod", Op::prod}, {"min", Op::min}, {"max", Op::max}, {"lor", Op::lor}, {"land", Op::land},
+      {"lxor", Op::lxor}, {"bor", Op::bor}, {"band", Op::band}, {"bxor", Op::bxor}};
+  int ran = 0, reduces = 0, halves = 0;
+  std::string line;
+  while (std::getline(f, line)) {
+    if (line.empty() || line[0] == '#') continue;
+    std::istringstream in(line);
+    std::string coll, dtype, opname;
+    int P = 0, dist = 0, root = 0;
+    unsigned seed = 0;
+    size_t n = 0;
+    std::vector<size_t> counts;
+    in >> coll >> P >> dtype >> opname;
+    if (coll != "reduce_scatterv") in >> n;
+    in >> dist >> seed;
+    if (coll == "reduce") in >> root;
+    if (coll == "reduce_scatterv")
+      for (int b = 0; b < P; ++b) { size_t c = 0; in >> c; counts.push_back(c); }
+    std::vector<std::string> want;
+    for (std::string w; in >> w;) want.push_back(w);
+    const bool scatter = coll == "reduce_scatter" || coll == "reduce_scatterv";
+    EXPECT(in.eof() && want.size() == (scatter ? (size_t)P : 1u) && ops.count(opname), "malformed line: %s", line.c_str());
+    if (want.size() != (scatter ? (size_t)P : 1u) || !ops.count(opname)) continue;
+    const Op op = ops.at(opname);
+#define RUN(NAME, T) if (dtype == NAME) run_mpich_case<T>(coll, P, op, n, dist, seed, root, counts, want, stream); else
+    RUN("i8", signed char) RUN("u8", unsigned char) RUN("i16", short) RUN("u16", unsigned short) RUN("i32", int)
+    RUN("u32", unsigned int) RUN("i64", long long) RUN("u64", unsigned long long) RUN("f16", Al::amd::half_bits)
+    RUN("bf16", Al::amd::bfloat16_bits) RUN("f32", float) RUN("f64", double)
+    EXPECT(false, "unknown dtype in %s", line.c_str());
+#undef RUN
+    ++ran;
+    reduces += coll == "reduce";
+    halves += dtype == "f16" || dtype == "bf16";
+  }
+  EXPECT(ran >= 800 && reduces >= 250 && halves >= 150, "too few cases: %d in all, %d reduces, %d of 16-bit floats", ran,
+         reduces, halves);
+}
+
+// One rank's thread polls Test on its request while another thread makes the last call, which launches
+// the operation, or fails to: the outcome reaches the polling thread through the request alone.
+static void test_request_polled_while_launching() {
+  const size_t n = 4096;
+  for (int round = 0; round < 200; ++round) {
+    const bool fail = round % 4 == 3;  // band on floats: the last call finds that the operation cannot be launched
+    const Op op = fail ? Op::band : Op::sum;
+    hipStream_t s0, s1;
+    HIPCHK(hipStreamCreateWithFlags(&s0, hipStreamNonBlocking));
+    HIPCHK(hipStreamCreateWithFlags(&s1, hipStreamNonBlocking));
+    {
+      DevBuf<float> a(n), b(n);
+      a.up(gen<float>(n, ALO_DIST_UNIFORM_PM1, 1));
+      b.up(gen<float>(n, ALO_DIST_UNIFORM_PM1, 2));
+      Al::amd::World world(std::vector<hipStream_t>{s0, s1});
+      Backend::req_type r0;
+      Al::NonblockingAllreduce<Backend>(a.p, n, op, world.comm(0), r0);
+      std::atomic<int> outcome{0};  // 1: completed, 2: threw
+      std::thread poller([&] {
+        try {
+          while (!Al::Test<Backend>(r0)) std::this_thread::yield();
+          outcome = 1;
+        } catch (const Al::al_exception &) { outcome = 2; }
+      });
+      Backend::req_type r1;
+      bool threw = false;
+      try {
+        Al::NonblockingAllreduce<Backend>(b.p, n, op, world.comm(1), r1);
+      } catch (const Al::al_exception &) { threw = true; }
+      poller.join();
+      EXPECT(threw == fail, "round %d: the last call %s", round, fail ? "should have thrown" : "threw");
+      EXPECT(outcome == (fail ? 2 : 1), "round %d: the polling rank saw outcome %d", round, outcome.load());
+      EXPECT(r0 == Backend::null_req, "round %d: request not reset", round);
+      if (!fail) Al::Wait<Backend>(r1);
+      HIPCHK(hipStreamSynchronize(s0));
+      HIPCHK(hipStreamSynchronize(s1));
+    }
+    HIPCHK(hipStreamDestroy(s0));
+    HIPCHK(hipStreamDestroy(s1));
+  }
+}
+
 // Several collectives in flight, posted by P threads, each rank on its own stream.
 static void test_threads_and_streams() {
   const int P = 4;
@@ -583,9 +718,19 @@ int main() {
       test_v_variants<float>(P, inplace, stream);
       test_v_variants<double>(P, inplace, stream);
     }
+  for (int P : {3, 5, 8})
+    for (size_t n : {size_t(7), size_t(600), size_t(70001)})
+      for (int root : {0, 1, P - 1}) {
+        test_reduce<double>(P, n, Op::prod, root, stream, -1, false, ALO_DIST_UNIFORM_09_11);
+        test_reduce<Al::amd::bfloat16_bits>(P, n, Op::sum, root, stream, -1, true, ALO_DIST_NORMAL);
+        test_reduce<float>(P, n, Op::max, root, stream, -1, false, ALO_DIST_UNIFORM_PM1, Algo::tree_binomial);
+        test_reduce<float>(P, n, Op::sum, root, stream, -1, false, ALO_DIST_UNIFORM_PM1, Algo::tree_reduce_scatter_gather);
+      }
+  test_automatic_against_mpich(stream);
   test_errors(stream);
   test_error_recovery(stream);
   test_threads_and_streams();
+  test_request_polled_while_launching();
   test_stream_order(false);
   test_stream_order(true);
   test_stream_order_shared_stream();

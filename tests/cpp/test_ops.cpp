@@ -8,7 +8,7 @@
 //
 // usage: test_ops --op allreduce|reduce|reduce_scatter|allgather|reduce_scatterv|allgatherv
 //                 [--backend hip] [--inplace] [--nonblocking] [--reduction-op sum|prod|min|max|lor|land|lxor|bor|band|bxor]
-//                 [--algorithm automatic|rank_order|tree_doubling|tree_halving|tree_binomial|pairwise|ring|ring_fused]
+//                 [--algorithm automatic|rank_order|tree_doubling|tree_halving|tree_binomial|tree_reduce_scatter_gather|pairwise|ring|ring_fused]
 //                 [--root R] [--size N | --min-size N --max-size N] [--odd-sizes] [--datatype float|...]
 //                 [--trials N] [--ranks P] [--threads N]
 #include <map>
@@ -127,7 +127,7 @@ int main(int argc, char **argv) {
   static const std::map<std::string, Algo> algos = {
       {"automatic", Algo::automatic}, {"", Algo::automatic}, {"rank_order", Algo::rank_order},
       {"tree_doubling", Algo::tree_doubling}, {"tree_halving", Algo::tree_halving},
-      {"tree_binomial", Algo::tree_binomial}, {"pairwise", Algo::pairwise}, {"ring", Algo::ring},
+      {"tree_binomial", Algo::tree_binomial}, {"tree_reduce_scatter_gather", Algo::tree_reduce_scatter_gather}, {"pairwise", Algo::pairwise}, {"ring", Algo::ring},
       {"ring_fused", Algo::ring_fused}};
   static const char *ops[] = {"allreduce", "reduce", "reduce_scatter", "allgather", "reduce_scatterv", "allgatherv"};
   bool op_ok = false;

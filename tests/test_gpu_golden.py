@@ -1,8 +1,11 @@
 """The HIP library against the MPICH golden vectors in tests/golden, through the C ABI and with
-no oracle in between: what MPI_Allreduce / MPI_Reduce_scatter_block / MPI_Reduce_scatter of
+no oracle in between: what MPI_Allreduce / MPI_Reduce / MPI_Reduce_scatter_block / MPI_Reduce_scatter of
 MPICH 3.3.2 returned for these inputs (the calls the reference's MPI backend forwards to,
-include/aluminum/mpi/allreduce.hpp:38-44, mpi/reduce_scatter.hpp:40-46) is what the GPU must
-return, bit for bit, under the order the front end's `automatic` picks for that message size."""
+include/aluminum/mpi/allreduce.hpp:38-44, mpi/reduce.hpp:41-49, mpi/reduce_scatter.hpp:40-46, and whose
+non-blocking forms its host-transfer backend makes, include/aluminum/ht/reduce.hpp:72-82) is what the GPU
+must return, bit for bit, under the order that alamd_reference_order names for that collective, root,
+type and message size - including the cases with NaNs, zeros of both signs and infinities planted in
+every operand position, where the bits depend on which operand of every pair is the inoutvec."""
 import glob
 import gzip
 import json
@@ -12,12 +15,14 @@ import numpy as np
 import pytest
 
 import oracle
-from util import assert_bits_equal, dev_empty, to_dev, to_host
+from util import assert_bits_equal, dev_empty, mpich_order, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
 
-GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "mpich_P*.json.gz")))
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "mpich_P*.json.gz")),
+                key=lambda p: int(os.path.basename(p)[7:-8]))
 IDS = [os.path.basename(p)[:-8] for p in GOLDEN]
+COLL = {"allreduce": 0, "reduce": 1, "reduce_scatter": 2, "reduce_scatterv": 2}
 
 
 def load(path):
@@ -29,6 +34,20 @@ def arr(hexstr, dtype):
     return np.frombuffer(bytes.fromhex(hexstr), dtype=oracle.NP_CARRIER[dtype]).copy()
 
 
+def inputs_of(c, P, n):
+    if "in" in c:
+        return [arr(h, c["dtype"]) for h in c["in"]]
+    return [oracle.fill(n, c["dtype"], c["dist"], c["seed_base"] + r) for r in range(P)]
+
+
+def library_order(al, coll, P, count, dtype, root=0):
+    """What the library itself picks; the tests also hold it against the table in util.mpich_order."""
+    order, start = al.reference_order(coll, P, count, dtype, root)
+    want = mpich_order(coll, dtype, count if coll in ("allreduce", "reduce") else 0, P, root, total=count)
+    assert (order, start) == want, (coll, P, count, dtype, root, order, start, want)
+    return order, start
+
+
 @pytest.mark.parametrize("path", GOLDEN, ids=IDS)
 def test_allreduce_vectors_on_the_gpu(al, path):
     import torch
@@ -38,19 +57,46 @@ def test_allreduce_vectors_on_the_gpu(al, path):
         if c["coll"] != "allreduce":
             continue
         dt, op, n = c["dtype"], c["op"], c["n"]
-        ins = [arr(h, dt) for h in c["in"]]
+        ins = inputs_of(c, P, n)
         want = arr(c["out"][0], dt)
-        # Al::Allreduce, automatic: binomial tree up to 2048 bytes, doubling tree above
-        order = "tree_binomial" if n * ins[0].itemsize <= 2048 else "tree_dbl"
+        order, start = library_order(al, "allreduce", P, n, dt)
         d_ins = [to_dev(a) for a in ins]
         outs = [dev_empty(n, ins[0].dtype) for _ in range(P)]
-        al.combine(outs, d_ins, op, order=order, dtype=dt, count=n)
+        al.combine(outs, d_ins, op, order=order, start=start, dtype=dt, count=n)
         torch.cuda.synchronize()
-        what = "P=%d %s %s n=%d %s" % (P, dt, op, n, c["note"])
+        what = "P=%d %s %s n=%d %s (%s)" % (P, dt, op, n, c["note"], order)
         for r in range(P):
             assert_bits_equal(to_host(outs[r], ins[0].dtype), want, dt, what + " rank %d" % r)
         seen += 1
-    assert seen >= 12
+    assert seen >= 18
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=IDS)
+def test_reduce_vectors_on_the_gpu(al, path):
+    """MPI_Reduce to the first, second and last rank."""
+    import torch
+    doc = load(path)
+    P, seen, roots = doc["P"], 0, set()
+    for c in doc["cases"]:
+        if c["coll"] != "reduce":
+            continue
+        dt, op, n, root = c["dtype"], c["op"], c["n"], c["root"]
+        npdt = oracle.NP_CARRIER[dt]
+        order, start = library_order(al, "reduce", P, n, dt, root)
+        d_ins = [to_dev(a) for a in inputs_of(c, P, n)]
+        out = dev_empty(n, npdt)
+        al.combine([out], d_ins, op, order=order, start=start, dtype=dt, count=n)
+        torch.cuda.synchronize()
+        got = to_host(out, npdt)
+        what = "P=%d %s %s n=%d root %d %s (%s)" % (P, dt, op, n, root, c["note"], order)
+        if "out" in c:
+            assert_bits_equal(got, arr(c["out"], dt), dt, what)
+        else:
+            assert "%016x" % oracle.checksum(got) == c["out_checksum"], what
+            assert_bits_equal(got[:8], arr(c["out_head"], dt), dt, what)
+        seen += 1
+        roots.add(root)
+    assert seen >= 30 and roots == {0, 1, P - 1}
 
 
 @pytest.mark.parametrize("path", GOLDEN, ids=IDS)
@@ -63,43 +109,48 @@ def test_reduce_scatter_vectors_on_the_gpu(al, path):
             continue
         dt, op, count = c["dtype"], c["op"], c["n"]
         npdt = oracle.NP_CARRIER[dt]
-        if "in" in c:  # short message: recursive halving
-            ins = [arr(h, dt) for h in c["in"]]
-            order = "tree_halv"
-        else:          # long message: pairwise exchange; inputs are the generator's, outputs kept as checksums
-            ins = [oracle.fill(P * count, dt, c["dist"], c["seed_base"] + r) for r in range(P)]
-            order = "pairwise_desc"
+        order, _ = library_order(al, "reduce_scatter", P, P * count, dt)
+        ins = inputs_of(c, P, P * count)
         d_sends = [to_dev(a) for a in ins]
         d_recvs = [dev_empty(count, npdt) for _ in range(P)]
         al.reduce_scatter(d_recvs, d_sends, op, order=order, dtype=dt, count=count)
         torch.cuda.synchronize()
         for r in range(P):
             got = to_host(d_recvs[r], npdt)
-            if "in" in c:
-                assert_bits_equal(got, arr(c["out"][r], dt), dt, "reduce_scatter short P=%d rank %d" % (P, r))
+            if "out" in c:
+                assert_bits_equal(got, arr(c["out"][r], dt), dt, "reduce_scatter short P=%d %s rank %d" % (P, dt, r))
             else:
-                assert "%016x" % oracle.checksum(got) == c["out_checksum"][r], (P, r)
+                assert "%016x" % oracle.checksum(got) == c["out_checksum"][r], (P, dt, r)
                 assert_bits_equal(got[:8], arr(c["out_head"][r], dt), dt, "head")
         seen += 1
-    assert seen >= 4
+    assert seen >= 8
 
 
 @pytest.mark.parametrize("path", GOLDEN, ids=IDS)
 def test_reduce_scatterv_vectors_on_the_gpu(al, path):
+    """MPI_Reduce_scatter with uneven counts, below and above 512 KiB in all."""
     import torch
     doc = load(path)
     P = doc["P"]
-    for c in [c for c in doc["cases"] if c["coll"] == "reduce_scatterv"]:
-        dt, counts = c["dtype"], c["counts"]
+    cases = [c for c in doc["cases"] if c["coll"] == "reduce_scatterv"]
+    assert len(cases) == 8
+    for c in cases:
+        dt, counts, total = c["dtype"], c["counts"], c["n"]
         npdt = oracle.NP_CARRIER[dt]
-        ins = [arr(h, dt) for h in c["in"]]
-        d_sends = [to_dev(a) for a in ins]
+        order, _ = library_order(al, "reduce_scatter", P, total, dt)
+        d_sends = [to_dev(a) for a in inputs_of(c, P, total)]
         d_recvs = [dev_empty(max(k, 1), npdt) for k in counts]
-        al.reduce_scatterv(d_recvs, d_sends, counts, c["op"], order="tree_halv", dtype=dt)
+        al.reduce_scatterv(d_recvs, d_sends, counts, c["op"], order=order, dtype=dt)
         torch.cuda.synchronize()
         for b in range(P):
-            want = arr(c["out"][b], dt)[:counts[b]]
-            assert_bits_equal(to_host(d_recvs[b], npdt)[:counts[b]], want, dt, "reduce_scatterv P=%d rank %d" % (P, b))
+            got = to_host(d_recvs[b], npdt)[:counts[b]]
+            what = "reduce_scatterv P=%d %s rank %d (%s)" % (P, dt, b, order)
+            if "out" in c:
+                assert_bits_equal(got, arr(c["out"][b], dt)[:counts[b]], dt, what)
+            else:
+                assert "%016x" % oracle.checksum(got) == c["out_checksum"][b], what
+                if counts[b]:
+                    assert_bits_equal(got[:8], arr(c["out_head"][b], dt), dt, what)
 
 
 MPIEXEC = "/opt/conda/bin/mpiexec"
@@ -109,22 +160,24 @@ MPI_PROGRAM = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__fil
 @pytest.mark.skipif(not (os.path.exists(MPIEXEC) and os.path.exists(MPI_PROGRAM)),
                     reason="needs mpiexec and the built oracle/mpi_baseline")
 @pytest.mark.parametrize("P", (2, 3, 4, 5, 8))
-def test_live_mpi_allreduce_against_the_gpu(al, P):
-    """MPI_Allreduce(MPI_SUM, MPI_FLOAT) run now, on this machine's host cores, over generated inputs
-    (uniform[-1,1), seed 1000+rank), against the GPU's combine of the same inputs: equal checksums."""
+def test_live_mpi_allreduce_and_reduce_against_the_gpu(al, P):
+    """MPI_Allreduce and MPI_Reduce (MPI_SUM, MPI_FLOAT) run now, on this machine's host cores, over
+    generated inputs (uniform[-1,1), seed 1000+rank), against the GPU's combine of the same inputs under
+    the order the library names: equal checksums."""
     import subprocess
     import torch
     for n in (300, 513, (1 << 16) + 1, 1 << 20):
-        p = subprocess.run([MPIEXEC, "-n", str(P), MPI_PROGRAM, str(n), "0", "1"], capture_output=True, text=True,
-                           timeout=120)
-        line = [l for l in p.stdout.splitlines() if l.startswith("{")]
-        assert p.returncode == 0 and line, (p.stdout, p.stderr)
-        want = json.loads(line[-1])["checksum"]
-        ins = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(P)]
-        out = torch.empty(n, dtype=torch.float32, device="cuda")
-        for r in range(P):
-            al.fill(ins[r], "uniform_pm1", 1000 + r)
-        order = "tree_binomial" if n * 4 <= 2048 else "tree_dbl"
-        al.combine([out], ins, "sum", order=order)
-        torch.cuda.synchronize()
-        assert "%016x" % oracle.checksum(out.cpu().numpy()) == want, "P=%d n=%d" % (P, n)
+        for root in (-1, 0, P - 1):  # -1: allreduce
+            p = subprocess.run([MPIEXEC, "-n", str(P), MPI_PROGRAM, str(n), "0", "1", str(root)], capture_output=True,
+                               text=True, timeout=120)
+            line = [l for l in p.stdout.splitlines() if l.startswith("{")]
+            assert p.returncode == 0 and line, (p.stdout, p.stderr)
+            want = json.loads(line[-1])["checksum"]
+            ins = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(P)]
+            out = torch.empty(n, dtype=torch.float32, device="cuda")
+            for r in range(P):
+                al.fill(ins[r], "uniform_pm1", 1000 + r)
+            order, start = library_order(al, "allreduce" if root < 0 else "reduce", P, n, "f32", max(root, 0))
+            al.combine([out], ins, "sum", order=order, start=start)
+            torch.cuda.synchronize()
+            assert "%016x" % oracle.checksum(out.cpu().numpy()) == want, "P=%d n=%d root=%d" % (P, n, root)
