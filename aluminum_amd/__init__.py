@@ -12,7 +12,8 @@ from . import capi  # noqa: F401
 from .capi import (  # noqa: F401
     AlError, DTYPES, OPS, ORDERS, DISTS, RING_MODES, FLAG_MODES,
     load, lib_path, combine, reduce_scatter, allgather, reduce_scatterv, reduce_scatterv_noalloc, allgatherv,
-    reduce_scatterv_wait_expired, set_chain_poll_limit, tune, tuned, reference_order,
+    reduce_scatterv_wait_expired, set_chain_poll_limit, tune, tuned, reference_order, reserve_scratch,
+    release_scratch, CHAIN_POLLS_NONE, planned_launches,
     ring_allreduce,
     ring_reduce_scatter, ring_allgather, halo_pack, halo_unpack, halo_face_elems,
     fill, narrow_f32, widen_f32, copy, Flag, torch_dtype, dtype_size, check_op,

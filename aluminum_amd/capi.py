@@ -67,9 +67,13 @@ def load():
     L.alamd_allgatherv.argtypes = [pvp, pvp, i, C.POINTER(sz), C.POINTER(sz), i, vp]
     L.alamd_reduce_scatterv_wait_expired.argtypes = []
     L.alamd_set_chain_poll_limit.argtypes = [C.c_uint]
+    L.alamd_reserve_scratch.argtypes = [vp, sz]
+    L.alamd_release_scratch.argtypes = [vp]
     L.alamd_tune.argtypes = [C.c_char_p, sz]
     L.alamd_tuned.argtypes = [C.c_char_p]
     L.alamd_tuned.restype = sz
+    L.alamd_planned_launches.argtypes = [i, sz, i]
+    L.alamd_planned_launches.restype = sz
     L.alamd_ring_allreduce.argtypes = [pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_allreduce_from.argtypes = [pvp, pvp, i, sz, i, i, sz, i, vp]
     L.alamd_ring_reduce_scatter.argtypes = [pvp, i, sz, i, i, sz, i, vp]
@@ -218,9 +222,21 @@ def reduce_scatterv_wait_expired():
     return bool(load().alamd_reduce_scatterv_wait_expired())
 
 
+CHAIN_POLLS_NONE = 0xffffffff  # every wait the tiling calls for gives up without looking
+
+
 def set_chain_poll_limit(polls):
-    """Polls after which such a wait gives up (0: the default); for tests of that path."""
+    """Polls after which such a wait gives up (0: the default; CHAIN_POLLS_NONE); for tests of that path."""
     _check(load().alamd_set_chain_poll_limit(polls))
+
+
+def reserve_scratch(max_block_bytes, stream=None):
+    """alamd_reserve_scratch: scratch for in-place Reduce_scatterv blocks of up to that many bytes on `stream`."""
+    _check(load().alamd_reserve_scratch(_stream(stream), max_block_bytes))
+
+
+def release_scratch(stream=None):
+    _check(load().alamd_release_scratch(_stream(stream)))
 
 
 def tune(name, value):
@@ -230,6 +246,11 @@ def tune(name, value):
 
 def tuned(name):
     return int(load().alamd_tuned(name.encode()))
+
+
+def planned_launches(P, count, dtype):
+    """Kernel launches of one alamd_combine call with one output (alamd_planned_launches)."""
+    return int(load().alamd_planned_launches(P, count, _dt(dtype)))
 
 
 def allgatherv(recvs, sends, counts, displs, dtype=None, stream=None):

@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <atomic>
 #include <type_traits>
 
 #include "aluminum_amd.h"
@@ -32,16 +33,19 @@ int device_cus();
 
 // The sizes the launch planners work with (what each one means, and the measurements behind its default,
 // stands where it is used).  Defaults suit an MI355X; alamd_tune() changes them for comparisons.
+// Process-wide; every field is an atomic, so that a setting changed while calls run is a clean old-or-new
+// value for each of them, never a torn one.
 struct Tunables {
-  size_t launch_bytes = (size_t)800 << 20;          // bytes one fold / tree launch moves
-  size_t two_step_min_total_bytes = (size_t)128 << 20;  // fold + spread instead of one kernel: from this many
-                                                        // bytes written in all (outputs x bytes each) ...
-  size_t two_step_min_outputs = 3;                  // ... and this many outputs up
-  size_t two_step_piece_bytes = (size_t)128 << 20;  // piece of the result the two steps alternate over
-  size_t ring_piece_bytes = (size_t)256 << 20;      // the same for the fused ring allreduce
-  size_t spread_launch_bytes = (size_t)288 << 20;   // bytes one spread launch moves
-  size_t spread_hbm_chunk_tiles = 1024, spread_hbm_launch_chunks = 2;      // slices read from HBM
-  size_t spread_cache_chunk_tiles = 512, spread_cache_launch_chunks = 16;  // a result just written
+  std::atomic<size_t> launch_bytes{(size_t)800 << 20};          // bytes one fold / tree launch moves
+  std::atomic<size_t> two_step_min_total_bytes{(size_t)128 << 20};  // fold + spread instead of one kernel: from this
+                                                                    // many bytes written in all (outputs x bytes each) ...
+  std::atomic<size_t> two_step_min_outputs{3};                  // ... and this many outputs up
+  std::atomic<size_t> two_step_piece_bytes{(size_t)128 << 20};  // piece of the result the two steps alternate over
+  std::atomic<size_t> ring_piece_bytes{(size_t)256 << 20};      // the same for the fused ring allreduce
+  std::atomic<size_t> spread_launch_bytes{(size_t)288 << 20};   // bytes one spread launch moves
+  std::atomic<size_t> spread_hbm_chunk_tiles{1024}, spread_hbm_launch_chunks{2};      // slices read from HBM
+  std::atomic<size_t> spread_cache_chunk_tiles{512}, spread_cache_launch_chunks{16};  // a result just written
+  std::atomic<size_t> halo_load_policy{0};  // grid loads of a halo pack: 0 plain, 1 nt, 2 sc1, 3 sc0 sc1, 4 sc0 sc1 nt
 };
 Tunables &tunables();
 

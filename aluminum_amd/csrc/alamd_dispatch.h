@@ -186,7 +186,9 @@ __device__ __forceinline__ void chain_gate(const ChainParams &c, unsigned self, 
       long long hi = (a1 + tb - 1) / tb - 1;           // ceil - 1
       if (hi > (long long)self - 1) hi = (long long)self - 1;
       if (hi > (long long)c.nvec_tiles - 1) hi = (long long)c.nvec_tiles - 1;
-      for (long long t = lo; t <= hi; ++t) {
+      // max_polls == 0 (a test's setting): a wait that the tiling calls for gives up without looking
+      if (c.max_polls == 0 && lo <= hi) __hip_atomic_store(c.error, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      for (long long t = lo; t <= hi && c.max_polls != 0; ++t) {
         unsigned spins = 0;
         while (__hip_atomic_load(&c.flags[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) == 0u) {
           __builtin_amdgcn_s_sleep(2);

@@ -10,6 +10,7 @@
 
 #include "alamd_dispatch.h"
 #include "alamd_tile.h"
+#include "aluminum_amd_support.h"
 
 namespace alamd {
 
@@ -144,7 +145,7 @@ constexpr size_t kChainMinTileBytes = 4096;
 struct ChainPool {
   std::mutex mutex;
   std::map<std::pair<int, hipStream_t>, ChainScratch> live;
-  std::vector<void *> retired;
+  std::map<std::pair<int, hipStream_t>, std::vector<void *>> retired;
 };
 ChainPool &chain_pool() {
   static ChainPool *pool = new ChainPool;  // never destroyed: device memory outlives static destruction order
@@ -194,10 +195,15 @@ ChainScratch scratch_at(void *base, size_t bytes) {
   return cs;
 }
 
-int chain_scratch_for(hipStream_t stream, size_t tiles, ChainScratch &out) {
+// The scratch of `stream` for `tiles` tile flags.  may_allocate: a buffer that is missing or too small is
+// allocated here (hipMalloc, nothing else: every chained launch clears what it uses on its own stream
+// first); otherwise its absence is an error.  A stream that is being captured never allocates.
+int chain_scratch_for(hipStream_t stream, size_t tiles, bool may_allocate, ChainScratch &out) {
   int dev = 0;
   ALAMD_HIP(hipGetDevice(&dev));
-  if (int rc = expired_word_init()) return rc;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  ALAMD_HIP(hipStreamIsCapturing(stream, &capturing));
+  if (capturing != hipStreamCaptureStatusNone) may_allocate = false;
   ChainPool &pool = chain_pool();
   std::lock_guard<std::mutex> lock(pool.mutex);
   auto key = std::make_pair(dev, stream);
@@ -207,13 +213,20 @@ int chain_scratch_for(hipStream_t stream, size_t tiles, ChainScratch &out) {
     finish_scratch(out);
     return ALAMD_OK;
   }
+  if (!may_allocate)
+    return set_error(ALAMD_ERR_INVALID_ARG,
+                     "an in-place block that overlaps its own input needs %zu bytes of scratch on this stream, and a "
+                     "stream that is being captured cannot allocate them: call alamd_reserve_scratch first",
+                     kChainHeaderBytes + tiles * sizeof(unsigned));
+  if (int rc = expired_word_init()) return rc;
   size_t cap = (size_t)1 << 16;
   while (cap < tiles) cap *= 2;
   const size_t bytes = kChainHeaderBytes + cap * sizeof(unsigned);
   void *mem = nullptr;
   ALAMD_HIP(hipMalloc(&mem, bytes));
-  ALAMD_HIP(hipMemset(mem, 0, kChainHeaderBytes));
-  if (it != pool.live.end()) pool.retired.push_back(it->second.ticket);
+  // work already enqueued may still use the buffer this one replaces: it is kept until the stream's
+  // scratch is released
+  if (it != pool.live.end()) pool.retired[key].push_back(it->second.ticket);
   out = scratch_at(mem, bytes);
   pool.live[key] = out;
   finish_scratch(out);
@@ -230,20 +243,64 @@ namespace {
 
 std::mutex g_static_mutex;
 unsigned char *g_static_ptr[64];
+// Who used a device's array last: the stream, and an event recorded behind its chained launch.  A call on
+// another stream that comes before that event has completed would share counter and flags with work still
+// running, and is refused.  (Launches recorded into a graph are not tracked: what runs beside a replay is
+// the caller's to order.)
+struct StaticOwner { hipStream_t stream = nullptr; hipEvent_t event = nullptr; bool pending = false; };
+StaticOwner g_static_owner[64];
 
-int static_chain_scratch(ChainScratch &out) {
+// Set-up, once per device, by alamd_init: the array's address on the current device and the owner's event.
+int static_scratch_setup() {
   int dev = 0;
   ALAMD_HIP(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64) return set_error(ALAMD_ERR_HIP, "device index %d out of range", dev);
   std::lock_guard<std::mutex> lock(g_static_mutex);
-  if (!g_static_ptr[dev]) {
-    unsigned char *ptr = nullptr;
-    ALAMD_HIP(hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)));
-    if (!ptr) return set_error(ALAMD_ERR_HIP, "hipGetSymbolAddress returned a null address");
-    g_static_ptr[dev] = ptr;
+  if (g_static_ptr[dev]) return ALAMD_OK;
+  unsigned char *ptr = nullptr;
+  ALAMD_HIP(hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch)));
+  if (!ptr) return set_error(ALAMD_ERR_HIP, "hipGetSymbolAddress returned a null address");
+  ALAMD_HIP(hipEventCreateWithFlags(&g_static_owner[dev].event, hipEventDisableTiming));
+  g_static_ptr[dev] = ptr;
+  return ALAMD_OK;
+}
+
+// The fixed array as scratch for a call on `stream`.  Allocates nothing: without alamd_init on this device
+// it is an error.
+int static_chain_scratch(hipStream_t stream, ChainScratch &out) {
+  int dev = 0;
+  ALAMD_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return set_error(ALAMD_ERR_HIP, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (!g_static_ptr[dev] || !g_expired_host)
+    return set_error(ALAMD_ERR_INVALID_ARG, "alamd_reduce_scatterv_noalloc needs alamd_init to have run on this device "
+                                            "(it looks up the fixed scratch array and allocates nothing later)");
+  StaticOwner &own = g_static_owner[dev];
+  if (own.pending && own.stream != stream) {
+    const hipError_t e = hipEventQuery(own.event);
+    if (e == hipErrorNotReady)
+      return set_error(ALAMD_ERR_INVALID_ARG, "the fixed scratch array is still in use by a chained launch on another "
+                                              "stream of this device: keep such calls on one stream, or order them");
+    if (e != hipSuccess) return set_error(ALAMD_ERR_HIP, "hipEventQuery failed: %s", hipGetErrorString(e));
+    own.pending = false;
   }
   out = scratch_at(g_static_ptr[dev], ALAMD_NOALLOC_SCRATCH_BYTES);
   finish_scratch(out);
+  return ALAMD_OK;
+}
+
+// Called behind a chained launch that used the fixed array.
+int static_scratch_used(hipStream_t stream) {
+  int dev = 0;
+  ALAMD_HIP(hipGetDevice(&dev));
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  ALAMD_HIP(hipStreamIsCapturing(stream, &capturing));
+  if (capturing != hipStreamCaptureStatusNone) return ALAMD_OK;
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  StaticOwner &own = g_static_owner[dev];
+  ALAMD_HIP(hipEventRecord(own.event, stream));
+  own.stream = stream;
+  own.pending = true;
   return ALAMD_OK;
 }
 
@@ -349,8 +406,7 @@ int check_common(int P, size_t count, int dtype) {
 
 int chain_static_init() {
   if (int rc = expired_word_init()) return rc;
-  ChainScratch cs;
-  return static_chain_scratch(cs);
+  return static_scratch_setup();
 }
 
 int chain_clear(const ChainScratch &cs, size_t tiles, hipStream_t stream) {
@@ -591,10 +647,11 @@ int reduce_scatterv_in_place(void *const *recvs, const void *const *sends, int P
             return set_error(ALAMD_ERR_INVALID_ARG,
                              "in-place block %d of %zu bytes is beyond the %zu bytes the fixed scratch covers", b,
                              n * es, cs.max_tiles * kChainMinTileBytes);
-        } else if ((rc = chain_scratch_for(stream, tiles, cs))) {
+        } else if ((rc = chain_scratch_for(stream, tiles, true, cs))) {
           return rc;
         }
         rc = launch_order(out_tab, ins, P, lay, dtype, op, order, stream, &cs, displ[b] * es);
+        if (rc == ALAMD_OK && fixed) rc = static_scratch_used(stream);
       } else {
         rc = launch_order(out_tab, ins, P, lay, dtype, op, order, stream);
       }
@@ -822,7 +879,7 @@ int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P, c
 int alamd_reduce_scatterv_noalloc(void *const *recvs, const void *const *sends, int P, const size_t *counts,
                                   int dtype, int op, int order, void *stream) {
   ChainScratch cs;
-  const int rc = static_chain_scratch(cs);
+  const int rc = static_chain_scratch(as_stream(stream), cs);
   if (rc) return rc;
   return reduce_scatterv_impl(recvs, sends, P, counts, dtype, op, order, stream, &cs);
 }
@@ -830,7 +887,46 @@ int alamd_reduce_scatterv_noalloc(void *const *recvs, const void *const *sends, 
 int alamd_reduce_scatterv_wait_expired(void) { return take_expired() ? 1 : 0; }
 
 int alamd_set_chain_poll_limit(unsigned polls) {
-  g_chain_polls.store(polls ? polls : kChainDefaultPolls);
+  g_chain_polls.store(polls == ALAMD_CHAIN_POLLS_NONE ? 0u : polls ? polls : kChainDefaultPolls);
+  return ALAMD_OK;
+}
+
+size_t alamd_planned_launches(int P, size_t count, int dtype) {
+  const size_t es = alamd_dtype_size(dtype);
+  if (P < 1 || P > ALAMD_MAX_RANKS || es == 0 || count == 0) return 0;
+  // the planner of the fold kernels, run without launching anything
+  constexpr size_t kTileBytes = Tile<8, 128>::BYTES;
+  SegParams seg = make_seg(count, 0, 0, OUT_ALL, 1);
+  size_t launches = 0;
+  plan_launches(seg, 1, count, kTileBytes / es, launch_tiles(P, kTileBytes, tunables().launch_bytes),
+                [&](size_t, size_t, unsigned, unsigned) { ++launches; });
+  return launches;
+}
+
+int alamd_reserve_scratch(void *stream, size_t max_block_bytes) {
+  if (max_block_bytes == 0) return ALAMD_OK;
+  ChainScratch cs;
+  const size_t tiles = (max_block_bytes + kChainMinTileBytes - 1) / kChainMinTileBytes;
+  return chain_scratch_for(as_stream(stream), tiles, true, cs);
+}
+
+int alamd_release_scratch(void *stream) {
+  int dev = 0;
+  ALAMD_HIP(hipGetDevice(&dev));
+  ALAMD_HIP(hipStreamSynchronize(as_stream(stream)));
+  ChainPool &pool = chain_pool();
+  std::lock_guard<std::mutex> lock(pool.mutex);
+  const auto key = std::make_pair(dev, as_stream(stream));
+  auto it = pool.live.find(key);
+  if (it != pool.live.end()) {
+    ALAMD_HIP(hipFree(it->second.ticket));
+    pool.live.erase(it);
+  }
+  auto old = pool.retired.find(key);
+  if (old != pool.retired.end()) {
+    for (void *mem : old->second) ALAMD_HIP(hipFree(mem));
+    pool.retired.erase(old);
+  }
   return ALAMD_OK;
 }
 

@@ -35,7 +35,7 @@ Tunables &tunables() {
 namespace {
 // least: the pieces of a two-step call at least 64 KiB (smaller ones would turn one call into millions
 // of launches; less than one element, into a loop that never ends)
-struct TunableName { const char *name; size_t Tunables::*field; size_t least; };
+struct TunableName { const char *name; std::atomic<size_t> Tunables::*field; size_t least; };
 const TunableName kTunableNames[] = {
     {"launch_bytes", &Tunables::launch_bytes, 1},
     {"two_step_min_total_bytes", &Tunables::two_step_min_total_bytes, 1},
@@ -47,6 +47,7 @@ const TunableName kTunableNames[] = {
     {"spread_hbm_launch_chunks", &Tunables::spread_hbm_launch_chunks, 1},
     {"spread_cache_chunk_tiles", &Tunables::spread_cache_chunk_tiles, 1},
     {"spread_cache_launch_chunks", &Tunables::spread_cache_launch_chunks, 1},
+    {"halo_load_policy", &Tunables::halo_load_policy, 0},
 };
 }  // namespace
 
@@ -116,7 +117,7 @@ int alamd_tune(const char *name, size_t value) {
     if (std::string(name) == t.name) {
       if (value != 0 && value < t.least)
         return alamd::set_error(ALAMD_ERR_INVALID_ARG, "%s must be at least %zu (0 restores the default)", name, t.least);
-      alamd::tunables().*(t.field) = value ? value : defaults.*(t.field);
+      (alamd::tunables().*(t.field)).store(value ? value : (defaults.*(t.field)).load());
       return ALAMD_OK;
     }
   return alamd::set_error(ALAMD_ERR_INVALID_ARG, "no launch-planner size is called %s", name);
@@ -125,7 +126,7 @@ int alamd_tune(const char *name, size_t value) {
 size_t alamd_tuned(const char *name) {
   if (name)
     for (const auto &t : alamd::kTunableNames)
-      if (std::string(name) == t.name) return alamd::tunables().*(t.field);
+      if (std::string(name) == t.name) return (alamd::tunables().*(t.field)).load();
   return 0;
 }
 

@@ -70,7 +70,22 @@ template <int UB> __device__ __forceinline__ void store_through(char *p, typenam
   else asm volatile("global_store_byte %0, %1, off sc0 sc1" ::"v"(p), "v"((uint32_t)v) : "memory");
 }
 
-template <int UB, bool PACK>
+// The grid loads of a pack under another cache policy (16-byte units only; Tunables::halo_load_policy, a
+// measurement setting).  An x face needs 16 bytes of every 128-byte line it touches, so a policy under
+// which the L2 asked memory for 32- or 64-byte sectors instead of whole lines would cut its traffic.  None
+// does: under every policy below every read request that leaves the L2 is 128 bytes (329 k requests for
+// both x faces, 462 k for all six, none of 32 bytes, 352 of 64), and the times are the same within 1 %
+// (nt: +20 % on the six-face launch).  The plain load stays.
+template <int LP> __device__ __forceinline__ u32x4 load_policy(const char *p) {
+  u32x4 v;
+  if constexpr (LP == 1) asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(v) : "v"(p) : "memory");
+  else if constexpr (LP == 2) asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+  else if constexpr (LP == 3) asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+  else asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1 nt" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+
+template <int UB, bool PACK, int LP = 0>
 __global__ void __launch_bounds__(kThreads) halo_kernel(const HaloParams p) {
   using Unit = typename unit_of<UB>::type;
   constexpr int U = kPasses;
@@ -104,9 +119,16 @@ __global__ void __launch_bounds__(kThreads) halo_kernel(const HaloParams p) {
            (unsigned long long)c1 * UB + (second ? f.delta2 : 0u);
     b[u] = (second ? f.buf2 : f.buf) + ((unsigned long long)r * f.upr + c1) * UB;
   }
+  if constexpr (LP > 0 && UB == 16 && PACK) {
 #pragma unroll
-  for (int u = 0; u < U; ++u)
-    if (ok[u]) v[u] = *reinterpret_cast<const Unit *>(PACK ? g[u] : b[u]);
+    for (int u = 0; u < U; ++u)
+      if (ok[u]) v[u] = load_policy<LP>(g[u]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the compiler does not count loads made by asm statements
+  } else {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (ok[u]) v[u] = *reinterpret_cast<const Unit *>(PACK ? g[u] : b[u]);
+  }
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (ok[u]) {
@@ -190,7 +212,13 @@ int halo_launch(void *grid, void *const bufs[6], const size_t dims[3], size_t ha
   }
   void (*kern)(const HaloParams) = nullptr;
   switch (unit) {
-  case 16: kern = pack ? halo_kernel<16, true> : halo_kernel<16, false>; break;
+  case 16: {
+    const size_t lp = tunables().halo_load_policy;
+    kern = !pack ? halo_kernel<16, false>
+           : lp == 1 ? halo_kernel<16, true, 1> : lp == 2 ? halo_kernel<16, true, 2> : lp == 3 ? halo_kernel<16, true, 3>
+           : lp == 4 ? halo_kernel<16, true, 4> : halo_kernel<16, true>;
+    break;
+  }
   case 8: kern = pack ? halo_kernel<8, true> : halo_kernel<8, false>; break;
   case 4: kern = pack ? halo_kernel<4, true> : halo_kernel<4, false>; break;
   case 2: kern = pack ? halo_kernel<2, true> : halo_kernel<2, false>; break;

@@ -25,7 +25,7 @@ WORKLOADS = {
     # name: (dtype, count per rank, op, dist, seed base, order)
     "c2_f32_sum": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "rank_asc"),
     "c2_f32_prod": ("f32", 1 << 26, "prod", "uniform_09_11", 1000, "rank_asc"),
-    "c2_f32_sum_tree": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "tree_dbl"),
+    "c2_f32_sum_tree": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "tree_rsg"),
     "c2_bf16_sum": ("bf16", 1 << 27, "sum", "normal", 2000, "rank_asc"),
     "c4_i32_max": ("i32", 1 << 28, "max", "fullrange", 3000, "rank_asc"),
     "c4_i64_bxor": ("i64", 1 << 28, "bxor", "fullrange", 3000, "rank_asc"),
@@ -53,7 +53,7 @@ KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false /*o
 # Every configuration of the headline benchmark beside the primary workload: C2 in the tree order, prod and bf16, the same over
 # buffers no earlier call has touched, C4 (integer / bitwise / logical), C3 (ring, both modes), C5 (halo
 # faces), the stream flags, and the layouts an Allreduce / Reduce_scatter / Allgather reaches the kernels in.
-DEFAULT_ALSO = ("c2_f32_sum_rotating,c2_f32_sum_tree,c2_f32_prod,c2_bf16_sum,c2_bf16_sum_rotating,c4_i32_max,c4_i64_bxor,"
+DEFAULT_ALSO = ("c2_sum_rotating_pair,c2_f32_sum_tree,c2_f32_prod,c2_bf16_sum,c4_i32_max,c4_i64_bxor,"
                 "c4_u8_lxor,c3_ring_stepwise,c3_ring_fused,c5_halo,flags,c2_f32_allreduce,"
                 "c2_f32_allreduce_rotating,c2_f32_reduce_scatter,c2_f32_reduce_scatter_rotating,"
                 "c2_f32_allgather,c2_f32_allgather_rotating,c2_f32_reduce_scatterv_in_place")
@@ -74,6 +74,113 @@ def measured_traffic(workload):
     if not m:
         return None, "%s holds no 'B per call' line" % rel
     return int(m.group(2)), "%s (sha1 %s)" % (rel, hashlib.sha1(text.encode()).hexdigest()[:12])
+
+
+def halo_traffic():
+    """((bytes the six-face pack moves, bytes the six-face unpack moves), source) out of the committed counter
+    profile of the halo kernel, or (None, why)."""
+    import hashlib
+    import re
+    rel = "profiles/halo_kernel_f64_c5.md"
+    try:
+        text = open(os.path.join(ROOT, rel)).read()
+    except OSError:
+        return None, "%s is missing" % rel
+    m = re.search(r"Pack:.*?In all (\d+) B", text, re.S)
+    n = re.search(r"Unpack:.*?; (\d+) B", text, re.S)
+    if not (m and n):
+        return None, "%s holds no byte totals" % rel
+    return (int(m.group(1)), int(n.group(1))), "%s (sha1 %s)" % (rel, hashlib.sha1(text.encode()).hexdigest()[:12])
+
+
+def run_pair_workload(al, torch, steps, warmup):
+    """C2 as fp32 and as bf16 over the SAME memory: four rotating sets of eight 256 MiB buffers plus an output
+    (9 GiB in all, so nothing a call touches was touched by the three calls before it), filled once with
+    bf16 normal(0,1) values and read as 2^27 bf16 or as 2^26 fp32 elements, the two taking turns.  Where the
+    buffers lie in HBM moves a rate by up to 3 points from one allocation to the next; measured this way the
+    difference between the two types is the kernels' alone."""
+    import numpy as np
+    import oracle
+    nbytes = 256 << 20
+    raw = []
+    for _ in range(4):
+        ins = [torch.empty(nbytes // 2, dtype=torch.int16, device="cuda") for _ in range(P)]
+        out = torch.empty(nbytes // 2, dtype=torch.int16, device="cuda")
+        for r in range(P):
+            al.fill(ins[r], "normal", 2000 + r, dtype="bf16")
+        raw.append((ins, out))
+    views = {"f32": torch.float32, "bf16": torch.int16}
+    calls = {dt: [lambda ins=ins, out=out, dt=dt, v=v: al.combine([out.view(v)], [t.view(v) for t in ins], "sum",
+                                                                  order="rank_asc", dtype=dt) for ins, out in raw]
+             for dt, v in views.items()}
+    # parity: both views of the first and last 2^18 bytes of every set against the oracle's fold of the same bytes
+    ok, m = True, 1 << 18
+    for dt in views:
+        np_dt = oracle.NP_CARRIER[dt]
+        for k, (ins, out) in enumerate(raw):
+            calls[dt][k]()
+            torch.cuda.synchronize()
+            for lo in (0, nbytes - m):
+                host = [t.view(torch.uint8)[lo:lo + m].cpu().numpy().view(np_dt) for t in ins]
+                want = oracle.combine(host, dt, "sum", "rank_asc")
+                got = out.view(torch.uint8)[lo:lo + m].cpu().numpy().view(np_dt)
+                ok = ok and got.tobytes() == want.tobytes()
+    alg = (P + 1) * nbytes
+    rates = {dt: [] for dt in views}
+    turn = {dt: 0 for dt in views}
+    for _ in range(5):
+        for dt in views:
+            def step(dt=dt):
+                calls[dt][turn[dt] % 4]()
+                turn[dt] += 1
+            _, kms = timed(torch, step, steps, max(4, warmup))
+            rates[dt].append(alg / (kms * 1e-3) * 1e-9)
+    med = {dt: sorted(r)[len(r) // 2] for dt, r in rates.items()}
+    diffs = sorted(b - a for a, b in zip(rates["f32"], rates["bf16"]))
+    return {"workload": "c2_sum_rotating_pair", "P": P, "bytes_per_buffer": nbytes, "buffer_sets": 4, "op": "sum",
+            "order": "rank_asc", "algorithmic_bytes": alg, "rounds": 5,
+            "gbps_kernel_f32": med["f32"], "gbps_kernel_bf16": med["bf16"],
+            "frac_f32": med["f32"] / HBM_PEAK_GBPS, "frac_bf16": med["bf16"] / HBM_PEAK_GBPS,
+            "bf16_minus_f32_gbps_median_of_paired": diffs[len(diffs) // 2], "parity_vs_oracle": bool(ok)}
+
+
+def run_halo_policy_workload(al, torch, steps, warmup):
+    """The pack of both x faces, and of all six faces, of the C5 grid with the grid loads under each cache
+    policy the library can be set to (a measurement: see alamd_tune, halo_load_policy)."""
+    import ctypes as C
+    n, h = 512, 2
+    dims, side = (n, n, n), n + 2 * h
+    grid = torch.empty(side ** 3, dtype=torch.float64, device="cuda")
+    al.fill(grid, "uniform_01", 4000)
+    bufs = {f: torch.empty(al.halo_face_elems(dims, h, f), dtype=torch.float64, device="cuda") for f in range(6)}
+    L = al.load()
+    tab = (C.c_void_p * 6)(*[bufs[f].data_ptr() for f in range(6)])
+    cdims = (C.c_size_t * 3)(*dims)
+    gp = C.c_void_p(grid.data_ptr())
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def pack(mask):
+        assert L.alamd_halo_pack(tab, gp, cdims, h, 8, mask, st) == 0
+
+    pack(0x3f)
+    torch.cuda.synchronize()
+    ref = {f: bufs[f].clone() for f in range(6)}
+    names = ["plain", "nt", "sc1", "sc0 sc1", "sc0 sc1 nt"]
+    res = {"workload": "c5_halo_load_policy", "dtype": "f64", "policies": {}}
+    try:
+        for lp, name in enumerate(names):
+            al.tune("halo_load_policy", lp)
+            _, kx = timed(torch, lambda: pack(3), steps, warmup)
+            _, ka = timed(torch, lambda: pack(0x3f), steps, warmup)
+            for f in range(6):
+                bufs[f].zero_()
+            pack(0x3f)
+            torch.cuda.synchronize()
+            res["policies"][name] = {"pack_x_pair_us": kx * 1e3, "pack_all_us": ka * 1e3,
+                                     "same_bytes_as_plain": all(bool(torch.equal(bufs[f], ref[f])) for f in range(6))}
+    finally:
+        al.tune("halo_load_policy", 0)
+    return res
 
 
 def run_combine_workload(al, torch, name, steps, warmup, check=True):
@@ -106,7 +213,7 @@ def run_combine_workload(al, torch, name, steps, warmup, check=True):
     alg_bytes = (P + 1) * count * es
     res = {
         "workload": name, "dtype": dtype, "op": op, "order": order, "P": P, "count": count,
-        "buffer_sets": nsets, "launches_per_step": -(-(count * es) // (4096 * 16384)),
+        "buffer_sets": nsets, "launches_per_step": al.planned_launches(P, count, dtype),
         "algorithmic_bytes": alg_bytes, "ms_per_step": wall * 1e3 / steps, "kernel_ms": kernel_ms,
         "gbps_wall": alg_bytes / (wall / steps) * 1e-9, "gbps_kernel": alg_bytes / (kernel_ms * 1e-3) * 1e-9,
     }
@@ -173,9 +280,7 @@ def run_ring_workload(al, torch, mode, steps, warmup):
     # P-1 allgather steps reads one and writes one; fused: every buffer is read once and written once
     alg = 5 * (P - 1) * count * es if mode == "stepwise" else 2 * P * count * es
     return {"workload": "c3_ring_" + mode, "dtype": dtype, "op": "sum", "P": P, "count": count,
-            "chunk_bytes": chunk, "launches_per_step": 2 * (P - 1) if mode == "stepwise" else None,  # fused: a fold pass and a spread
-            # pass per 256 MiB piece, each cut into launches by the planner
-            "algorithmic_bytes": alg, "ms_per_step": wall * 1e3, "kernel_ms": kms,
+            "chunk_bytes": chunk, "algorithmic_bytes": alg, "ms_per_step": wall * 1e3, "kernel_ms": kms,
             "gbps_wall": alg / wall * 1e-9, "gbps_kernel": alg / (kms * 1e-3) * 1e-9,
             "parity_vs_oracle": bool(ok)}
 
@@ -187,7 +292,7 @@ LAYOUTS.append("c2_f32_reduce_scatterv_in_place")
 def run_layout_workload(al, torch, name, steps, warmup):
     """The two write-heavy layouts at the C2 shape (P = 8 fp32 ranks, seed 1000+rank):
     c2_f32_allreduce - the combine delivered to all eight ranks' receive buffers (8 reads + 8 writes of
-    2^26 elements, order tree_dbl: what Al::Allreduce yields above 2 KiB);
+    2^26 elements, order tree_rsg: what Al::Allreduce yields above 2 KiB);
     c2_f32_allgather - eight slices of 2^23 elements gathered into eight receive buffers of 2^26
     (each slice read once, written eight times);
     c2_f32_reduce_scatter - eight send buffers of 2^26 elements, block b folded into receive buffer b of
@@ -210,13 +315,14 @@ def run_layout_workload(al, torch, name, steps, warmup):
             outs = [torch.empty(count, dtype=torch.float32, device="cuda") for _ in range(P)]
             for r in range(P):
                 al.fill(ins[r], "uniform_pm1", 1000 + r)
-            fn = lambda ins=ins, outs=outs: al.combine(outs, ins, "sum", order="tree_dbl")
+            fn = lambda ins=ins, outs=outs: al.combine(outs, ins, "sum", order="tree_rsg")
             alg = 2 * P * count * 4
-            launches = count * 4 // (64 << 20) + count * 4 // (32 << 20)
             fn()
             torch.cuda.synchronize()
             for j in (0, P - 1):
                 for lo in (0, count - m):
+                    # (for a sum the reduce-scatter + gather order gives the bits of the doubling tree
+                    # wherever the element lies, so a slice can be checked on its own)
                     want = oracle.combine_generated(P, m, "f32", "sum", "tree_dbl", 0, "uniform_pm1", 1000, lo)
                     ok = ok and outs[j][lo:lo + m].cpu().numpy().tobytes() == want.tobytes()
         elif base == "c2_f32_reduce_scatter":
@@ -228,7 +334,6 @@ def run_layout_workload(al, torch, name, steps, warmup):
             fn = lambda sends=sends, recvs=recvs: al.reduce_scatter(recvs, sends, "sum", order="pairwise_desc",
                                                                     count=count)
             alg = (P + 1) * P * count * 4
-            launches = P * count * 4 // (64 << 20)
             fn()
             torch.cuda.synchronize()
             for b in (0, P - 1):
@@ -244,7 +349,6 @@ def run_layout_workload(al, torch, name, steps, warmup):
                 al.fill(sends[r], "uniform_pm1", 1000 + r)
             fn = lambda sends=sends, recvs=recvs: al.allgather(recvs, sends, count=count)
             alg = (P + P * P) * count * 4
-            launches = P
             fn()
             torch.cuda.synchronize()
             for j in (0, P - 1):
@@ -261,7 +365,6 @@ def run_layout_workload(al, torch, name, steps, warmup):
             fn = lambda bufs=bufs, counts=counts: al.reduce_scatterv(bufs, bufs, counts, "sum",
                                                                      order="pairwise_desc", dtype="f32")
             alg = (P + 1) * count * 4
-            launches = 3  # the one-element block, the clearing of the tile flags, the chained fold
             fn()  # later calls fold what this one left: the same traffic, other values
             torch.cuda.synchronize()
             for lo in (0, count - 1 - m):
@@ -276,7 +379,7 @@ def run_layout_workload(al, torch, name, steps, warmup):
         fns[turn[0] % len(fns)]()
         turn[0] += 1
     wall, kms = timed(torch, step, steps, warmup)
-    return {"workload": name, "dtype": "f32", "op": "sum", "P": P, "count": count, "launches_per_step": launches,
+    return {"workload": name, "dtype": "f32", "op": "sum", "P": P, "count": count,
             "buffer_sets": len(fns), "algorithmic_bytes": alg, "ms_per_step": wall * 1e3, "kernel_ms": kms,
             "gbps_wall": alg / wall * 1e-9, "gbps_kernel": alg / (kms * 1e-3) * 1e-9, "parity_vs_oracle": bool(ok)}
 
@@ -328,9 +431,11 @@ def run_halo_workload(al, torch, steps, warmup):
     # what the six-face launches really move (one 128-byte line per 16-byte run of an x face, 1.26 lines
     # per row when both x faces go together; ghost runs written as 32-byte pieces): from the counter
     # profile profiles/halo_kernel_f64_c5.md
-    res["pack_all_hbm_bytes"], res["unpack_all_hbm_bytes"] = 84243968, 59262464
-    res["pack_all_hbm_gbps"] = res["pack_all_hbm_bytes"] / (kms * 1e-3) * 1e-9
-    res["unpack_all_hbm_gbps"] = res["unpack_all_hbm_bytes"] / (kms2 * 1e-3) * 1e-9
+    hbm, res["hbm_bytes_source"] = halo_traffic()
+    if hbm:
+        res["pack_all_hbm_bytes"], res["unpack_all_hbm_bytes"] = hbm
+        res["pack_all_hbm_gbps"] = hbm[0] / (kms * 1e-3) * 1e-9
+        res["unpack_all_hbm_gbps"] = hbm[1] / (kms2 * 1e-3) * 1e-9
     for f, name in enumerate(("-x", "+x", "-y", "+y", "-z", "+z")):
         _, k1 = timed(torch, lambda: pack(1 << f), steps, warmup)
         _, k2 = timed(torch, lambda: unpack(1 << f), steps, warmup)
@@ -406,7 +511,8 @@ def c1_gpu_checksum(al, torch):
     out = torch.empty(n, dtype=torch.float32, device="cuda")
     for r in range(ranks):
         al.fill(ins[r], "uniform_pm1", 1000 + r)
-    al.combine([out], ins, "sum", order="tree_dbl")
+    order, start = al.reference_order("allreduce", ranks, n, "f32")
+    al.combine([out], ins, "sum", order=order, start=start)
     torch.cuda.synchronize()
     return "%016x" % oracle.checksum(out.cpu().numpy())
 
@@ -420,7 +526,7 @@ def c1_gpu_time(al, torch):
     outs = [torch.empty(n, dtype=torch.float32, device="cuda") for _ in range(ranks)]
     for r in range(ranks):
         al.fill(ins[r], "uniform_pm1", 1000 + r)
-    call = lambda: al.combine(outs, ins, "sum", order="tree_dbl")
+    call = lambda: al.combine(outs, ins, "sum", order="tree_rsg")
     for _ in range(10):
         call()
     torch.cuda.synchronize()
@@ -512,7 +618,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2_f32_sum",
-                    choices=sorted(WORKLOADS) + ["c3_ring_stepwise", "c3_ring_fused", "c5_halo", "flags"] + LAYOUTS)
+                    choices=sorted(WORKLOADS) + ["c3_ring_stepwise", "c3_ring_fused", "c5_halo", "c5_halo_load_policy",
+                                                 "flags", "c2_sum_rotating_pair"] + LAYOUTS)
     ap.add_argument("--also", default=DEFAULT_ALSO,
                     help="comma-separated extra workloads reported under 'also' ('' for none)")
     ap.add_argument("--batch", default="",
@@ -543,6 +650,10 @@ def main():
             res = run_ring_workload(al, torch, name[len("c3_ring_"):], steps, warmup)
         elif name == "c5_halo":
             res = run_halo_workload(al, torch, steps, warmup)
+        elif name == "c5_halo_load_policy":
+            res = run_halo_policy_workload(al, torch, steps, warmup)
+        elif name == "c2_sum_rotating_pair":
+            res = run_pair_workload(al, torch, steps, warmup)
         elif name == "flags":
             res = run_flag_workload()
         elif name in LAYOUTS:
@@ -585,8 +696,7 @@ def main():
         line = [l for l in p.stdout.splitlines() if l.startswith("{")]
         also = json.loads(line[-1]) if p.returncode == 0 and line else {"error": p.stderr[-300:]}
     traffic, traffic_source = measured_traffic(args.workload)
-    untouched = {k: also[k]["frac"] for k in ("c2_f32_sum_rotating", "c2_bf16_sum_rotating")
-                 if isinstance(also.get(k), dict) and "frac" in also[k]}
+    pair = also.get("c2_sum_rotating_pair") if isinstance(also.get("c2_sum_rotating_pair"), dict) else {}
 
     out = {
         "metric": METRIC, "value": main_res["gbps_wall"], "unit": "GB/s", "n_gpus": 1,
@@ -603,9 +713,10 @@ def main():
         "roofline": {"bound": "hbm", "achieved": main_res["gbps_kernel"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": main_res["gbps_kernel"] / HBM_PEAK_GBPS,
                      # the same kernel over four rotating buffer sets: nothing a call reads or writes was
-                     # touched by the three calls before it, so the 256 MiB memory-side cache cannot help
-                     "frac_untouched": untouched.get("c2_f32_sum_rotating"),
-                     "frac_untouched_bf16": untouched.get("c2_bf16_sum_rotating"),
+                     # touched by the three calls before it, so the 256 MiB memory-side cache cannot help;
+                     # fp32 and bf16 read the same memory, taking turns (also.c2_sum_rotating_pair)
+                     "frac_untouched": pair.get("frac_f32"),
+                     "frac_untouched_bf16": pair.get("frac_bf16"),
                      # HBM bytes (fetched + written) per call and per launch, read from the committed
                      # counter profile, not measured by this run
                      "traffic": traffic,
@@ -613,7 +724,7 @@ def main():
                      "traffic_source": traffic_source,
                      "kernel": KERNEL_NAME.get(args.workload, "alamd::fold_vec_kernel"),
                      "kernel_ms": main_res["kernel_ms"],
-                     # one call is cut into launches of at most 4096 tiles of 16 KiB per stream
+                     # the launches one call is cut into, as the library's planner reports them
                      "launches_per_step": main_res["launches_per_step"],
                      "launch_avg_us": main_res["kernel_ms"] * 1e3 / main_res["launches_per_step"],
                      "algorithmic_bytes_per_launch": main_res["algorithmic_bytes"] // main_res["launches_per_step"],

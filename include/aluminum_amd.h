@@ -5,8 +5,11 @@
  * C ABI.  No C++ or HIP types cross this boundary: streams are passed as
  * `void *` (a hipStream_t; NULL is the default stream), buffers as device
  * pointers.  Every call that takes a stream only enqueues work on it and
- * returns; buffers are caller-owned and must stay valid until the stream has
- * passed the call (reference contract: docs/comm.rst:18, docs/index.rst:33-40).
+ * returns (the set-up calls alamd_reserve_scratch / alamd_release_scratch
+ * aside; the one collective that may need memory of the library's own says so:
+ * alamd_reduce_scatterv); buffers are caller-owned and must stay valid until
+ * the stream has passed the call (reference contract: docs/comm.rst:18,
+ * docs/index.rst:33-40).
  * Calls return ALAMD_OK or a small positive status code; the message of
  * the last error on the calling thread is alamd_last_error().  The library is
  * thread-compatible: concurrent calls are fine as long as they do not share a
@@ -69,7 +72,10 @@ typedef enum {
  * ALAMD_SUM, followed by one division by the number of ranks P in the element
  * type's own arithmetic: IEEE division for fp32 / fp64; for fp16 / bf16 the
  * sum is widened, divided in fp32 and narrowed round-to-nearest-even; for the
- * integer types C division, which truncates toward zero. */
+ * integer types C division, which truncates toward zero.  Parity unpinned: the
+ * reference holds no values for avg, and the library its NCCL backend hands it
+ * to may scale every contribution by 1/P before summing instead, so float
+ * results need not agree with Al::NCCLBackend bit for bit. */
 typedef enum {
   ALAMD_SUM = 0, ALAMD_PROD = 1, ALAMD_MIN = 2, ALAMD_MAX = 3, ALAMD_LOR = 4,
   ALAMD_LAND = 5, ALAMD_LXOR = 6, ALAMD_BOR = 7, ALAMD_BAND = 8, ALAMD_BXOR = 9,
@@ -139,10 +145,14 @@ size_t alamd_dtype_size(int dtype);
  * MPI defines the logical and bitwise ops for integers only; avg for every
  * type, see alamd_op). */
 int alamd_check_op(int dtype, int op);
-/* Selects nothing and allocates nothing; checks that the current device is a
- * gfx950 and caches its compute-unit count.  Optional: every entry point
- * performs it on first use.  (Replaces internal::cuda::init,
- * src/cuda/cuda.cpp:52-78.) */
+/* Set-up for the current device, once per device (calling it again is cheap):
+ * checks that the device is a gfx950, caches its compute-unit count, allocates
+ * one line of pinned host memory (where a bounded wait that gives up leaves
+ * its mark, see alamd_reduce_scatterv_wait_expired), looks up the address of
+ * the fixed scratch array of alamd_reduce_scatterv_noalloc and creates the
+ * event that guards it.  Required before alamd_reduce_scatterv_noalloc, which
+ * may not allocate; every other entry point works without it.  (Replaces
+ * internal::cuda::init, src/cuda/cuda.cpp:52-78.) */
 int alamd_init(void);
 
 /* The order (and its start rank) under which the reference's result comes
@@ -206,13 +216,31 @@ int alamd_allgather(void *const *recvs, const void *const *sends, int P,
  * buffer than it is long is read and overwritten at a displacement: in two
  * launches no longer than the displacement where they suffice, else in one
  * launch whose workgroups order themselves through a ticket counter and one
- * flag per tile in device scratch memory (allocated per stream on first need
- * and kept).
+ * flag per tile in device scratch memory of the library's own, kept per
+ * stream.  That scratch is the one thing a collective here may have to
+ * allocate: the first such launch on a stream calls hipMalloc (4 bytes per
+ * 4 KiB of the block, at least 256 KiB) unless alamd_reserve_scratch has been
+ * called for the stream; a stream that is being captured into a graph never
+ * allocates, and the call then fails with ALAMD_ERR_INVALID_ARG if nothing was
+ * reserved.  Everything the launch needs cleared is cleared by a small kernel
+ * on the stream itself.
  * Replaces MPI_Ireduce_scatter on the host copy
  * (include/aluminum/ht/reduce_scatterv.hpp:40-87). */
 int alamd_reduce_scatterv(void *const *recvs, const void *const *sends, int P,
                           const size_t *counts, int dtype, int op, int order,
                           void *stream);
+
+/* Set-up calls, not stream-ordered work.  alamd_reserve_scratch makes sure that
+ * `stream` (on the current device) owns scratch for in-place Reduce_scatterv
+ * blocks of up to max_block_bytes that overlap their own input, allocating it
+ * now if need be, so that no later alamd_reduce_scatterv on that stream
+ * allocates and the call can be captured into a graph.  alamd_release_scratch
+ * synchronises the stream and frees what it holds (call it before destroying a
+ * stream whose scratch should not outlive it).  No counterpart in the
+ * reference, whose host-transfer backend draws staging memory from a pool
+ * (include/aluminum/mempool.hpp) inside the call. */
+int alamd_reserve_scratch(void *stream, size_t max_block_bytes);
+int alamd_release_scratch(void *stream);
 
 /* The waits inside a chained in-place launch (see alamd_reduce_scatterv) are
  * bounded, so that a device that loses a workgroup cannot hang the stream; a
@@ -235,9 +263,14 @@ int alamd_reduce_scatterv_wait_expired(void);
  * such a block may be at most ALAMD_NOALLOC_MAX_BLOCK_BYTES long unless it
  * starts at least a 32nd of its length into its buffer (then up to 32 plain
  * launches do; ALAMD_ERR_INVALID_ARG otherwise; blocks that do not overlap their own
- * input, and separate receive buffers, have no limit).  All calls on one device
- * share the array: calls that overlap in time on one device (different
- * streams, different threads) race; keep them on one stream. */
+ * input, and separate receive buffers, have no limit).  alamd_init must have
+ * run on the device (ALAMD_ERR_INVALID_ARG otherwise): it looks the array up.
+ * All calls on one device share the array, which keeps the last call's
+ * contents (every call clears what it uses): calls that overlap in time on one
+ * device would race, so keep them on one stream.  A call made on another
+ * stream while the last chained launch that used the array is still running is
+ * refused (ALAMD_ERR_INVALID_ARG); launches recorded into a graph are not
+ * tracked that way, and what runs beside a replay is the caller's to order. */
 #define ALAMD_NOALLOC_SCRATCH_BYTES ((size_t)1 << 20)
 #define ALAMD_NOALLOC_MAX_BLOCK_BYTES (((ALAMD_NOALLOC_SCRATCH_BYTES - 256) / 4) * 4096)
 int alamd_reduce_scatterv_noalloc(void *const *recvs, const void *const *sends, int P,

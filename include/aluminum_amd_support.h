@@ -36,17 +36,31 @@ int alamd_fill(void *dst, size_t count, int dtype, int dist, uint64_t seed,
 int alamd_narrow_f32(void *dst16, const float *src, size_t count, int dtype, void *stream);
 int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void *stream);
 /* The sizes the launch planners cut their work by, for comparisons on a given
- * machine (not thread-safe against running calls; value 0 restores the
- * default): launch_bytes, two_step_min_total_bytes, two_step_min_outputs,
+ * machine (they exist for measurements, not for production code).  The
+ * settings are process-wide atomics: a call that runs while one changes sees
+ * the old or the new value of each.  Value 0 restores the default.  Names:
+ * launch_bytes, two_step_min_total_bytes, two_step_min_outputs,
  * two_step_piece_bytes, ring_piece_bytes, spread_launch_bytes,
  * spread_hbm_chunk_tiles, spread_hbm_launch_chunks, spread_cache_chunk_tiles,
- * spread_cache_launch_chunks.  Piece sizes below 64 KiB are refused.
- * Results never depend on them, only speed. */
+ * spread_cache_launch_chunks; halo_load_policy (the cache policy of the grid
+ * loads of a halo pack: 0 plain, 1 nt, 2 sc1, 3 sc0 sc1, 4 sc0 sc1 nt).  Piece
+ * sizes below 64 KiB are refused.  Results never depend on them, only speed. */
 int alamd_tune(const char *name, size_t value);
 size_t alamd_tuned(const char *name);
+/* The number of kernel launches that alamd_combine makes for one output of
+ * `count` elements folded from P ranks under a fold order (the launch planner's
+ * own answer under the current settings; 0 for arguments it would refuse), so
+ * that a benchmark can turn a call's duration into a launch's. */
+size_t alamd_planned_launches(int P, size_t count, int dtype);
 /* Polls after which a wait inside a chained in-place Reduce_scatterv launch
  * gives up (0 restores the default, 2^24): lets a test make waits expire
- * without anything being wrong with the device. */
+ * without anything being wrong with the device.  ALAMD_CHAIN_POLLS_NONE: every
+ * wait that the tiling calls for gives up without looking at its flag, whether
+ * the neighbouring tile has loaded or not - the same outcome on every device
+ * and at every speed; every kernel still runs to its end.  Not synchronised
+ * against running calls, like alamd_tune: a test's setting, made while
+ * nothing else uses the library. */
+#define ALAMD_CHAIN_POLLS_NONE 0xffffffffu
 int alamd_set_chain_poll_limit(unsigned polls);
 #ifdef __cplusplus
 }

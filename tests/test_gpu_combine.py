@@ -505,29 +505,30 @@ def test_collectives_in_a_hip_graph(al):
 
 
 def test_reduce_scatterv_chained_wait_that_gives_up_is_reported(al):
-    """The waits inside a chained in-place launch are bounded.  With the bound set to a single poll
-    (a hook for this test; nothing is wrong with the device and every kernel ends normally) some tile
-    finds its neighbour's loads not yet done and gives up: the result of that call is not valid, the
-    query says so once, and so does the next Reduce_scatterv, after which everything works again."""
+    """The waits inside a chained in-place launch are bounded.  With the test's setting under which every
+    wait that the tiling calls for gives up without looking at its flag (nothing is wrong with the device,
+    every kernel ends normally, and the outcome does not depend on how fast anything runs) the result of
+    the call is not valid: the query says so once, and a Reduce_scatterv that follows an unreported expiry
+    refuses with ALAMD_ERR_TIMEOUT, after which everything works again."""
     import torch
     P, counts = 4, [1, 6_000_000, 3, 0]
     sends = make_inputs(P, sum(counts), "f32", "sum")
     want = oracle.reduce_scatterv(sends, counts, "f32", "sum", "rank_asc")
     assert not al.reduce_scatterv_wait_expired()
     try:
-        al.set_chain_poll_limit(1)
+        al.set_chain_poll_limit(al.CHAIN_POLLS_NONE)
         bufs = [to_dev(a) for a in sends]
         al.reduce_scatterv(bufs, bufs, counts, "sum", order="rank_asc", dtype="f32")
         torch.cuda.synchronize()
-        assert al.reduce_scatterv_wait_expired(), "no wait gave up although one poll was all they had"
+        assert al.reduce_scatterv_wait_expired(), "no wait gave up although none was allowed a poll"
         assert not al.reduce_scatterv_wait_expired(), "reported once only"
         bufs = [to_dev(a) for a in sends]
-        al.reduce_scatterv(bufs, bufs, counts, "sum", order="rank_asc", dtype="f32")
+        al.reduce_scatterv(bufs, bufs, counts, "sum", order="rank_asc", dtype="f32")  # expires again, not queried
         torch.cuda.synchronize()
     finally:
         al.set_chain_poll_limit(0)
     bufs = [to_dev(a) for a in sends]
-    with pytest.raises(al.AlError, match="gave up waiting") as e:  # the second call's waits gave up as well
+    with pytest.raises(al.AlError, match="gave up waiting") as e:  # the next call reports it instead of running
         al.reduce_scatterv(bufs, bufs, counts, "sum", order="rank_asc", dtype="f32")
     assert e.value.code == 7
     al.reduce_scatterv(bufs, bufs, counts, "sum", order="rank_asc", dtype="f32")
@@ -535,6 +536,55 @@ def test_reduce_scatterv_chained_wait_that_gives_up_is_reported(al):
     assert not al.reduce_scatterv_wait_expired()
     for b in range(P):
         assert_bits_equal(to_host(bufs[b], np.float32)[:counts[b]], want[b], "f32", "after the report, rank %d" % b)
+
+
+def test_reduce_scatterv_captured_without_a_warm_up(al):
+    """An in-place Reduce_scatterv whose block overlaps its own input, captured into a HIP graph on a stream
+    that has never run one: the library may not allocate under capture, so without a reservation the call
+    is refused with a message that names the remedy, and with alamd_reserve_scratch made beforehand the
+    capture succeeds cold and every replay gives the oracle's bits."""
+    import torch
+    P, counts = 3, [1, 2_000_003, 7]
+    total = sum(counts)
+    src = [dev_empty(total, np.float32) for _ in range(P)]
+    work = [dev_empty(total, np.float32) for _ in range(P)]
+
+    def run():
+        for r in range(P):
+            al.copy(work[r], src[r])
+        al.reduce_scatterv(work, work, counts, "sum", order="pairwise_desc", dtype="f32")
+
+    cold = torch.cuda.Stream()
+    with pytest.raises(al.AlError, match="alamd_reserve_scratch") as e:
+        g0 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g0, stream=cold):
+            run()
+    assert e.value.code == 1
+    torch.cuda.synchronize()
+    del g0
+
+    s = torch.cuda.Stream()
+    al.reserve_scratch(counts[1] * 4, stream=s.cuda_stream)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        run()  # first ever call on this stream: nothing allocated, nothing synchronised
+    for rep in range(3):
+        fresh = [oracle.fill(total, "f32", "uniform_pm1", 900 + 10 * rep + r) for r in range(P)]
+        for t, a in zip(src, fresh):
+            t.copy_(torch.from_numpy(a))  # eager work between the replays
+        for t in work:
+            t.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        want = oracle.reduce_scatterv(fresh, counts, "f32", "sum", "pairwise_desc")
+        for b in range(P):
+            got = to_host(work[b], np.float32)
+            assert_bits_equal(got[:counts[b]], want[b], "f32", "graph replay %d rank %d" % (rep, b))
+            assert got[counts[b]:].tobytes() == fresh[b][counts[b]:].tobytes(), "bytes behind the result changed"
+    del g
+    al.release_scratch(stream=s.cuda_stream)
+    al.release_scratch(stream=s.cuda_stream)  # nothing left to free: still fine
 
 
 SETTINGS = [

@@ -165,6 +165,26 @@ def test_halo_pack_unpack(al, np_dtype, dims, h):
     assert to_host(d_grid2, np_dtype).tobytes() == w2.tobytes(), "subset unpack"
 
 
+def test_halo_pack_does_not_depend_on_the_load_policy(al):
+    """The cache policy of the pack's grid loads is a measurement setting: every policy packs the same bytes."""
+    import torch
+    nx, ny, nz, h = 64, 40, 24, 2
+    rng = np.random.default_rng(4100)
+    grid = rng.random((nz + 2 * h, ny + 2 * h, nx + 2 * h))
+    d_grid = to_dev(grid.reshape(-1))
+    want = [oracle.halo_pack(grid.reshape(-1), nx, ny, nz, h, f) for f in range(6)]
+    try:
+        for policy in range(5):
+            al.tune("halo_load_policy", policy)
+            bufs = {f: dev_empty(oracle.halo_face_elems(nx, ny, nz, h, f), np.float64) for f in range(6)}
+            al.halo_pack(bufs, d_grid, (nx, ny, nz), h)
+            torch.cuda.synchronize()
+            for f in range(6):
+                assert to_host(bufs[f], np.float64).tobytes() == want[f].tobytes(), "policy %d face %d" % (policy, f)
+    finally:
+        al.tune("halo_load_policy", 0)
+
+
 def test_halo_errors(al):
     grid = to_dev(np.zeros(6 * 6 * 6, np.float64))
     buf = {0: dev_empty(8, np.float64)}

@@ -89,13 +89,9 @@ def test_noalloc_in_a_hip_graph(al):
             al.copy(work[r], src[r])
         al.reduce_scatterv_noalloc(work, work, counts, "sum", order="tree_halv", dtype="f32")
 
-    for t in src:
-        t.zero_()
-    run()  # eager warm-up outside the capture
-    torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g):
-        run()
+        run()  # no eager call beforehand: the entry point needs no warm-up
     for rep in range(3):
         fresh = [oracle.fill(total, "f32", "uniform_pm1", 700 + 10 * rep + r) for r in range(P)]
         for t, a in zip(src, fresh):
@@ -110,3 +106,37 @@ def test_noalloc_in_a_hip_graph(al):
             got = to_host(work[b], np.float32)
             assert_bits_equal(got[:counts[b]], want[b], "f32", "graph replay %d rank %d" % (rep, b))
             assert got[counts[b]:].tobytes() == fresh[b][counts[b]:].tobytes(), "bytes behind the result changed"
+
+
+def test_noalloc_refuses_a_second_stream_while_the_array_is_in_use(al):
+    """Every call on a device shares the one fixed array.  A chained launch is held back on its stream by a
+    flag that the host has not signalled yet; a call on another stream that would need the array meanwhile
+    is refused; once the first has run, the second stream's call goes through and is right."""
+    import torch
+    P, counts = 2, [1, 300_001]
+    total = sum(counts)
+    sends = [oracle.fill(total, "f32", "uniform_pm1", 40 + r) for r in range(P)]
+    want = oracle.reduce_scatterv(sends, counts, "f32", "sum", "rank_asc")
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    first = [to_dev(x) for x in sends]
+    second = [to_dev(x) for x in sends]
+    torch.cuda.synchronize()
+    flag = al.Flag(0)
+    try:
+        flag.wait(1, mode="kernel", max_spins=1 << 34, stream=a)  # bounded: the stream goes on by itself in the end
+        al.reduce_scatterv_noalloc(first, first, counts, "sum", dtype="f32", stream=a)
+        with pytest.raises(al.AlError, match="still in use") as e:
+            al.reduce_scatterv_noalloc(second, second, counts, "sum", dtype="f32", stream=b)
+        assert e.value.code == 1
+        # the same stream may queue another one behind its own
+        al.reduce_scatterv_noalloc(first, first, [1, 1000], "sum", dtype="f32", stream=a)
+    finally:
+        flag.signal(1)
+    a.synchronize()
+    assert not flag.timed_out()
+    second = [to_dev(x) for x in sends]
+    al.reduce_scatterv_noalloc(second, second, counts, "sum", dtype="f32", stream=b)
+    torch.cuda.synchronize()
+    for r in range(P):
+        assert_bits_equal(to_host(second[r], np.float32)[:counts[r]], want[r], "f32", "second stream, rank %d" % r)
+    flag.destroy()
