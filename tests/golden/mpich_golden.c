@@ -165,6 +165,7 @@ static void plant_specials(void *buf, size_t n, int dt) {
 /* More than two ranks: every element of every rank is drawn from a pool of
  * special values (and two ordinary ones) by a fixed rule, so that NaNs, zeros
  * of both signs and infinities meet in every position of the combine order. */
+/* (tests/util.py restates this rule, so that long cases need not repeat their inputs) */
 static void plant_specials_many(void *buf, size_t n, int dt) {
   static const unsigned pool[] = {0x7fc00000u, 0xbf800000u, 0x00000000u, 0x80000000u, 0x7f800000u,
                                   0xff800000u, 0x00000001u, 0x80000001u, 0x3f800000u, 0x7f7fffffu,
@@ -178,7 +179,9 @@ static void plant_specials_many(void *buf, size_t n, int dt) {
     float f;
     memcpy(&f, &u, 4);
     if (dt == ALO_F32) ((float *)buf)[i] = f;
-    else ((double *)buf)[i] = (double)f;
+    else if (dt == ALO_F64) ((double *)buf)[i] = (double)f;
+    else if (dt == ALO_BF16) ((unsigned short *)buf)[i] = alo_f32_to_bf16(f);
+    else ((unsigned short *)buf)[i] = alo_f32_to_f16(f);
   }
 }
 
@@ -199,19 +202,20 @@ static void case_allreduce(int dt, int op, size_t n, int dist, int specials,
   head("allreduce", dt, op, n, dist, seed, note);
   emit_nb(same);
   /* inputs are repeated for short messages and planted values; the others are the generator's */
-  if (!is_half(dt) && (specials || n * es <= 2048)) emit_list("in", in, n * es);
+  if ((specials && n * es <= 2048) || (!is_half(dt) && (specials || n * es <= 2048))) emit_list("in", in, n * es);
   emit_list("out", out, n * es);
   tail();
   free(in); free(out); free(nb);
 }
 
 /* count = elements per rank; send buffer holds P*count. */
-static void case_reduce_scatter(int dt, int op, size_t count, int dist, int full,
-                                const char *note) {
+static void case_reduce_scatter_x(int dt, int op, size_t count, int dist, int full, int specials,
+                                  const char *note) {
   const unsigned long long seed = 1000;
   size_t es = alo_dtype_size(dt), n = count * (size_t)P_;
   void *in = malloc(n * es), *out = malloc(count * es);
   alo_fill(in, n, dt, dist, seed + (unsigned long long)rank_, 0);
+  if (specials) plant_specials(in, n, dt);
   MPI_Reduce_scatter_block(in, out, (int)count, mpi_type(dt), op_for(dt, op), MPI_COMM_WORLD);
   void *nb = malloc(n * es);
   MPI_Request req;
@@ -223,7 +227,7 @@ static void case_reduce_scatter(int dt, int op, size_t count, int dist, int full
   head("reduce_scatter", dt, op, count, dist, seed, note);
   emit_nb(same);
   if (full) {
-    if (!is_half(dt)) emit_list("in", in, n * es);
+    if (!is_half(dt) || specials) emit_list("in", in, n * es);
     emit_list("out", out, count * es);
   } else {
     emit_sums("out_checksum", out, count * es);
@@ -231,6 +235,10 @@ static void case_reduce_scatter(int dt, int op, size_t count, int dist, int full
   }
   tail();
   free(in); free(out);
+}
+
+static void case_reduce_scatter(int dt, int op, size_t count, int dist, int full, const char *note) {
+  case_reduce_scatter_x(dt, op, count, dist, full, 0, note);
 }
 
 /* MPI_Reduce_scatter with uneven counts: rank b receives 3 + 2*((b*5) % 4) elements, rank 1 none. */
@@ -414,6 +422,21 @@ int main(int argc, char **argv) {
       case_reduce_scatter(hdt[d], ALO_SUM, (size_t)(1u << 20) / (size_t)P_ / 2 + 64, ALO_DIST_UNIFORM_PM1, 0,
                           "long message");
       case_reduce_scatterv_long(hdt[d], ALO_SUM, ALO_DIST_UNIFORM_PM1, "uneven counts, long message");
+    }
+  }
+
+  /* operand roles of the reduce-scatter orders and of the 16-bit user-defined operations: special values
+   * planted in every position (long cases keep checksums; their inputs follow plant_specials_many) */
+  if (P_ == 3 || P_ == 4 || P_ == 8) {
+    for (int op = ALO_MIN; op <= ALO_MAX; op++) {
+      case_reduce_scatter_x(ALO_F32, op, 24, ALO_DIST_UNIFORM_PM1, 1, 1, "specials");
+      case_reduce_scatter_x(ALO_BF16, op, 24, ALO_DIST_UNIFORM_PM1, 1, 1, "specials");
+      if (big)
+        case_reduce_scatter_x(ALO_F32, op, (size_t)(1u << 20) / (size_t)P_ / 4 + 64, ALO_DIST_UNIFORM_PM1, 0, 1,
+                              "specials");
+      case_allreduce(ALO_BF16, op, 96, ALO_DIST_UNIFORM_PM1, 1, "specials");
+      case_allreduce(ALO_F16, op, 96, ALO_DIST_UNIFORM_PM1, 1, "specials");
+      case_allreduce(ALO_BF16, op, 2048 / 2 + 8, ALO_DIST_UNIFORM_PM1, 1, "specials");
     }
   }
 

@@ -111,6 +111,12 @@ OPS_SWEEPS = [
     "--op allgather --datatype short --inplace --nonblocking --odd-sizes --max-size 65536 --ranks 8",
     "--op reduce_scatterv --datatype double --nonblocking --odd-sizes --max-size 16384 --ranks 5",
     "--op allgatherv --datatype char --inplace --nonblocking --odd-sizes --max-size 16384 --ranks 8",
+    # the orders of a rooted reduce: binomial to the root (automatic below 2 KiB and for 16-bit floats),
+    # reduce-scatter + gather above
+    "--op reduce --datatype bfloat16 --root 6 --odd-sizes --max-size 65536 --ranks 7",
+    "--op reduce --datatype float --reduction-op max --root 3 --algorithm tree_reduce_scatter_gather --odd-sizes --max-size 65536 --ranks 5",
+    "--op allreduce --datatype double --reduction-op min --algorithm tree_reduce_scatter_gather --inplace --max-size 65536 --ranks 7",
+    "--op reduce_scatter --datatype float --reduction-op min --algorithm tree_halving --odd-sizes --max-size 16384 --ranks 6",
     # non-blocking operations that move more than 256 MiB in all take the internal stream
     "--op allreduce --datatype double --nonblocking --odd-sizes --min-size 1048576 --max-size 4194304 --ranks 8",
     "--op reduce_scatter --datatype float --nonblocking --inplace --min-size 1048576 --max-size 2097152 --ranks 8",

@@ -15,7 +15,7 @@ import numpy as np
 import pytest
 
 import oracle
-from util import assert_bits_equal, dev_empty, mpich_order, to_dev, to_host
+from util import assert_bits_equal, dev_empty, mpich_order, planted_specials, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
 
@@ -37,6 +37,8 @@ def arr(hexstr, dtype):
 def inputs_of(c, P, n):
     if "in" in c:
         return [arr(h, c["dtype"]) for h in c["in"]]
+    if c["note"] == "specials":
+        return [planted_specials(n, c["dtype"], r) for r in range(P)]
     return [oracle.fill(n, c["dtype"], c["dist"], c["seed_base"] + r) for r in range(P)]
 
 

@@ -19,7 +19,7 @@ import numpy as np
 import pytest
 
 import oracle
-from util import assert_bits_equal, mpich_order
+from util import assert_bits_equal, mpich_order, planted_specials
 
 GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "mpich_P*.json.gz")),
                 key=lambda p: int(os.path.basename(p)[7:-8]))
@@ -40,6 +40,8 @@ def inputs_of(c, P, n):
     does not repeat them."""
     if "in" in c:
         return [arr(h, c["dtype"]) for h in c["in"]]
+    if c["note"] == "specials":
+        return [planted_specials(n, c["dtype"], r) for r in range(P)]
     return [oracle.fill(n, c["dtype"], c["dist"], c["seed_base"] + r) for r in range(P)]
 
 
@@ -69,6 +71,10 @@ def test_allreduce_vectors(path):
             # the committed inputs are what the generator makes
             for r in range(P):
                 assert oracle.fill(n, dt, c["dist"], c["seed_base"] + r).tobytes() == ins[r].tobytes()
+        if "in" in c and c["note"] == "specials" and P > 2:
+            # ... and the planted ones follow the rule that the long cases, which do not repeat them, rely on
+            for r in range(P):
+                assert planted_specials(n, dt, r).tobytes() == ins[r].tobytes(), (P, dt, n, r)
         order, start = mpich_order("allreduce", dt, n, P)
         want = outs[0]
         got = oracle.combine(ins, dt, op, order, start)
@@ -125,10 +131,14 @@ def test_reduce_scatter_vectors(path):
         else:
             # long: pairwise exchange, rank r folds x_r, x_{r-1}, ... ; outputs kept as checksums
             assert order == "pairwise_desc"
+            planted = inputs_of(c, P, P * count) if c["note"] == "specials" else None
             for r in range(P):
-                got = oracle.combine_generated(P, count, dt, op, order, r, c["dist"],
-                                               c["seed_base"], r * count)
-                assert "%016x" % oracle.checksum(got) == c["out_checksum"][r], (P, dt, r)
+                if planted:
+                    got = oracle.combine([a[r * count:(r + 1) * count] for a in planted], dt, op, order, r)
+                else:
+                    got = oracle.combine_generated(P, count, dt, op, order, r, c["dist"], c["seed_base"], r * count)
+                # (a min / max result is one of its operands bit for bit, the one planted NaN included)
+                assert "%016x" % oracle.checksum(got) == c["out_checksum"][r], (P, dt, r, c["note"])
                 assert_bits_equal(got[:8], arr(c["out_head"][r], dt), dt, "head")
         seen += 1
     assert seen >= 8

@@ -88,3 +88,41 @@ def assert_bits_equal(got, want, dtype, what=""):
         i = int(bad[0])
         raise AssertionError("%s: %d of %d elements differ; first at %d: got %r want %r" % (
             what, bad.size, got.size, i, got.reshape(-1)[i], want.reshape(-1)[i]))
+
+
+_POOL = np.array([0x7fc00000, 0xbf800000, 0x00000000, 0x80000000, 0x7f800000, 0xff800000, 0x00000001, 0x80000001,
+                  0x3f800000, 0x7f7fffff, 0x00800000, 0x00400000, 0x3e99999a], dtype=np.uint32)
+
+
+def _fin64(z):
+    z = z ^ (z >> np.uint64(30))
+    z = z * np.uint64(0xBF58476D1CE4E5B9)
+    z = z ^ (z >> np.uint64(27))
+    z = z * np.uint64(0x94D049BB133111EB)
+    return z ^ (z >> np.uint64(31))
+
+
+def mix64(seed, idx):
+    """The generator's hash (oracle.mix64) over an array of indices."""
+    g = np.uint64(0x9E3779B97F4A7C15)
+    with np.errstate(over="ignore"):
+        return _fin64(_fin64(np.uint64(seed) + g) + (idx.astype(np.uint64) + np.uint64(1)) * g)
+
+
+def planted_specials(n, dtype, rank):
+    """The inputs that the golden generator plants for more than two ranks (tests/golden/mpich_golden.c,
+    plant_specials_many): element i of `rank` is drawn from a pool of NaN, zeros of both signs, infinities,
+    denormals and a few ordinary values by a fixed rule; every fourth element is a zero of one sign or the other."""
+    import oracle
+    i = np.arange(n, dtype=np.uint64)
+    h = mix64(77, i * np.uint64(64) + np.uint64(rank))
+    u = _POOL[(h % np.uint64(len(_POOL))).astype(np.int64)]
+    fourth = (i % np.uint64(4)) == 0
+    neg = fourth & (((h >> np.uint64(32)) % np.uint64(3)) == 0)
+    u = np.where(fourth, np.where(neg, np.uint32(0x80000000), np.uint32(0)), u).astype(np.uint32)
+    f = u.view(np.float32)
+    if dtype == "f32":
+        return f.copy()
+    if dtype == "f64":
+        return f.astype(np.float64)
+    return oracle.f32_to_bf16(f) if dtype == "bf16" else oracle.f32_to_f16(f)
