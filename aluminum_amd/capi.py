@@ -14,7 +14,7 @@ _LIB = os.path.join(_HERE, "libaluminum_amd.so")
 DTYPES = ["i8", "u8", "i16", "u16", "i32", "u32", "i64", "u64", "f16", "bf16", "f32", "f64"]
 OPS = ["sum", "prod", "min", "max", "lor", "land", "lxor", "bor", "band", "bxor", "avg"]
 ORDERS = {"rank_asc": 0, "tree_dbl": 1, "tree_halv": 2, "pairwise_desc": 3, "ring": 4,
-          "tree_binomial": 5, "tree_rsg": 6}
+          "tree_binomial": 5, "tree_rsg": 6, "tree_rsg_spread": 7}
 DISTS = {"uniform_pm1": 0, "uniform_09_11": 1, "uniform_01": 2, "fullrange": 3, "bool01": 4,
          "normal": 5, "smallint": 6}
 RING_MODES = {"stepwise": 0, "fused": 1}
@@ -175,7 +175,7 @@ def combine(outs, ins, op, order="rank_asc", start=0, dtype=None, count=None, st
                                 _op(op), _order(order), start, _stream(stream)))
 
 
-COLLECTIVES = {"allreduce": 0, "reduce": 1, "reduce_scatter": 2}
+COLLECTIVES = {"allreduce": 0, "reduce": 1, "reduce_scatter": 2, "allreduce_blocking": 3, "reduce_blocking": 4}
 _ORDER_NAMES = {v: k for k, v in ORDERS.items()}
 
 

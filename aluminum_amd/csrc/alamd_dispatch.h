@@ -244,6 +244,7 @@ struct TreeParams {
   int role_start0, role_stride;      // ROLE_PER_SEGMENT: segment s is for rank (role_start0 + s * role_stride) mod P
   unsigned long long role_base;      // ROLE_PER_BLOCK: element 0 of a segment is element role_base of the message,
   unsigned long long role_count;     // which has role_count elements (0: the segment is the message)
+  int role_spread;                   // ROLE_PER_BLOCK: how the message is cut into blocks, see role_mask_of_elem
 };
 
 __host__ __device__ inline unsigned role_bit_reverse(unsigned v, int bits) {
@@ -257,12 +258,19 @@ __host__ __device__ inline unsigned role_mask_of_rank(const TreeParams &p, int r
   const int o = rank < 2 * p.role_rem ? rank / 2 : rank - p.role_rem;
   return role_bit_reverse((unsigned)o, p.role_bits);
 }
-// ROLE_PER_BLOCK: the message is cut into 2^role_bits blocks of count >> role_bits elements (the last
-// one takes the remainder); block k ends up on survivor bit_reverse(k).
+// ROLE_PER_BLOCK: the message is cut into 2^role_bits blocks of count >> role_bits elements; what that
+// leaves over goes to the last block (TREE_RSG) or, role_spread, one element each to the first blocks
+// (TREE_RSG_SPREAD).  Block k ends up on survivor bit_reverse(k).
 __host__ __device__ inline unsigned role_mask_of_elem(const TreeParams &p, size_t seg_len, size_t e) {
   const unsigned long long n = p.role_count ? p.role_count : seg_len, blk = n >> p.role_bits;
-  const unsigned long long last = (1ull << p.role_bits) - 1;
-  unsigned long long k = blk ? (p.role_base + e) / blk : last;
+  const unsigned long long last = (1ull << p.role_bits) - 1, x = p.role_base + e;
+  unsigned long long k;
+  if (p.role_spread) {
+    const unsigned long long longer = n & last, cut = longer * (blk + 1);  // `longer` blocks of blk + 1 come first
+    k = x < cut ? x / (blk + 1) : (blk ? longer + (x - cut) / blk : last);
+  } else {
+    k = blk ? x / blk : last;
+  }
   if (k > last) k = last;
   return role_bit_reverse((unsigned)k, p.role_bits);
 }

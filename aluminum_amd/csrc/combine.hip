@@ -42,9 +42,10 @@ bool order_start_per_block(int order) {
 }
 bool order_is_tree(int order) {
   return order == ALAMD_ORDER_TREE_DBL || order == ALAMD_ORDER_TREE_HALV || order == ALAMD_ORDER_TREE_BINOMIAL ||
-         order == ALAMD_ORDER_TREE_RSG;
+         order == ALAMD_ORDER_TREE_RSG || order == ALAMD_ORDER_TREE_RSG_SPREAD;
 }
-bool order_valid(int order) { return order >= ALAMD_ORDER_RANK_ASC && order <= ALAMD_ORDER_TREE_RSG; }
+bool order_is_rsg(int order) { return order == ALAMD_ORDER_TREE_RSG || order == ALAMD_ORDER_TREE_RSG_SPREAD; }
+bool order_valid(int order) { return order >= ALAMD_ORDER_RANK_ASC && order <= ALAMD_ORDER_TREE_RSG_SPREAD; }
 
 // Fills the slot tables of a tree order over the P inputs `ins`.  start: the root of the binomial tree.
 int build_tree(TreeParams &tp, const void *const *ins, int P, int order, int start) {
@@ -53,6 +54,7 @@ int build_tree(TreeParams &tp, const void *const *ins, int P, int order, int sta
   tp.role_mode = ROLE_FIXED;
   tp.role_rem = tp.role_bits = tp.role_start0 = tp.role_stride = 0;
   tp.role_base = tp.role_count = 0;
+  tp.role_spread = order == ALAMD_ORDER_TREE_RSG_SPREAD;
   if (order == ALAMD_ORDER_TREE_BINOMIAL) {
     // the ranks counted from the root, with wrap
     for (int j = 0; j < P; ++j) tp.a[j] = static_cast<const char *>(ins[(j + start) % P]);
@@ -62,8 +64,8 @@ int build_tree(TreeParams &tp, const void *const *ins, int P, int order, int sta
   const int pof2 = floor_pow2(P), rem = P - pof2;
   const char *la[ALAMD_MAX_RANKS], *lb[ALAMD_MAX_RANKS];
   // pre-fold of the first 2 * rem ranks: the slot holds step(in = la, inout = lb).  The odd rank
-  // keeps the result, except under TREE_RSG, where the even one does.
-  const int keep = order == ALAMD_ORDER_TREE_RSG ? 0 : 1;
+  // keeps the result, except under TREE_RSG(_SPREAD), where the even one does.
+  const int keep = order_is_rsg(order) ? 0 : 1;
   for (int j = 0; j < pof2; ++j) {
     if (j < rem) { la[j] = static_cast<const char *>(ins[2 * j + 1 - keep]); lb[j] = static_cast<const char *>(ins[2 * j + keep]); }
     else { la[j] = static_cast<const char *>(ins[j + rem]); lb[j] = nullptr; }
@@ -73,7 +75,7 @@ int build_tree(TreeParams &tp, const void *const *ins, int P, int order, int sta
   tp.role_rem = rem;
   tp.role_bits = bits;
   if (order == ALAMD_ORDER_TREE_HALV) tp.role_mode = ROLE_PER_SEGMENT;
-  if (order == ALAMD_ORDER_TREE_RSG) tp.role_mode = ROLE_PER_BLOCK;
+  if (order_is_rsg(order)) tp.role_mode = ROLE_PER_BLOCK;
   for (int k = 0; k < pof2; ++k) {
     // pairing at distance pof2/2, ..., 1 is the adjacent-pair tree over the
     // bit-reversed slot order
@@ -90,7 +92,7 @@ struct Layout {
   SegParams seg;
   size_t max_len;
   int start0, start_stride;  // segment s is for rank (start0 + s * start_stride) mod P (orders with a start)
-  // TREE_RSG, when the launch covers part of a message only: where element 0 of a segment lies in the
+  // TREE_RSG(_SPREAD), when the launch covers part of a message only: where element 0 of a segment lies in the
   // message, and the message's length (0: every segment is a message of its own)
   size_t msg_base = 0, msg_count = 0;
 };

@@ -140,22 +140,27 @@ int alamd_reference_order(int collective, int P, size_t count, int dtype, int ro
   *start = 0;
   switch (collective) {
   case ALAMD_COLL_ALLREDUCE:
-  case ALAMD_COLL_REDUCE: {
-    if (collective == ALAMD_COLL_REDUCE && (root < 0 || root >= P))
+  case ALAMD_COLL_REDUCE:
+  case ALAMD_COLL_ALLREDUCE_BLOCKING:
+  case ALAMD_COLL_REDUCE_BLOCKING: {
+    const bool rooted = collective == ALAMD_COLL_REDUCE || collective == ALAMD_COLL_REDUCE_BLOCKING;
+    const bool blocking = collective == ALAMD_COLL_ALLREDUCE_BLOCKING || collective == ALAMD_COLL_REDUCE_BLOCKING;
+    if (rooted && (root < 0 || root >= P))
       return alamd::set_error(ALAMD_ERR_INVALID_ARG, "root %d outside [0, %d)", root, P);
     // An allreduce among ranks of one host is a reduce to rank 0 followed by a broadcast.  The reduce
     // is a binomial tree to the root, over the ranks counted from it, for short messages, for fewer
     // elements than the largest power of two of ranks and for every operation that is not one of the
     // library's own (fp16 and bf16 are user-defined operations to it); otherwise a reduce-scatter by
-    // recursive halving followed by a gather, which does not depend on the root.
+    // recursive halving followed by a gather, which does not depend on the root; the blocking calls
+    // cut its blocks differently from the non-blocking ones.
     size_t pof2 = 1;
     while (2 * pof2 <= (size_t)P) pof2 *= 2;
     const bool user_op = dtype == ALAMD_F16 || dtype == ALAMD_BF16;
     if (user_op || count * es <= 2048 || count < pof2) {
       *order = ALAMD_ORDER_TREE_BINOMIAL;
-      *start = collective == ALAMD_COLL_REDUCE ? root : 0;
+      *start = rooted ? root : 0;
     } else {
-      *order = ALAMD_ORDER_TREE_RSG;
+      *order = blocking ? ALAMD_ORDER_TREE_RSG_SPREAD : ALAMD_ORDER_TREE_RSG;
     }
     return ALAMD_OK;
   }

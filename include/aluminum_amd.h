@@ -112,13 +112,18 @@ typedef enum {
  *                  survivor whose bit d equals that survivor's bit d keeps.
  *                  For sum and prod this gives the bits of TREE_DBL; it differs
  *                  where a float min / max meets a tie (+0 / -0) or a NaN.
+ *   TREE_RSG_SPREAD  the same, but what count / 2^k leaves over goes one
+ *                  element each to the first blocks instead of to the last one.
  * Which of two operands is the inout one only shows in float min / max (a tie
  * or a NaN lets the in operand through); every other result depends on the
  * shape of the tree alone.
  * With MPICH 3.3.2 on one host the reference's MPI and host-transfer backends
  * produce: Allreduce and Reduce of native types - TREE_BINOMIAL with s = root
- * (Allreduce: 0) up to 2048 bytes or when count < 2^k, TREE_RSG above, whatever
- * the root; of fp16 / bf16, which are user-defined operations to the MPI
+ * (Allreduce: 0) up to 2048 bytes or when count < 2^k; above that, whatever the
+ * root, TREE_RSG where the backend calls MPI_Ireduce / MPI_Iallreduce (the
+ * host-transfer backend always, the MPI backend in its non-blocking calls) and
+ * TREE_RSG_SPREAD where it calls MPI_Reduce / MPI_Allreduce (the MPI backend's
+ * blocking calls); of fp16 / bf16, which are user-defined operations to the MPI
  * library - TREE_BINOMIAL at every size; Reduce_scatter, with equal or unequal
  * counts - TREE_HALV with s = receiving rank below 512 KiB in total,
  * PAIRWISE_DESC with s = receiving rank from there on. */
@@ -129,7 +134,8 @@ typedef enum {
   ALAMD_ORDER_PAIRWISE_DESC = 3,
   ALAMD_ORDER_RING = 4,
   ALAMD_ORDER_TREE_BINOMIAL = 5,
-  ALAMD_ORDER_TREE_RSG = 6
+  ALAMD_ORDER_TREE_RSG = 6,
+  ALAMD_ORDER_TREE_RSG_SPREAD = 7
 } alamd_order;
 
 /* ---- library ---------------------------------------------------------- */
@@ -163,13 +169,22 @@ int alamd_init(void);
  * (include/aluminum/mpi/allreduce.hpp:38-44, mpi/reduce.hpp:41-49,
  * mpi/reduce_scatter.hpp:40-46, include/aluminum/ht/allreduce.hpp:76-79,
  * ht/reduce.hpp:72-82, ht/reduce_scatter.hpp:71-74, ht/reduce_scatterv.hpp:76-79);
- * the table was read off that library's results for 2 to 16 ranks.
- * `count`: elements per rank for ALAMD_COLL_ALLREDUCE and ALAMD_COLL_REDUCE,
- * elements in a whole send buffer for ALAMD_COLL_REDUCE_SCATTER (with equal or
- * unequal counts).  `root` is ignored except for ALAMD_COLL_REDUCE.  *start is
- * what alamd_combine takes; alamd_reduce_scatter(v) add the receiving rank
- * themselves. */
-typedef enum { ALAMD_COLL_ALLREDUCE = 0, ALAMD_COLL_REDUCE = 1, ALAMD_COLL_REDUCE_SCATTER = 2 } alamd_collective;
+ * the table was read off that library's results for 2 to 64 ranks.
+ * ALAMD_COLL_ALLREDUCE and ALAMD_COLL_REDUCE stand for the non-blocking MPI
+ * calls (every call of the host-transfer backend), the _BLOCKING ones for
+ * MPI_Allreduce and MPI_Reduce (the MPI backend's blocking calls), which differ
+ * in how a long message is cut into blocks; a reduce-scatter is the same in both.
+ * `count`: elements per rank for an allreduce or reduce, elements in a whole
+ * send buffer for ALAMD_COLL_REDUCE_SCATTER (with equal or unequal counts).
+ * `root` is ignored except for a reduce.  *start is what alamd_combine takes;
+ * alamd_reduce_scatter(v) add the receiving rank themselves. */
+typedef enum {
+  ALAMD_COLL_ALLREDUCE = 0,
+  ALAMD_COLL_REDUCE = 1,
+  ALAMD_COLL_REDUCE_SCATTER = 2,
+  ALAMD_COLL_ALLREDUCE_BLOCKING = 3,
+  ALAMD_COLL_REDUCE_BLOCKING = 4
+} alamd_collective;
 int alamd_reference_order(int collective, int P, size_t count, int dtype, int root, int *order, int *start);
 
 /* ---- combine: the element-wise fold of P rank contributions ----------- */
@@ -193,7 +208,7 @@ int alamd_combine(void *const *outs, int nout, const void *const *ins, int P,
 /* Reduce_scatter over P logical ranks: sends[r] holds P*count elements;
  * recvs[b] receives count elements, the fold of block b of every sends[r],
  * with start = b under PAIRWISE_DESC, RING and TREE_HALV (TREE_BINOMIAL: 0;
- * TREE_RSG: every block is a message of its own).  In-place form
+ * TREE_RSG, TREE_RSG_SPREAD: every block is a message of its own).  In-place form
  * (recvs[b] == sends[b]) puts the result at the start of the buffer.
  * Replaces MPI_Ireduce_scatter_block on the host copy
  * (include/aluminum/ht/reduce_scatter.hpp:45-74; layout docs/comm.rst:284-285). */

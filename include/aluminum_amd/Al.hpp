@@ -168,17 +168,23 @@ AL_AMD_TYPEMAP(__hip_bfloat16, ALAMD_BF16);
 
 /** Combine orders and ring modes a caller can ask for by name. */
 enum class CombineAlgorithm {
-  automatic,      /**< what the reference's MPI and host-transfer backends yield with MPICH
-                       3.3.2 on one host (alamd_reference_order): Allreduce and Reduce - binomial
-                       tree to the root up to 2048 bytes and for fp16 / bf16, reduce-scatter +
-                       gather above; Reduce_scatter(v) - distance-halving tree below 512 KiB in
-                       total, descending pairwise fold from there on */
+  automatic,      /**< what the reference's host-transfer backend (and the non-blocking calls of its
+                       MPI backend) yield with MPICH 3.3.2 on one host (alamd_reference_order):
+                       Allreduce and Reduce - binomial tree to the root up to 2048 bytes and for
+                       fp16 / bf16, reduce-scatter + gather above; Reduce_scatter(v) -
+                       distance-halving tree below 512 KiB in total, descending pairwise fold from
+                       there on */
+  automatic_mpi_blocking,  /**< what the blocking calls of the reference's MPI backend yield there:
+                       as `automatic`, except that MPI_Allreduce and MPI_Reduce cut a long message
+                       into the blocks of tree_reduce_scatter_gather_spread */
   rank_order,     /**< ((x0 . x1) . x2) ... */
   tree_doubling,
   tree_halving,
   tree_binomial,  /**< to the root of a Reduce, to rank 0 otherwise */
   tree_reduce_scatter_gather,  /**< the doubling tree with the operand roles of a reduce-scatter by
                                     recursive halving of the data followed by a gather */
+  tree_reduce_scatter_gather_spread,  /**< the same, with what the count is not a multiple of spread
+                                    over the first blocks instead of left to the last one */
   pairwise,       /**< x_r . x_{r-1} . x_{r-2} ... for the block of rank r */
   ring,           /**< ring reduce-scatter + allgather, one launch per ring step */
   ring_fused      /**< the same values with every segment folded in one pass */
@@ -661,11 +667,17 @@ inline void World::launch(PendingOp &p) {
                                 &start) != ALAMD_OK)
         AL_AMD_THROW(std::string(alamd_last_error()));
       break;
+    case CombineAlgorithm::automatic_mpi_blocking:
+      if (alamd_reference_order(rooted ? ALAMD_COLL_REDUCE_BLOCKING : ALAMD_COLL_ALLREDUCE_BLOCKING, P, p.count,
+                                p.dtype, p.root, &order, &start) != ALAMD_OK)
+        AL_AMD_THROW(std::string(alamd_last_error()));
+      break;
     case CombineAlgorithm::rank_order: order = ALAMD_ORDER_RANK_ASC; break;
     case CombineAlgorithm::tree_doubling: order = ALAMD_ORDER_TREE_DBL; break;
     case CombineAlgorithm::tree_halving: order = ALAMD_ORDER_TREE_HALV; break;
     case CombineAlgorithm::tree_binomial: order = ALAMD_ORDER_TREE_BINOMIAL; start = rooted ? p.root : 0; break;
     case CombineAlgorithm::tree_reduce_scatter_gather: order = ALAMD_ORDER_TREE_RSG; break;
+    case CombineAlgorithm::tree_reduce_scatter_gather_spread: order = ALAMD_ORDER_TREE_RSG_SPREAD; break;
     case CombineAlgorithm::ring:
     case CombineAlgorithm::ring_fused: ring = true; break;
     default: AL_AMD_THROW("Invalid algorithm");
@@ -687,6 +699,7 @@ inline void World::launch(PendingOp &p) {
     int order = ALAMD_ORDER_RANK_ASC, start = 0;
     switch (p.algo) {
     case CombineAlgorithm::automatic:
+    case CombineAlgorithm::automatic_mpi_blocking:
       if (alamd_reference_order(ALAMD_COLL_REDUCE_SCATTER, P, p.count * static_cast<size_t>(P), p.dtype, 0, &order,
                                 &start) != ALAMD_OK)
         AL_AMD_THROW(std::string(alamd_last_error()));
@@ -703,7 +716,8 @@ inline void World::launch(PendingOp &p) {
     break;
   }
   case OpKind::allgather:
-    if (p.algo != CombineAlgorithm::automatic) AL_AMD_THROW("Invalid algorithm");
+    if (p.algo != CombineAlgorithm::automatic && p.algo != CombineAlgorithm::automatic_mpi_blocking)
+      AL_AMD_THROW("Invalid algorithm");
     rc = alamd_allgather(recvs.data(), sends.data(), P, p.count, p.dtype, target);
     break;
   case OpKind::reduce_scatterv: {
@@ -712,6 +726,7 @@ inline void World::launch(PendingOp &p) {
     int order = ALAMD_ORDER_RANK_ASC, start = 0;
     switch (p.algo) {
     case CombineAlgorithm::automatic:
+    case CombineAlgorithm::automatic_mpi_blocking:
       if (alamd_reference_order(ALAMD_COLL_REDUCE_SCATTER, P, total, p.dtype, 0, &order, &start) != ALAMD_OK)
         AL_AMD_THROW(std::string(alamd_last_error()));
       break;
@@ -726,7 +741,8 @@ inline void World::launch(PendingOp &p) {
     break;
   }
   case OpKind::allgatherv:
-    if (p.algo != CombineAlgorithm::automatic) AL_AMD_THROW("Invalid algorithm");
+    if (p.algo != CombineAlgorithm::automatic && p.algo != CombineAlgorithm::automatic_mpi_blocking)
+      AL_AMD_THROW("Invalid algorithm");
     rc = alamd_allgatherv(recvs.data(), sends.data(), P, p.counts.data(), p.displs.data(), p.dtype, target);
     break;
   }

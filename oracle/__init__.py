@@ -18,7 +18,7 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 DTYPES = ["i8", "u8", "i16", "u16", "i32", "u32", "i64", "u64", "f16", "bf16", "f32", "f64"]
 OPS = ["sum", "prod", "min", "max", "lor", "land", "lxor", "bor", "band", "bxor", "avg"]
 ORDERS = {"rank_asc": 0, "tree_dbl": 1, "tree_halv": 2, "pairwise_desc": 3, "ring": 4,
-          "tree_binomial": 5, "tree_rsg": 6}
+          "tree_binomial": 5, "tree_rsg": 6, "tree_rsg_spread": 7}
 DISTS = {"uniform_pm1": 0, "uniform_09_11": 1, "uniform_01": 2, "fullrange": 3, "bool01": 4,
          "normal": 5, "smallint": 6}
 

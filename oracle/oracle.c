@@ -430,7 +430,8 @@ int alo_schedule(int P, int order, int start, int *pairs, int *result) {
       }
     *result = start;
     return np;
-  case ALO_ORDER_TREE_RSG: {
+  case ALO_ORDER_TREE_RSG:
+  case ALO_ORDER_TREE_RSG_SPREAD: {
     /* Reduce-scatter by recursive halving of the data at distance 1, 2, 4, ...
      * followed by a gather.  Non-power-of-two P: the odd ranks among the first
      * 2*rem send to the even rank below them, which keeps the result.  The
@@ -497,18 +498,25 @@ int alo_schedule(int P, int order, int start, int *pairs, int *result) {
   }
 }
 
-/* TREE_RSG: the n elements are cut into pof2 blocks of n / pof2 (the last one
- * takes the remainder); block k ends up on survivor bit_reverse(k): the first
- * exchange, at distance 1, already halves the data, the lower half staying with
- * the survivors whose lowest bit is clear. */
+/* TREE_RSG, TREE_RSG_SPREAD: the n elements are cut into pof2 blocks of
+ * n / pof2; the n % pof2 elements left over go to the last block (TREE_RSG:
+ * MPI_Ireduce, MPI_Iallreduce) or one each to the first n % pof2 blocks
+ * (TREE_RSG_SPREAD: MPI_Reduce, MPI_Allreduce).  Block k ends up on survivor
+ * bit_reverse(k): the first exchange, at distance 1, already halves the data,
+ * the lower half staying with the survivors whose lowest bit is clear. */
 int alo_rsg_blocks(int P) { return floor_pow2(P); }
-void alo_rsg_block(int P, size_t n, int k, size_t *lo, size_t *hi, int *owner) {
+void alo_rsg_block(int P, size_t n, int k, int spread, size_t *lo, size_t *hi, int *owner) {
   int pof2 = floor_pow2(P), bits = 0, o = 0;
-  size_t b = n / (size_t)pof2;
+  size_t b = n / (size_t)pof2, left = n % (size_t)pof2;
   while ((1 << bits) < pof2) bits++;
   for (int j = 0; j < bits; j++) if (k & (1 << j)) o |= 1 << (bits - 1 - j);
-  *lo = (size_t)k * b;
-  *hi = k == pof2 - 1 ? n : (size_t)(k + 1) * b;
+  if (spread) {
+    *lo = (size_t)k * b + ((size_t)k < left ? (size_t)k : left);
+    *hi = *lo + b + ((size_t)k < left ? 1 : 0);
+  } else {
+    *lo = (size_t)k * b;
+    *hi = k == pof2 - 1 ? n : (size_t)(k + 1) * b;
+  }
   *owner = o;
 }
 
@@ -528,13 +536,14 @@ static int combine_impl(void *out, const void *const *in, int P, size_t n,
   int *pairs = (int *)malloc(sizeof(int) * 2 * (size_t)(P > 1 ? P : 1));
   if (!pairs) return 3;
   int fail = 0;
-  /* one schedule for the whole range, except under TREE_RSG: one per block */
-  const int nblocks = order == ALO_ORDER_TREE_RSG ? alo_rsg_blocks(P) : 1;
-  if (order == ALO_ORDER_TREE_RSG && start != 0) { free(pairs); return 4; }
+  /* one schedule for the whole range, except under TREE_RSG(_SPREAD): one per block */
+  const int rsg = order == ALO_ORDER_TREE_RSG || order == ALO_ORDER_TREE_RSG_SPREAD;
+  const int nblocks = rsg ? alo_rsg_blocks(P) : 1;
+  if (rsg && start != 0) { free(pairs); return 4; }
   for (int k = 0; k < nblocks && !fail; k++) {
     size_t b_lo = 0, b_hi = n;
     int owner = start, result = 0;
-    if (order == ALO_ORDER_TREE_RSG) alo_rsg_block(P, n, k, &b_lo, &b_hi, &owner);
+    if (rsg) alo_rsg_block(P, n, k, order == ALO_ORDER_TREE_RSG_SPREAD, &b_lo, &b_hi, &owner);
     int np = alo_schedule(P, order, owner, pairs, &result);
     if (np < 0) { free(pairs); return 4; }
     const size_t bn = b_hi - b_lo, ntiles = (bn + ALO_TILE - 1) / ALO_TILE;

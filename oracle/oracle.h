@@ -25,16 +25,18 @@
  *     with (invec, inoutvec) argument order.
  *
  * Pin status (what checks each function against something other than itself):
- *   alo_step (int / f32 / f64), the TREE_BINOMIAL / TREE_RSG / TREE_DBL /
- *     TREE_HALV / PAIRWISE_DESC schedules: MPICH 3.3.2 golden vectors in
- *     tests/golden (MPI_Allreduce, MPI_Reduce to the first, second and last
- *     rank, MPI_Reduce_scatter_block, MPI_Reduce_scatter with uneven counts;
- *     the exact calls the reference makes; 2 to 16 ranks; fp32 / fp64 and, as
+ *   alo_step (int / f32 / f64), the TREE_BINOMIAL / TREE_RSG /
+ *     TREE_RSG_SPREAD / TREE_DBL / TREE_HALV / PAIRWISE_DESC schedules: MPICH
+ *     3.3.2 golden vectors in tests/golden (MPI_Allreduce, MPI_Reduce to the
+ *     first, second and last rank, MPI_Reduce_scatter_block, MPI_Reduce_scatter
+ *     with uneven counts, and their non-blocking in-place forms; the exact
+ *     calls the reference makes; 2 to 64 ranks; fp32 / fp64 and, as
  *     user-defined operations on MPI_SHORT the way the reference registers
  *     them, fp16 / bf16), numpy closed forms for the order-free integer ops.
  *     The vectors with NaN, signed zeros and infinities planted in every
- *     operand position (3, 4 and 8 ranks) pin which operand of every pair is
- *     the inoutvec, i.e. which one a tie or a NaN lets through.
+ *     operand position (3 to 64 ranks) pin which operand of every pair is
+ *     the inoutvec, i.e. which one a tie or a NaN lets through, and how the
+ *     blocking and the non-blocking calls cut a long message into blocks.
  *   alo_step (f16 / bf16): numpy float16 and torch bfloat16 arithmetic
  *     (library round-to-nearest-even narrowing), exhaustive over all 2^16
  *     values for widening, sampled + edge cases for narrowing.
@@ -88,12 +90,16 @@ enum {
                                   the running partial is the `in` operand    */
   ALO_ORDER_TREE_BINOMIAL = 5, /* binomial tree to rank s over the ranks
                                   counted from s with wrap (rooted reduce)   */
-  ALO_ORDER_TREE_RSG = 6       /* reduce-scatter + gather (MPI_Reduce and
-                                  MPI_Allreduce of long messages): the tree
+  ALO_ORDER_TREE_RSG = 6,      /* reduce-scatter + gather (MPI_Ireduce and
+                                  MPI_Iallreduce of long messages): the tree
                                   of TREE_DBL, but which rank of a pair keeps
                                   the result depends on the element's block;
                                   s must be 0 (in alo_schedule: the block's
                                   owner among the survivors)                 */
+  ALO_ORDER_TREE_RSG_SPREAD = 7 /* the same with the blocks that MPI_Reduce and
+                                  MPI_Allreduce cut: what count / 2^k leaves
+                                  over goes one element each to the first
+                                  blocks, not to the last block              */
 };
 
 /* Input distributions of the counter-based generator. */
@@ -146,10 +152,11 @@ int alo_divide(void *x, size_t n, int dtype, int ranks);
  * slot *result.  Returns the number of pairs, or -1 on bad arguments. */
 int alo_schedule(int P, int order, int start, int *pairs, int *result);
 
-/* TREE_RSG: the blocks the n elements are cut into, and the survivor that
- * ends up owning block k (what alo_schedule takes as `start`). */
+/* TREE_RSG (spread = 0) and TREE_RSG_SPREAD (spread = 1): the blocks the n
+ * elements are cut into, and the survivor that ends up owning block k (what
+ * alo_schedule takes as `start`). */
 int alo_rsg_blocks(int P);
-void alo_rsg_block(int P, size_t n, int k, size_t *lo, size_t *hi, int *owner);
+void alo_rsg_block(int P, size_t n, int k, int spread, size_t *lo, size_t *hi, int *owner);
 /* The `start` a Reduce_scatter passes for the block that rank b receives. */
 int alo_order_start(int order, int b);
 

@@ -206,8 +206,10 @@ int main(int argc, char **argv) {
       {"lxor", Al::ReductionOperator::lxor}, {"bor", Al::ReductionOperator::bor}, {"band", Al::ReductionOperator::band},
       {"bxor", Al::ReductionOperator::bxor}, {"avg", Al::ReductionOperator::avg}};
   const std::map<std::string, Algo> algos = {
-      {"automatic", Algo::automatic}, {"rank_order", Algo::rank_order}, {"tree_doubling", Algo::tree_doubling},
-      {"tree_halving", Algo::tree_halving}, {"tree_binomial", Algo::tree_binomial}, {"tree_reduce_scatter_gather", Algo::tree_reduce_scatter_gather}, {"pairwise", Algo::pairwise},
+      {"automatic", Algo::automatic}, {"automatic_mpi_blocking", Algo::automatic_mpi_blocking},
+      {"rank_order", Algo::rank_order}, {"tree_doubling", Algo::tree_doubling},
+      {"tree_halving", Algo::tree_halving}, {"tree_binomial", Algo::tree_binomial}, {"tree_reduce_scatter_gather", Algo::tree_reduce_scatter_gather},
+      {"tree_reduce_scatter_gather_spread", Algo::tree_reduce_scatter_gather_spread}, {"pairwise", Algo::pairwise},
       {"ring", Algo::ring}, {"ring_fused", Algo::ring_fused}};
   if (!rops.count(o.redop) || !algos.count(o.algo) || o.min_size == 0 ||
       (o.op != "allreduce" && o.op != "reduce" && o.op != "reduce_scatter" && o.op != "allgather" &&

@@ -54,6 +54,30 @@ template <typename T> std::vector<T> gen(size_t n, int dist, unsigned seed) {
   return v;
 }
 
+// The special values that tests/golden/mpich_golden.c (plant_specials_many) plants for more than two ranks:
+// element i of `rank` comes from a pool of NaN, zeros of both signs, infinities, denormals and a few
+// ordinary values by a fixed rule; every fourth element is a zero of one sign or the other.
+template <typename T> std::vector<T> planted(size_t n, int rank) {
+  static const uint32_t pool[] = {0x7fc00000u, 0xbf800000u, 0x00000000u, 0x80000000u, 0x7f800000u,
+                                  0xff800000u, 0x00000001u, 0x80000001u, 0x3f800000u, 0x7f7fffffu,
+                                  0x00800000u, 0x00400000u, 0x3e99999au};
+  const size_t cnt = sizeof(pool) / sizeof(pool[0]);
+  std::vector<T> v(n);
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t h = alo_mix64(77, (uint64_t)i * 64u + (uint64_t)rank);
+    uint32_t u = pool[(size_t)(h % cnt)];
+    if (i % 4 == 0) u = (h >> 32) % 3 == 0 ? 0x80000000u : 0u;
+    float f;
+    std::memcpy(&f, &u, 4);
+    if constexpr (std::is_same<T, float>::value) v[i] = f;
+    else if constexpr (std::is_same<T, double>::value) v[i] = (double)f;
+    else if constexpr (std::is_same<T, Al::amd::bfloat16_bits>::value) v[i].bits = alo_f32_to_bf16(f);
+    else if constexpr (std::is_same<T, Al::amd::half_bits>::value) v[i].bits = alo_f32_to_f16(f);
+    else v[i] = T();
+  }
+  return v;
+}
+
 // NaN payloads are outside the parity claim; the seeded inputs hold no NaN.
 template <typename T> bool same_bits(const std::vector<T> &a, const std::vector<T> &b) {
   return a.size() == b.size() && (a.empty() || std::memcmp(a.data(), b.data(), a.size() * sizeof(T)) == 0);
@@ -62,34 +86,34 @@ template <typename T> bool same_bits(const std::vector<T> &a, const std::vector<
 // The oracle's order for an algorithm of the front end.  `automatic` is stated here on its own, not
 // asked of the library: what MPICH 3.3.2 does on one host (pinned by the golden vectors in tests/golden;
 // test_backend's test_automatic_against_mpich checks the front end itself against that library's bits).
-static int order_of(Algo a, size_t bytes, bool reduce_scatter, size_t total_bytes) {
+static int order_of(Algo a, size_t total_bytes) {
   switch (a) {
-  case Algo::automatic:
+  case Algo::automatic:  // Reduce_scatter(v); Allreduce and Reduce go through rooted_order
+  case Algo::automatic_mpi_blocking:
     return total_bytes < (512u << 10) ? ALO_ORDER_TREE_HALV : ALO_ORDER_PAIRWISE_DESC;
   case Algo::rank_order: return ALO_ORDER_RANK_ASC;
   case Algo::tree_doubling: return ALO_ORDER_TREE_DBL;
   case Algo::tree_halving: return ALO_ORDER_TREE_HALV;
   case Algo::tree_binomial: return ALO_ORDER_TREE_BINOMIAL;
   case Algo::tree_reduce_scatter_gather: return ALO_ORDER_TREE_RSG;
+  case Algo::tree_reduce_scatter_gather_spread: return ALO_ORDER_TREE_RSG_SPREAD;
   case Algo::pairwise: return ALO_ORDER_PAIRWISE_DESC;
   default: return ALO_ORDER_RING;
   }
-  (void)bytes;
-  (void)reduce_scatter;
 }
 
 struct OrderPick { int order, start; };
 // Allreduce (root = 0) and Reduce.
 static OrderPick rooted_order(Algo a, int dt, size_t count, size_t elem_size, int P, int root) {
-  if (a == Algo::automatic) {
+  if (a == Algo::automatic || a == Algo::automatic_mpi_blocking) {
     size_t pof2 = 1;
     while (2 * pof2 <= (size_t)P) pof2 *= 2;
     const bool user_op = dt == ALO_F16 || dt == ALO_BF16;
     if (user_op || count * elem_size <= 2048 || count < pof2) return {ALO_ORDER_TREE_BINOMIAL, root};
-    return {ALO_ORDER_TREE_RSG, 0};
+    return {a == Algo::automatic ? ALO_ORDER_TREE_RSG : ALO_ORDER_TREE_RSG_SPREAD, 0};
   }
   if (a == Algo::tree_binomial) return {ALO_ORDER_TREE_BINOMIAL, root};
-  return {order_of(a, 0, false, 0), 0};
+  return {order_of(a, 0), 0};
 }
 
 template <typename T>
@@ -217,7 +241,7 @@ void test_reduce_scatter(int P, size_t count, Op op, Algo algo, bool inplace, hi
   std::vector<void *> rp;
   for (int r = 0; r < P; ++r) { sp.push_back(in[r].data()); rp.push_back(want[r].data()); }
   alo_reduce_scatter(rp.data(), sp.data(), P, count, dt, (int)op,
-                     algo == Algo::ring_fused ? ALO_ORDER_RING : order_of(algo, 0, true, n * sizeof(T)));
+                     algo == Algo::ring_fused ? ALO_ORDER_RING : order_of(algo, n * sizeof(T)));
   for (int r = 0; r < P; ++r) {
     auto got = inplace ? send[r]->down() : recv[r]->down();
     got.resize(count);  // in place the result is at the start of the buffer
@@ -294,7 +318,7 @@ void test_v_variants(int P, bool inplace, hipStream_t stream, bool nonblocking =
     for (int r = 0; r < P; ++r) { want.emplace_back(counts[r] ? counts[r] : 1); sp.push_back(in[r].data()); }
     for (int r = 0; r < P; ++r) rp.push_back(want[r].data());
     alo_reduce_scatterv(rp.data(), sp.data(), P, counts.data(), dt, (int)op,
-                        order_of(Algo::automatic, 0, true, total * sizeof(T)));
+                        order_of(Algo::automatic, total * sizeof(T)));
     for (int r = 0; r < P; ++r) {
       auto got = inplace ? send[r]->down() : recv[r]->down();
       got.resize(counts[r]);

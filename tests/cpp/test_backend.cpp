@@ -56,9 +56,13 @@ static void test_errors(hipStream_t stream) {
 // above each size at which that library changes algorithm, fp32 / fp64 / fp16 / bf16 and integers).
 // The front end, left to choose its order, must return the same bytes.  No oracle in between.
 template <typename T>
-static void run_mpich_case(const std::string &coll, int P, Op op, size_t n, int dist, unsigned seed, int root,
+static void run_mpich_case(std::string coll, int P, Op op, size_t n, int dist, unsigned seed, int root,
                            const std::vector<size_t> &counts, const std::vector<std::string> &want, hipStream_t stream) {
   const int dt = Al::amd::TypeMap<T>::value;
+  // "..._blocking": what MPI_Allreduce / MPI_Reduce returned, the others what the non-blocking calls did
+  Algo algo = Algo::automatic;
+  const size_t tag = coll.find("_blocking");
+  if (tag != std::string::npos) { coll = coll.substr(0, tag); algo = Algo::automatic_mpi_blocking; }
   const bool scatter = coll == "reduce_scatter" || coll == "reduce_scatterv";
   size_t in_len = n;
   if (coll == "reduce_scatter") in_len = n * (size_t)P;
@@ -67,7 +71,9 @@ static void run_mpich_case(const std::string &coll, int P, Op op, size_t n, int 
   for (int r = 0; r < P; ++r) {
     send.emplace_back(new DevBuf<T>(in_len));
     recv.emplace_back(new DevBuf<T>(in_len));
-    if (alamd_fill(send[r]->p, in_len, dt, dist, seed + (unsigned)r, 0, stream) != ALAMD_OK) {
+    if (dist == 99) {  // planted special values
+      send[r]->up(planted<T>(in_len, r));
+    } else if (alamd_fill(send[r]->p, in_len, dt, dist, seed + (unsigned)r, 0, stream) != ALAMD_OK) {
       EXPECT(false, "alamd_fill: %s", alamd_last_error());
       return;
     }
@@ -76,8 +82,8 @@ static void run_mpich_case(const std::string &coll, int P, Op op, size_t n, int 
   for (int r = 0; r < P; ++r) {
     auto &comm = world.comm(r);
     const T *src = send[r]->p;
-    if (coll == "allreduce") Al::Allreduce<Backend>(src, recv[r]->p, n, op, comm);
-    else if (coll == "reduce") Al::Reduce<Backend>(src, recv[r]->p, n, op, root, comm);
+    if (coll == "allreduce") Al::Allreduce<Backend>(src, recv[r]->p, n, op, comm, algo);
+    else if (coll == "reduce") Al::Reduce<Backend>(src, recv[r]->p, n, op, root, comm, algo);
     else if (coll == "reduce_scatter") Al::Reduce_scatter<Backend>(src, recv[r]->p, n, op, comm);
     else Al::Reduce_scatterv<Backend>(src, recv[r]->p, counts, op, comm);
   }
@@ -89,8 +95,8 @@ static void run_mpich_case(const std::string &coll, int P, Op op, size_t n, int 
     char cs[32];
     std::snprintf(cs, sizeof(cs), "%016llx", (unsigned long long)alo_checksum(got.data(), len * sizeof(T)));
     const std::string &w = scatter ? want[(size_t)r] : want[0];
-    EXPECT(w == cs, "%s against MPICH: P=%d dt=%d op=%d n=%zu root=%d rank %d: %s, MPICH %s", coll.c_str(), P, dt, (int)op,
-           len, root, r, cs, w.c_str());
+    EXPECT(w == cs, "%s%s against MPICH: P=%d dt=%d op=%d n=%zu root=%d rank %d: %s, MPICH %s", coll.c_str(),
+           algo == Algo::automatic ? "" : " (blocking)", P, dt, (int)op, len, root, r, cs, w.c_str());
   }
 }
 
@@ -107,7 +113,7 @@ static void test_automatic_against_mpich(hipStream_t stream) {
   static const std::map<std::string, Op> ops = {
       {"sum", Op::sum}, {"prod", Op::prod}, {"min", Op::min}, {"max", Op::max}, {"lor", Op::lor}, {"land", Op::land},
       {"lxor", Op::lxor}, {"bor", Op::bor}, {"band", Op::band}, {"bxor", Op::bxor}};
-  int ran = 0, reduces = 0, halves = 0;
+  int ran = 0, reduces = 0, halves = 0, blocking = 0, specials = 0, many = 0;
   std::string line;
   while (std::getline(f, line)) {
     if (line.empty() || line[0] == '#') continue;
@@ -120,7 +126,7 @@ static void test_automatic_against_mpich(hipStream_t stream) {
     in >> coll >> P >> dtype >> opname;
     if (coll != "reduce_scatterv") in >> n;
     in >> dist >> seed;
-    if (coll == "reduce") in >> root;
+    if (coll == "reduce" || coll == "reduce_blocking") in >> root;
     if (coll == "reduce_scatterv")
       for (int b = 0; b < P; ++b) { size_t c = 0; in >> c; counts.push_back(c); }
     std::vector<std::string> want;
@@ -138,9 +144,13 @@ static void test_automatic_against_mpich(hipStream_t stream) {
     ++ran;
     reduces += coll == "reduce";
     halves += dtype == "f16" || dtype == "bf16";
+    blocking += coll.find("_blocking") != std::string::npos;
+    specials += dist == 99;
+    many += P >= 32;
   }
-  EXPECT(ran >= 800 && reduces >= 250 && halves >= 150, "too few cases: %d in all, %d reduces, %d of 16-bit floats", ran,
-         reduces, halves);
+  EXPECT(ran >= 1000 && reduces >= 250 && halves >= 150 && blocking >= 150 && specials >= 100 && many >= 50,
+         "too few cases: %d in all, %d reduces, %d of 16-bit floats, %d of the blocking calls, %d with special values, "
+         "%d for 32 ranks and more", ran, reduces, halves, blocking, specials, many);
 }
 
 // One rank's thread polls Test on its request while another thread makes the last call, which launches

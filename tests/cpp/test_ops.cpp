@@ -8,7 +8,8 @@
 //
 // usage: test_ops --op allreduce|reduce|reduce_scatter|allgather|reduce_scatterv|allgatherv
 //                 [--backend hip] [--inplace] [--nonblocking] [--reduction-op sum|prod|min|max|lor|land|lxor|bor|band|bxor]
-//                 [--algorithm automatic|rank_order|tree_doubling|tree_halving|tree_binomial|tree_reduce_scatter_gather|pairwise|ring|ring_fused]
+//                 [--algorithm automatic|automatic_mpi_blocking|rank_order|tree_doubling|tree_halving|tree_binomial|
+//                  tree_reduce_scatter_gather|tree_reduce_scatter_gather_spread|pairwise|ring|ring_fused]
 //                 [--root R] [--size N | --min-size N --max-size N] [--odd-sizes] [--datatype float|...]
 //                 [--trials N] [--ranks P] [--threads N]
 #include <map>
@@ -125,9 +126,11 @@ int main(int argc, char **argv) {
       {"sum", Op::sum}, {"prod", Op::prod}, {"min", Op::min}, {"max", Op::max}, {"lor", Op::lor}, {"land", Op::land},
       {"lxor", Op::lxor}, {"bor", Op::bor}, {"band", Op::band}, {"bxor", Op::bxor}, {"avg", Op::avg}};
   static const std::map<std::string, Algo> algos = {
-      {"automatic", Algo::automatic}, {"", Algo::automatic}, {"rank_order", Algo::rank_order},
+      {"automatic", Algo::automatic}, {"", Algo::automatic}, {"automatic_mpi_blocking", Algo::automatic_mpi_blocking},
+      {"rank_order", Algo::rank_order},
       {"tree_doubling", Algo::tree_doubling}, {"tree_halving", Algo::tree_halving},
-      {"tree_binomial", Algo::tree_binomial}, {"tree_reduce_scatter_gather", Algo::tree_reduce_scatter_gather}, {"pairwise", Algo::pairwise}, {"ring", Algo::ring},
+      {"tree_binomial", Algo::tree_binomial}, {"tree_reduce_scatter_gather", Algo::tree_reduce_scatter_gather},
+      {"tree_reduce_scatter_gather_spread", Algo::tree_reduce_scatter_gather_spread}, {"pairwise", Algo::pairwise}, {"ring", Algo::ring},
       {"ring_fused", Algo::ring_fused}};
   static const char *ops[] = {"allreduce", "reduce", "reduce_scatter", "allgather", "reduce_scatterv", "allgatherv"};
   bool op_ok = false;

@@ -1,6 +1,10 @@
 """Writes mpich_front_end_cases.txt from the mpich_P*.json.gz fixtures next to it: one line per case whose
-inputs are the generator's, with the checksum of what MPICH returned.  The C++ front end's tests read it
-(no JSON or gzip there) to check that `automatic` gives MPICH's bits for every collective, root and size.
+inputs are the generator's (or, distribution 99, the special values planted by the rule of mpich_golden.c's
+plant_specials_many: float min / max only, whose result is one of the operands bit for bit), with the
+checksum of what MPICH returned.  The C++ front end's tests read it (no JSON or gzip there) to check that
+`automatic` gives MPICH's bits for every collective, root and size.  "allreduce" and "reduce" lines hold what
+the non-blocking calls returned (`automatic`); for long messages of native types "allreduce_blocking" and
+"reduce_blocking" lines hold what MPI_Allreduce and MPI_Reduce returned (`automatic_mpi_blocking`).
 
     python tests/golden/export_front_end_cases.py
 """
@@ -29,15 +33,24 @@ def main():
             doc = json.load(f)
         P = doc["P"]
         for c in doc["cases"]:
-            if c["note"] == "specials":
+            planted = c["note"] == "specials"
+            if planted and (P == 2 or c["op"] not in ("min", "max") or c["coll"] not in ("allreduce", "reduce")):
                 continue
             head = "%s %d %s %s" % (c["coll"], P, c["dtype"], c["op"])
-            gen = "%d %d" % (c["dist"], c["seed_base"])
+            gen = "%d %d" % (99 if planted else c["dist"], c["seed_base"])
+            long_native = c["dtype"] not in ("f16", "bf16") and c["n"] * oracle.dtype_size(c["dtype"]) > 2048
             if c["coll"] == "allreduce":
-                lines.append("%s %d %s %s" % (head, c["n"], gen, cs_hex(c["out"][0])))
+                lines.append("%s %d %s %s" % (head, c["n"], gen, cs_hex(c.get("out_nonblocking", c["out"][0]))))
+                if long_native:
+                    lines.append("allreduce_blocking %s %d %s %s" % (head.split(" ", 1)[1], c["n"], gen, cs_hex(c["out"][0])))
             elif c["coll"] == "reduce":
                 cs = c["out_checksum"] if "out_checksum" in c else cs_hex(c["out"])
-                lines.append("%s %d %s %d %s" % (head, c["n"], gen, c["root"], cs))
+                nb = cs
+                if not c["nonblocking_in_place_same"]:
+                    nb = c["out_nonblocking_checksum"] if "out_nonblocking_checksum" in c else cs_hex(c["out_nonblocking"])
+                lines.append("%s %d %s %d %s" % (head, c["n"], gen, c["root"], nb))
+                if long_native:
+                    lines.append("reduce_blocking %s %d %s %d %s" % (head.split(" ", 1)[1], c["n"], gen, c["root"], cs))
             elif c["coll"] == "reduce_scatter":
                 cs = c["out_checksum"] if "out_checksum" in c else [cs_hex(h) for h in c["out"]]
                 lines.append("%s %d %s %s" % (head, c["n"], gen, " ".join(cs)))

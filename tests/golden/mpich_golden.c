@@ -83,7 +83,10 @@ static int on_all(int mine) {
 
 /* The host-transfer backend makes the non-blocking, in-place form of every call
  * (include/aluminum/ht/allreduce.hpp:76-79, ht/reduce.hpp:72-82, ht/reduce_scatter.hpp:71-74,
- * ht/reduce_scatterv.hpp:76-79); every case records whether that form returned the same bytes. */
+ * ht/reduce_scatterv.hpp:76-79); every case records whether that form returned the same bytes, and
+ * what it returned where it did not ("out_nonblocking": MPI_Ireduce and MPI_Iallreduce cut a long
+ * message into blocks differently from MPI_Reduce and MPI_Allreduce, which shows where a float
+ * min / max meets a tie or a NaN and the count is not a multiple of the power of two of ranks). */
 static void emit_nb(int same) {
   if (rank_ == 0) printf(", \"nonblocking_in_place_same\": %s", same ? "true" : "false");
 }
@@ -95,6 +98,9 @@ static void print_hex(const unsigned char *p, size_t nbytes) {
 }
 
 static int first_case = 1;
+/* 32 ranks and more: an allreduce keeps rank 0's output only (and records that every rank received the
+ * same bytes), and no case repeats its inputs. */
+static int lean_ = 0;
 
 /* Gather `nbytes` from every rank to rank 0 and print as a JSON list. */
 static void emit_list(const char *key, const void *mine, size_t nbytes) {
@@ -201,9 +207,31 @@ static void case_allreduce(int dt, int op, size_t n, int dist, int specials,
   int same = on_all(memcmp(nb, out, n * es) == 0);
   head("allreduce", dt, op, n, dist, seed, note);
   emit_nb(same);
-  /* inputs are repeated for short messages and planted values; the others are the generator's */
-  if ((specials && n * es <= 2048) || (!is_half(dt) && (specials || n * es <= 2048))) emit_list("in", in, n * es);
-  emit_list("out", out, n * es);
+  if (!same) { /* rank 0's, and whether every rank received those bytes */
+    void *nb0 = malloc(n * es);
+    memcpy(nb0, nb, n * es);
+    MPI_Bcast(nb0, (int)(n * es), MPI_BYTE, 0, MPI_COMM_WORLD);
+    int nb_same = on_all(memcmp(nb0, nb, n * es) == 0);
+    if (rank_ == 0) {
+      printf(", \"nonblocking_all_ranks_same\": %s, \"out_nonblocking\": ", nb_same ? "true" : "false");
+      print_hex((unsigned char *)nb, n * es);
+    }
+    free(nb0);
+  }
+  if (lean_) {
+    memcpy(nb, out, n * es);
+    MPI_Bcast(nb, (int)(n * es), MPI_BYTE, 0, MPI_COMM_WORLD);
+    int all_same = on_all(memcmp(nb, out, n * es) == 0);
+    if (rank_ == 0) {
+      printf(", \"all_ranks_same\": %s, \"out\": [", all_same ? "true" : "false");
+      print_hex((unsigned char *)out, n * es);
+      printf("]");
+    }
+  } else {
+    /* inputs are repeated for short messages; the others are the generator's, or planted by rule */
+    if (n * es <= 2048 && (specials || !is_half(dt))) emit_list("in", in, n * es);
+    emit_list("out", out, n * es);
+  }
   tail();
   free(in); free(out); free(nb);
 }
@@ -227,7 +255,7 @@ static void case_reduce_scatter_x(int dt, int op, size_t count, int dist, int fu
   head("reduce_scatter", dt, op, count, dist, seed, note);
   emit_nb(same);
   if (full) {
-    if (!is_half(dt) || specials) emit_list("in", in, n * es);
+    if ((!is_half(dt) || specials) && !lean_) emit_list("in", in, n * es);
     emit_list("out", out, count * es);
   } else {
     emit_sums("out_checksum", out, count * es);
@@ -287,17 +315,23 @@ static void case_reduce(int dt, int op, size_t n, int dist, int root, int specia
   else MPI_Ireduce(nb, NULL, (int)n, mpi_type(dt), op_for(dt, op), root, MPI_COMM_WORLD, &req);
   MPI_Wait(&req, MPI_STATUS_IGNORE);
   int same = on_all(rank_ != root || memcmp(nb, out, n * es) == 0);
-  free(nb);
-  if (root != 0) { /* bring the root's result to rank 0, which prints */
+  if (root != 0) { /* bring the root's results to rank 0, which prints */
     if (rank_ == root) MPI_Send(out, (int)(n * es), MPI_BYTE, 0, 7, MPI_COMM_WORLD);
     if (rank_ == 0) MPI_Recv(out, (int)(n * es), MPI_BYTE, root, 7, MPI_COMM_WORLD, MPI_STATUS_IGNORE);
+    if (rank_ == root) MPI_Send(nb, (int)(n * es), MPI_BYTE, 0, 8, MPI_COMM_WORLD);
+    if (rank_ == 0) MPI_Recv(nb, (int)(n * es), MPI_BYTE, root, 8, MPI_COMM_WORLD, MPI_STATUS_IGNORE);
   }
   head("reduce", dt, op, n, dist, seed, note);
   if (rank_ == 0) printf(", \"root\": %d", root);
   emit_nb(same);
+  if (!same && rank_ == 0) {
+    if (n <= 1024) { printf(", \"out_nonblocking\": "); print_hex((unsigned char *)nb, n * es); }
+    else printf(", \"out_nonblocking_checksum\": \"%016llx\"", (unsigned long long)alo_checksum(nb, n * es));
+  }
+  free(nb);
   if (n <= 1024) {
-    /* inputs other than the planted ones are the generator's and not repeated here */
-    if (specials) emit_list("in", in, n * es);
+    /* inputs are repeated for short messages; the others are the generator's, or planted by rule */
+    if (specials && !lean_ && n * es <= 2048) emit_list("in", in, n * es);
     if (rank_ == 0) { printf(", \"out\": "); print_hex((unsigned char *)out, n * es); }
   } else if (rank_ == 0) {
     printf(", \"out_checksum\": \"%016llx\", \"out_head\": ", (unsigned long long)alo_checksum(out, n * es));
@@ -356,6 +390,35 @@ int main(int argc, char **argv) {
     printf("{\"mpi\": \"%s\", \"P\": %d, \"cases\": [", ver, P_);
   }
 
+  if (P_ >= 32) {
+    /* Many ranks (the tree orders over 32 slots and over two halves of 32; pre-folds of up to 31 pairs): a
+     * small set, outputs only.  Inputs are the generator's, or planted by rule. */
+    lean_ = 1;
+    const size_t nlong = 2048 / 4 + 8;
+    const int roots[3] = {0, 1, P_ - 1};
+    case_allreduce(ALO_F32, ALO_SUM, 16, ALO_DIST_UNIFORM_PM1, 0, "short message");
+    case_allreduce(ALO_F32, ALO_SUM, nlong, ALO_DIST_UNIFORM_PM1, 0, "long message");
+    case_allreduce(ALO_F32, ALO_PROD, nlong, ALO_DIST_UNIFORM_09_11, 0, "long message");
+    case_allreduce(ALO_F64, ALO_SUM, nlong, ALO_DIST_UNIFORM_PM1, 0, "long message");
+    case_allreduce(ALO_BF16, ALO_SUM, 2 * nlong, ALO_DIST_UNIFORM_PM1, 0, "long message");
+    case_allreduce(ALO_F32, ALO_MIN, nlong + 3, ALO_DIST_UNIFORM_PM1, 1, "specials");
+    case_allreduce(ALO_F32, ALO_MAX, 96, ALO_DIST_UNIFORM_PM1, 1, "specials");
+    for (int k = 0; k < 3; k++) {
+      case_reduce(ALO_F32, ALO_SUM, 16, ALO_DIST_UNIFORM_PM1, roots[k], 0, "short message");
+      case_reduce(ALO_F32, ALO_SUM, nlong, ALO_DIST_UNIFORM_PM1, roots[k], 0, "long message");
+      case_reduce(ALO_BF16, ALO_SUM, 2 * nlong, ALO_DIST_UNIFORM_PM1, roots[k], 0, "long message");
+      case_reduce(ALO_F32, ALO_MAX, nlong + 3, ALO_DIST_UNIFORM_PM1, roots[k], 1, "specials");
+    }
+    case_reduce_scatter(ALO_F32, ALO_SUM, 8, ALO_DIST_UNIFORM_PM1, 1, "short message");
+    case_reduce_scatter_x(ALO_F32, ALO_MIN, 8, ALO_DIST_UNIFORM_PM1, 1, 1, "specials");
+    if (big)
+      case_reduce_scatter(ALO_F32, ALO_SUM, (size_t)(1u << 20) / (size_t)P_ / 4 + 64, ALO_DIST_UNIFORM_PM1, 0,
+                          "long message");
+    if (rank_ == 0) printf("\n]}\n");
+    MPI_Finalize();
+    return 0;
+  }
+
   /* fp sum / prod: 16 elements (<= 2048 bytes) and just over 2048 bytes. */
   const int fdt[2] = {ALO_F32, ALO_F64};
   for (int d = 0; d < 2; d++) {
@@ -370,10 +433,10 @@ int main(int argc, char **argv) {
       for (int op = ALO_SUM; op <= ALO_MAX; op++)
         case_allreduce(fdt[d], op, 48, ALO_DIST_UNIFORM_PM1, 1, "specials");
     }
-    if (P_ == 3 || P_ == 4 || P_ == 8) { /* special values under a whole order; every rank's output is kept */
+    if (P_ == 3 || P_ == 4 || P_ == 7 || P_ == 8 || P_ == 16) { /* special values under a whole order; every rank's output is kept */
       for (int op = ALO_SUM; op <= ALO_MAX; op++) {
         case_allreduce(fdt[d], op, 96, ALO_DIST_UNIFORM_PM1, 1, "specials");
-        case_allreduce(fdt[d], op, nlong, ALO_DIST_UNIFORM_PM1, 1, "specials");
+        case_allreduce(fdt[d], op, nlong + 3, ALO_DIST_UNIFORM_PM1, 1, "specials"); /* not a multiple of 2^k */
       }
     }
     /* rooted reduce: first, second and last rank as root, below and above 2048 bytes */
@@ -385,10 +448,10 @@ int main(int argc, char **argv) {
       case_reduce(fdt[d], ALO_PROD, 16, ALO_DIST_UNIFORM_09_11, roots[k], 0, "short message");
       case_reduce(fdt[d], ALO_PROD, nlong, ALO_DIST_UNIFORM_09_11, roots[k], 0, "long message");
       if (big) case_reduce(fdt[d], ALO_SUM, (size_t)(1u << 18) + 3, ALO_DIST_UNIFORM_PM1, roots[k], 0, "1 MiB and more");
-      if ((P_ == 3 || P_ == 4 || P_ == 8) && (d == 0 || k == 1))
+      if ((P_ == 3 || P_ == 4 || P_ == 7 || P_ == 8 || P_ == 16) && (d == 0 || k == 1))
         for (int op = ALO_MIN; op <= ALO_MAX; op++) {
           case_reduce(fdt[d], op, 96, ALO_DIST_UNIFORM_PM1, roots[k], 1, "specials");
-          case_reduce(fdt[d], op, nlong, ALO_DIST_UNIFORM_PM1, roots[k], 1, "specials");
+          case_reduce(fdt[d], op, nlong + 3, ALO_DIST_UNIFORM_PM1, roots[k], 1, "specials");
         }
     }
     case_reduce_scatter(fdt[d], ALO_SUM, 8, ALO_DIST_UNIFORM_PM1, 1, "short message");

@@ -117,6 +117,8 @@ OPS_SWEEPS = [
     "--op reduce --datatype float --reduction-op max --root 3 --algorithm tree_reduce_scatter_gather --odd-sizes --max-size 65536 --ranks 5",
     "--op allreduce --datatype double --reduction-op min --algorithm tree_reduce_scatter_gather --inplace --max-size 65536 --ranks 7",
     "--op reduce_scatter --datatype float --reduction-op min --algorithm tree_halving --odd-sizes --max-size 16384 --ranks 6",
+    "--op allreduce --datatype float --reduction-op min --algorithm tree_reduce_scatter_gather_spread --odd-sizes --max-size 65536 --ranks 6",
+    "--op reduce --datatype double --root 2 --algorithm automatic_mpi_blocking --odd-sizes --max-size 65536 --ranks 12",
     # non-blocking operations that move more than 256 MiB in all take the internal stream
     "--op allreduce --datatype double --nonblocking --odd-sizes --min-size 1048576 --max-size 4194304 --ranks 8",
     "--op reduce_scatter --datatype float --nonblocking --inplace --min-size 1048576 --max-size 2097152 --ranks 8",

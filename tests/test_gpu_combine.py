@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from util import (ALL_DTYPES, FLOAT_DTYPES, INT_DTYPES, ORDERS, assert_bits_equal, dev_empty,
+from util import (ALL_DTYPES, FLOAT_DTYPES, INT_DTYPES, ORDERS, assert_bits_equal, dev_empty, planted_specials,
                   ops_of, to_dev, to_host)
 
 pytestmark = pytest.mark.gpu
@@ -195,6 +195,38 @@ def test_combine_special_values(al, dtype):
             want = oracle.combine(ins, dtype, op, order, start)
             got = run_combine(al, ins, dtype, op, order, start)[0]
             assert_bits_equal(got, want, dtype, "%s %s %s" % (dtype, op, order))
+
+
+@pytest.mark.parametrize("P", (3, 5, 8, 12, 16, 33, 48, 64))
+def test_float_min_max_operand_roles_over_many_tiles(al, P):
+    """Zeros of both signs and NaNs in every operand position (the inputs of the golden vectors' special
+    cases), over messages of many tiles whose blocks end inside tiles and whose length is no multiple of
+    the power of two of ranks: which operand of every pair lets a tie through depends on the order, the
+    start and, under the reduce-scatter + gather orders, on the block the element lies in."""
+    import torch
+    for dtype, n in (("f32", 70001), ("bf16", 33333), ("f64", 20011)):
+        ins = [planted_specials(n, dtype, r) for r in range(P)]
+        d_ins = [to_dev(a) for a in ins]
+        for op in ("min", "max"):
+            for order, start in (("tree_rsg", 0), ("tree_rsg_spread", 0), ("tree_halv", 0), ("tree_halv", P - 1),
+                                 ("tree_halv", P // 2), ("tree_binomial", P // 3), ("tree_dbl", 0)):
+                want = oracle.combine(ins, dtype, op, order, start)
+                outs = [dev_empty(n, ins[0].dtype) for _ in range(2)]
+                al.combine(outs, d_ins, op, order=order, start=start, dtype=dtype, count=n)
+                torch.cuda.synchronize()
+                for o in outs:
+                    assert_bits_equal(to_host(o, ins[0].dtype), want, dtype, "%s %s P=%d %s start %d" % (dtype, op, P, order, start))
+    # ... and a reduce-scatter, whose tree orders take the receiving rank as start block by block
+    count = 1031
+    sends = [planted_specials(P * count, "f32", r) for r in range(P)]
+    d_sends = [to_dev(a) for a in sends]
+    for order in ("tree_halv", "tree_rsg", "tree_rsg_spread"):
+        want = oracle.reduce_scatter(sends, "f32", "min", order)
+        recvs = [dev_empty(count, np.float32) for _ in range(P)]
+        al.reduce_scatter(recvs, d_sends, "min", order=order, dtype="f32", count=count)
+        torch.cuda.synchronize()
+        for r in range(P):
+            assert_bits_equal(to_host(recvs[r], np.float32), want[r], "f32", "reduce_scatter min P=%d %s rank %d" % (P, order, r))
 
 
 @pytest.mark.parametrize("dtype", ("f32", "bf16", "u8", "i64"))

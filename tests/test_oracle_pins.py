@@ -250,8 +250,8 @@ def test_orders_against_brute_force(P):
         if dist == "bool01":
             ins = [np.where(a == 0, np.where(np.arange(n) % (r + 2) == 0, -0.0, 0.0), a) for r, a in enumerate(ins)]
         for order in oracle.ORDERS:
-            if order == "tree_rsg":
-                continue  # depends on the element's position: see the simulation below
+            if order in ("tree_rsg", "tree_rsg_spread"):
+                continue  # depend on the element's position: see the simulation below
             starts = range(P) if order in ("pairwise_desc", "ring", "tree_binomial", "tree_halv") else (0,)
             for start in starts:
                 got = oracle.combine(ins, "f64", op, order, start)
@@ -259,11 +259,13 @@ def test_orders_against_brute_force(P):
                 assert got.tobytes() == want.tobytes(), (P, op, order, start)
 
 
-def simulate_reduce_scatter_gather(ins, dtype, op):
+def simulate_reduce_scatter_gather(ins, dtype, op, spread=False):
     """P ranks exchanging messages: a reduce-scatter by recursive halving of the data at distance 1, 2,
     4, ... (odd ranks among the first 2 * rem hand their data to the even rank below them first; what
     a rank receives is the invec of its step, what it holds the inoutvec), then the blocks gathered from
-    their owners.  The vector that MPI_Reduce and MPI_Allreduce of a long message leave at the root."""
+    their owners.  The vector that a reduce or allreduce of a long message leaves at the root; what the
+    count is not a multiple of goes to the last block (MPI_Ireduce, MPI_Iallreduce) or, `spread`, one
+    element each to the first blocks (MPI_Reduce, MPI_Allreduce)."""
     P, n = len(ins), ins[0].size
     pof2 = 1 << (P.bit_length() - 1)
     rem = P - pof2
@@ -272,7 +274,12 @@ def simulate_reduce_scatter_gather(ins, dtype, op):
     for j in range(rem):
         buf[2 * j] = oracle.step(buf[2 * j], buf[2 * j + 1], dtype, op)
     cnts = [n // pof2] * pof2
-    cnts[-1] = n - (n // pof2) * (pof2 - 1)
+    if spread:
+        for k in range(n % pof2):
+            cnts[k] += 1
+    else:
+        cnts[-1] = n - (n // pof2) * (pof2 - 1)
+    assert sum(cnts) == n
     disps = [sum(cnts[:k]) for k in range(pof2 + 1)]
     lo_hi = {nr: (0, pof2) for nr in range(pof2)}  # the blocks a rank still works on
     mask = 1
@@ -343,9 +350,10 @@ def test_tree_rsg_against_a_message_passing_simulation(P):
             continue
         for op in ("sum", "min", "max"):
             ins = [specials(n, 900 + r) if op != "sum" else oracle.fill(n, "f32", "uniform_pm1", 900 + r) for r in range(P)]
-            got = oracle.combine(ins, "f32", op, "tree_rsg")
-            want = simulate_reduce_scatter_gather(ins, "f32", op)
-            assert_same(got, want, (P, n, op))
+            for spread in (False, True):
+                got = oracle.combine(ins, "f32", op, "tree_rsg_spread" if spread else "tree_rsg")
+                want = simulate_reduce_scatter_gather(ins, "f32", op, spread)
+                assert_same(got, want, (P, n, op, spread))
 
 
 @pytest.mark.parametrize("P", (2, 3, 4, 5, 6, 7, 8, 12, 16))

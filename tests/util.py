@@ -9,7 +9,8 @@ INT_DTYPES = ("i8", "u8", "i16", "u16", "i32", "u32", "i64", "u64")
 ALL_DTYPES = INT_DTYPES + FLOAT_DTYPES
 FP_OPS = ("sum", "prod", "min", "max", "avg")
 INT_OPS = ("sum", "prod", "min", "max", "lor", "land", "lxor", "bor", "band", "bxor", "avg")
-ORDERS = ("rank_asc", "tree_dbl", "tree_halv", "pairwise_desc", "ring", "tree_binomial", "tree_rsg")
+ORDERS = ("rank_asc", "tree_dbl", "tree_halv", "pairwise_desc", "ring", "tree_binomial", "tree_rsg",
+          "tree_rsg_spread")
 
 
 def floor_pow2(p):
@@ -19,20 +20,23 @@ def floor_pow2(p):
     return q
 
 
-def mpich_order(coll, dtype, count, P, root=0, total=None):
+def mpich_order(coll, dtype, count, P, root=0, total=None, blocking=False):
     """(order, start) that MPICH 3.3.2 on one host follows for the call the reference makes - what the
     golden vectors in tests/golden establish.  Rooted reduce and allreduce (the latter is a reduce to
     rank 0 followed by a broadcast): binomial tree to the root over the ranks counted from it, up to
     2048 bytes, for fewer elements than the largest power of two of ranks, and for every user-defined
     operation (fp16 / bf16); above that a reduce-scatter by recursive halving plus gather, whatever the
-    root.  Reduce_scatter (block or not): recursive halving below 512 KiB in all, pairwise exchange from
+    root - MPI_Ireduce and MPI_Iallreduce (which the host-transfer backend and the MPI backend's
+    non-blocking calls make) leave what the count is not a multiple of to the last block, MPI_Reduce and
+    MPI_Allreduce (`blocking`: the MPI backend's blocking calls) spread it over the first blocks.
+    Reduce_scatter (block or not): recursive halving below 512 KiB in all, pairwise exchange from
     there on; `start` is then added per receiving rank by the collective itself."""
     es = {"f16": 2, "bf16": 2, "f32": 4, "f64": 8}.get(dtype) or int("".join(c for c in dtype if c.isdigit())) // 8
     if coll in ("allreduce", "reduce"):
         r = root if coll == "reduce" else 0
         if dtype in ("f16", "bf16") or count * es <= 2048 or count < floor_pow2(P):
             return "tree_binomial", r
-        return "tree_rsg", 0
+        return ("tree_rsg_spread" if blocking else "tree_rsg"), 0
     if coll in ("reduce_scatter", "reduce_scatterv"):
         total = count * P if total is None else total
         return ("tree_halv" if total * es < (512 << 10) else "pairwise_desc"), 0
