@@ -101,6 +101,8 @@ static int first_case = 1;
 /* 32 ranks and more: an allreduce keeps rank 0's output only (and records that every rank received the
  * same bytes), and no case repeats its inputs. */
 static int lean_ = 0;
+/* Set while cases are made whose inputs, the generator's, need not be repeated whatever their size. */
+static int no_inputs_ = 0;
 
 /* Gather `nbytes` from every rank to rank 0 and print as a JSON list. */
 static void emit_list(const char *key, const void *mine, size_t nbytes) {
@@ -229,7 +231,7 @@ static void case_allreduce(int dt, int op, size_t n, int dist, int specials,
     }
   } else {
     /* inputs are repeated for short messages; the others are the generator's, or planted by rule */
-    if (n * es <= 2048 && (specials || !is_half(dt))) emit_list("in", in, n * es);
+    if (n * es <= 2048 && (specials || !is_half(dt)) && !no_inputs_) emit_list("in", in, n * es);
     emit_list("out", out, n * es);
   }
   tail();
@@ -461,6 +463,23 @@ int main(int argc, char **argv) {
                           ALO_DIST_UNIFORM_PM1, 0, "long message");
       case_reduce_scatterv_long(fdt[d], ALO_SUM, ALO_DIST_UNIFORM_PM1, "uneven counts, long message");
     }
+    /* the sizes at which the library changes algorithm, exactly: 2048 bytes (still the short-message
+     * tree; 5 and 7 ranks, where the two trees differ in shape) and 512 KiB in all (already the pairwise
+     * exchange), with one element less or more beside them */
+    no_inputs_ = 1;
+    if (P_ == 5 || P_ == 7) {
+      const size_t edge = 2048 / alo_dtype_size(fdt[d]);
+      for (size_t n = edge - 1; n <= edge + 1; n++) {
+        case_allreduce(fdt[d], ALO_SUM, n, ALO_DIST_UNIFORM_PM1, 0, "at 2048 bytes");
+        case_reduce(fdt[d], ALO_SUM, n, ALO_DIST_UNIFORM_PM1, P_ - 1, 0, "at 2048 bytes");
+      }
+    }
+    if (big && P_ == 4 && d == 0) {
+      const size_t edge = (size_t)(512u << 10) / 4 / alo_dtype_size(fdt[d]);
+      for (size_t n = edge - 1; n <= edge + 1; n++)
+        case_reduce_scatter(fdt[d], ALO_SUM, n, ALO_DIST_UNIFORM_PM1, 0, "at 512 KiB");
+    }
+    no_inputs_ = 0;
   }
 
   /* fp16 / bf16 through user-defined commutative operations on MPI_SHORT, as the reference
