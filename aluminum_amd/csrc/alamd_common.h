@@ -36,7 +36,7 @@ int device_cus();
 // Process-wide; every field is an atomic, so that a setting changed while calls run is a clean old-or-new
 // value for each of them, never a torn one.
 struct Tunables {
-  std::atomic<size_t> launch_bytes{(size_t)800 << 20};          // bytes one fold / tree launch moves
+  std::atomic<size_t> launch_bytes{(size_t)4 << 30};            // bytes one fold / tree launch moves
   std::atomic<size_t> two_step_min_total_bytes{(size_t)128 << 20};  // fold + spread instead of one kernel: from this
                                                                     // many bytes written in all (outputs x bytes each) ...
   std::atomic<size_t> two_step_min_outputs{3};                  // ... and this many outputs up
@@ -45,6 +45,7 @@ struct Tunables {
   std::atomic<size_t> spread_launch_bytes{(size_t)288 << 20};   // bytes one spread launch moves
   std::atomic<size_t> spread_hbm_chunk_tiles{1024}, spread_hbm_launch_chunks{2};      // slices read from HBM
   std::atomic<size_t> spread_cache_chunk_tiles{512}, spread_cache_launch_chunks{16};  // a result just written
+  std::atomic<size_t> fold_front3_ranks{0};  // ranks from which a fold asks for three streams up front (0: by type)
   std::atomic<size_t> halo_load_policy{0};  // grid loads of a halo pack: 0 plain, 1 nt, 2 sc1, 3 sc0 sc1, 4 sc0 sc1 nt
 };
 Tunables &tunables();

@@ -245,6 +245,11 @@ struct TreeParams {
   unsigned long long role_base;      // ROLE_PER_BLOCK: element 0 of a segment is element role_base of the message,
   unsigned long long role_count;     // which has role_count elements (0: the segment is the message)
   int role_spread;                   // ROLE_PER_BLOCK: how the message is cut into blocks, see role_mask_of_elem
+  // ROLE_PER_BLOCK, filled in by the launcher when every segment's message has the same known length:
+  // that length, its block length and the reciprocals of the two block lengths there are, so that a
+  // workgroup finds its block without a 64-bit division
+  unsigned long long role_n, role_blk;
+  double role_inv_blk, role_inv_blk1;
 };
 
 __host__ __device__ inline unsigned role_bit_reverse(unsigned v, int bits) {
@@ -261,17 +266,33 @@ __host__ __device__ inline unsigned role_mask_of_rank(const TreeParams &p, int r
 // ROLE_PER_BLOCK: the message is cut into 2^role_bits blocks of count >> role_bits elements; what that
 // leaves over goes to the last block (TREE_RSG) or, role_spread, one element each to the first blocks
 // (TREE_RSG_SPREAD).  Block k ends up on survivor bit_reverse(k).
-__host__ __device__ inline unsigned role_mask_of_elem(const TreeParams &p, size_t seg_len, size_t e) {
-  const unsigned long long n = p.role_count ? p.role_count : seg_len, blk = n >> p.role_bits;
+// x / d from the reciprocal of d (x < 2^53, d > 0): the rounded product is within one of the quotient.
+__host__ __device__ inline unsigned long long role_div(unsigned long long x, unsigned long long d, double inv) {
+  unsigned long long q = (unsigned long long)((double)x * inv);
+  if (q * d > x) --q;
+  else if ((q + 1) * d <= x) ++q;
+  return q;
+}
+// *end: the element of the segment at which that block ends (for the last block: beyond every element).
+__host__ __device__ inline unsigned role_mask_of_elem(const TreeParams &p, size_t seg_len, size_t e,
+                                                      unsigned long long *end = nullptr) {
+  const bool fast = p.role_n != 0;
+  const unsigned long long n = fast ? p.role_n : (p.role_count ? p.role_count : seg_len);
+  const unsigned long long blk = fast ? p.role_blk : n >> p.role_bits;
   const unsigned long long last = (1ull << p.role_bits) - 1, x = p.role_base + e;
-  unsigned long long k;
+  unsigned long long k, stop;
   if (p.role_spread) {
     const unsigned long long longer = n & last, cut = longer * (blk + 1);  // `longer` blocks of blk + 1 come first
-    k = x < cut ? x / (blk + 1) : (blk ? longer + (x - cut) / blk : last);
+    if (x < cut) k = fast ? role_div(x, blk + 1, p.role_inv_blk1) : x / (blk + 1);
+    else k = blk ? longer + (fast ? role_div(x - cut, blk, p.role_inv_blk) : (x - cut) / blk) : last;
+    if (k > last) k = last;
+    stop = k * blk + (k < longer ? k : longer) + blk + (k < longer ? 1 : 0);
   } else {
-    k = blk ? x / blk : last;
+    k = blk ? (fast ? role_div(x, blk, p.role_inv_blk) : x / blk) : last;
+    if (k > last) k = last;
+    stop = (k + 1) * blk;
   }
-  if (k > last) k = last;
+  if (end) *end = k == last ? ~0ull : stop - p.role_base;
   return role_bit_reverse((unsigned)k, p.role_bits);
 }
 

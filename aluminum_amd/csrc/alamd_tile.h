@@ -26,16 +26,17 @@ constexpr unsigned kRsrcFlags = 0x00020000u;
 
 // Workgroups are handed to the eight XCDs round-robin and each XCD then works
 // through its share at its own pace, so over a long launch the XCDs drift
-// apart and the addresses in flight spread over more DRAM pages.  Longer inputs
-// are therefore cut into consecutive launches on the same stream.  The best
-// cut shrinks with the number of streams, and cuts that are not powers of two
-// run 1 to 2 points lower than their power-of-two neighbours.  Measured on
-// untouched buffers of 256 MiB per rank, % of the HBM peak by tiles of 16 KiB
-// per stream and launch (2048 / 4096 / 8192 / 16384 / 32768):
-//   P = 2: 68 75 78 79 79     P = 3: 72 76 77 77 77     P = 4: 73 76 77 76 77
-//   P = 6: 74 76 76 75 74     P = 8: 76 77 76 75 75     P = 12: 76 75 74 72 72
-// The rule below picks 16384, 8192, 8192, 4096, 4096 and 2048 for these.
-constexpr size_t kLaunchBytes = (size_t)800 << 20;
+// apart and the addresses in flight spread over more DRAM pages.  Very long
+// inputs are therefore cut into consecutive launches on the same stream, each
+// of which costs about 4.5 us of launch, ramp and drain.  The best cut shrinks
+// with the number of streams.  Measured with the streaming fold on untouched
+// fp32 buffers of 4.5 to 9 GiB in all, % of the HBM peak by MiB per stream and
+// launch (32 / 64 / 128 / 256 / 512 / 1024 / 2048):
+//   P = 2:  70 76 80 82 83 83 84    P = 4:  72 79 82 84 86 86     P = 8:  75 80 82 83 83 83
+//   P = 12: 76 79 81 82 81          P = 16: 77 80 80 79 79        P = 32: 77 79 77 76
+//   P = 64: 80 80 78
+// The rule below picks 1024, 512, 256, 256, 128, 64 and 32 MiB for these.
+constexpr size_t kLaunchBytes = (size_t)4 << 30;
 // Tiles (of `tile_bytes` per stream) in one launch of a kernel that reads `nin` streams and
 // writes one: the largest power of two that keeps the launch within launch_bytes.
 inline size_t floor_pow2(size_t v) {
@@ -65,6 +66,9 @@ __host__ __device__ inline size_t head_count(size_t elem_size, const char *out, 
 template <typename T> __device__ __forceinline__ size_t head_elems(const char *out, const char *first, size_t len) {
   return head_count(sizeof(T), out, first, len);
 }
+
+// Bytes per stream of a tile of the streaming fold and tree kernels (one wave, one vector per lane).
+constexpr size_t kStreamTileBytes = 1024;
 
 template <int U, int THREADS> struct Tile {
   static constexpr size_t BYTES = (size_t)THREADS * U * 16;

@@ -3,7 +3,7 @@
 // contributions resident in HBM.  Bandwidth-bound: every input byte is read
 // once, every output byte written once.
 //
-// One workgroup per tile, all loads of a lane issued before the first use,
+// One workgroup per tile, a bounded number of loads in flight per wave (see Shape),
 // buffer instructions with per-tile descriptors (see alamd_tile.h); buffers
 // need only be aligned to their element type.  The len % N elements behind the
 // last whole vector of a segment are folded one per thread.
@@ -42,43 +42,54 @@ __device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, siz
   for (int j = j0; j < j0 + nj; ++j) st_elem<T>(p.out[j] + out_bytes + e * sizeof(T), acc);
 }
 
-// Tile shape: 128 threads x 8 vectors per stream for every type (byte sums and
-// products, the most arithmetic per byte, are done a dword at a time and keep up).
-template <typename T, int OP> struct Shape {
-  static constexpr int U = 8;
-  static constexpr int THREADS = 128;
-  // P = 8 body: streams whose loads are issued before the first use (0: left to the compiler, which
-  // keeps as many in flight as the registers hold).  bf16 spends seven instructions per dword and
-  // step where the other types spend one; with everything requested up front the compiler ends up
-  // with a schedule that asks for 36 vectors, works through 27 of them and only then asks for the
-  // rest.  Two streams up front and one more requested for every one consumed is worth 0.3 to 0.5
-  // points to bf16 (6253 against 6227 GB/s, and 6250 against 6210, on buffers that are not reused)
-  // and nothing to fp32 (6144 / 6122, 6179 / 6173); three to seven streams up front, or more than
-  // two waves per SIMD with two, lose 1 to 5 points for both.
-  static constexpr int FRONT = std::is_same<T, bf16_t>::value ? 2 : 0;
+// Shape of a launch.
+//
+// An ordinary launch streams: one wave per workgroup, one 128-bit vector per lane and stream (1 KiB per
+// wave and stream), FRONT streams requested before the first use and one more for every stream consumed,
+// up to five waves per SIMD.  What counts is how many read requests the device keeps in flight: the
+// memory system is at its best with about 5 KiB per SIMD (some 40 thousand 128-byte requests in all) and
+// loses up to 25 points with a third of that and 5 to 8 points with three times as much.  Measured on
+// buffers that no recent launch has touched, fp32 sum, % of the HBM peak, by streams in flight per wave
+// (FRONT - 1 once the fold is under way) and waves per SIMD:
+//   P = 2:  FRONT 2: 3 waves 77, 4 83, 5 85, 6 85, 8 85        FRONT 3: 3 waves 77, 4 83, 5 84, 6 85
+//   P = 8:  FRONT 2: 3 waves 68, 4 80, 5 86, 6 84, 8 82        FRONT 3: 3 waves 72, 4 83, 5 84, 6 83
+//   P = 16: FRONT 2: 3 waves 64, 4 75, 5 83, 6 82, 8 79        FRONT 3: 3 waves 66, 4 78, 5 84, 6 82
+//   P = 64: FRONT 2: 3 waves 61, 4 74, 5 83, 6 84, 8 81        FRONT 3: 3 waves 62, 4 75, 5 84, 6 85
+// Workgroups of two or four waves with the same in flight run 2 to 4 points lower, and so does every shape
+// that asks for all of a lane's vectors up front (128 threads x 8 vectors x 8 streams: 79 %).
+//
+// A chained launch (see CHAIN below) keeps tiles of 16 KiB per stream, 128 threads x 8 vectors, all of a
+// batch of streams requested up front, two waves per SIMD: its tiles are handed out by a counter and wait
+// for one another through one flag per tile, which small tiles would make sixteen times as many of.
+template <typename T, int OP, bool CHAIN = false> struct Shape {
+  static constexpr int U = CHAIN ? 8 : 1;
+  static constexpr int THREADS = CHAIN ? 128 : 64;
+  static constexpr int WAVES = CHAIN ? 2 : 5;
 };
+// Ordinary launches are built with FRONT = 2 and FRONT = 3; the host takes three from this many ranks on
+// (16-bit floats, which spend seven instructions per dword and step where the others spend one, earlier).
+template <typename T> constexpr int front3_from_ranks() {
+  return (std::is_same<T, f16_t>::value || std::is_same<T, bf16_t>::value) ? 8 : 12;
+}
 
-// amdgpu_waves_per_eu(1, 2): the loads in flight are the point of this kernel;
-// the register allocator must not trade them away for more resident waves.
 // HEAD = false: no segment has leading elements to handle one by one (every buffer on a 64-byte
-// boundary).  With the head a compile-time zero the fp32 fold runs 1.6 points faster (83.8 % of the HBM
-// peak against 82.2 %) and the fp32 tree 2.8; both bodies in one kernel behind a uniform branch ran slower
-// than either (82.7 %, bf16 80.8 % against 82.2 %), so there are two kernels and the host picks.
-// (The body must stay in the kernel itself: moved into an inlined device function it was compiled
-// with 161 instead of 249 VGPRs, i.e. with fewer loads in flight, and lost 1.5 points.)
+// boundary); two kernels, and the host picks, so that the usual case carries no trace of the other.
+// FRONT: see Shape (0 in a chained launch).
 // CHAIN: the output overlaps one of the inputs at a displacement; tiles come from a ticket counter and
 // a tile's stores wait for the loads of the tiles that read what it writes (see ChainParams).  Always
 // with HEAD = false (no leading elements: the vectors start at the output's first element) and one
 // segment with one output.
-template <typename T, int OP, bool ACC_IS_IN, int PT, bool HEAD, bool CHAIN = false>
-__global__ void __launch_bounds__((Shape<T, OP>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
+template <typename T, int OP, bool ACC_IS_IN, int FRONT, bool HEAD, bool CHAIN = false>
+__global__ void __launch_bounds__((Shape<T, OP, CHAIN>::THREADS))
+__attribute__((amdgpu_waves_per_eu(1, Shape<T, OP, CHAIN>::WAVES)))
 fold_vec_kernel(const FoldParams p) {
   static_assert(!(CHAIN && HEAD), "a chained launch has no head");
-  constexpr int U = Shape<T, OP>::U, THREADS = Shape<T, OP>::THREADS;
+  static_assert(CHAIN ? FRONT == 0 : (FRONT >= 2 && FRONT <= 4), "streams requested up front");
+  constexpr int U = Shape<T, OP, CHAIN>::U, THREADS = Shape<T, OP, CHAIN>::THREADS;
   constexpr int N = 16 / sizeof(T);
   using TL = Tile<U, THREADS>;
   const TL tl;
-  const int P = PT ? PT : p.P;
+  const int P = p.P;
   // The general case looks its segment up in several tables, one dependent scalar load after the
   // other; a launch over one whole segment into one output needs none of that.
   unsigned seg = 0;
@@ -104,72 +115,49 @@ fold_vec_kernel(const FoldParams p) {
     const size_t rem = vec_bytes - tb;
     const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
     u32x4 acc[U];
-    if constexpr (PT == 8 && Shape<T, OP>::FRONT >= 2) {
-      // FRONT streams have their loads issued before the first use; every vector consumed then frees
-      // four registers, which the same vector of the next stream not yet requested takes.
-      constexpr int FRONT = Shape<T, OP>::FRONT;
-      u32x4 x[PT][U];
-      __amdgpu_buffer_rsrc_t r[PT];
-      int idx = s;
+    if constexpr (!CHAIN) {
+      static_assert(U == 1, "the streaming body holds one vector per lane and stream");
+      // Stream k lives in x[k % FRONT].  A later load takes its offset from an empty asm statement that
+      // reads the result of the step before it, so that it cannot be issued any earlier; the empty
+      // statement on the accumulator keeps the steps themselves in order.
+      u32x4 x[FRONT];
+      // the rank whose stream is requested next, and its buffer: the pointer is fetched one request
+      // ahead, so that its scalar load is not part of the chain from one request to the next
+      int req = s;
+      const char *next_in = p.in[req];
 #pragma unroll
-      for (int k = 0; k < PT; ++k) {
-        r[k] = TL::rsrc(p.in[idx] + vin + tb, nrec);
-        idx = next_rank(idx, p.dir, PT);
-      }
-#pragma unroll
-      for (int k = 0; k < FRONT; ++k) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) x[k][u] = tl.load(r[k], u);
+      for (int j = 0; j < FRONT; ++j) {
+        if (j < P) {
+          x[j] = tl.load(TL::rsrc(next_in + vin + tb, nrec), 0);
+          req = next_rank(req, p.dir, P);
+          next_in = p.in[req];
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
-      // a later load takes its offset from an empty asm statement that reads the step's result, so
-      // that it cannot be issued earlier
-      auto load_after = [&](__amdgpu_buffer_rsrc_t rs, int u, const u32x4 &after) {
+      auto load_after = [&](__amdgpu_buffer_rsrc_t rs, const u32x4 &after) {
         unsigned vo = tl.vo;
         asm volatile("" : "+v"(vo) : "v"(after));
-        return __builtin_amdgcn_raw_buffer_load_b128(rs, vo + (unsigned)u * 1024u, 0, kAuxLoadStream);
+        return __builtin_amdgcn_raw_buffer_load_b128(rs, vo, 0, kAuxLoadStream);
       };
+      acc[0] = x[0];
+      for (int base = 0; base < P; base += FRONT) {
 #pragma unroll
-      for (int k = 1; k < PT; ++k) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const u32x4 a = k == 1 ? x[0][u] : acc[u];
-          acc[u] = ACC_IS_IN ? step_vec<T, OP>(a, x[k][u]) : step_vec<T, OP>(x[k][u], a);
-          const int nx = FRONT + k - 1;  // the stream requested next
-          if (nx < PT) x[nx < PT ? nx : 0][u] = load_after(r[nx < PT ? nx : 0], u, acc[u]);
+        for (int j = 0; j < FRONT; ++j) {
+          const int k = base + j;
+          if (k >= 1 && k < P) {
+            acc[0] = ACC_IS_IN ? step_vec<T, OP>(acc[0], x[j]) : step_vec<T, OP>(x[j], acc[0]);
+            if (k + FRONT - 1 < P) {
+              x[(j + FRONT - 1) % FRONT] = load_after(TL::rsrc(next_in + vin + tb, nrec), acc[0]);
+              req = next_rank(req, p.dir, P);
+              next_in = p.in[req];
+            }
+            asm volatile("" : "+v"(acc[0]));
+          }
         }
-        // an empty asm statement per accumulator: the steps of stream k can neither sink below it nor
-        // mix with those of stream k + 1
-#pragma unroll
-        for (int u = 0; u < U; ++u) asm volatile("" : "+v"(acc[u]));
-      }
-    } else if constexpr (PT > 0) {
-      u32x4 x[PT][U];
-      int idx = s;
-#pragma unroll
-      for (int k = 0; k < PT; ++k) {
-        const auto r = TL::rsrc(p.in[idx] + vin + tb, nrec);
-#pragma unroll
-        for (int u = 0; u < U; ++u) x[k][u] = tl.load(r, u);
-        idx = next_rank(idx, p.dir, PT);
-      }
-      // stream-major, the order the loads were issued in (they return in
-      // order): every accumulator advances as soon as a stream has arrived
-#pragma unroll
-      for (int u = 0; u < U; ++u) acc[u] = x[0][u];
-#pragma unroll
-      for (int k = 1; k < PT; ++k) {
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-          acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[k][u]) : step_vec<T, OP>(x[k][u], acc[u]);
       }
     } else {
-      // Run-time rank count: the streams are taken in batches of a compile-time size - the pointers
-      // of a batch, then all its loads, then all its steps, no branch in between - so that up to
-      // seven ranks have every stream in flight at once, like the P = 8 body above.  (With one
-      // branch per stream the compiler fetched each stream's pointer, waited for it and only then
-      // issued that stream's loads: 1.5 % slower at P = 12 and 16, and for 16-bit and 8-bit types
-      // at P = 4.  A compile-time P = 4 body gains another 0.5 to 1 %, not worth its kernels.)
+      // The streams are taken in batches of a compile-time size - the pointers of a batch, then all its
+      // loads, then all its steps, no branch in between.
       int idx = s;
       auto batch = [&](auto rc, auto first_c) {
         constexpr int R = decltype(rc)::value;
@@ -202,11 +190,10 @@ fold_vec_kernel(const FoldParams p) {
       using No = std::false_type;
       // Up to seven streams in one batch; beyond that a first batch that leaves a multiple of six.
       // For 8- and 16-bit types, whose arithmetic needs registers as well, the kernel then no longer
-      // fits two waves per SIMD.  Batches of five and four, which do, ran 1 to 3 % slower all the
-      // same - except in a chained launch, where the second wave hides the waits for the
-      // neighbouring tile (bf16, a block one element into its buffer: 5.2 TB/s against 4.5).
-      constexpr bool kTwoWaves = CHAIN && sizeof(T) <= 2;
-      constexpr int B0 = kTwoWaves ? 5 : 7, B = kTwoWaves ? 4 : 6;
+      // fits two waves per SIMD, and the second wave is what hides the waits for the neighbouring
+      // tile (bf16, a block one element into its buffer: 5.2 TB/s against 4.5): batches of five and four.
+      constexpr bool kSmall = sizeof(T) <= 2;
+      constexpr int B0 = kSmall ? 5 : 7, B = kSmall ? 4 : 6;
       int left = P;
       switch (P <= B0 ? P : (P - 1) % B + 1) {
       case 7: if constexpr (B0 >= 7) { batch(std::integral_constant<int, 7>{}, Yes{}); left -= 7; } break;
@@ -240,10 +227,12 @@ fold_vec_kernel(const FoldParams p) {
     }
   } else {
     // the head elements and the vlen % N elements behind the last whole vector, one per thread of the
-    // segment's first workgroup
-    if (p.seg.tile0 == 0 && blockIdx.x == 0 && threadIdx.x < head + vlen % N) {
-      const size_t e = threadIdx.x < head ? threadIdx.x : (vlen / N) * N + threadIdx.x;
-      fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
+    // segment's first workgroup (up to 63 and 15 of them)
+    if (p.seg.tile0 == 0 && blockIdx.x == 0) {
+      for (size_t t = threadIdx.x; t < head + vlen % N; t += THREADS) {
+        const size_t e = t < head ? t : (vlen / N) * N + t;
+        fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
+      }
     }
   }
 }
@@ -258,7 +247,10 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
     constexpr bool FP_MINMAX = (std::is_same<T, float>::value || std::is_same<T, double>::value ||
                                 std::is_same<T, f16_t>::value || std::is_same<T, bf16_t>::value) &&
                                (OP == ALAMD_MIN || OP == ALAMD_MAX);
-    const size_t tile_elems = Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES / sizeof(T);
+    using Stream = Shape<T, OP, false>;
+    using Chained = Shape<T, OP, true>;
+    static_assert(Tile<Stream::U, Stream::THREADS>::BYTES == kStreamTileBytes, "alamd_planned_launches counts in these tiles");
+    const size_t tile_elems = Tile<Stream::U, Stream::THREADS>::BYTES / sizeof(T);
     FoldParams q = p;
     q.div = make_divisor(p.P);
     q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0, 0};
@@ -267,8 +259,8 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
       // one segment, one output, every tile in one launch, tiles handed out by the ticket counter
       if (nseg != 1) return set_error(ALAMD_ERR_INVALID_ARG, "a chained fold has one segment");
       constexpr size_t N = 16 / sizeof(T);
-      const size_t nvec = (max_len / N * 16 + Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES - 1) /
-                          Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES;
+      constexpr size_t kChainTile = Tile<Chained::U, Chained::THREADS>::BYTES;
+      const size_t nvec = (max_len / N * 16 + kChainTile - 1) / kChainTile;
       const size_t tickets = nvec + (max_len % N ? 1 : 0);
       if (nvec > chain->max_tiles || tickets > 0x7fffffffull)
         return set_error(ALAMD_ERR_INVALID_ARG, "in-place block of %zu elements needs %zu tile flags, the scratch holds %zu",
@@ -280,12 +272,9 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
       q.seg.seg0 = 0;
       q.seg.mapped = 0;
       void (*ck)(const FoldParams) = nullptr;
-      // Always the run-time-P body: with the gate in it the P = 8 body no longer fits two waves per SIMD,
-      // and a second wave is what hides a tile's wait for its neighbour (a block one element into its
-      // buffer: 3 to 11 % faster than with the P = 8 body; from a few MiB in, 3 % slower).
       if constexpr (FP_MINMAX) ck = roles ? fold_vec_kernel<T, OP, true, 0, false, true> : fold_vec_kernel<T, OP, false, 0, false, true>;
       else ck = fold_vec_kernel<T, OP, false, 0, false, true>;
-      hipLaunchKernelGGL(ck, dim3((unsigned)tickets, 1, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
+      hipLaunchKernelGGL(ck, dim3((unsigned)tickets, 1, 1), dim3(Chained::THREADS, 1, 1), 0, stream, q);
       ALAMD_HIP(hipGetLastError());
       return ALAMD_OK;
     }
@@ -301,28 +290,29 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
     }
     q.seg.simple = nseg == 1 && !q.seg.ragged && q.seg.seg_rem == 0 && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1 &&
                    !q.seg.any_head && p.start0 >= 0 && p.start0 < p.P;
-    auto pick = [&](auto acc_is_in_t, auto pt_t) -> void (*)(const FoldParams) {
+    auto pick = [&](auto acc_is_in_t, auto front_t) -> void (*)(const FoldParams) {
       constexpr bool A = decltype(acc_is_in_t)::value;
-      constexpr int PT = decltype(pt_t)::value;
-      return q.seg.any_head ? fold_vec_kernel<T, OP, A, PT, true> : fold_vec_kernel<T, OP, A, PT, false>;
+      constexpr int FRONT = decltype(front_t)::value;
+      return q.seg.any_head ? fold_vec_kernel<T, OP, A, FRONT, true> : fold_vec_kernel<T, OP, A, FRONT, false>;
     };
     using No = std::false_type;
     using Yes = std::true_type;
-    using P8 = std::integral_constant<int, 8>;
-    using PN = std::integral_constant<int, 0>;
+    using F2 = std::integral_constant<int, 2>;
+    using F3 = std::integral_constant<int, 3>;
     void (*kern)(const FoldParams) = nullptr;
-    if (p.P == 8) {
-      if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, P8{}) : pick(No{}, P8{});
-      else kern = pick(No{}, P8{});
+    const size_t front3 = tunables().fold_front3_ranks;
+    if ((size_t)p.P >= (front3 ? front3 : (size_t)front3_from_ranks<T>())) {
+      if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, F3{}) : pick(No{}, F3{});
+      else kern = pick(No{}, F3{});
     } else {
-      if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, PN{}) : pick(No{}, PN{});
-      else kern = pick(No{}, PN{});
+      if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, F2{}) : pick(No{}, F2{});
+      else kern = pick(No{}, F2{});
     }
-    const size_t per_launch = launch_tiles(p.P, Tile<Shape<T, OP>::U, Shape<T, OP>::THREADS>::BYTES, tunables().launch_bytes);
+    const size_t per_launch = launch_tiles(p.P, Tile<Stream::U, Stream::THREADS>::BYTES, tunables().launch_bytes);
     plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
       q.seg.tile0 = t0;
       q.seg.seg0 = s0;
-      hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(Shape<T, OP>::THREADS, 1, 1), 0, stream, q);
+      hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(Stream::THREADS, 1, 1), 0, stream, q);
     });
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;

@@ -57,12 +57,23 @@ __device__ __forceinline__ void tree_elem(const TreeParams &p, size_t in_bytes, 
 // two), which needs room for up to twice as many loads in flight.
 enum { TREE_FULL = 0, TREE_PARTIAL = 1, TREE_PREFOLD = 2 };
 
-template <typename T, int OP, int SLOTS, int MODE> struct TreeShape {
+// An ordinary launch streams like the fold does (see Shape there): one wave per workgroup, one vector per
+// lane and slot, the two slots of a pair requested together and the next pair as soon as a pair has been
+// combined, partial results combined as soon as both halves of a subtree are there.  Untouched
+// buffers, 8 slots, sum, % of the HBM peak by waves per SIMD (2 / 3 / 4 / 5 / 6): fp32 72 85 84 82 82,
+// fp64 72 85 84 82 82, fp16 71 85 84 82 82, bf16 66 82 84 82 81; a second pair requested ahead changes
+// nothing, every slot requested up front (128 threads x 8 vectors) gives 79.  A float min / max, whose
+// workgroups first work out which operand of every pair keeps the result, wants a fourth wave as well
+// (fp32 under the reduce-scatter + gather order: 77 with three, 85 with four).
+// A chained launch keeps tiles of 4 to 16 KiB per slot with every load issued up front (see the fold).
+template <typename T, int OP, int SLOTS, int MODE, bool CHAIN = false> struct TreeShape {
   static constexpr bool heavy = sizeof(T) <= 2;
-  static constexpr int budget = heavy ? 32 : 64;  // 128-bit loads in flight per lane
+  static constexpr int budget = heavy ? 32 : 64;  // chained: 128-bit loads in flight per lane
   static constexpr int streams = MODE == TREE_PREFOLD ? 2 * SLOTS : SLOTS;
-  static constexpr int U = budget / streams >= 8 ? (heavy ? 4 : 8) : (budget / streams >= 1 ? budget / streams : 1);
-  static constexpr int THREADS = U == 8 ? 128 : 256;
+  static constexpr int chained_u = budget / streams >= 8 ? (heavy ? 4 : 8) : (budget / streams >= 1 ? budget / streams : 1);
+  static constexpr int U = CHAIN ? chained_u : 1;
+  static constexpr int THREADS = CHAIN ? (chained_u == 8 ? 128 : 256) : 64;
+  static constexpr int WAVES = CHAIN ? 2 : (heavy || OP == ALAMD_MIN || OP == ALAMD_MAX ? 4 : 3);
 };
 
 __host__ __device__ inline void tree_out_select(const TreeParams &p, unsigned seg, size_t off_bytes,
@@ -79,10 +90,11 @@ __host__ __device__ inline void tree_out_select(const TreeParams &p, unsigned se
 // of one.
 // CHAIN: the output overlaps one of the inputs at a displacement (see ChainParams and the fold kernel).
 template <typename T, int OP, int SLOTS, int MODE, bool HEAD, int HALVES, bool CHAIN = false>
-__global__ void __launch_bounds__((TreeShape<T, OP, SLOTS, MODE>::THREADS)) __attribute__((amdgpu_waves_per_eu(1, 2)))
+__global__ void __launch_bounds__((TreeShape<T, OP, SLOTS, MODE, CHAIN>::THREADS))
+__attribute__((amdgpu_waves_per_eu(1, TreeShape<T, OP, SLOTS, MODE, CHAIN>::WAVES)))
 tree_vec_kernel(const TreeParams p) {
   static_assert(!(CHAIN && HEAD), "a chained launch has no head");
-  constexpr int U = TreeShape<T, OP, SLOTS, MODE>::U, THREADS = TreeShape<T, OP, SLOTS, MODE>::THREADS;
+  constexpr int U = TreeShape<T, OP, SLOTS, MODE, CHAIN>::U, THREADS = TreeShape<T, OP, SLOTS, MODE, CHAIN>::THREADS;
   constexpr int N = 16 / sizeof(T);
   static_assert(HALVES == 1 || MODE != TREE_PREFOLD, "a pre-fold never meets more than 32 slots");
   using TL = Tile<U, THREADS>;
@@ -117,8 +129,9 @@ tree_vec_kernel(const TreeParams p) {
     } else if (p.role_mode == ROLE_PER_BLOCK && tb < vec_bytes) {
       const size_t rem = vec_bytes - tb, nb = rem > TL::BYTES ? TL::BYTES : rem;
       const size_t e0 = head + tb / sizeof(T);
-      w = role_mask_of_elem(p, len, e0);
-      mixed = role_mask_of_elem(p, len, e0 + nb / sizeof(T) - 1) != w;
+      unsigned long long block_end;
+      w = role_mask_of_elem(p, len, e0, &block_end);
+      mixed = e0 + nb / sizeof(T) > block_end;
     }
   }
   if (ROLES && !CHAIN && mixed) {
@@ -133,6 +146,82 @@ tree_vec_kernel(const TreeParams p) {
     const size_t rem = vec_bytes - tb;
     const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
     u32x4 res[U];
+    if constexpr (!CHAIN) {
+      static_assert(U == 1, "the streaming body holds one vector per lane and slot");
+      // a later load takes its offset from an empty asm statement that reads the result of the pair
+      // before it, so that it cannot be issued any earlier
+      auto load_after = [&](const char *base, const u32x4 &after) {
+        unsigned vo = tl.vo;
+        asm volatile("" : "+v"(vo) : "v"(after));
+        return __builtin_amdgcn_raw_buffer_load_b128(TL::rsrc(base + vin + tb, nrec), vo, 0, kAuxLoadStream);
+      };
+#pragma unroll
+      for (int h = 0; h < HALVES; ++h) {
+        const int base = h * SLOTS;
+        const int nvalid = MODE == TREE_FULL ? SLOTS : p.nvalid - base;
+        if (h > 0 && nvalid <= 0) break;
+        // la / lb: what slot j and the rank pre-folded into it have sent; v: the partial results
+        u32x4 la[SLOTS], lb[SLOTS], v[SLOTS];
+        // the buffers of slot j (with a mask in play their table index is only known here): fetched a
+        // pair ahead of their request, so that no scalar load sits between one request and the next
+        const char *pa[SLOTS], *pb[SLOTS];
+        auto fetch = [&](int j) {
+          if (j < SLOTS && j < nvalid) {
+            const int sl = ROLES ? (base + j) ^ (int)w : base + j;
+            pa[j] = p.a[sl];
+            if constexpr (MODE == TREE_PREFOLD) pb[j] = p.b[sl];
+          }
+        };
+        auto request = [&](int j, const u32x4 &after, bool first) {
+          if (j < nvalid) {
+            la[j] = first ? tl.load(TL::rsrc(pa[j] + vin + tb, nrec), 0) : load_after(pa[j], after);
+            if constexpr (MODE == TREE_PREFOLD) {
+              if (pb[j] != nullptr) lb[j] = first ? tl.load(TL::rsrc(pb[j] + vin + tb, nrec), 0) : load_after(pb[j], after);
+            }
+          }
+        };
+        // the leaf of slot j: its own data, with the pre-folded rank's combined in (the odd rank keeps
+        // step(in = even rank, inout = odd rank))
+        auto leaf = [&](int j) {
+          u32x4 x = la[j];
+          if constexpr (MODE == TREE_PREFOLD) {
+            if (pb[j] != nullptr) x = step_vec<T, OP>(x, lb[j]);
+          }
+          return x;
+        };
+        const u32x4 none = {0u, 0u, 0u, 0u};
+        fetch(0);
+        fetch(1);
+        request(0, none, true);
+        request(1, none, true);
+        fetch(2);
+        fetch(3);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < SLOTS; j += 2) {
+          if (j < nvalid) {
+            v[j] = leaf(j);
+            if (j + 1 < nvalid) v[j] = step_vec<T, OP>(leaf(j + 1), v[j]);
+            if (j + 2 < SLOTS) request(j + 2, v[j], false);
+            if (j + 3 < SLOTS) request(j + 3, v[j], false);
+            fetch(j + 4);
+            fetch(j + 5);
+            asm volatile("" : "+v"(v[j]));
+          }
+          // the subtrees that end with this pair: distance 2, 4, ...
+#pragma unroll
+          for (int d = 2; d < SLOTS; d *= 2) {
+            if ((j + 2) % (2 * d) != 0) break;
+            const int i = j + 2 - 2 * d;
+            if (i + d < nvalid) {
+              v[i] = step_vec<T, OP>(v[i + d], v[i]);
+              asm volatile("" : "+v"(v[i]));
+            }
+          }
+        }
+        res[0] = h == 0 ? v[0] : step_vec<T, OP>(v[0], res[0]);
+      }
+    } else {
 #pragma unroll
     for (int h = 0; h < HALVES; ++h) {
       const int base = h * SLOTS;
@@ -180,6 +269,7 @@ tree_vec_kernel(const TreeParams p) {
 #pragma unroll
       for (int u = 0; u < U; ++u) res[u] = h == 0 ? v[0][u] : step_vec<T, OP>(v[0][u], res[u]);
     }
+    }
 #pragma unroll
     for (int u = 0; u < U; ++u) res[u] = finish_vec<T, OP>(res[u], p.div);
     if constexpr (CHAIN) chain_gate(p.chain, bx, tb, (unsigned long long)nrec, (unsigned)TL::BYTES);
@@ -201,10 +291,12 @@ tree_vec_kernel(const TreeParams p) {
     }
   } else {
     // the head elements and the vlen % N elements behind the last whole vector
-    if (p.seg.tile0 == 0 && blockIdx.x == 0 && threadIdx.x < head + vlen % N) {
-      const size_t e = threadIdx.x < head ? threadIdx.x : (vlen / N) * N + threadIdx.x;
-      tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e,
-                                      ROLES && p.role_mode == ROLE_PER_BLOCK ? role_mask_of_elem(p, len, e) : w);
+    if (p.seg.tile0 == 0 && blockIdx.x == 0) {
+      for (size_t t = threadIdx.x; t < head + vlen % N; t += THREADS) {
+        const size_t e = t < head ? t : (vlen / N) * N + t;
+        tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e,
+                                        ROLES && p.role_mode == ROLE_PER_BLOCK ? role_mask_of_elem(p, len, e) : w);
+      }
     }
   }
 }
@@ -214,20 +306,34 @@ struct ChainArgs { const ChainScratch *scratch; size_t displ_bytes; };
 
 template <typename T, int OP, int SLOTS, int MODE, int HALVES = 1>
 int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStream_t stream, ChainArgs chain) {
-  using S = TreeShape<T, OP, SLOTS, MODE>;
+  using S = TreeShape<T, OP, SLOTS, MODE, false>;
+  using C = TreeShape<T, OP, SLOTS, MODE, true>;
+  static_assert(Tile<S::U, S::THREADS>::BYTES == kStreamTileBytes, "the tile of a streaming launch");
   const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
   const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES, tunables().launch_bytes);
   TreeParams q = p;
   q.div = make_divisor(p.P);
   q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0, 0};
   q.seg.simple = 0;
+  q.role_n = q.role_blk = 0;
+  q.role_inv_blk = q.role_inv_blk1 = 0.0;
+  if (p.role_mode == ROLE_PER_BLOCK) {
+    // the message every segment belongs to, if it is the same for all and short enough for exact doubles
+    const unsigned long long n = p.role_count ? p.role_count : (!p.seg.ragged && p.seg.seg_rem == 0 ? p.seg.seg_base : 0);
+    if (n != 0 && n < (1ull << 52)) {
+      q.role_n = n;
+      q.role_blk = n >> p.role_bits;
+      q.role_inv_blk = q.role_blk ? 1.0 / (double)q.role_blk : 0.0;
+      q.role_inv_blk1 = 1.0 / (double)(q.role_blk + 1);
+    }
+  }
   if (chain.scratch) {
     if (nseg != 1) return set_error(ALAMD_ERR_INVALID_ARG, "a chained combine has one segment");
     if (op_has_roles<OP>() && p.role_mode == ROLE_PER_BLOCK)
       return set_error(ALAMD_ERR_INVALID_ALGO, "a float min / max under the reduce-scatter + gather order is not available "
                        "for an in-place block that overlaps its own input");
     constexpr size_t N = 16 / sizeof(T);
-    const size_t tile_bytes = Tile<S::U, S::THREADS>::BYTES;
+    const size_t tile_bytes = Tile<C::U, C::THREADS>::BYTES;
     const size_t nvec = (max_len / N * 16 + tile_bytes - 1) / tile_bytes;
     const size_t tickets = nvec + (max_len % N ? 1 : 0);
     if (nvec > chain.scratch->max_tiles || tickets > 0x7fffffffull)
@@ -243,7 +349,7 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
     // only the most general variants are built for chained launches
     if constexpr (MODE == TREE_PREFOLD || (HALVES == 2 && MODE == TREE_PARTIAL)) {
       hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE, false, HALVES, true>), dim3((unsigned)tickets, 1, 1),
-                         dim3(S::THREADS, 1, 1), 0, stream, q);
+                         dim3(C::THREADS, 1, 1), 0, stream, q);
       ALAMD_HIP(hipGetLastError());
       return ALAMD_OK;
     } else {
