@@ -45,6 +45,7 @@ struct Tunables {
   std::atomic<size_t> spread_launch_bytes{(size_t)288 << 20};   // bytes one spread launch moves
   std::atomic<size_t> spread_hbm_chunk_tiles{1024}, spread_hbm_launch_chunks{2};      // slices read from HBM
   std::atomic<size_t> spread_cache_chunk_tiles{512}, spread_cache_launch_chunks{16};  // a result just written
+  std::atomic<size_t> stream_wgs_per_cu{0};  // workgroups per CU of a streaming fold / tree launch (0: the kernels' own)
   std::atomic<size_t> fold_front3_ranks{0};  // ranks from which a fold asks for three streams up front (0: by type)
   std::atomic<size_t> halo_load_policy{0};  // grid loads of a halo pack: 0 plain, 1 nt, 2 sc1, 3 sc0 sc1, 4 sc0 sc1 nt
 };

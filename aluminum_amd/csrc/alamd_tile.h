@@ -69,6 +69,37 @@ template <typename T> __device__ __forceinline__ size_t head_elems(const char *o
 
 // Bytes per stream of a tile of the streaming fold and tree kernels (one wave, one vector per lane).
 constexpr size_t kStreamTileBytes = 1024;
+// The streaming kernels are compiled for up to kStreamMaxWaves waves per SIMD; how many a launch really
+// gets is set when it is launched, through the LDS it asks for: a CU has 160 KiB and a workgroup is one
+// wave, so with 160 KiB / n bytes each n workgroups fit a CU (LDS is handed out by the KiB, so the
+// counts that can be had are 32, 26, 22, 20, 17, 16, 14, 13, 12, ...).  The kernels never touch that memory.
+// What counts is how many read requests the device keeps in flight: with one or two KiB per wave, as
+// the streaming kernels have them, the memory system is at its best with 22 waves per CU for a fold
+// and 16 for a tree (which has a pair of slots in flight where the fold has one stream); it loses 5 to
+// 25 points with fewer and 2 to 6 with more.  Untouched fp32 buffers, % of the HBM peak by workgroups
+// per CU (12 / 14 / 16 / 20 / 22 / 26 / 32):
+//   fold  P = 2:  69 73 81 82 84 85 85    P = 4:  66 70 81 84 83 81 79    P = 8:  63 66 77 80 84 82 80
+//         P = 16 (three streams up front): 62 65 75 80 84 81 80          P = 64 (three): 58 61 74 76 82 80 81
+//   tree  P = 2:  71 75 82 83 84 85 84    P = 4:  79 82 81 80 79 80 79    P = 8:  80 83 81 81 80 80 80
+//         P = 16: 79 80 82 81 79 79 79    P = 64: 84 84 83 80 80 80 81
+//   (a tree of 16-bit floats or a float min / max, P = 8: 14: 75, 16: 84, 20: 83, 26: 81)
+// Launches that move less than 256 MiB in all, much of which the caches hold, want more: 32 and 26
+// (16 MiB per rank, P = 8, repeated on the same buffers: 23.0 us against 25.1 us with 22).
+constexpr int kStreamMaxWaves = 8;
+inline unsigned stream_lds_bytes(int wgs_per_cu) {
+  const int n = wgs_per_cu < 4 ? 4 : (wgs_per_cu > 4 * kStreamMaxWaves ? 4 * kStreamMaxWaves : wgs_per_cu);
+  return (unsigned)((160u * 1024u / (unsigned)n) & ~127u);
+}
+// A launch that writes every tile to three or more buffers is better off with 16 whatever its size
+// (8 MiB per rank to 8 buffers, repeated: 22.2 us against 24.1 us; 16 MiB, untouched: 51.0 against 52.8).
+// Workgroups per CU of a streaming launch over `streams` inputs that moves `total_bytes` in all and
+// writes every tile to `outputs` buffers.
+inline int stream_wgs_per_cu(bool tree, int streams, int outputs, size_t total_bytes) {
+  if (outputs >= 3) return 16;
+  if (total_bytes < ((size_t)256 << 20)) return tree ? 26 : 32;
+  if (streams <= 2) return 26;
+  return tree ? 16 : 22;
+}
 
 template <int U, int THREADS> struct Tile {
   static constexpr size_t BYTES = (size_t)THREADS * U * 16;

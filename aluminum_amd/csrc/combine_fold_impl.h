@@ -45,18 +45,12 @@ __device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, siz
 // Shape of a launch.
 //
 // An ordinary launch streams: one wave per workgroup, one 128-bit vector per lane and stream (1 KiB per
-// wave and stream), FRONT streams requested before the first use and one more for every stream consumed,
-// up to five waves per SIMD.  What counts is how many read requests the device keeps in flight: the
-// memory system is at its best with about 5 KiB per SIMD (some 40 thousand 128-byte requests in all) and
-// loses up to 25 points with a third of that and 5 to 8 points with three times as much.  Measured on
-// buffers that no recent launch has touched, fp32 sum, % of the HBM peak, by streams in flight per wave
-// (FRONT - 1 once the fold is under way) and waves per SIMD:
-//   P = 2:  FRONT 2: 3 waves 77, 4 83, 5 85, 6 85, 8 85        FRONT 3: 3 waves 77, 4 83, 5 84, 6 85
-//   P = 8:  FRONT 2: 3 waves 68, 4 80, 5 86, 6 84, 8 82        FRONT 3: 3 waves 72, 4 83, 5 84, 6 83
-//   P = 16: FRONT 2: 3 waves 64, 4 75, 5 83, 6 82, 8 79        FRONT 3: 3 waves 66, 4 78, 5 84, 6 82
-//   P = 64: FRONT 2: 3 waves 61, 4 74, 5 83, 6 84, 8 81        FRONT 3: 3 waves 62, 4 75, 5 84, 6 85
-// Workgroups of two or four waves with the same in flight run 2 to 4 points lower, and so does every shape
-// that asks for all of a lane's vectors up front (128 threads x 8 vectors x 8 streams: 79 %).
+// wave and stream), FRONT streams requested before the first use and one more for every stream consumed
+// (so FRONT - 1 loads of a wave are in flight once the fold is under way), and a number of waves per CU
+// that the host sets per launch (see stream_lds_bytes and stream_wgs_per_cu in alamd_tile.h, which also
+// hold the measurements).  Workgroups of two or four waves with the same amount in flight run 2 to 4
+// points lower, and so does every shape that asks for all of a lane's vectors up front (128 threads x
+// 8 vectors x 8 streams, two waves per SIMD: 79 % of the HBM peak where this shape reaches 85 %).
 //
 // A chained launch (see CHAIN below) keeps tiles of 16 KiB per stream, 128 threads x 8 vectors, all of a
 // batch of streams requested up front, two waves per SIMD: its tiles are handed out by a counter and wait
@@ -64,13 +58,11 @@ __device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, siz
 template <typename T, int OP, bool CHAIN = false> struct Shape {
   static constexpr int U = CHAIN ? 8 : 1;
   static constexpr int THREADS = CHAIN ? 128 : 64;
-  static constexpr int WAVES = CHAIN ? 2 : 5;
+  static constexpr int WAVES = CHAIN ? 2 : kStreamMaxWaves;  // compiled for; see stream_lds_bytes
 };
 // Ordinary launches are built with FRONT = 2 and FRONT = 3; the host takes three from this many ranks on
-// (16-bit floats, which spend seven instructions per dword and step where the others spend one, earlier).
-template <typename T> constexpr int front3_from_ranks() {
-  return (std::is_same<T, f16_t>::value || std::is_same<T, bf16_t>::value) ? 8 : 12;
-}
+// (P = 8: 84 against 84 %, P = 12: 82 and 82, P = 16: 84 against 81, P = 64: 82 against 79).
+constexpr int kFront3FromRanks = 12;
 
 // HEAD = false: no segment has leading elements to handle one by one (every buffer on a 64-byte
 // boundary); two kernels, and the host picks, so that the usual case carries no trace of the other.
@@ -301,7 +293,7 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
     using F3 = std::integral_constant<int, 3>;
     void (*kern)(const FoldParams) = nullptr;
     const size_t front3 = tunables().fold_front3_ranks;
-    if ((size_t)p.P >= (front3 ? front3 : (size_t)front3_from_ranks<T>())) {
+    if ((size_t)p.P >= (front3 ? front3 : (size_t)kFront3FromRanks)) {
       if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, F3{}) : pick(No{}, F3{});
       else kern = pick(No{}, F3{});
     } else {
@@ -309,10 +301,13 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
       else kern = pick(No{}, F2{});
     }
     const size_t per_launch = launch_tiles(p.P, Tile<Stream::U, Stream::THREADS>::BYTES, tunables().launch_bytes);
+    const size_t wgs = tunables().stream_wgs_per_cu;
+    const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + 1);
+    const unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(false, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes));
     plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
       q.seg.tile0 = t0;
       q.seg.seg0 = s0;
-      hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(Stream::THREADS, 1, 1), 0, stream, q);
+      hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(Stream::THREADS, 1, 1), lds, stream, q);
     });
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;

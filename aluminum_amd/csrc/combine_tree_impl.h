@@ -20,7 +20,9 @@ template <int OP> constexpr bool op_has_roles() { return OP == ALAMD_MIN || OP =
 template <typename T, int OP, int SLOTS, int HALVES>
 __device__ __forceinline__ T tree_elem_value(const TreeParams &p, size_t in_bytes, size_t e, unsigned w = 0) {
   T res;
-#pragma unroll
+  // (rolled: unrolled over 64 slots, the table lookups below make the compiler copy the whole argument
+  // structure into scratch memory for every wave)
+#pragma unroll 1
   for (int h = 0; h < HALVES; ++h) {
     const int base = h * SLOTS;
     const int nvalid = p.nvalid - base;
@@ -50,6 +52,26 @@ __device__ __forceinline__ void tree_elem(const TreeParams &p, size_t in_bytes, 
   for (int j = j0; j < j0 + nj; ++j) st_elem<T>(p.out[j] + out_bytes + e * sizeof(T), res);
 }
 
+// The elements [lo, hi) of a segment one by one, a workgroup's threads side by side.  per_block: the
+// mask changes from block to block of the message (ROLE_PER_BLOCK); the range is then walked block by
+// block, so that the mask is the same in every lane and may index the argument tables.
+template <typename T, int OP, int SLOTS, int HALVES, int THREADS>
+__device__ __forceinline__ void tree_elems(const TreeParams &p, size_t len, size_t in_bytes, int j0, int nj,
+                                           size_t out_bytes, size_t lo, size_t hi, unsigned w, bool per_block) {
+  if (!per_block) {
+    for (size_t e = lo + threadIdx.x; e < hi; e += THREADS) tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e, w);
+    return;
+  }
+  size_t e0 = lo;
+  while (e0 < hi) {
+    unsigned long long block_end;
+    const unsigned m = (unsigned)__builtin_amdgcn_readfirstlane((int)role_mask_of_elem(p, len, e0, &block_end));
+    const size_t stop = block_end < hi ? (size_t)block_end : hi;
+    for (size_t e = e0 + threadIdx.x; e < stop; e += THREADS) tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e, m);
+    e0 = stop;
+  }
+}
+
 // Kernel variants: every slot occupied and none pre-folded (P a power of two:
 // straight-line code, no uniform branches between the loads and their uses);
 // some slots empty (binomial order, P not a power of two); some slots
@@ -59,12 +81,9 @@ enum { TREE_FULL = 0, TREE_PARTIAL = 1, TREE_PREFOLD = 2 };
 
 // An ordinary launch streams like the fold does (see Shape there): one wave per workgroup, one vector per
 // lane and slot, the two slots of a pair requested together and the next pair as soon as a pair has been
-// combined, partial results combined as soon as both halves of a subtree are there.  Untouched
-// buffers, 8 slots, sum, % of the HBM peak by waves per SIMD (2 / 3 / 4 / 5 / 6): fp32 72 85 84 82 82,
-// fp64 72 85 84 82 82, fp16 71 85 84 82 82, bf16 66 82 84 82 81; a second pair requested ahead changes
-// nothing, every slot requested up front (128 threads x 8 vectors) gives 79.  A float min / max, whose
-// workgroups first work out which operand of every pair keeps the result, wants a fourth wave as well
-// (fp32 under the reduce-scatter + gather order: 77 with three, 85 with four).
+// combined, partial results combined as soon as both halves of a subtree are there; the waves per CU
+// are the host's choice per launch (stream_wgs_per_cu in alamd_tile.h).  A second pair requested ahead
+// changes nothing; every slot requested up front (128 threads x 8 vectors) runs 5 points lower.
 // A chained launch keeps tiles of 4 to 16 KiB per slot with every load issued up front (see the fold).
 template <typename T, int OP, int SLOTS, int MODE, bool CHAIN = false> struct TreeShape {
   static constexpr bool heavy = sizeof(T) <= 2;
@@ -73,7 +92,7 @@ template <typename T, int OP, int SLOTS, int MODE, bool CHAIN = false> struct Tr
   static constexpr int chained_u = budget / streams >= 8 ? (heavy ? 4 : 8) : (budget / streams >= 1 ? budget / streams : 1);
   static constexpr int U = CHAIN ? chained_u : 1;
   static constexpr int THREADS = CHAIN ? (chained_u == 8 ? 128 : 256) : 64;
-  static constexpr int WAVES = CHAIN ? 2 : (heavy || OP == ALAMD_MIN || OP == ALAMD_MAX ? 4 : 3);
+  static constexpr int WAVES = CHAIN ? 2 : kStreamMaxWaves;  // compiled for; see stream_lds_bytes
 };
 
 __host__ __device__ inline void tree_out_select(const TreeParams &p, unsigned seg, size_t off_bytes,
@@ -133,15 +152,15 @@ tree_vec_kernel(const TreeParams p) {
       w = role_mask_of_elem(p, len, e0, &block_end);
       mixed = e0 + nb / sizeof(T) > block_end;
     }
+    // (the same in every lane; said explicitly, because it indexes the argument tables)
+    w = (unsigned)__builtin_amdgcn_readfirstlane((int)w);
   }
   if (ROLES && !CHAIN && mixed) {
-    // one element per access, every element under its own mask (never in a chained launch: the host
-    // refuses that combination)
+    // one element per access, block by block (never in a chained launch: the host refuses that
+    // combination)
     const size_t rem = vec_bytes - tb, nb = rem > TL::BYTES ? TL::BYTES : rem;
     const size_t e0 = head + tb / sizeof(T), ne = nb / sizeof(T);
-#pragma unroll 1
-    for (size_t k = threadIdx.x; k < ne; k += THREADS)
-      tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e0 + k, role_mask_of_elem(p, len, e0 + k));
+    tree_elems<T, OP, SLOTS, HALVES, THREADS>(p, len, in_bytes, j0, nj, out_bytes, e0, e0 + ne, w, true);
   } else if (tb < vec_bytes) {
     const size_t rem = vec_bytes - tb;
     const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
@@ -155,7 +174,10 @@ tree_vec_kernel(const TreeParams p) {
         asm volatile("" : "+v"(vo) : "v"(after));
         return __builtin_amdgcn_raw_buffer_load_b128(TL::rsrc(base + vin + tb, nrec), vo, 0, kAuxLoadStream);
       };
-#pragma unroll
+      // (the two halves of 33 to 64 slots run through the same code one after the other: unrolled, the
+      // body outgrows what the compiler will unroll of the loop over the slots, and the arrays below
+      // end up in scratch memory)
+#pragma unroll 1
       for (int h = 0; h < HALVES; ++h) {
         const int base = h * SLOTS;
         const int nvalid = MODE == TREE_FULL ? SLOTS : p.nvalid - base;
@@ -285,18 +307,18 @@ tree_vec_kernel(const TreeParams p) {
       const bool mine = threadIdx.x < vlen % N;
       const size_t e = (vlen / N) * N + threadIdx.x;
       T val = T();
-      if (mine) val = tree_elem_value<T, OP, SLOTS, HALVES>(p, in_bytes, e, ROLES && p.role_mode == ROLE_PER_BLOCK ? role_mask_of_elem(p, len, e) : w);
+      // (never with a mask per block: the host refuses that combination)
+      if (mine) val = tree_elem_value<T, OP, SLOTS, HALVES>(p, in_bytes, e, w);
       chain_gate(p.chain, bx, vec_bytes, (vlen % N) * sizeof(T), (unsigned)TL::BYTES);
       if (mine) st_elem<T>(p.out[j0] + out_bytes + e * sizeof(T), val);
     }
   } else {
     // the head elements and the vlen % N elements behind the last whole vector
     if (p.seg.tile0 == 0 && blockIdx.x == 0) {
-      for (size_t t = threadIdx.x; t < head + vlen % N; t += THREADS) {
-        const size_t e = t < head ? t : (vlen / N) * N + t;
-        tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e,
-                                        ROLES && p.role_mode == ROLE_PER_BLOCK ? role_mask_of_elem(p, len, e) : w);
-      }
+      const bool per_block = ROLES && p.role_mode == ROLE_PER_BLOCK;
+      const size_t tail = head + (vlen / N) * N;
+      tree_elems<T, OP, SLOTS, HALVES, THREADS>(p, len, in_bytes, j0, nj, out_bytes, 0, head, w, per_block);
+      tree_elems<T, OP, SLOTS, HALVES, THREADS>(p, len, in_bytes, j0, nj, out_bytes, tail, tail + vlen % N, w, per_block);
     }
   }
 }
@@ -367,12 +389,15 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   }
   q.seg.simple = nseg == 1 && !q.seg.ragged && q.seg.seg_rem == 0 && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1 &&
                  !q.seg.any_head;
+  const size_t wgs = tunables().stream_wgs_per_cu;
+  const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + 1);
+  const unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(true, SLOTS * HALVES, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes));
   void (*kern)(const TreeParams) =
       q.seg.any_head ? tree_vec_kernel<T, OP, SLOTS, MODE, true, HALVES> : tree_vec_kernel<T, OP, SLOTS, MODE, false, HALVES>;
   plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
     q.seg.tile0 = t0;
     q.seg.seg0 = s0;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(S::THREADS, 1, 1), 0, stream, q);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(S::THREADS, 1, 1), lds, stream, q);
   });
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;
