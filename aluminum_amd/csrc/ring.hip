@@ -14,9 +14,9 @@ namespace alamd {
 
 namespace {
 
-// A ring step streams like a fold of two ranks (see alamd_tile.h): one wave per workgroup, one vector per
-// lane from each of the two buffers.
-constexpr int kThreads = 64;
+// (A ring step keeps tiles of 256 threads x 8 vectors: on C3, whose segments the previous step has just
+// written, the streaming shape of the fold kernels gains nothing - 1358 us per allreduce against 1349.)
+constexpr int kThreads = 256;
 
 struct RingParams {
   char *buf[ALAMD_MAX_RANKS];
@@ -37,9 +37,9 @@ __device__ __forceinline__ void ring_seg(const RingParams &p, int seg, size_t &o
 // A chunk is a run of tiles_per_chunk tiles; no tile crosses a chunk boundary.
 // OP < 0: plain copy (allgather step).  FIN: the last reduce-scatter step of an
 // avg, which ends with the division by the number of ranks.
-constexpr int kRingU = 1;
+constexpr int kRingU = 8;
 template <typename T, int OP, bool FIN>
-__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, kStreamMaxWaves)))
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
 ring_step_vec_kernel(const RingParams p) {
   using TL = Tile<kRingU, kThreads>;
   const TL tl;
@@ -56,18 +56,16 @@ ring_step_vec_kernel(const RingParams p) {
   const size_t vlen = len - head;
   // the head elements and the vlen % N elements after the last whole vector, one per thread of the
   // segment's first workgroup
-  if (blockIdx.x == 0) {
-    for (size_t t = threadIdx.x; t < head + vlen % N; t += kThreads) {
-      const size_t e = t < head ? t : (vlen / N) * N + t;
-      const T a = ld_elem<T>(recv + e * sizeof(T));
-      if constexpr (OP >= 0) {
-        const T b = ld_elem<T>(local + e * sizeof(T));
-        T v = Step<T, (OP >= 0 ? OP : 0)>::apply(a, b);
-        if constexpr (FIN) v = finish_elem<T, OP>(v, p.div);
-        st_elem<T>(local + e * sizeof(T), v);
-      } else {
-        st_elem<T>(local + e * sizeof(T), a);
-      }
+  if (blockIdx.x == 0 && threadIdx.x < head + vlen % N) {
+    const size_t e = threadIdx.x < head ? threadIdx.x : (vlen / N) * N + threadIdx.x;
+    const T a = ld_elem<T>(recv + e * sizeof(T));
+    if constexpr (OP >= 0) {
+      const T b = ld_elem<T>(local + e * sizeof(T));
+      T v = Step<T, (OP >= 0 ? OP : 0)>::apply(a, b);
+      if constexpr (FIN) v = finish_elem<T, OP>(v, p.div);
+      st_elem<T>(local + e * sizeof(T), v);
+    } else {
+      st_elem<T>(local + e * sizeof(T), a);
     }
   }
   local += head * sizeof(T);
@@ -153,10 +151,6 @@ int make_plan(RingPlan &pl, void *const *bufs, int P, size_t count, int dtype, s
 // last: the final reduce-scatter step, after which every rank holds its fully reduced segment
 int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, bool last, hipStream_t stream) {
   const dim3 grid(pl.gx, pl.rp.P, 1), block(kThreads, 1, 1);
-  const size_t wgs = tunables().stream_wgs_per_cu;
-  // C3 (bf16, 8 x 256 MiB in place), us per allreduce by workgroups per CU (16 / 20 / 22 / 26 / 32):
-  // 1571 1469 1367 1285 1218; with tiles of 256 threads x 8 vectors and two waves per SIMD: 1349
-  const unsigned lds = stream_lds_bytes(wgs ? (int)wgs : 32);
   if (!reduce) {
     // a copy only needs the element size
     void (*kern)(const RingParams) = nullptr;
@@ -166,7 +160,7 @@ int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, bool last, h
     case 4: kern = ring_step_vec_kernel<uint32_t, -1, false>; break;
     default: kern = ring_step_vec_kernel<uint64_t, -1, false>; break;
     }
-    hipLaunchKernelGGL(kern, grid, block, lds, stream, pl.rp);
+    hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;
   }
@@ -177,7 +171,7 @@ int launch_step(const RingPlan &pl, int dtype, int op, bool reduce, bool last, h
     if constexpr (OP == ALAMD_AVG) {
       if (last) kern = ring_step_vec_kernel<T, OP, true>;
     }
-    hipLaunchKernelGGL(kern, grid, block, lds, stream, pl.rp);
+    hipLaunchKernelGGL(kern, grid, block, 0, stream, pl.rp);
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;
   });

@@ -42,9 +42,13 @@ int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void
  * launch_bytes, two_step_min_total_bytes, two_step_min_outputs,
  * two_step_piece_bytes, ring_piece_bytes, spread_launch_bytes,
  * spread_hbm_chunk_tiles, spread_hbm_launch_chunks, spread_cache_chunk_tiles,
- * spread_cache_launch_chunks; halo_load_policy (the cache policy of the grid
- * loads of a halo pack: 0 plain, 1 nt, 2 sc1, 3 sc0 sc1, 4 sc0 sc1 nt).  Piece
- * sizes below 64 KiB are refused.  Results never depend on them, only speed. */
+ * spread_cache_launch_chunks (chunk lengths in units of 16 KiB);
+ * stream_wgs_per_cu (one-wave workgroups per CU of a fold / tree launch; 0:
+ * the library's choice by size, rank count and outputs), fold_front3_ranks
+ * (rank count from which a fold asks for three streams up front instead of
+ * two; 0: 12); halo_load_policy (the cache policy of the grid loads of a halo
+ * pack: 0 plain, 1 nt, 2 sc1, 3 sc0 sc1, 4 sc0 sc1 nt).  Piece sizes below
+ * 64 KiB are refused.  Results never depend on them, only speed. */
 int alamd_tune(const char *name, size_t value);
 size_t alamd_tuned(const char *name);
 /* The number of kernel launches that alamd_combine makes for one output of

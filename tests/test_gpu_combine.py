@@ -628,13 +628,18 @@ SETTINGS = [
      "spread_launch_bytes": 1 << 40, "ring_piece_bytes": 1 << 40},
     {"two_step_min_total_bytes": 1, "two_step_min_outputs": 2, "two_step_piece_bytes": 1 << 20,
      "spread_cache_chunk_tiles": 16, "spread_cache_launch_chunks": 2, "launch_bytes": 3 << 20},
+    # the streaming kernels: few waves per CU and three streams up front for every rank count, ...
+    {"stream_wgs_per_cu": 4, "fold_front3_ranks": 2},
+    # ... as many as fit and two up front for every rank count
+    {"stream_wgs_per_cu": 32, "fold_front3_ranks": 1000, "launch_bytes": 1 << 22},
 ]
 
 
 @pytest.mark.parametrize("k", range(len(SETTINGS)))
 def test_results_do_not_depend_on_the_launch_planners_sizes(al, k):
     """The sizes the launch planners cut their work by (bytes per launch, the thresholds and pieces of
-    the two-step calls, the spread's chunks) only decide how the same work is spread over launches:
+    the two-step calls, the spread's chunks, the waves per CU and streams requested up front of the
+    streaming kernels) only decide how the same work is spread over launches and waves:
     extreme settings give the bits of the defaults, i.e. the oracle's."""
     import torch
     P, n = 5, 1_300_007
