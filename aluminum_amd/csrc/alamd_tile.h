@@ -126,4 +126,25 @@ template <int U, int THREADS> struct Tile {
   }
 };
 
+// Stores one tile's result to out[j0 .. j0 + nj): the pointers are fetched four at a time, so that a
+// wave that writes several buffers does not wait for one scalar load per buffer, one after the other.
+template <typename TL, int U>
+__device__ __forceinline__ void store_to_outputs(const TL &tl, char *const *out, int j0, int nj, size_t byte_off,
+                                                 int nrec, const u32x4 (&v)[U]) {
+  const int end = j0 + nj;
+  for (int j = j0; j < end; j += 4) {
+    char *o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o[k] = out[j + k < end ? j + k : end - 1];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (j + k < end) {
+        const auto r = TL::rsrc(o[k] + byte_off, nrec);
+#pragma unroll
+        for (int u = 0; u < U; ++u) tl.store(r, u, v[u]);
+      }
+    }
+  }
+}
+
 }  // namespace alamd

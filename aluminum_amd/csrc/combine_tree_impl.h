@@ -295,11 +295,7 @@ tree_vec_kernel(const TreeParams p) {
 #pragma unroll
     for (int u = 0; u < U; ++u) res[u] = finish_vec<T, OP>(res[u], p.div);
     if constexpr (CHAIN) chain_gate(p.chain, bx, tb, (unsigned long long)nrec, (unsigned)TL::BYTES);
-    for (int j = j0; j < j0 + nj; ++j) {
-      const auto r = TL::rsrc(p.out[j] + vout + tb, nrec);
-#pragma unroll
-      for (int u = 0; u < U; ++u) tl.store(r, u, res[u]);
-    }
+    store_to_outputs<TL, U>(tl, p.out, j0, nj, vout + tb, nrec, res);
   }
   if constexpr (CHAIN) {
     // the vlen % N elements behind the last whole vector are the last ticket

@@ -12,7 +12,7 @@
 //                  tree_halving|tree_binomial|tree_reduce_scatter_gather|pairwise|ring|ring_fused] [--ranks P] [--root R]
 //                  [--inplace] [--nonblocking] [--min-size N] [--max-size N] [--size N] [--num-iters N]
 //                  [--num-warmup N] [--summarize] [--save-to-file FILE] [--no-print-table] [--backend hip]
-//                  [--stream-per-rank]
+//                  [--stream-per-rank] [--tune name=value ...]
 // (--summarize: per size "Size Mean Median Stdev Min Max" over the timed trials, benchmark_ops.cpp:211-224;
 // --save-to-file / --no-print-table: where the table of rows goes, :225-230.)
 #include <hip/hip_runtime_api.h>
@@ -188,6 +188,14 @@ int main(int argc, char **argv) {
     else if (a == "--save-to-file") o.save_to = next();
     else if (a == "--no-print-table") o.print_table = false;
     else if (a == "--stream-per-rank") o.stream_per_rank = true;
+    else if (a == "--tune") {  // name=value: one of the launch planner's settings (alamd_tune)
+      const std::string kv = next();
+      const size_t eq = kv.find('=');
+      if (eq == std::string::npos || alamd_tune(kv.substr(0, eq).c_str(), std::strtoull(kv.c_str() + eq + 1, nullptr, 10)) != ALAMD_OK) {
+        std::fprintf(stderr, "bad --tune %s\n", kv.c_str());
+        return 2;
+      }
+    }
     else if (a == "--backend") { if (next() != "hip") { std::fprintf(stderr, "this program benchmarks the hip backend only\n"); return 2; } }
     else if (a == "--help") { std::printf("see the usage comment at the top of tests/cpp/bench_ops.cpp\n"); return 0; }
     else if (a == "--ranks") o.ranks = std::atoi(next().c_str());
