@@ -1,6 +1,7 @@
 // Host-only property test of the launch planner (plan_launches, alamd_dispatch.h): whatever the
 // segment lengths and the launch size, the launches it asks for cover every (segment, tile) exactly
-// once, in grids the device accepts.  Needs no GPU: nothing is launched.
+// once, in grids the device accepts.  Also: the block lookup of the role masks against its definition,
+// and the LDS sizing of the streaming launches.  Needs no GPU: nothing is launched.
 //
 // usage: test_planner [trials, default 4000]
 #include <cstdio>
@@ -9,6 +10,7 @@
 #include <vector>
 
 #include "alamd_dispatch.h"
+#include "alamd_tile.h"
 
 using namespace alamd;
 
@@ -81,6 +83,59 @@ int main(int argc, char **argv) {
     launches_total += launches;
     idle_total += idle;
     busy_total += busy;
+  }
+  // The block of a message that an element lies in (role_mask_of_elem): the lookup through prepared
+  // reciprocals gives what the 64-bit divisions give, and the block ends where it says - for both ways
+  // of cutting a message, every number of blocks, bases inside the message, and lengths up to 2^40.
+  for (int trial = 0; trial < trials && g_fail < 10; ++trial) {
+    TreeParams tp = {};
+    tp.role_bits = (int)pick(0, 6);
+    tp.role_spread = (int)pick(0, 1);
+    const unsigned long long n = trial % 3 == 0 ? pick(1, 5000) : (trial % 3 == 1 ? pick(1, (size_t)1 << 40) : ((size_t)1 << pick(6, 40)) + pick(0, 70));
+    const unsigned long long base = pick(0, n - 1), seg_len = n - base;
+    tp.role_base = base;
+    tp.role_count = n;
+    TreeParams fast = tp;
+    fast.role_n = n;
+    fast.role_blk = n >> tp.role_bits;
+    fast.role_inv_blk = fast.role_blk ? 1.0 / (double)fast.role_blk : 0.0;
+    fast.role_inv_blk1 = 1.0 / (double)(fast.role_blk + 1);
+    const unsigned long long blocks = 1ull << tp.role_bits, blk = n >> tp.role_bits, longer = n & (blocks - 1);
+    for (int k = 0; k < 200; ++k) {
+      // elements at and around the block boundaries, and anywhere
+      unsigned long long x;
+      if (k < 150 && blk > 0) {
+        const unsigned long long b = pick(0, blocks - 1);
+        const unsigned long long start = tp.role_spread ? b * blk + (b < longer ? b : longer) : b * blk;
+        x = start + pick(0, 2) - 1;
+        if (x >= n) x = n - 1;
+      } else {
+        x = pick(0, n - 1);
+      }
+      if (x < base) x = base;
+      const size_t e = (size_t)(x - base);
+      unsigned long long end_slow = 0, end_fast = 0;
+      const unsigned ms = role_mask_of_elem(tp, (size_t)seg_len, e, &end_slow), mf = role_mask_of_elem(fast, (size_t)seg_len, e, &end_fast);
+      EXPECT(ms == mf && end_slow == end_fast, "block lookup: n %llu bits %d spread %d element %llu: mask %u / %u, end %llu / %llu", n,
+             tp.role_bits, tp.role_spread, x, ms, mf, end_slow, end_fast);
+      // the block by its definition
+      unsigned long long kb = 0, lo = 0, hi = 0;
+      for (kb = 0; kb < blocks; ++kb) {
+        lo = tp.role_spread ? kb * blk + (kb < longer ? kb : longer) : kb * blk;
+        hi = kb == blocks - 1 ? n : (tp.role_spread ? lo + blk + (kb < longer ? 1 : 0) : lo + blk);
+        if (x >= lo && x < hi) break;
+      }
+      EXPECT(kb < blocks && ms == role_bit_reverse((unsigned)kb, tp.role_bits), "block lookup: n %llu bits %d spread %d element %llu is in block %llu", n,
+             tp.role_bits, tp.role_spread, x, kb);
+      EXPECT(kb == blocks - 1 ? end_slow == ~0ull : end_slow == hi - base, "block lookup: end of block %llu: %llu, expected %llu", kb, end_slow, hi - base);
+    }
+  }
+  // The LDS a streaming launch asks for lets exactly the wanted number of one-wave workgroups into a CU's
+  // 160 KiB, up to the eight waves per SIMD the kernels are compiled for.
+  for (int n = 1; n <= 40; ++n) {
+    const unsigned lds = stream_lds_bytes(n);
+    const int want = n < 4 ? 4 : (n > 32 ? 32 : n);
+    EXPECT(lds >= 128 && 160u * 1024u / lds >= (unsigned)want && 160u * 1024u / (lds + 128) <= (unsigned)want, "LDS for %d workgroups per CU: %u bytes", n, lds);
   }
   // workgroups that find nothing to do: a planner that put every segment side by side in one grid
   // would idle far more than it works on the "one long among short" shapes

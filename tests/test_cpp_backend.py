@@ -21,7 +21,9 @@ def test_front_end_compiles_with_the_host_compiler():
 
 def test_launch_planner_covers_every_tile_once():
     """plan_launches (alamd_dispatch.h) on random segment tables, on the host: every tile of every
-    segment in exactly one launch, grids within the device's limits."""
+    segment in exactly one launch, grids within the device's limits; the block lookup of the role masks
+    (through prepared reciprocals) against 64-bit division and against the definition of the blocks;
+    the LDS sizing of the streaming launches."""
     exe = os.path.join(ROOT, "tests", "cpp", "test_planner")
     if not os.path.exists(exe):
         subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp"), "test_planner"], check=True,
