@@ -77,16 +77,16 @@ struct SegParams {
   unsigned long long tile0;  // index of the first tile of this launch
   unsigned seg0;             // position of the first segment of this launch
   int mapped;                // 1: the segment at position i is order[i], 0: it is i
-  unsigned char order[ALAMD_MAX_RANKS];
-  // leading elements of each segment handled one by one (see head_count); the host fills this in, so
-  // that no workgroup has to wait for the output pointer before it can issue its loads
-  unsigned char seg_head[ALAMD_MAX_RANKS];
-  int any_head;              // 0: every seg_head is zero (all buffers 64-byte aligned: the usual case)
+  alignas(4) unsigned char order[ALAMD_MAX_RANKS];
+  // leading elements of each segment handled one by one (see stream_head_count); the host fills this
+  // in, so that no workgroup has to wait for the output pointer before it can issue its loads
+  alignas(4) unsigned short seg_head[ALAMD_MAX_RANKS];
+  int any_head;              // 0: every seg_head is zero (all buffers 1 KiB aligned: the usual case)
   int in_blocked;   // 1: inputs are read at the segment's offset, 0: at 0
   int out_mode;     // OUT_ALL / OUT_SEG / OUT_OWNER
   int owner_shift;  // OUT_OWNER: output index is (segment + owner_shift) mod P
   int nout;         // OUT_ALL: number of outputs written
-  int simple;       // 1: one segment from element 0, one output, no head (the kernels then skip the lookups)
+  int simple;       // 1: one segment from element 0, one output (the kernels then skip the lookups)
   int ragged;       // 1: segments are given by the two tables below
   unsigned long long seg_off[ALAMD_MAX_RANKS];
   unsigned long long seg_len[ALAMD_MAX_RANKS];
@@ -108,8 +108,18 @@ inline SegParams make_seg(size_t seg_base, size_t seg_rem, int in_blocked, int o
 // (These lookups are a chain of dependent scalar loads, one branch per mode.  Reading every table
 // whatever the mode and choosing afterwards shortens the chain but ran 2 to 3 % slower for a
 // Reduce_scatter; the launches that need no lookup at all skip them instead: SegParams::simple.)
+// Entry i of a table of bytes or of 16-bit numbers in the kernel's arguments, i the same in every lane:
+// read as the dword it lies in, which is a scalar load; read as what it is, it would be a vector load
+// (there are no scalar loads of less than a dword), i.e. a round trip through the memory pipeline that
+// a workgroup's first requests would wait for.  Both tables start on a dword.
+__device__ __forceinline__ unsigned arg_u8(const unsigned char *table, unsigned i) {
+  return (reinterpret_cast<const unsigned *>(table)[i >> 2] >> ((i & 3u) * 8u)) & 0xffu;
+}
+__device__ __forceinline__ unsigned arg_u16(const unsigned short *table, unsigned i) {
+  return (reinterpret_cast<const unsigned *>(table)[i >> 1] >> ((i & 1u) * 16u)) & 0xffffu;
+}
 __device__ __forceinline__ unsigned seg_of(const SegParams &s, unsigned pos) {
-  return s.mapped ? s.order[pos] : pos;
+  return s.mapped ? arg_u8(s.order, pos) : pos;
 }
 
 __host__ __device__ inline void seg_range(const SegParams &s, unsigned seg, size_t &off, size_t &len) {

@@ -49,6 +49,9 @@ inline size_t launch_tiles(int nin, size_t tile_bytes, size_t launch_bytes = kLa
   return t < 8 ? 8 : t;
 }
 
+// Bytes per stream of a tile of the streaming fold and tree kernels (one wave, one vector per lane).
+constexpr size_t kStreamTileBytes = 1024;
+
 // Loads of 128 bits run at full rate from any 4-byte-aligned address; from an
 // address that splits its dwords they lose about a fifth of the bandwidth.
 // Stores want whole 64-byte lines: on buffers that no earlier launch has
@@ -63,12 +66,25 @@ __host__ __device__ inline size_t head_count(size_t elem_size, const char *out, 
   const size_t h = bytes / elem_size;
   return h < len ? h : len;
 }
+// The streaming kernels (one wave and 1 KiB per stream and tile) want more: a tile that starts off a
+// 1 KiB boundary of its streams shares its first and last 128-byte lines with its neighbours, which run
+// at the same time on other XCDs, and both fetch them.  P = 8 fold of f32, 256 MiB per rank, every
+// buffer the same number of bytes off a 2 MiB boundary: 0: 85 % of the HBM peak, 1 KiB and more: 85,
+// 512: 83.5, 256: 83, 128: 82, 64: 74.  From kBigHeadFromBytes per segment on, the leading elements
+// therefore reach to the first input's next 1 KiB boundary (f32, every buffer 4 bytes off: 73 -> 84 %;
+// output 20 bytes off the inputs: 73 -> 77 %: reads that split lines cost more than writes that do),
+// spread over the segment's first workgroups, 64 elements each; shorter segments keep the rule above,
+// since their few workgroups would spend longer on the elements than on the tiles.
+constexpr size_t kBigHeadFromBytes = (size_t)64 << 10;
+__host__ __device__ inline size_t stream_head_count(size_t elem_size, const char *out, const char *first, size_t len) {
+  if (len * elem_size < kBigHeadFromBytes) return head_count(elem_size, out, first, len);
+  const uintptr_t f = reinterpret_cast<uintptr_t>(first);
+  return ((kStreamTileBytes - (size_t)(f & (kStreamTileBytes - 1))) & (kStreamTileBytes - 1)) / elem_size;
+}
 template <typename T> __device__ __forceinline__ size_t head_elems(const char *out, const char *first, size_t len) {
   return head_count(sizeof(T), out, first, len);
 }
 
-// Bytes per stream of a tile of the streaming fold and tree kernels (one wave, one vector per lane).
-constexpr size_t kStreamTileBytes = 1024;
 // The streaming kernels are compiled for up to kStreamMaxWaves waves per SIMD; how many a launch really
 // gets is set when it is launched, through the LDS it asks for: a CU has 160 KiB and a workgroup is one
 // wave, so with 160 KiB / n bytes each n workgroups fit a CU (LDS is handed out by the KiB, so the

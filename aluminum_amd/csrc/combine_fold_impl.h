@@ -64,8 +64,8 @@ template <typename T, int OP, bool CHAIN = false> struct Shape {
 // (P = 8: 84 against 84 %, P = 12: 82 and 82, P = 16: 84 against 81, P = 64: 82 against 79).
 constexpr int kFront3FromRanks = 12;
 
-// HEAD = false: no segment has leading elements to handle one by one (every buffer on a 64-byte
-// boundary); two kernels, and the host picks, so that the usual case carries no trace of the other.
+// HEAD = false: no segment has leading elements to handle one by one (see stream_head_count); two
+// kernels, and the host picks, so that the usual case carries no trace of the other.
 // FRONT: see Shape (0 in a chained launch).
 // CHAIN: the output overlaps one of the inputs at a displacement; tiles come from a ticket counter and
 // a tile's stores wait for the loads of the tiles that read what it writes (see ChainParams).  Always
@@ -96,7 +96,7 @@ fold_vec_kernel(const FoldParams p) {
     out_select(p.seg, P, seg, off_bytes, j0, nj, out_bytes);
   }
 
-  const size_t head = HEAD ? p.seg.seg_head[seg] : 0;
+  const size_t head = HEAD ? arg_u16(p.seg.seg_head, seg) : 0;
   const size_t vlen = len - head;
   const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
   const size_t vec_bytes = (vlen / N) * 16;
@@ -214,12 +214,16 @@ fold_vec_kernel(const FoldParams p) {
       if (mine) st_elem<T>(p.out[j0] + out_bytes + e * sizeof(T), val);
     }
   } else {
-    // the head elements and the vlen % N elements behind the last whole vector, one per thread of the
-    // segment's first workgroup (up to 63 and 15 of them)
-    if (p.seg.tile0 == 0 && blockIdx.x == 0) {
-      for (size_t t = threadIdx.x; t < head + vlen % N; t += THREADS) {
-        const size_t e = t < head ? t : (vlen / N) * N + t;
-        fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
+    // the head elements and the vlen % N elements behind the last whole vector (up to 1 KiB's worth and
+    // 15 of them), one per thread of the segment's first workgroups
+    const size_t loose = head + vlen % N;
+    if (loose) {
+      const size_t ntiles = vec_bytes ? (vec_bytes + TL::BYTES - 1) / TL::BYTES : 1, mine = (size_t)p.seg.tile0 + blockIdx.x;
+      if (mine < ntiles) {
+        for (size_t t = mine * THREADS + threadIdx.x; t < loose; t += ntiles * THREADS) {
+          const size_t e = t < head ? t : (vlen / N) * N + t;
+          fold_elem<T, OP, ACC_IS_IN>(p, P, s, in_bytes, j0, nj, out_bytes, e);
+        }
       }
     }
   }
@@ -272,12 +276,12 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
       seg_range(p.seg, sg, off, len);
       out_select(p.seg, p.P, sg, off * sizeof(T), j0, nj, out_bytes);
       const int first = (p.start0 + (int)sg * p.start_stride) % p.P;
-      q.seg.seg_head[sg] = (unsigned char)head_count(sizeof(T), p.out[j0] + out_bytes,
+      q.seg.seg_head[sg] = (unsigned short)stream_head_count(sizeof(T), p.out[j0] + out_bytes,
                                                      p.in[first] + (p.seg.in_blocked ? off * sizeof(T) : 0), len);
       if (q.seg.seg_head[sg]) q.seg.any_head = 1;
     }
     q.seg.simple = nseg == 1 && !q.seg.ragged && q.seg.seg_rem == 0 && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1 &&
-                   !q.seg.any_head && p.start0 >= 0 && p.start0 < p.P;
+                   p.start0 >= 0 && p.start0 < p.P;
     auto pick = [&](auto acc_is_in_t, auto front_t) -> void (*)(const FoldParams) {
       constexpr bool A = decltype(acc_is_in_t)::value;
       constexpr int FRONT = decltype(front_t)::value;

@@ -57,9 +57,10 @@ __device__ __forceinline__ void tree_elem(const TreeParams &p, size_t in_bytes, 
 // block, so that the mask is the same in every lane and may index the argument tables.
 template <typename T, int OP, int SLOTS, int HALVES, int THREADS>
 __device__ __forceinline__ void tree_elems(const TreeParams &p, size_t len, size_t in_bytes, int j0, int nj,
-                                           size_t out_bytes, size_t lo, size_t hi, unsigned w, bool per_block) {
+                                           size_t out_bytes, size_t lo, size_t hi, unsigned w, bool per_block,
+                                           size_t first = threadIdx.x, size_t stride = THREADS) {
   if (!per_block) {
-    for (size_t e = lo + threadIdx.x; e < hi; e += THREADS) tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e, w);
+    for (size_t e = lo + first; e < hi; e += stride) tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e, w);
     return;
   }
   size_t e0 = lo;
@@ -67,7 +68,7 @@ __device__ __forceinline__ void tree_elems(const TreeParams &p, size_t len, size
     unsigned long long block_end;
     const unsigned m = (unsigned)__builtin_amdgcn_readfirstlane((int)role_mask_of_elem(p, len, e0, &block_end));
     const size_t stop = block_end < hi ? (size_t)block_end : hi;
-    for (size_t e = e0 + threadIdx.x; e < stop; e += THREADS) tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e, m);
+    for (size_t e = e0 + first; e < stop; e += stride) tree_elem<T, OP, SLOTS, HALVES>(p, in_bytes, j0, nj, out_bytes, e, m);
     e0 = stop;
   }
 }
@@ -130,7 +131,7 @@ tree_vec_kernel(const TreeParams p) {
     tree_out_select(p, seg, off_bytes, in_bytes, j0, nj, out_bytes);
   }
 
-  const size_t head = HEAD ? p.seg.seg_head[seg] : 0;
+  const size_t head = HEAD ? arg_u16(p.seg.seg_head, seg) : 0;
   const size_t vlen = len - head;
   const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
   const size_t vec_bytes = (vlen / N) * 16;
@@ -309,12 +310,16 @@ tree_vec_kernel(const TreeParams p) {
       if (mine) st_elem<T>(p.out[j0] + out_bytes + e * sizeof(T), val);
     }
   } else {
-    // the head elements and the vlen % N elements behind the last whole vector
-    if (p.seg.tile0 == 0 && blockIdx.x == 0) {
-      const bool per_block = ROLES && p.role_mode == ROLE_PER_BLOCK;
-      const size_t tail = head + (vlen / N) * N;
-      tree_elems<T, OP, SLOTS, HALVES, THREADS>(p, len, in_bytes, j0, nj, out_bytes, 0, head, w, per_block);
-      tree_elems<T, OP, SLOTS, HALVES, THREADS>(p, len, in_bytes, j0, nj, out_bytes, tail, tail + vlen % N, w, per_block);
+    // the head elements and the vlen % N elements behind the last whole vector, spread over the
+    // segment's first workgroups
+    if (head + vlen % N) {
+      const size_t ntiles = vec_bytes ? (vec_bytes + TL::BYTES - 1) / TL::BYTES : 1, mine = (size_t)p.seg.tile0 + blockIdx.x;
+      if (mine < ntiles) {
+        const bool per_block = ROLES && p.role_mode == ROLE_PER_BLOCK;
+        const size_t tail = head + (vlen / N) * N, first = mine * THREADS + threadIdx.x, stride = ntiles * THREADS;
+        tree_elems<T, OP, SLOTS, HALVES, THREADS>(p, len, in_bytes, j0, nj, out_bytes, 0, head, w, per_block, first, stride);
+        tree_elems<T, OP, SLOTS, HALVES, THREADS>(p, len, in_bytes, j0, nj, out_bytes, tail, tail + vlen % N, w, per_block, first, stride);
+      }
     }
   }
 }
@@ -380,11 +385,10 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
     seg_range(p.seg, sg, off, len);
     const size_t in_bytes = p.seg.in_blocked ? off * sizeof(T) : 0;
     tree_out_select(p, sg, off * sizeof(T), in_bytes, j0, nj, out_bytes);
-    q.seg.seg_head[sg] = (unsigned char)head_count(sizeof(T), p.out[j0] + out_bytes, p.a[0] + in_bytes, len);
+    q.seg.seg_head[sg] = (unsigned short)stream_head_count(sizeof(T), p.out[j0] + out_bytes, p.a[0] + in_bytes, len);
     if (q.seg.seg_head[sg]) q.seg.any_head = 1;
   }
-  q.seg.simple = nseg == 1 && !q.seg.ragged && q.seg.seg_rem == 0 && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1 &&
-                 !q.seg.any_head;
+  q.seg.simple = nseg == 1 && !q.seg.ragged && q.seg.seg_rem == 0 && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1;
   const size_t wgs = tunables().stream_wgs_per_cu;
   const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + 1);
   const unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(true, SLOTS * HALVES, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes));

@@ -137,6 +137,28 @@ int main(int argc, char **argv) {
     const int want = n < 4 ? 4 : (n > 32 ? 32 : n);
     EXPECT(lds >= 128 && 160u * 1024u / lds >= (unsigned)want && 160u * 1024u / (lds + 128) <= (unsigned)want, "LDS for %d workgroups per CU: %u bytes", n, lds);
   }
+  // The leading elements of a segment: never more than the segment, whole elements, below 1 KiB's worth;
+  // long segments then have their first input on a 1 KiB boundary, short ones their output on a 64-byte
+  // boundary where the first input's vectors then start on a dword (else the first input on a dword).
+  {
+    std::mt19937_64 rng(4242);
+    const size_t sizes[] = {1, 2, 4, 8};
+    for (int t = 0; t < 20000; ++t) {
+      const size_t es = sizes[rng() % 4];
+      const uintptr_t out = (uintptr_t)((rng() % (1u << 20)) * es), first = (uintptr_t)((rng() % (1u << 20)) * es);
+      const size_t len = t % 3 == 0 ? rng() % 200 : (t % 3 == 1 ? kBigHeadFromBytes / es - 2 + rng() % 5 : rng() % (1u << 22));
+      const size_t h = stream_head_count(es, reinterpret_cast<const char *>(out), reinterpret_cast<const char *>(first), len);
+      EXPECT(h <= len && h * es < kStreamTileBytes, "head of %zu elements of %zu bytes, segment of %zu", h, es, len);
+      if (h == len) continue;
+      if (len * es >= kBigHeadFromBytes) {
+        EXPECT((first + h * es) % kStreamTileBytes == 0, "long segment: first input %zu bytes off a tile boundary", (size_t)((first + h * es) % kStreamTileBytes));
+      } else if ((out ^ first) % 4 == 0) {
+        EXPECT((out + h * es) % 64 == 0 && (first + h * es) % 4 == 0, "short segment: output %zu bytes off a line", (size_t)((out + h * es) % 64));
+      } else {
+        EXPECT((first + h * es) % 4 == 0, "short segment: first input splits its dwords (%zu)", (size_t)((first + h * es) % 4));
+      }
+    }
+  }
   // workgroups that find nothing to do: a planner that put every segment side by side in one grid
   // would idle far more than it works on the "one long among short" shapes
   EXPECT(idle_total < busy_total, "idle workgroups %zu against %zu busy ones", idle_total, busy_total);

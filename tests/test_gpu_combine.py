@@ -149,6 +149,56 @@ def test_head_up_to_the_outputs_64_byte_boundary(al, dtype):
 
 
 @pytest.mark.parametrize("dtype", ("u8", "bf16", "f32", "f64"))
+def test_head_up_to_the_first_inputs_1kib_boundary(al, dtype):
+    """From 64 KiB per segment on, the streaming kernels walk the leading elements one by one until the
+    first input reaches a 1 KiB boundary (up to 1023 bytes' worth, spread over the segment's first
+    workgroups): lengths just below, at and above that size, inputs and outputs at the same and at
+    different offsets from one element to one short of 1 KiB, fold and tree orders, two outputs, one
+    launch and many; float min under a reduce-scatter + gather order, whose operand roles change from
+    block to block, heads included; the ragged segments of a Reduce_scatterv."""
+    import torch
+    P = 3
+    es = oracle.dtype_size(dtype)
+    kib = 1024 // es
+    for in_off, out_off in ((1, 1), (kib - 1, kib - 1), (kib // 2 + 1, 3), (0, 5), (7, 0)):
+        for n in (64 * kib - 1, 64 * kib, 64 * kib + 1, 300 * kib + 37):
+            ins = make_inputs(P, n, dtype, "sum", seed=70 + in_off)
+            views = [_offset_view(a, in_off + (r if in_off != out_off else 0)) for r, a in enumerate(ins)]
+            for order, launch_bytes in (("rank_asc", 0), ("tree_dbl", 0), ("rank_asc", 1 << 18), ("tree_halv", 1 << 18)):
+                want = oracle.combine(ins, dtype, "sum", order)
+                raws = [dev_empty(n + out_off + 16, ins[0].dtype) for _ in range(2)]
+                try:
+                    al.tune("launch_bytes", launch_bytes)
+                    al.combine([r[out_off:out_off + n] for r in raws], views, "sum", order=order, dtype=dtype, count=n)
+                    torch.cuda.synchronize()
+                finally:
+                    al.tune("launch_bytes", 0)
+                for r in raws:
+                    assert_bits_equal(to_host(r, ins[0].dtype)[out_off:out_off + n], want, dtype,
+                                      "%s %s out+%d in+%d n=%d launches of %d" % (dtype, order, out_off, in_off, n, launch_bytes))
+    if dtype in ("bf16", "f32", "f64"):
+        n = 200 * kib + 11
+        ins = [planted_specials(n, dtype, r) for r in range(5)]
+        views = [_offset_view(a, 3) for a in ins]
+        for order in ("tree_rsg", "tree_rsg_spread", "rank_asc"):
+            want = oracle.combine(ins, dtype, "min", order)
+            raw = dev_empty(n + 3, ins[0].dtype)
+            al.combine([raw[3:]], views, "min", order=order, dtype=dtype, count=n)
+            torch.cuda.synchronize()
+            assert_bits_equal(to_host(raw, ins[0].dtype)[3:], want, dtype, "%s min %s, buffers 3 elements in" % (dtype, order))
+    counts = [70 * kib + 3, 0, 65 * kib + 1, 5, 129 * kib - 7]
+    sends = make_inputs(len(counts), sum(counts), dtype, "sum", seed=77)
+    d_sends = [_offset_view(a, 1) for a in sends]
+    for order in ("rank_asc", "tree_halv"):
+        want = oracle.reduce_scatterv(sends, counts, dtype, "sum", order)
+        recvs = [dev_empty(c + 2, sends[0].dtype)[2:] for c in counts]
+        al.reduce_scatterv(recvs, d_sends, counts, "sum", order=order, dtype=dtype)
+        torch.cuda.synchronize()
+        for b, c in enumerate(counts):
+            assert_bits_equal(to_host(recvs[b], sends[0].dtype)[:c], want[b], dtype, "reduce_scatterv %s rank %d" % (order, b))
+
+
+@pytest.mark.parametrize("dtype", ("u8", "bf16", "f32", "f64"))
 @pytest.mark.parametrize("inplace", (False, True))
 def test_reduce_scatter_odd_block_sizes(al, dtype, inplace):
     """Block sizes that put every block but the first off a 16-byte boundary."""
