@@ -22,7 +22,8 @@ METRIC = "combine HBM GB/s (% of 8 TB/s peak), P=8 fp32/bf16 sum, 2 GiB buffers"
 HBM_PEAK_GBPS = 8000.0
 
 WORKLOADS = {
-    # name: (dtype, count per rank, op, dist, seed base, order)
+    # name: (dtype, count per rank, op, dist, seed base, order[, buffer sets[, (elements the inputs, the
+    # output start into their allocations)]])
     "c2_f32_sum": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "rank_asc"),
     "c2_f32_prod": ("f32", 1 << 26, "prod", "uniform_09_11", 1000, "rank_asc"),
     "c2_f32_sum_tree": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "tree_rsg"),
@@ -41,6 +42,11 @@ WORKLOADS = {
     # launch reads or writes was touched by the three launches before it
     "c2_f32_sum_rotating": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "rank_asc", 4),
     "c2_bf16_sum_rotating": ("bf16", 1 << 27, "sum", "normal", 2000, "rank_asc", 4),
+    # the same with buffers that start off the 1 KiB boundaries the kernels' tiles like: every buffer one
+    # element into its allocation; the inputs at the start of theirs and the output five elements in
+    "c2_f32_sum_rotating_one_element_in": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "rank_asc", 4, (1, 1)),
+    "c2_f32_sum_rotating_output_five_elements_in": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "rank_asc", 4, (0, 5)),
+    "c2_f32_sum_tree_rotating_one_element_in": ("f32", 1 << 26, "sum", "uniform_pm1", 1000, "tree_rsg", 4, (1, 1)),
 }
 P = 8
 
@@ -186,12 +192,13 @@ def run_halo_policy_workload(al, torch, steps, warmup):
 def run_combine_workload(al, torch, name, steps, warmup, check=True):
     dtype, count, op, dist, seed, order = WORKLOADS[name][:6]
     nsets = WORKLOADS[name][6] if len(WORKLOADS[name]) > 6 else 1
+    in_off, out_off = WORKLOADS[name][7] if len(WORKLOADS[name]) > 7 else (0, 0)
     es = al.dtype_size(dtype)
     carrier = al.torch_dtype(dtype)
     sets = []
     for _ in range(nsets):
-        ins = [torch.empty(count, dtype=carrier, device="cuda") for _ in range(P)]
-        out = torch.empty(count, dtype=carrier, device="cuda")
+        ins = [torch.empty(count + in_off, dtype=carrier, device="cuda")[in_off:] for _ in range(P)]
+        out = torch.empty(count + out_off, dtype=carrier, device="cuda")[out_off:]
         for r in range(P):
             al.fill(ins[r], dist, seed + r, dtype=dtype)
         sets.append((ins, out))
@@ -213,7 +220,7 @@ def run_combine_workload(al, torch, name, steps, warmup, check=True):
     alg_bytes = (P + 1) * count * es
     res = {
         "workload": name, "dtype": dtype, "op": op, "order": order, "P": P, "count": count,
-        "buffer_sets": nsets, "launches_per_step": al.planned_launches(P, count, dtype),
+        "buffer_sets": nsets, "elements_into_allocation": {"inputs": in_off, "output": out_off}, "launches_per_step": al.planned_launches(P, count, dtype),
         "algorithmic_bytes": alg_bytes, "ms_per_step": wall * 1e3 / steps, "kernel_ms": kernel_ms,
         "gbps_wall": alg_bytes / (wall / steps) * 1e-9, "gbps_kernel": alg_bytes / (kernel_ms * 1e-3) * 1e-9,
     }
