@@ -35,6 +35,7 @@ int device_cus();
 // stands where it is used).  Defaults suit an MI355X; alamd_tune() changes them for comparisons.
 // Process-wide; every field is an atomic, so that a setting changed while calls run is a clean old-or-new
 // value for each of them, never a torn one.
+constexpr size_t kBlockShapeFromBytes = (size_t)32 << 20, kBlockShapeBelowBytes = (size_t)384 << 20;
 struct Tunables {
   std::atomic<size_t> launch_bytes{(size_t)4 << 30};            // bytes one fold / tree launch moves
   std::atomic<size_t> two_step_min_total_bytes{(size_t)128 << 20};  // fold + spread instead of one kernel: from this
@@ -46,6 +47,8 @@ struct Tunables {
   std::atomic<size_t> spread_hbm_chunk_tiles{1024}, spread_hbm_launch_chunks{2};      // slices read from HBM
   std::atomic<size_t> spread_cache_chunk_tiles{512}, spread_cache_launch_chunks{16};  // a result just written
   std::atomic<size_t> stream_wgs_per_cu{0};  // workgroups per CU of a streaming fold / tree launch (0: the kernels' own)
+  // a fold / tree launch that moves this much in all and less than that takes the block shape (alamd_tile.h)
+  std::atomic<size_t> block_shape_from_bytes{kBlockShapeFromBytes}, block_shape_below_bytes{kBlockShapeBelowBytes};
   std::atomic<size_t> fold_front3_ranks{0};  // ranks from which a fold asks for three streams up front (0: by type)
   std::atomic<size_t> halo_load_policy{0};  // grid loads of a halo pack: 0 plain, 1 nt, 2 sc1, 3 sc0 sc1, 4 sc0 sc1 nt
 };

@@ -66,6 +66,13 @@ template <typename F> int dispatch_any(int dtype, int op, F &&f) {
   }
 }
 
+// Whether a fold / tree launch that reads and writes total_bytes in all takes the block shape
+// (the measurements are in alamd_tile.h, above Tile).
+enum { FOLD_STREAM = 0, FOLD_BLOCK = 1, FOLD_CHAINED = 2 };  // the KIND of a fold / tree kernel
+inline bool use_block_shape(size_t total_bytes) {
+  return total_bytes >= tunables().block_shape_from_bytes && total_bytes < tunables().block_shape_below_bytes;
+}
+
 // ---- parameters of the two combine kernel families -------------------------
 
 // Work is a grid of segments (blockIdx.y) x tiles (blockIdx.x).  Segment s

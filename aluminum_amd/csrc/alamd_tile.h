@@ -85,6 +85,8 @@ template <typename T> __device__ __forceinline__ size_t head_elems(const char *o
   return head_count(sizeof(T), out, first, len);
 }
 
+// ... and of the fold's block shape (128 threads x 8 vectors).
+constexpr size_t kBlockTileBytes = 16384;
 // The streaming kernels are compiled for up to kStreamMaxWaves waves per SIMD; how many a launch really
 // gets is set when it is launched, through the LDS it asks for: a CU has 160 KiB and a workgroup is one
 // wave, so with 160 KiB / n bytes each n workgroups fit a CU (LDS is handed out by the KiB, so the
@@ -116,6 +118,20 @@ inline int stream_wgs_per_cu(bool tree, int streams, int outputs, size_t total_b
   if (streams <= 2) return 26;
   return tree ? 16 : 22;
 }
+
+// Between 32 and 384 MiB (bytes a launch reads and writes in all) the fold and tree kernels take the
+// block shape instead (128 or 256 threads x 4 or 8 vectors, every load of a lane issued up front, two
+// waves per SIMD): a launch of tens of microseconds, much of whose data the caches hold, gains more from
+// having a sixteenth of the workgroups to hand out and from workgroups that are done after one trip to
+// memory than it loses by what queues up in front of the L2.  The bare patterns (8 streams read, 1 or 8
+// written, the same buffers again and again), us per launch, streaming (best setting) against block:
+//   MiB per stream        4            8             16            32           64     128
+//   1 written       4.8 / 4.1   10.8 / 10.3   21.6 / 20.8   43.9 / 43.0   88 / 93   178 / 187
+//   8 written      10.0 / 7.5   20.9 / 19.2   40.3 / 37.8   76.2 / 78.8
+// Below, a launch is over before the second round of workgroups starts, and what counts is how many
+// start at once (library calls, P = 8, 64 KiB to 2 MiB per rank: 3.5 to 5.0 us streaming, 4.3 to 5.4 us
+// in blocks).
+// (kBlockShapeFromBytes and kBlockShapeBelowBytes, with the other sizes the planner goes by, in alamd_common.h.)
 
 template <int U, int THREADS> struct Tile {
   static constexpr size_t BYTES = (size_t)THREADS * U * 16;

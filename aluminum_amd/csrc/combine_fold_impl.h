@@ -44,7 +44,7 @@ __device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, siz
 
 // Shape of a launch.
 //
-// An ordinary launch streams: one wave per workgroup, one 128-bit vector per lane and stream (1 KiB per
+// A large or a small launch streams: one wave per workgroup, one 128-bit vector per lane and stream (1 KiB per
 // wave and stream), FRONT streams requested before the first use and one more for every stream consumed
 // (so FRONT - 1 loads of a wave are in flight once the fold is under way), and a number of waves per CU
 // that the host sets per launch (see stream_lds_bytes and stream_wgs_per_cu in alamd_tile.h, which also
@@ -52,13 +52,17 @@ __device__ __forceinline__ void fold_elem(const FoldParams &p, int P, int s, siz
 // points lower, and so does every shape that asks for all of a lane's vectors up front (128 threads x
 // 8 vectors x 8 streams, two waves per SIMD: 79 % of the HBM peak where this shape reaches 85 %).
 //
-// A chained launch (see CHAIN below) keeps tiles of 16 KiB per stream, 128 threads x 8 vectors, all of a
-// batch of streams requested up front, two waves per SIMD: its tiles are handed out by a counter and wait
-// for one another through one flag per tile, which small tiles would make sixteen times as many of.
-template <typename T, int OP, bool CHAIN = false> struct Shape {
-  static constexpr int U = CHAIN ? 8 : 1;
-  static constexpr int THREADS = CHAIN ? 128 : 64;
-  static constexpr int WAVES = CHAIN ? 2 : kStreamMaxWaves;  // compiled for; see stream_lds_bytes
+// The block shape keeps tiles of 16 KiB per stream, 128 threads x 8 vectors, all of a batch of streams
+// requested up front, two waves per SIMD.  A launch of middling size takes it (see use_block_shape in
+// alamd_dispatch.h and the measurements above Tile in alamd_tile.h): sixteen times fewer workgroups to hand out, each done after one trip to memory instead
+// of P / FRONT of them, which is what counts while a launch lasts tens of microseconds and much of what
+// it reads sits in the caches.  A chained launch (see KIND below) takes it as well: its tiles are handed
+// out by a counter and wait for one another through one flag per tile, which small tiles would make
+// sixteen times as many of.
+template <typename T, int OP, bool BLOCK = false> struct Shape {
+  static constexpr int U = BLOCK ? 8 : 1;
+  static constexpr int THREADS = BLOCK ? 128 : 64;
+  static constexpr int WAVES = BLOCK ? 2 : kStreamMaxWaves;  // compiled for; see stream_lds_bytes
 };
 // Ordinary launches are built with FRONT = 2 and FRONT = 3; the host takes three from this many ranks on
 // (P = 8: 84 against 84 %, P = 12: 82 and 82, P = 16: 84 against 81, P = 64: 82 against 79).
@@ -66,18 +70,20 @@ constexpr int kFront3FromRanks = 12;
 
 // HEAD = false: no segment has leading elements to handle one by one (see stream_head_count); two
 // kernels, and the host picks, so that the usual case carries no trace of the other.
-// FRONT: see Shape (0 in a chained launch).
-// CHAIN: the output overlaps one of the inputs at a displacement; tiles come from a ticket counter and
-// a tile's stores wait for the loads of the tiles that read what it writes (see ChainParams).  Always
-// with HEAD = false (no leading elements: the vectors start at the output's first element) and one
-// segment with one output.
-template <typename T, int OP, bool ACC_IS_IN, int FRONT, bool HEAD, bool CHAIN = false>
-__global__ void __launch_bounds__((Shape<T, OP, CHAIN>::THREADS))
-__attribute__((amdgpu_waves_per_eu(1, Shape<T, OP, CHAIN>::WAVES)))
+// FRONT: see Shape (0 in the block shape).
+// KIND: FOLD_STREAM, FOLD_BLOCK (built with HEAD = true only: its few workgroups do not feel the lookup),
+// or FOLD_CHAINED: the output overlaps one of the inputs at a displacement; tiles in the block shape come
+// from a ticket counter and a tile's stores wait for the loads of the tiles that read what it writes
+// (see ChainParams).  Always with HEAD = false (no leading elements: the vectors start at the output's
+// first element) and one segment with one output.
+template <typename T, int OP, bool ACC_IS_IN, int FRONT, bool HEAD, int KIND = FOLD_STREAM>
+__global__ void __launch_bounds__((Shape<T, OP, KIND != FOLD_STREAM>::THREADS))
+__attribute__((amdgpu_waves_per_eu(1, Shape<T, OP, KIND != FOLD_STREAM>::WAVES)))
 fold_vec_kernel(const FoldParams p) {
+  constexpr bool CHAIN = KIND == FOLD_CHAINED, BLOCK = KIND != FOLD_STREAM;
   static_assert(!(CHAIN && HEAD), "a chained launch has no head");
-  static_assert(CHAIN ? FRONT == 0 : (FRONT >= 2 && FRONT <= 4), "streams requested up front");
-  constexpr int U = Shape<T, OP, CHAIN>::U, THREADS = Shape<T, OP, CHAIN>::THREADS;
+  static_assert(BLOCK ? FRONT == 0 : (FRONT >= 2 && FRONT <= 4), "streams requested up front");
+  constexpr int U = Shape<T, OP, BLOCK>::U, THREADS = Shape<T, OP, BLOCK>::THREADS;
   constexpr int N = 16 / sizeof(T);
   using TL = Tile<U, THREADS>;
   const TL tl;
@@ -107,7 +113,7 @@ fold_vec_kernel(const FoldParams p) {
     const size_t rem = vec_bytes - tb;
     const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
     u32x4 acc[U];
-    if constexpr (!CHAIN) {
+    if constexpr (!BLOCK) {
       static_assert(U == 1, "the streaming body holds one vector per lane and stream");
       // Stream k lives in x[k % FRONT].  A later load takes its offset from an empty asm statement that
       // reads the result of the step before it, so that it cannot be issued any earlier; the empty
@@ -180,14 +186,15 @@ fold_vec_kernel(const FoldParams p) {
       };
       using Yes = std::true_type;
       using No = std::false_type;
-      // Up to seven streams in one batch; beyond that a first batch that leaves a multiple of six.
+      // Up to eight streams in one batch; beyond that a first batch that leaves a multiple of six.
       // For 8- and 16-bit types, whose arithmetic needs registers as well, the kernel then no longer
       // fits two waves per SIMD, and the second wave is what hides the waits for the neighbouring
       // tile (bf16, a block one element into its buffer: 5.2 TB/s against 4.5): batches of five and four.
       constexpr bool kSmall = sizeof(T) <= 2;
-      constexpr int B0 = kSmall ? 5 : 7, B = kSmall ? 4 : 6;
+      constexpr int B0 = kSmall ? 5 : 8, B = kSmall ? 4 : 6;
       int left = P;
       switch (P <= B0 ? P : (P - 1) % B + 1) {
+      case 8: if constexpr (B0 >= 8) { batch(std::integral_constant<int, 8>{}, Yes{}); left -= 8; } break;
       case 7: if constexpr (B0 >= 7) { batch(std::integral_constant<int, 7>{}, Yes{}); left -= 7; } break;
       case 6: if constexpr (B0 >= 6) { batch(std::integral_constant<int, 6>{}, Yes{}); left -= 6; } break;
       case 5: batch(std::integral_constant<int, 5>{}, Yes{}); left -= 5; break;
@@ -201,7 +208,17 @@ fold_vec_kernel(const FoldParams p) {
 #pragma unroll
     for (int u = 0; u < U; ++u) acc[u] = finish_vec<T, OP>(acc[u], p.div);
     if constexpr (CHAIN) chain_gate(p.chain, bx, tb, (unsigned long long)nrec, (unsigned)TL::BYTES);
-    store_to_outputs<TL, U>(tl, p.out, j0, nj, vout + tb, nrec, acc);
+    if constexpr (BLOCK) {
+      // (one buffer after the other: with store_to_outputs the compiler keeps fewer of the loads above in
+      // flight, 194 instead of 254 registers in the fp32 tree over eight slots)
+      for (int j = j0; j < j0 + nj; ++j) {
+        const auto r = TL::rsrc(p.out[j] + vout + tb, nrec);
+#pragma unroll
+        for (int u = 0; u < U; ++u) tl.store(r, u, acc[u]);
+      }
+    } else {
+      store_to_outputs<TL, U>(tl, p.out, j0, nj, vout + tb, nrec, acc);
+    }
   }
   if constexpr (CHAIN) {
     // the vlen % N elements behind the last whole vector are the last ticket
@@ -241,8 +258,12 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
                                (OP == ALAMD_MIN || OP == ALAMD_MAX);
     using Stream = Shape<T, OP, false>;
     using Chained = Shape<T, OP, true>;
-    static_assert(Tile<Stream::U, Stream::THREADS>::BYTES == kStreamTileBytes, "alamd_planned_launches counts in these tiles");
-    const size_t tile_elems = Tile<Stream::U, Stream::THREADS>::BYTES / sizeof(T);
+    static_assert(Tile<Stream::U, Stream::THREADS>::BYTES == kStreamTileBytes && Tile<Chained::U, Chained::THREADS>::BYTES == kBlockTileBytes,
+                  "alamd_planned_launches counts in these tiles");
+    const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + (p.seg.out_mode == OUT_ALL ? p.seg.nout : 1));
+    const bool block = !chain && use_block_shape(total_bytes);
+    const size_t tile_bytes = block ? Tile<Chained::U, Chained::THREADS>::BYTES : Tile<Stream::U, Stream::THREADS>::BYTES;
+    const size_t tile_elems = tile_bytes / sizeof(T);
     FoldParams q = p;
     q.div = make_divisor(p.P);
     q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0, 0};
@@ -264,8 +285,8 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
       q.seg.seg0 = 0;
       q.seg.mapped = 0;
       void (*ck)(const FoldParams) = nullptr;
-      if constexpr (FP_MINMAX) ck = roles ? fold_vec_kernel<T, OP, true, 0, false, true> : fold_vec_kernel<T, OP, false, 0, false, true>;
-      else ck = fold_vec_kernel<T, OP, false, 0, false, true>;
+      if constexpr (FP_MINMAX) ck = roles ? fold_vec_kernel<T, OP, true, 0, false, FOLD_CHAINED> : fold_vec_kernel<T, OP, false, 0, false, FOLD_CHAINED>;
+      else ck = fold_vec_kernel<T, OP, false, 0, false, FOLD_CHAINED>;
       hipLaunchKernelGGL(ck, dim3((unsigned)tickets, 1, 1), dim3(Chained::THREADS, 1, 1), 0, stream, q);
       ALAMD_HIP(hipGetLastError());
       return ALAMD_OK;
@@ -300,14 +321,20 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
       if constexpr (FP_MINMAX) kern = roles ? pick(Yes{}, F2{}) : pick(No{}, F2{});
       else kern = pick(No{}, F2{});
     }
-    const size_t per_launch = launch_tiles(p.P, Tile<Stream::U, Stream::THREADS>::BYTES, tunables().launch_bytes);
+    const size_t per_launch = launch_tiles(p.P, tile_bytes, tunables().launch_bytes);
     const size_t wgs = tunables().stream_wgs_per_cu;
-    const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + 1);
-    const unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(false, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes));
+    unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(false, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes));
+    unsigned threads = Stream::THREADS;
+    if (block) {
+      if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 0, true, FOLD_BLOCK> : fold_vec_kernel<T, OP, false, 0, true, FOLD_BLOCK>;
+      else kern = fold_vec_kernel<T, OP, false, 0, true, FOLD_BLOCK>;
+      lds = 0;
+      threads = Chained::THREADS;
+    }
     plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
       q.seg.tile0 = t0;
       q.seg.seg0 = s0;
-      hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(Stream::THREADS, 1, 1), lds, stream, q);
+      hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(threads, 1, 1), lds, stream, q);
     });
     ALAMD_HIP(hipGetLastError());
     return ALAMD_OK;

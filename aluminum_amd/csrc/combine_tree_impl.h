@@ -80,20 +80,21 @@ __device__ __forceinline__ void tree_elems(const TreeParams &p, size_t len, size
 // two), which needs room for up to twice as many loads in flight.
 enum { TREE_FULL = 0, TREE_PARTIAL = 1, TREE_PREFOLD = 2 };
 
-// An ordinary launch streams like the fold does (see Shape there): one wave per workgroup, one vector per
+// A large or a small launch streams like the fold does (see Shape there): one wave per workgroup, one vector per
 // lane and slot, the two slots of a pair requested together and the next pair as soon as a pair has been
 // combined, partial results combined as soon as both halves of a subtree are there; the waves per CU
 // are the host's choice per launch (stream_wgs_per_cu in alamd_tile.h).  A second pair requested ahead
 // changes nothing; every slot requested up front (128 threads x 8 vectors) runs 5 points lower.
-// A chained launch keeps tiles of 4 to 16 KiB per slot with every load issued up front (see the fold).
-template <typename T, int OP, int SLOTS, int MODE, bool CHAIN = false> struct TreeShape {
+// The block shape (launches of middling size and chained launches: see the fold) keeps tiles of 4 to
+// 16 KiB per slot with every load issued up front.
+template <typename T, int OP, int SLOTS, int MODE, bool BLOCK = false> struct TreeShape {
   static constexpr bool heavy = sizeof(T) <= 2;
-  static constexpr int budget = heavy ? 32 : 64;  // chained: 128-bit loads in flight per lane
+  static constexpr int budget = heavy ? 32 : 64;  // block shape: 128-bit loads in flight per lane
   static constexpr int streams = MODE == TREE_PREFOLD ? 2 * SLOTS : SLOTS;
-  static constexpr int chained_u = budget / streams >= 8 ? (heavy ? 4 : 8) : (budget / streams >= 1 ? budget / streams : 1);
-  static constexpr int U = CHAIN ? chained_u : 1;
-  static constexpr int THREADS = CHAIN ? (chained_u == 8 ? 128 : 256) : 64;
-  static constexpr int WAVES = CHAIN ? 2 : kStreamMaxWaves;  // compiled for; see stream_lds_bytes
+  static constexpr int block_u = budget / streams >= 8 ? (heavy ? 4 : 8) : (budget / streams >= 1 ? budget / streams : 1);
+  static constexpr int U = BLOCK ? block_u : 1;
+  static constexpr int THREADS = BLOCK ? (block_u == 8 ? 128 : 256) : 64;
+  static constexpr int WAVES = BLOCK ? 2 : kStreamMaxWaves;  // compiled for; see stream_lds_bytes
 };
 
 __host__ __device__ inline void tree_out_select(const TreeParams &p, unsigned seg, size_t off_bytes,
@@ -108,13 +109,15 @@ __host__ __device__ inline void tree_out_select(const TreeParams &p, unsigned se
 // top level of a tree over 2 * SLOTS slots combines slot 0 with slot SLOTS, each the root of a tree
 // over SLOTS slots, so the two halves are loaded and reduced one after the other with the registers
 // of one.
-// CHAIN: the output overlaps one of the inputs at a displacement (see ChainParams and the fold kernel).
-template <typename T, int OP, int SLOTS, int MODE, bool HEAD, int HALVES, bool CHAIN = false>
-__global__ void __launch_bounds__((TreeShape<T, OP, SLOTS, MODE, CHAIN>::THREADS))
-__attribute__((amdgpu_waves_per_eu(1, TreeShape<T, OP, SLOTS, MODE, CHAIN>::WAVES)))
+// KIND: FOLD_STREAM, FOLD_BLOCK (built with HEAD = true only) or FOLD_CHAINED: the output overlaps one of
+// the inputs at a displacement (see ChainParams and the fold kernel).
+template <typename T, int OP, int SLOTS, int MODE, bool HEAD, int HALVES, int KIND = FOLD_STREAM>
+__global__ void __launch_bounds__((TreeShape<T, OP, SLOTS, MODE, KIND != FOLD_STREAM>::THREADS))
+__attribute__((amdgpu_waves_per_eu(1, TreeShape<T, OP, SLOTS, MODE, KIND != FOLD_STREAM>::WAVES)))
 tree_vec_kernel(const TreeParams p) {
+  constexpr bool CHAIN = KIND == FOLD_CHAINED, BLOCK = KIND != FOLD_STREAM;
   static_assert(!(CHAIN && HEAD), "a chained launch has no head");
-  constexpr int U = TreeShape<T, OP, SLOTS, MODE, CHAIN>::U, THREADS = TreeShape<T, OP, SLOTS, MODE, CHAIN>::THREADS;
+  constexpr int U = TreeShape<T, OP, SLOTS, MODE, BLOCK>::U, THREADS = TreeShape<T, OP, SLOTS, MODE, BLOCK>::THREADS;
   constexpr int N = 16 / sizeof(T);
   static_assert(HALVES == 1 || MODE != TREE_PREFOLD, "a pre-fold never meets more than 32 slots");
   using TL = Tile<U, THREADS>;
@@ -166,7 +169,7 @@ tree_vec_kernel(const TreeParams p) {
     const size_t rem = vec_bytes - tb;
     const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
     u32x4 res[U];
-    if constexpr (!CHAIN) {
+    if constexpr (!BLOCK) {
       static_assert(U == 1, "the streaming body holds one vector per lane and slot");
       // a later load takes its offset from an empty asm statement that reads the result of the pair
       // before it, so that it cannot be issued any earlier
@@ -296,7 +299,17 @@ tree_vec_kernel(const TreeParams p) {
 #pragma unroll
     for (int u = 0; u < U; ++u) res[u] = finish_vec<T, OP>(res[u], p.div);
     if constexpr (CHAIN) chain_gate(p.chain, bx, tb, (unsigned long long)nrec, (unsigned)TL::BYTES);
-    store_to_outputs<TL, U>(tl, p.out, j0, nj, vout + tb, nrec, res);
+    if constexpr (BLOCK) {
+      // (one buffer after the other: with store_to_outputs the compiler keeps fewer of the loads above in
+      // flight, 194 instead of 254 registers in the fp32 tree over eight slots)
+      for (int j = j0; j < j0 + nj; ++j) {
+        const auto r = TL::rsrc(p.out[j] + vout + tb, nrec);
+#pragma unroll
+        for (int u = 0; u < U; ++u) tl.store(r, u, res[u]);
+      }
+    } else {
+      store_to_outputs<TL, U>(tl, p.out, j0, nj, vout + tb, nrec, res);
+    }
   }
   if constexpr (CHAIN) {
     // the vlen % N elements behind the last whole vector are the last ticket
@@ -332,8 +345,11 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   using S = TreeShape<T, OP, SLOTS, MODE, false>;
   using C = TreeShape<T, OP, SLOTS, MODE, true>;
   static_assert(Tile<S::U, S::THREADS>::BYTES == kStreamTileBytes, "the tile of a streaming launch");
-  const size_t tile_elems = Tile<S::U, S::THREADS>::BYTES / sizeof(T);
-  const size_t per_launch = launch_tiles(p.P, Tile<S::U, S::THREADS>::BYTES, tunables().launch_bytes);
+  const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + (p.seg.out_mode == OUT_ALL ? p.seg.nout : 1));
+  const bool block = !chain.scratch && use_block_shape(total_bytes);
+  const size_t tile_bytes = block ? Tile<C::U, C::THREADS>::BYTES : Tile<S::U, S::THREADS>::BYTES;
+  const size_t tile_elems = tile_bytes / sizeof(T);
+  const size_t per_launch = launch_tiles(p.P, tile_bytes, tunables().launch_bytes);
   TreeParams q = p;
   q.div = make_divisor(p.P);
   q.chain = ChainParams{nullptr, nullptr, nullptr, 0, 0, 0};
@@ -371,7 +387,7 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
     q.seg.mapped = 0;
     // only the most general variants are built for chained launches
     if constexpr (MODE == TREE_PREFOLD || (HALVES == 2 && MODE == TREE_PARTIAL)) {
-      hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE, false, HALVES, true>), dim3((unsigned)tickets, 1, 1),
+      hipLaunchKernelGGL((tree_vec_kernel<T, OP, SLOTS, MODE, false, HALVES, FOLD_CHAINED>), dim3((unsigned)tickets, 1, 1),
                          dim3(C::THREADS, 1, 1), 0, stream, q);
       ALAMD_HIP(hipGetLastError());
       return ALAMD_OK;
@@ -390,14 +406,19 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   }
   q.seg.simple = nseg == 1 && !q.seg.ragged && q.seg.seg_rem == 0 && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1;
   const size_t wgs = tunables().stream_wgs_per_cu;
-  const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + 1);
-  const unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(true, SLOTS * HALVES, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes));
+  unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(true, SLOTS * HALVES, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes));
+  unsigned threads = S::THREADS;
   void (*kern)(const TreeParams) =
       q.seg.any_head ? tree_vec_kernel<T, OP, SLOTS, MODE, true, HALVES> : tree_vec_kernel<T, OP, SLOTS, MODE, false, HALVES>;
+  if (block) {
+    kern = tree_vec_kernel<T, OP, SLOTS, MODE, true, HALVES, FOLD_BLOCK>;
+    lds = 0;
+    threads = C::THREADS;
+  }
   plan_launches(q.seg, nseg, max_len, tile_elems, per_launch, [&](size_t t0, size_t nt, unsigned s0, unsigned ns) {
     q.seg.tile0 = t0;
     q.seg.seg0 = s0;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(S::THREADS, 1, 1), lds, stream, q);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nt, ns, 1), dim3(threads, 1, 1), lds, stream, q);
   });
   ALAMD_HIP(hipGetLastError());
   return ALAMD_OK;

@@ -47,6 +47,8 @@ const TunableName kTunableNames[] = {
     {"spread_hbm_launch_chunks", &Tunables::spread_hbm_launch_chunks, 1},
     {"spread_cache_chunk_tiles", &Tunables::spread_cache_chunk_tiles, 1},
     {"spread_cache_launch_chunks", &Tunables::spread_cache_launch_chunks, 1},
+    {"block_shape_from_bytes", &Tunables::block_shape_from_bytes, 1},
+    {"block_shape_below_bytes", &Tunables::block_shape_below_bytes, 1},
     {"fold_front3_ranks", &Tunables::fold_front3_ranks, 0},
     {"stream_wgs_per_cu", &Tunables::stream_wgs_per_cu, 0},
     {"halo_load_policy", &Tunables::halo_load_policy, 0},

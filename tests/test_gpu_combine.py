@@ -31,8 +31,20 @@ def run_combine(al, ins, dtype, op, order, start=0, nout=1):
     return [to_host(o, ins[0].dtype) for o in outs]
 
 
+@pytest.fixture(params=["shape by size", "block shape"])
+def shape(request, al):
+    """Runs a test twice: with the launch shapes the library picks by size (the streaming shape at the
+    sizes of these tests) and with every fold / tree launch in the block shape."""
+    if request.param == "block shape":
+        al.tune("block_shape_from_bytes", 1)
+        al.tune("block_shape_below_bytes", 1 << 60)
+    yield request.param
+    al.tune("block_shape_from_bytes", 0)
+    al.tune("block_shape_below_bytes", 0)
+
+
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
-def test_combine_all_ops_orders(al, dtype):
+def test_combine_all_ops_orders(al, dtype, shape):
     for op in ops_of(dtype):
         for P in (1, 2, 3, 5, 8):
             orders = ORDERS if dtype in FLOAT_DTYPES else ("rank_asc", "tree_halv")
@@ -47,7 +59,7 @@ def test_combine_all_ops_orders(al, dtype):
 
 @pytest.mark.parametrize("dtype", ("f32", "bf16", "i32"))
 @pytest.mark.parametrize("P", (4, 6, 7, 8, 13, 16, 31, 32, 33, 40, 48, 63, 64))
-def test_combine_many_ranks(al, dtype, P):
+def test_combine_many_ranks(al, dtype, P, shape):
     n = 5000
     for order in ORDERS:
         ins = make_inputs(P, n, dtype, "sum")
@@ -101,7 +113,7 @@ def _offset_view(a, off):
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
-def test_vector_path_at_any_element_alignment(al, dtype):
+def test_vector_path_at_any_element_alignment(al, dtype, shape):
     """Buffers that are only element-aligned (each input and the output at its own offset) go through the
     128-bit kernels: several tiles plus a ragged tail, fold and tree orders, two outputs."""
     import torch
@@ -119,7 +131,7 @@ def test_vector_path_at_any_element_alignment(al, dtype):
 
 
 @pytest.mark.parametrize("dtype", ("u8", "i16", "bf16", "f32", "f64"))
-def test_head_up_to_the_outputs_64_byte_boundary(al, dtype):
+def test_head_up_to_the_outputs_64_byte_boundary(al, dtype, shape):
     """The kernels walk the leading elements one by one until the output reaches a 64-byte boundary:
     outputs 1 element to 60 bytes past a boundary, inputs at the same or at other offsets, counts
     shorter than the head, equal to it and far beyond; fold and tree orders, combine and allgather."""
@@ -149,7 +161,7 @@ def test_head_up_to_the_outputs_64_byte_boundary(al, dtype):
 
 
 @pytest.mark.parametrize("dtype", ("u8", "bf16", "f32", "f64"))
-def test_head_up_to_the_first_inputs_1kib_boundary(al, dtype):
+def test_head_up_to_the_first_inputs_1kib_boundary(al, dtype, shape):
     """From 64 KiB per segment on, the streaming kernels walk the leading elements one by one until the
     first input reaches a 1 KiB boundary (up to 1023 bytes' worth, spread over the segment's first
     workgroups): lengths just below, at and above that size, inputs and outputs at the same and at
@@ -218,7 +230,7 @@ def test_reduce_scatter_odd_block_sizes(al, dtype, inplace):
 
 
 @pytest.mark.parametrize("dtype", ("f32", "f64", "bf16", "f16"))
-def test_combine_special_values(al, dtype):
+def test_combine_special_values(al, dtype, shape):
     # NaN, infinities, signed zeros, denormals and ties on every side
     f32 = np.array([np.nan, -1.0, np.nan, 0.0, -0.0, np.inf, -np.inf, 1e-45, -1e-45, 1.0,
                     3.4028235e38, 1.1754944e-38, 0.0, -0.0, np.inf, 5.877472e-39, 65504.0, 1e-8],
@@ -248,7 +260,7 @@ def test_combine_special_values(al, dtype):
 
 
 @pytest.mark.parametrize("P", (3, 5, 8, 12, 16, 33, 48, 64))
-def test_float_min_max_operand_roles_over_many_tiles(al, P):
+def test_float_min_max_operand_roles_over_many_tiles(al, P, shape):
     """Zeros of both signs and NaNs in every operand position (the inputs of the golden vectors' special
     cases), over messages of many tiles whose blocks end inside tiles and whose length is no multiple of
     the power of two of ranks: which operand of every pair lets a tie through depends on the order, the
@@ -281,7 +293,7 @@ def test_float_min_max_operand_roles_over_many_tiles(al, P):
 
 @pytest.mark.parametrize("dtype", ("f32", "bf16", "u8", "i64"))
 @pytest.mark.parametrize("order", ("rank_asc", "tree_halv", "pairwise_desc", "ring"))
-def test_reduce_scatter(al, dtype, order):
+def test_reduce_scatter(al, dtype, order, shape):
     import torch
     for P in (1, 2, 5, 8):
         for count in (1, 24, 1000, 4096):
@@ -328,7 +340,7 @@ def test_allgather(al, dtype):
 
 @pytest.mark.parametrize("dtype", ("f32", "bf16", "i16", "f64"))
 @pytest.mark.parametrize("order", ("rank_asc", "tree_halv", "pairwise_desc"))
-def test_reduce_scatterv(al, dtype, order):
+def test_reduce_scatterv(al, dtype, order, shape):
     import torch
     for P, counts in ((1, [9]), (3, [5, 0, 12]), (4, [1, 100, 3, 64]), (8, [4096, 8, 0, 1000, 8192, 1, 33, 4100])):
         total = sum(counts)
@@ -419,7 +431,7 @@ def test_allgatherv(al, dtype):
 
 
 @pytest.mark.parametrize("dtype", ALL_DTYPES)
-def test_avg_division_every_rank_count(al, dtype):
+def test_avg_division_every_rank_count(al, dtype, shape):
     """avg ends with one division by P: every 8- and 16-bit pattern (and edge values plus random ones of
     the wider types) as the sum, for every P up to 64, against the oracle's C division."""
     import torch
@@ -682,6 +694,12 @@ SETTINGS = [
     {"stream_wgs_per_cu": 4, "fold_front3_ranks": 2},
     # ... as many as fit and two up front for every rank count
     {"stream_wgs_per_cu": 32, "fold_front3_ranks": 1000, "launch_bytes": 1 << 22},
+    # every fold / tree launch in the block shape, ...
+    {"block_shape_from_bytes": 1, "block_shape_below_bytes": 1 << 60},
+    # ... in many launches, ...
+    {"block_shape_from_bytes": 1, "block_shape_below_bytes": 1 << 60, "launch_bytes": 1 << 20},
+    # ... and none
+    {"block_shape_below_bytes": 1},
 ]
 
 
@@ -689,7 +707,7 @@ SETTINGS = [
 def test_results_do_not_depend_on_the_launch_planners_sizes(al, k):
     """The sizes the launch planners cut their work by (bytes per launch, the thresholds and pieces of
     the two-step calls, the spread's chunks, the waves per CU and streams requested up front of the
-    streaming kernels) only decide how the same work is spread over launches and waves:
+    streaming kernels, the sizes between which a launch takes the block shape) only decide how the same work is spread over launches and waves:
     extreme settings give the bits of the defaults, i.e. the oracle's."""
     import torch
     P, n = 5, 1_300_007
