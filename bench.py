@@ -54,7 +54,7 @@ P = 8
 # WRITE_SIZE, each scaled by the same counter's reading for the 1 GiB copy kernel.
 TRAFFIC_PROFILE = {"c2_f32_sum": "profiles/fold_vec_kernel_f32_sum_P8_c2.md"}
 KERNEL_NAME = {"c2_f32_sum": "alamd::fold_vec_kernel<float, 0 /*sum*/, false /*operand roles*/, 2 /*streams requested "
-                             "up front*/, false /*no leading elements*/, false /*not chained*/>"}
+                             "up front*/, false /*no leading elements*/, 0 /*streaming launch*/>"}
 
 # Every configuration of the headline benchmark beside the primary workload: C2 in the tree order, prod and bf16, the same over
 # buffers no earlier call has touched, C4 (integer / bitwise / logical), C3 (ring, both modes), C5 (halo

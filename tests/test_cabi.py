@@ -114,6 +114,30 @@ def test_launch_planner_sizes_are_checked():
     assert al.tuned("two_step_piece_bytes") == 128 << 20
 
 
+def test_planned_launches_follow_the_launch_cut_and_the_shape():
+    """alamd_planned_launches runs the fold's planner without launching: one launch up to 4 GiB of traffic,
+    then a power of two of tiles per launch; a call of middling size counts in the 16 KiB tiles of the
+    block shape, the others in the 1 KiB tiles of the streaming shape."""
+    import aluminum_amd as al
+    assert al.tuned("launch_bytes") == 4 << 30
+    assert al.tuned("block_shape_from_bytes") == 32 << 20 and al.tuned("block_shape_below_bytes") == 384 << 20
+    assert al.planned_launches(8, 1 << 26, "f32") == 1      # the headline workload: 9 x 256 MiB
+    assert al.planned_launches(8, 1 << 28, "f32") == 4      # 9 GiB: 256 MiB per stream and launch
+    assert al.planned_launches(64, 1 << 28, "f32") == 32    # 65 GiB: 32 MiB per stream and launch
+    assert al.planned_launches(8, 1 << 22, "f32") == 1      # 144 MiB in all: block shape
+    assert al.planned_launches(8, 0, "f32") == 0
+    try:
+        al.tune("launch_bytes", 9 << 20)  # 1 MiB per stream and launch at P = 8, whatever the tile
+        assert al.planned_launches(8, 1 << 26, "f32") == 256
+        assert al.planned_launches(8, 1 << 22, "f32") == 16
+        al.tune("launch_bytes", 1)        # never fewer than eight tiles per launch: 8 KiB streaming, 128 KiB in blocks
+        assert al.planned_launches(8, 1 << 20, "f32") == 32    # 36 MiB in all: block shape
+        assert al.planned_launches(8, 1 << 18, "f32") == 128   # 9 MiB in all: streaming
+    finally:
+        al.tune("launch_bytes", 0)
+    assert al.tuned("launch_bytes") == 4 << 30
+
+
 def test_graft_entry_has_build_and_smoke():
     import importlib
     g = importlib.import_module("__graft_entry__")
