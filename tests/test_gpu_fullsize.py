@@ -47,6 +47,55 @@ def test_c2_bf16_full_size(al):
     assert_bits_equal(out.cpu().numpy().view(np.uint16), want, "bf16", "C2 bf16")
 
 
+@pytest.mark.parametrize("dtype,dist,seed", [("f32", "uniform_pm1", 1000), ("bf16", "normal", 2000), ("f64", "uniform_pm1", 1000),
+                                             ("i32", "fullrange", 3000)])
+def test_middling_sizes_in_the_block_shape(al, dtype, dist, seed):
+    """Calls that move between 32 and 384 MiB in all run in tiles of 16 KiB with every load issued up front,
+    by the library's own choice: 4 Mi + 37 elements per rank (buffers one element into their allocations,
+    so with leading elements), one output and eight, fold and tree orders, float min under the order whose
+    operand roles change from block to block; and the sizes either side of the two thresholds."""
+    import torch
+    assert al.tuned("block_shape_from_bytes") == 32 << 20 and al.tuned("block_shape_below_bytes") == 384 << 20
+    es = al.dtype_size(dtype)
+    carrier = al.torch_dtype(dtype)
+    np_dt = oracle.NP_CARRIER[dtype]
+    n = (1 << 22) + 37
+    raw = [torch.empty(n + 1, dtype=carrier, device="cuda") for _ in range(P)]
+    ins = [t[1:] for t in raw]
+    for r in range(P):
+        al.fill(ins[r], dist, seed + r, dtype=dtype)
+    host = [t.cpu().numpy().view(np_dt) for t in ins]
+    is_float = dtype in ("f32", "bf16", "f64")
+    cases = [("sum", "rank_asc", 1), ("sum", "rank_asc", 8)]
+    if is_float:
+        cases += [("sum", "tree_rsg", 1), ("min", "tree_rsg", 2), ("sum", "tree_dbl", 8)]
+    else:
+        cases += [("max", "pairwise_desc", 2)]
+    for op, order, nout in cases:
+        want = oracle.combine(host, dtype, op, order)
+        outs = [torch.empty(n + 1, dtype=carrier, device="cuda")[1:] for _ in range(nout)]
+        al.combine(outs, ins, op, order=order, dtype=dtype)
+        torch.cuda.synchronize()
+        for o in outs:
+            assert_bits_equal(o.cpu().numpy().view(np_dt), want, dtype, "%s %s %s to %d buffers" % (dtype, op, order, nout))
+    # one tile of 16 KiB either side of where the shape changes (totals of 32 MiB and 384 MiB)
+    for total in (32 << 20, 384 << 20):
+        for delta in (-4096 // es, 0, 4096 // es):
+            m = total // (P + 1) // es + delta
+            if m > n:
+                sub = [torch.empty(m, dtype=carrier, device="cuda") for _ in range(P)]
+                for r in range(P):
+                    al.fill(sub[r], dist, seed + r, dtype=dtype)
+            else:
+                sub = [t[:m] for t in ins]
+            out = torch.empty(m, dtype=carrier, device="cuda")
+            al.combine([out], sub, "sum", order="rank_asc", dtype=dtype)
+            torch.cuda.synchronize()
+            want = oracle.combine([t.cpu().numpy().view(np_dt) for t in sub], dtype, "sum", "rank_asc")
+            assert_bits_equal(out.cpu().numpy().view(np_dt), want, dtype, "%s, %d elements per rank" % (dtype, m))
+            del out, sub
+
+
 @pytest.mark.parametrize("mode", ("stepwise", "fused"))
 def test_c3_ring_full_size(al, mode):
     """C3: P=8 bf16 buffers of 2^27 elements, seed 2000+rank, 4 MiB chunks."""
