@@ -94,6 +94,7 @@ struct SegParams {
   int owner_shift;  // OUT_OWNER: output index is (segment + owner_shift) mod P
   int nout;         // OUT_ALL: number of outputs written
   int simple;       // 1: one segment from element 0, one output (the kernels then skip the lookups)
+  int xcd_run_log2; // > 0: runs of 2^k consecutive tiles go to one XCD (kernels with HEAD only; see tiles_by_output)
   int ragged;       // 1: segments are given by the two tables below
   unsigned long long seg_off[ALAMD_MAX_RANKS];
   unsigned long long seg_len[ALAMD_MAX_RANKS];
@@ -124,6 +125,15 @@ __device__ __forceinline__ unsigned arg_u8(const unsigned char *table, unsigned 
 }
 __device__ __forceinline__ unsigned arg_u16(const unsigned short *table, unsigned i) {
   return (reinterpret_cast<const unsigned *>(table)[i >> 1] >> ((i & 1u) * 16u)) & 0xffffu;
+}
+// Workgroup i of a launch of n -> tile, so that runs of 2^rl consecutive tiles fall to one XCD (workgroups
+// are dealt to the eight XCDs round-robin); the workgroups behind the last whole group of 8 * 2^rl keep
+// their own index.
+__host__ __device__ __forceinline__ unsigned xcd_run_tile(unsigned i, unsigned n, unsigned rl) {
+  const unsigned span = 8u << rl, full = n & ~(span - 1u);
+  if (i >= full) return i;
+  const unsigned w = i & (span - 1u);
+  return (i & ~(span - 1u)) + ((w & 7u) << rl) + (w >> 3);
 }
 __device__ __forceinline__ unsigned seg_of(const SegParams &s, unsigned pos) {
   return s.mapped ? arg_u8(s.order, pos) : pos;

@@ -76,10 +76,36 @@ __host__ __device__ inline size_t head_count(size_t elem_size, const char *out, 
 // spread over the segment's first workgroups, 64 elements each; shorter segments keep the rule above,
 // since their few workgroups would spend longer on the elements than on the tiles.
 constexpr size_t kBigHeadFromBytes = (size_t)64 << 10;
-__host__ __device__ inline size_t stream_head_count(size_t elem_size, const char *out, const char *first, size_t len) {
+// Where some input sits at another distance from a 64-byte boundary than the output, one side has to
+// split lines.  Then the output's tiles start on its 1 KiB boundary instead (whole lines written), and
+// the launch hands runs of four consecutive tiles to one XCD (kXcdRunLog2, xcd_run_tile in
+// alamd_dispatch.h), whose L2 then fetches most of the lines that neighbouring tiles share only once
+// (f32, output 20 bytes off the inputs: 77 % with the inputs on their boundary, 74 % with the output on
+// its boundary and the usual order of tiles, 80.5 % with runs of four; runs of two: 78, of eight: 79; on
+// buffers that split no lines runs cost up to a point, so only these launches take them).
+constexpr int kXcdRunLog2 = 2;
+__host__ __device__ inline size_t stream_head_count(size_t elem_size, const char *out, const char *first, size_t len,
+                                                    bool to_output = false) {
   if (len * elem_size < kBigHeadFromBytes) return head_count(elem_size, out, first, len);
-  const uintptr_t f = reinterpret_cast<uintptr_t>(first);
+  const uintptr_t f = reinterpret_cast<uintptr_t>(to_output ? out : first);
   return ((kStreamTileBytes - (size_t)(f & (kStreamTileBytes - 1))) & (kStreamTileBytes - 1)) / elem_size;
+}
+// Whether a segment's tiles go by the output (see above): some input at another distance from a 64-byte
+// boundary than the output, all of them on the output's dword grid (else the loads would split dwords,
+// which costs more), the segment long enough for tiles on 1 KiB boundaries.
+template <typename NextInput>
+inline bool tiles_by_output(size_t elem_size, const char *out, size_t len, int nin, NextInput input) {
+  if (len * elem_size < kBigHeadFromBytes) return false;
+  const uintptr_t o = reinterpret_cast<uintptr_t>(out);
+  bool differs = false;
+  for (int k = 0; k < nin; ++k) {
+    const char *in = input(k);
+    if (!in) continue;
+    const uintptr_t d = reinterpret_cast<uintptr_t>(in) ^ o;
+    if (d & 3u) return false;
+    differs = differs || ((reinterpret_cast<uintptr_t>(in) - o) & 63u) != 0;
+  }
+  return differs;
 }
 template <typename T> __device__ __forceinline__ size_t head_elems(const char *out, const char *first, size_t len) {
   return head_count(sizeof(T), out, first, len);

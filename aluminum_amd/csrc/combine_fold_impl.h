@@ -107,6 +107,7 @@ fold_vec_kernel(const FoldParams p) {
   const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
   const size_t vec_bytes = (vlen / N) * 16;
   unsigned bx = blockIdx.x;
+  if constexpr (HEAD && !BLOCK) { if (p.seg.xcd_run_log2) bx = xcd_run_tile(bx, gridDim.x, (unsigned)p.seg.xcd_run_log2); }
   if constexpr (CHAIN) bx = chain_take_tile(p.chain);
   const size_t tb = ((size_t)p.seg.tile0 + bx) * TL::BYTES;
   if (tb < vec_bytes) {
@@ -297,9 +298,11 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
       seg_range(p.seg, sg, off, len);
       out_select(p.seg, p.P, sg, off * sizeof(T), j0, nj, out_bytes);
       const int first = (p.start0 + (int)sg * p.start_stride) % p.P;
-      q.seg.seg_head[sg] = (unsigned short)stream_head_count(sizeof(T), p.out[j0] + out_bytes,
-                                                     p.in[first] + (p.seg.in_blocked ? off * sizeof(T) : 0), len);
-      if (q.seg.seg_head[sg]) q.seg.any_head = 1;
+      const size_t in_bytes = p.seg.in_blocked ? off * sizeof(T) : 0;
+      const bool by_output = !block && tiles_by_output(sizeof(T), p.out[j0] + out_bytes, len, p.P, [&](int k) { return p.in[k] + in_bytes; });
+      q.seg.seg_head[sg] = (unsigned short)stream_head_count(sizeof(T), p.out[j0] + out_bytes, p.in[first] + in_bytes, len, by_output);
+      if (by_output) q.seg.xcd_run_log2 = kXcdRunLog2;
+      if (q.seg.seg_head[sg] || by_output) q.seg.any_head = 1;
     }
     q.seg.simple = nseg == 1 && !q.seg.ragged && q.seg.seg_rem == 0 && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1 &&
                    p.start0 >= 0 && p.start0 < p.P;

@@ -139,6 +139,7 @@ tree_vec_kernel(const TreeParams p) {
   const size_t vin = in_bytes + head * sizeof(T), vout = out_bytes + head * sizeof(T);
   const size_t vec_bytes = (vlen / N) * 16;
   unsigned bx = blockIdx.x;
+  if constexpr (HEAD && !BLOCK) { if (p.seg.xcd_run_log2) bx = xcd_run_tile(bx, gridDim.x, (unsigned)p.seg.xcd_run_log2); }
   if constexpr (CHAIN) bx = chain_take_tile(p.chain);
   const size_t tb = ((size_t)p.seg.tile0 + bx) * TL::BYTES;
   // float min / max: the slot mask of this tile (uniform), or, where a tile straddles two blocks of a
@@ -401,8 +402,13 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
     seg_range(p.seg, sg, off, len);
     const size_t in_bytes = p.seg.in_blocked ? off * sizeof(T) : 0;
     tree_out_select(p, sg, off * sizeof(T), in_bytes, j0, nj, out_bytes);
-    q.seg.seg_head[sg] = (unsigned short)stream_head_count(sizeof(T), p.out[j0] + out_bytes, p.a[0] + in_bytes, len);
-    if (q.seg.seg_head[sg]) q.seg.any_head = 1;
+    const bool by_output = !block && tiles_by_output(sizeof(T), p.out[j0] + out_bytes, len, 2 * SLOTS * HALVES, [&](int k) {
+      const char *in = k < SLOTS * HALVES ? p.a[k] : p.b[k - SLOTS * HALVES];
+      return in ? in + in_bytes : nullptr;
+    });
+    q.seg.seg_head[sg] = (unsigned short)stream_head_count(sizeof(T), p.out[j0] + out_bytes, p.a[0] + in_bytes, len, by_output);
+    if (by_output) q.seg.xcd_run_log2 = kXcdRunLog2;
+    if (q.seg.seg_head[sg] || by_output) q.seg.any_head = 1;
   }
   q.seg.simple = nseg == 1 && !q.seg.ragged && q.seg.seg_rem == 0 && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1;
   const size_t wgs = tunables().stream_wgs_per_cu;

@@ -159,6 +159,39 @@ int main(int argc, char **argv) {
       }
     }
   }
+  // Runs of consecutive tiles per XCD: a permutation of the launch's tiles whatever its length; in every whole
+  // group the workgroups that go to one XCD (index mod 8) take 2^rl consecutive tiles, in order.
+  for (unsigned rl = 1; rl <= 5; ++rl) {
+    for (unsigned n : {1u, 7u, 8u, 31u, 32u, 33u, 255u, 256u, 1000u, 4096u, 5000u}) {
+      std::vector<int> seen(n, 0);
+      bool in_range = true, runs = true;
+      for (unsigned i = 0; i < n; ++i) {
+        const unsigned t = xcd_run_tile(i, n, rl);
+        if (t >= n) { in_range = false; break; }
+        ++seen[t];
+        const unsigned span = 8u << rl;
+        if (i + 8 < n && (i + 8) / span == i / span && i / span < n / span) runs = runs && xcd_run_tile(i + 8, n, rl) == t + 1;
+      }
+      bool once = in_range;
+      for (unsigned t = 0; once && t < n; ++t) once = seen[t] == 1;
+      EXPECT(once && runs, "tiles of a launch of %u in runs of %u per XCD: every tile once %d, consecutive %d", n, 1u << rl, (int)once, (int)runs);
+    }
+  }
+  // Tiles go by the output only where some input sits at another distance from a 64-byte boundary, every
+  // input is on the output's dword grid, and the segment is long.
+  {
+    const char *base = reinterpret_cast<const char *>((uintptr_t)1 << 30);
+    auto by_out = [&](size_t es, size_t out_off, std::vector<size_t> in_off, size_t len) {
+      return tiles_by_output(es, base + out_off, len, (int)in_off.size(), [&](int k) { return base + (1 << 20) * (k + 1) + in_off[(size_t)k]; });
+    };
+    EXPECT(!by_out(4, 0, {0, 0, 0}, 1 << 20), "aligned buffers");
+    EXPECT(!by_out(4, 4, {4, 4, 68}, 1 << 20), "a common distance (mod 64)");
+    EXPECT(by_out(4, 20, {0, 0, 0}, 1 << 20), "output 20 bytes off");
+    EXPECT(by_out(4, 0, {0, 12, 0}, 1 << 20), "one input 12 bytes off");
+    EXPECT(!by_out(4, 20, {0, 0, 0}, 1000), "short segment");
+    EXPECT(!by_out(2, 2, {0, 0}, 1 << 20), "inputs off the output's dword grid");
+    EXPECT(by_out(2, 4, {0, 0}, 1 << 20), "16-bit elements, output two elements off");
+  }
   // workgroups that find nothing to do: a planner that put every segment side by side in one grid
   // would idle far more than it works on the "one long among short" shapes
   EXPECT(idle_total < busy_total, "idle workgroups %zu against %zu busy ones", idle_total, busy_total);
