@@ -49,8 +49,10 @@ inline size_t launch_tiles(int nin, size_t tile_bytes, size_t launch_bytes = kLa
   return t < 8 ? 8 : t;
 }
 
-// Bytes per stream of a tile of the streaming fold and tree kernels (one wave, one vector per lane).
+// Bytes per stream of a tile of the streaming fold and tree kernels (one wave, one vector per lane) and
+// of the fold's block shape (128 threads x 8 vectors).
 constexpr size_t kStreamTileBytes = 1024;
+constexpr size_t kBlockTileBytes = 16384;
 
 // Loads of 128 bits run at full rate from any 4-byte-aligned address; from an
 // address that splits its dwords they lose about a fifth of the bandwidth.
@@ -72,8 +74,8 @@ __host__ __device__ inline size_t head_count(size_t elem_size, const char *out, 
 // buffer the same number of bytes off a 2 MiB boundary: 0: 85 % of the HBM peak, 1 KiB and more: 85,
 // 512: 83.5, 256: 83, 128: 82, 64: 74.  From kBigHeadFromBytes per segment on, the leading elements
 // therefore reach to the first input's next 1 KiB boundary (f32, every buffer 4 bytes off: 73 -> 84 %;
-// output 20 bytes off the inputs: 73 -> 77 %: reads that split lines cost more than writes that do),
-// spread over the segment's first workgroups, 64 elements each; shorter segments keep the rule above,
+// output 20 bytes off the inputs: 73 -> 77 %, reads that split lines costing more than writes that do;
+// such launches now do what stands below), spread over the segment's first workgroups, 64 elements each; shorter segments keep the rule above,
 // since their few workgroups would spend longer on the elements than on the tiles.
 constexpr size_t kBigHeadFromBytes = (size_t)64 << 10;
 // Where some input sits at another distance from a 64-byte boundary than the output, one side has to
@@ -111,8 +113,6 @@ template <typename T> __device__ __forceinline__ size_t head_elems(const char *o
   return head_count(sizeof(T), out, first, len);
 }
 
-// ... and of the fold's block shape (128 threads x 8 vectors).
-constexpr size_t kBlockTileBytes = 16384;
 // The streaming kernels are compiled for up to kStreamMaxWaves waves per SIMD; how many a launch really
 // gets is set when it is launched, through the LDS it asks for: a CU has 160 KiB and a workgroup is one
 // wave, so with 160 KiB / n bytes each n workgroups fit a CU (LDS is handed out by the KiB, so the
@@ -128,7 +128,8 @@ constexpr size_t kBlockTileBytes = 16384;
 //         P = 16: 79 80 82 81 79 79 79    P = 64: 84 84 83 80 80 80 81
 //   (a tree of 16-bit floats or a float min / max, P = 8: 14: 75, 16: 84, 20: 83, 26: 81)
 // Launches that move less than 256 MiB in all, much of which the caches hold, want more: 32 and 26
-// (16 MiB per rank, P = 8, repeated on the same buffers: 23.0 us against 25.1 us with 22).
+// (16 MiB per rank, P = 8, repeated on the same buffers: 23.0 us against 25.1 us with 22; of these only
+// the ones below 32 MiB still stream, the others take the block shape: see above Tile).
 constexpr int kStreamMaxWaves = 8;
 inline unsigned stream_lds_bytes(int wgs_per_cu) {
   const int n = wgs_per_cu < 4 ? 4 : (wgs_per_cu > 4 * kStreamMaxWaves ? 4 * kStreamMaxWaves : wgs_per_cu);
