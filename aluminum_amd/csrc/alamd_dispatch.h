@@ -66,11 +66,42 @@ template <typename F> int dispatch_any(int dtype, int op, F &&f) {
   }
 }
 
-// Whether a fold / tree launch that reads and writes total_bytes in all takes the block shape
-// (the measurements are in alamd_tile.h, above Tile).
+// Whether a fold / tree launch takes the block shape (the measurements are in alamd_tile.h, above Tile).
+// total_bytes: what it reads and writes in all; streams: ranks it reads; outputs: buffers every tile goes
+// to; tiles: how many block-shaped tiles it would have; cus: compute units of the device (<= 0: unknown).
+// With the two sizes at their defaults the rule is finer than the window between them:
+//  - three and more outputs: always (a streaming wave would write its KiB to every buffer in turn);
+//  - otherwise only if the tiles deal out evenly.  A CU gets through block-shaped tiles one at a time
+//    (one tile's loads are about what a CU can have in flight), so a launch of t tiles per CU lasts as
+//    long as ceil(t) of them: P = 32 fold, 140 / 186 / 279 / 372 / 558 tiles: 13.9 / 15.7 / 30.5 / 34.0 /
+//    53.2 us, where streaming takes 17.7 / 19.6 / 23.9 / 31.0 / 47.0 us; P = 8, 21.3 MiB per rank, 5.33
+//    tiles per CU: 31.5 us in blocks against 30.0 us streaming; 32 MiB per rank, 8 per CU: 45.7 against
+//    47.4.  Up to one tile per CU, or with up to 4 % of the CUs idle in the last round, it is taken.
+//    Powers of two from 4 MiB per rank on always deal out evenly;
+//  - up to four ranks into one or two buffers: never (every load up front buys little where there are few
+//    streams to wait for: P = 4, 8 / 16 / 32 MiB per rank: 12.5 / 23.2 / 48.0 us in blocks against 11.4 /
+//    22.0 / 46.9 us);
+//  - a tree whose block-shaped tiles are smaller than 16 KiB per slot (from 16 pre-folded slots or 32 slots
+//    on, where a lane's loads in flight are used up by the slots): never (48 ranks, 144 MiB in all: 29.0 us
+//    in blocks of 4 KiB against 23.0 us);
+//  - a fold over 24 ranks and more from half the size on (a streaming wave walks through its streams two
+//    or three at a time, P / 2 trips to memory one after the other: 64 ranks, 20 MiB in all: 20.0 us in
+//    blocks against 21.0 us, 96 MiB: 23.6 against 31.6).
 enum { FOLD_STREAM = 0, FOLD_BLOCK = 1, FOLD_CHAINED = 2 };  // the KIND of a fold / tree kernel
-inline bool use_block_shape(size_t total_bytes) {
-  return total_bytes >= tunables().block_shape_from_bytes && total_bytes < tunables().block_shape_below_bytes;
+inline bool use_block_shape(size_t total_bytes, int streams, int outputs, bool tree, size_t tiles, int cus,
+                            size_t tile_bytes = kBlockTileBytes) {
+  const size_t from = tunables().block_shape_from_bytes, below = tunables().block_shape_below_bytes;
+  const bool defaults = from == kBlockShapeFromBytes && below == kBlockShapeBelowBytes;
+  const bool many = streams >= 24;
+  if (total_bytes >= below) return false;
+  if (total_bytes < (defaults && many && !tree ? from / 2 : from)) return false;
+  if (!defaults) return true;
+  if (tile_bytes < kBlockTileBytes) return false;
+  if (outputs >= 3) return true;
+  if (streams <= 4) return false;
+  if (cus <= 0 || tiles <= (size_t)cus) return true;
+  const size_t per_cu = (tiles + (size_t)cus - 1) / (size_t)cus;  // ceil(t)
+  return (per_cu * (size_t)cus - tiles) * 25 <= per_cu * (size_t)cus;  // idle share <= 4 %
 }
 
 // ---- parameters of the two combine kernel families -------------------------

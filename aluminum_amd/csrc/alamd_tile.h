@@ -157,7 +157,8 @@ inline int stream_wgs_per_cu(bool tree, int streams, int outputs, size_t total_b
 //   8 written      10.0 / 7.5   20.9 / 19.2   40.3 / 37.8   76.2 / 78.8
 // Below, a launch is over before the second round of workgroups starts, and what counts is how many
 // start at once (library calls, P = 8, 64 KiB to 2 MiB per rank: 3.5 to 5.0 us streaming, 4.3 to 5.4 us
-// in blocks).
+// in blocks).  The figures above are for powers of two, whose tiles deal out evenly over the CUs; which
+// launches between the two sizes really take the block shape is use_block_shape's rule (alamd_dispatch.h).
 // (kBlockShapeFromBytes and kBlockShapeBelowBytes, with the other sizes the planner goes by, in alamd_common.h.)
 
 template <int U, int THREADS> struct Tile {

@@ -897,7 +897,8 @@ size_t alamd_planned_launches(int P, size_t count, int dtype) {
   const size_t es = alamd_dtype_size(dtype);
   if (P < 1 || P > ALAMD_MAX_RANKS || es == 0 || count == 0) return 0;
   // the planner of the fold kernels, run without launching anything
-  const size_t kTileBytes = use_block_shape(count * es * (size_t)(P + 1)) ? kBlockTileBytes : kStreamTileBytes;
+  const size_t kTileBytes = use_block_shape(count * es * (size_t)(P + 1), P, 1, false, (count * es + kBlockTileBytes - 1) / kBlockTileBytes, 256)
+                                ? kBlockTileBytes : kStreamTileBytes;  // (as on a device with 256 CUs: no device is asked here)
   SegParams seg = make_seg(count, 0, 0, OUT_ALL, 1);
   size_t launches = 0;
   plan_launches(seg, 1, count, kTileBytes / es, launch_tiles(P, kTileBytes, tunables().launch_bytes),

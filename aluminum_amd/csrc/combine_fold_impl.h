@@ -262,8 +262,10 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
     static_assert(Tile<Stream::U, Stream::THREADS>::BYTES == kStreamTileBytes && Tile<Chained::U, Chained::THREADS>::BYTES == kBlockTileBytes,
                   "alamd_planned_launches counts in these tiles");
     const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + (p.seg.out_mode == OUT_ALL ? p.seg.nout : 1));
-    const bool block = !chain && use_block_shape(total_bytes);
-    const size_t tile_bytes = block ? Tile<Chained::U, Chained::THREADS>::BYTES : Tile<Stream::U, Stream::THREADS>::BYTES;
+    constexpr size_t kBlockTile = Tile<Chained::U, Chained::THREADS>::BYTES;
+    const size_t block_tiles = (size_t)nseg * ((max_len * sizeof(T) + kBlockTile - 1) / kBlockTile);
+    const bool block = !chain && use_block_shape(total_bytes, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, false, block_tiles, device_cus());
+    const size_t tile_bytes = block ? kBlockTile : Tile<Stream::U, Stream::THREADS>::BYTES;
     const size_t tile_elems = tile_bytes / sizeof(T);
     FoldParams q = p;
     q.div = make_divisor(p.P);

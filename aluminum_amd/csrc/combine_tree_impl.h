@@ -347,8 +347,10 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   using C = TreeShape<T, OP, SLOTS, MODE, true>;
   static_assert(Tile<S::U, S::THREADS>::BYTES == kStreamTileBytes, "the tile of a streaming launch");
   const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + (p.seg.out_mode == OUT_ALL ? p.seg.nout : 1));
-  const bool block = !chain.scratch && use_block_shape(total_bytes);
-  const size_t tile_bytes = block ? Tile<C::U, C::THREADS>::BYTES : Tile<S::U, S::THREADS>::BYTES;
+  constexpr size_t kBlockTile = Tile<C::U, C::THREADS>::BYTES;
+  const size_t block_tiles = (size_t)nseg * ((max_len * sizeof(T) + kBlockTile - 1) / kBlockTile);
+  const bool block = !chain.scratch && use_block_shape(total_bytes, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, true, block_tiles, device_cus(), kBlockTile);
+  const size_t tile_bytes = block ? kBlockTile : Tile<S::U, S::THREADS>::BYTES;
   const size_t tile_elems = tile_bytes / sizeof(T);
   const size_t per_launch = launch_tiles(p.P, tile_bytes, tunables().launch_bytes);
   TreeParams q = p;

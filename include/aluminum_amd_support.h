@@ -48,8 +48,10 @@ int alamd_widen_f32(float *dst, const void *src16, size_t count, int dtype, void
  * (rank count from which a fold asks for three streams up front instead of
  * two; 0: 12); block_shape_from_bytes and block_shape_below_bytes (a fold /
  * tree launch that reads and writes at least the first and less than the
- * second in all works in tiles of 16 KiB with every load issued up front
- * instead of streaming; defaults 32 MiB and 384 MiB); halo_load_policy (the cache policy of the grid loads of a halo
+ * second in all may work in tiles of 16 KiB with every load issued up front
+ * instead of streaming; defaults 32 MiB and 384 MiB, between which the library
+ * also looks at outputs, rank count and how evenly the tiles deal out over
+ * the CUs; with other values every launch in the window does); halo_load_policy (the cache policy of the grid loads of a halo
  * pack: 0 plain, 1 nt, 2 sc1, 3 sc0 sc1, 4 sc0 sc1 nt).  Piece sizes below
  * 64 KiB are refused.  Results never depend on them, only speed. */
 int alamd_tune(const char *name, size_t value);

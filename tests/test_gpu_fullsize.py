@@ -50,16 +50,17 @@ def test_c2_bf16_full_size(al):
 @pytest.mark.parametrize("dtype,dist,seed", [("f32", "uniform_pm1", 1000), ("bf16", "normal", 2000), ("f64", "uniform_pm1", 1000),
                                              ("i32", "fullrange", 3000)])
 def test_middling_sizes_in_the_block_shape(al, dtype, dist, seed):
-    """Calls that move between 32 and 384 MiB in all run in tiles of 16 KiB with every load issued up front,
-    by the library's own choice: 4 Mi + 37 elements per rank (buffers one element into their allocations,
-    so with leading elements), one output and eight, fold and tree orders, float min under the order whose
-    operand roles change from block to block; and the sizes either side of the two thresholds."""
+    """Calls that move between 32 and 384 MiB in all and whose tiles of 16 KiB deal out evenly over the CUs
+    run in such tiles with every load issued up front, by the library's own choice: 4 Mi elements per rank
+    (buffers one element into their allocations, so with leading elements and a ragged last tile), one
+    output and eight, fold and tree orders, float min under the order whose operand roles change from
+    block to block; and the sizes either side of the two thresholds."""
     import torch
     assert al.tuned("block_shape_from_bytes") == 32 << 20 and al.tuned("block_shape_below_bytes") == 384 << 20
     es = al.dtype_size(dtype)
     carrier = al.torch_dtype(dtype)
     np_dt = oracle.NP_CARRIER[dtype]
-    n = (1 << 22) + 37
+    n = 1 << 22
     raw = [torch.empty(n + 1, dtype=carrier, device="cuda") for _ in range(P)]
     ins = [t[1:] for t in raw]
     for r in range(P):
