@@ -12,6 +12,9 @@
 #include "alamd_dispatch.h"
 #include "alamd_tile.h"
 
+// (the library defines this in core.hip; this program links no library)
+namespace alamd { Tunables &tunables() { static Tunables t; return t; } }
+
 using namespace alamd;
 
 static int g_fail = 0, g_checks = 0;
@@ -191,6 +194,24 @@ int main(int argc, char **argv) {
     EXPECT(!by_out(4, 20, {0, 0, 0}, 1000), "short segment");
     EXPECT(!by_out(2, 2, {0, 0}, 1 << 20), "inputs off the output's dword grid");
     EXPECT(by_out(2, 4, {0, 0}, 1 << 20), "16-bit elements, output two elements off");
+  }
+  // Which launches take the block shape (the sizes at their defaults; 256 CUs).
+  {
+    const size_t MiB = (size_t)1 << 20;
+    EXPECT(use_block_shape(144 * MiB, 8, 1, false, 1024, 256), "P = 8, 16 MiB per rank: four tiles per CU");
+    EXPECT(!use_block_shape(144 * MiB, 8, 1, false, 1025, 256), "one tile more: a fifth round for one CU");
+    EXPECT(use_block_shape(192 * MiB, 8, 1, true, 2731 - 171, 256), "ten tiles per CU exactly");
+    EXPECT(use_block_shape(192 * MiB, 8, 1, true, 2550, 256), "0.4 %% of the CUs idle in the last round");
+    EXPECT(!use_block_shape(192 * MiB, 8, 1, true, 1365, 256), "5.33 tiles per CU");
+    EXPECT(use_block_shape(40 * MiB, 8, 1, false, 200, 256), "fewer tiles than CUs");
+    EXPECT(use_block_shape(144 * MiB, 8, 8, false, 1025, 256), "eight outputs: whatever the tiles");
+    EXPECT(!use_block_shape(144 * MiB, 4, 1, false, 1024, 256), "four ranks");
+    EXPECT(use_block_shape(144 * MiB, 4, 3, false, 1024, 256), "four ranks, three outputs");
+    EXPECT(use_block_shape(20 * MiB, 64, 1, false, 20, 256), "a fold over 64 ranks from 16 MiB on");
+    EXPECT(!use_block_shape(20 * MiB, 64, 1, true, 20, 256) && !use_block_shape(20 * MiB, 8, 1, false, 142, 256), "others from 32 MiB on");
+    EXPECT(!use_block_shape(144 * MiB, 48, 1, true, 256, 256, 4096) && !use_block_shape(144 * MiB, 48, 8, true, 256, 256, 8192), "tree tiles under 16 KiB");
+    EXPECT(!use_block_shape(384 * MiB, 8, 1, false, 2048, 256) && !use_block_shape(31 * MiB, 8, 8, false, 256, 256), "outside the window");
+    EXPECT(use_block_shape(144 * MiB, 8, 1, false, 1025, 0), "unknown device: the window alone");
   }
   // workgroups that find nothing to do: a planner that put every segment side by side in one grid
   // would idle far more than it works on the "one long among short" shapes

@@ -23,7 +23,8 @@ def test_launch_planner_covers_every_tile_once():
     """plan_launches (alamd_dispatch.h) on random segment tables, on the host: every tile of every
     segment in exactly one launch, grids within the device's limits; the block lookup of the role masks
     (through prepared reciprocals) against 64-bit division and against the definition of the blocks;
-    the LDS sizing of the streaming launches."""
+    the LDS sizing of the streaming launches; the leading elements of a segment; the runs of tiles per XCD;
+    which launches take the block shape."""
     exe = os.path.join(ROOT, "tests", "cpp", "test_planner")
     if not os.path.exists(exe):
         subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp"), "test_planner"], check=True,
