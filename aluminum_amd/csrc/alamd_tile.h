@@ -139,11 +139,27 @@ inline unsigned stream_lds_bytes(int wgs_per_cu) {
 // (8 MiB per rank to 8 buffers, repeated: 22.2 us against 24.1 us; 16 MiB, untouched: 51.0 against 52.8).
 // Workgroups per CU of a streaming launch over `streams` inputs that moves `total_bytes` in all and
 // writes every tile to `outputs` buffers.
-inline int stream_wgs_per_cu(bool tree, int streams, int outputs, size_t total_bytes) {
+// A launch of few rounds (`tiles` workgroups in all over `cus` CUs; 0: unknown) is a matter of whole
+// rounds where a wave lives long, i.e. over many ranks: 64 ranks, 6048 tiles: 83 us with 22 per CU (two
+// rounds, the second all but empty), 59 us with 26 (one); 48 ranks, 6672 tiles: 63 us with 22 or 26, 49 us
+// with 32; 16 ranks, 23120 tiles: 62 / 59 / 58 us.  A fold of up to five rounds therefore takes the
+// setting with the fewest rounds; from there on the rounds overlap and the rule above holds (16 ranks,
+// 30832 tiles, six rounds: 79 us with 22, 83 us with 32; P = 8, 262144 tiles: 85 % with 22, 80 % with 32).  A tree, with twice the loads per wave, only goes from two
+// rounds to one where 22 or 26 per CU do that (64 ranks, 4528 tiles: 59 -> 46 us); more per CU cost it
+// more than the round saves.
+inline int stream_wgs_per_cu(bool tree, int streams, int outputs, size_t total_bytes, size_t tiles = 0, int cus = 0) {
   if (outputs >= 3) return 16;
-  if (total_bytes < ((size_t)256 << 20)) return tree ? 26 : 32;
-  if (streams <= 2) return 26;
-  return tree ? 16 : 22;
+  int n = tree ? 16 : 22;
+  if (total_bytes < ((size_t)256 << 20)) n = tree ? 26 : 32;
+  else if (streams <= 2) n = 26;
+  if (tiles == 0 || cus <= 0) return n;
+  auto rounds = [&](int m) { return (tiles + (size_t)m * (size_t)cus - 1) / ((size_t)m * (size_t)cus); };
+  size_t best = rounds(n);
+  if (tree ? best != 2 : (best < 2 || best > 5)) return n;
+  const int more[3] = {22, 26, tree ? 26 : 32};
+  for (int m : more)
+    if (m > n && rounds(m) < best && (!tree || rounds(m) == 1)) { best = rounds(m); n = m; }
+  return n;
 }
 
 // Between 32 and 384 MiB (bytes a launch reads and writes in all) the fold and tree kernels take the

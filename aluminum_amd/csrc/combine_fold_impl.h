@@ -328,7 +328,8 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
     }
     const size_t per_launch = launch_tiles(p.P, tile_bytes, tunables().launch_bytes);
     const size_t wgs = tunables().stream_wgs_per_cu;
-    unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(false, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes));
+    unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(false, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes,
+                                                                           (size_t)nseg * ((max_len * sizeof(T) + kStreamTileBytes - 1) / kStreamTileBytes), device_cus()));
     unsigned threads = Stream::THREADS;
     if (block) {
       if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 0, true, FOLD_BLOCK> : fold_vec_kernel<T, OP, false, 0, true, FOLD_BLOCK>;

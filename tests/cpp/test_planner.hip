@@ -195,6 +195,23 @@ int main(int argc, char **argv) {
     EXPECT(!by_out(2, 2, {0, 0}, 1 << 20), "inputs off the output's dword grid");
     EXPECT(by_out(2, 4, {0, 0}, 1 << 20), "16-bit elements, output two elements off");
   }
+  // Workgroups per CU of a streaming launch: by size, streams and outputs; a launch of few rounds takes
+  // the setting with the fewest whole rounds (a tree only from two rounds to one).
+  {
+    const size_t MiB = (size_t)1 << 20;
+    EXPECT(stream_wgs_per_cu(false, 8, 1, 2304 * MiB, 262144, 256) == 22 && stream_wgs_per_cu(true, 8, 1, 2304 * MiB, 262144, 256) == 16, "large launches");
+    EXPECT(stream_wgs_per_cu(false, 8, 1, 20 * MiB, 2276, 256) == 32 && stream_wgs_per_cu(true, 8, 1, 20 * MiB, 2276, 256) == 26, "small launches");
+    EXPECT(stream_wgs_per_cu(false, 8, 8, 2304 * MiB, 262144, 256) == 16 && stream_wgs_per_cu(false, 2, 1, 768 * MiB, 262144, 256) == 26, "outputs, two streams");
+    EXPECT(stream_wgs_per_cu(false, 64, 1, 384 * MiB, 6048, 256) == 26, "6048 tiles: one round with 26 per CU");
+    EXPECT(stream_wgs_per_cu(false, 64, 1, 448 * MiB, 7056, 256) == 32, "7056 tiles: one round with 32");
+    EXPECT(stream_wgs_per_cu(false, 48, 1, 448 * MiB, 9360, 256) == 22, "9360 tiles: two rounds whatever the setting");
+    EXPECT(stream_wgs_per_cu(false, 32, 1, 384 * MiB, 11904, 256) == 26, "11904 tiles: three rounds with 22, two with 26");
+    EXPECT(stream_wgs_per_cu(false, 8, 1, 512 * MiB, 58240, 256) == 22 && stream_wgs_per_cu(false, 16, 1, 512 * MiB, 30832, 256) == 22, "more than five rounds: by size alone");
+    EXPECT(stream_wgs_per_cu(false, 16, 1, 384 * MiB, 23120, 256) == 32, "five rounds with 22, three with 32");
+    EXPECT(stream_wgs_per_cu(true, 64, 1, 288 * MiB, 4528, 256) == 22 && stream_wgs_per_cu(true, 64, 1, 384 * MiB, 6048, 256) == 26, "a tree: from two rounds to one");
+    EXPECT(stream_wgs_per_cu(true, 64, 1, 448 * MiB, 7056, 256) == 16 && stream_wgs_per_cu(true, 32, 1, 512 * MiB, 15872, 256) == 16, "a tree: otherwise by size");
+    EXPECT(stream_wgs_per_cu(false, 64, 1, 384 * MiB) == 22, "unknown tile count");
+  }
   // Which launches take the block shape (the sizes at their defaults; 256 CUs).
   {
     const size_t MiB = (size_t)1 << 20;
