@@ -159,6 +159,15 @@ template <int OP> struct Step<bf16_t, OP> {
   }
 };
 
+// One 16-bit operation per byte of a dword: a byte of either operand selected as source and one byte of
+// the result written, the first instruction clearing the others and the later ones keeping them.
+// d = a NAME b, byte by byte; SRC0 / SRC1 are "%1" / "%2" or "sext(%1)" / "sext(%2)".
+#define ALAMD_PER_BYTE(NAME, SRC0, SRC1)                                                                             \
+asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0 src1_sel:BYTE_0" : "=v"(d) : "v"(a), "v"(b)); \
+asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_1 src1_sel:BYTE_1" : "+v"(d) : "v"(a), "v"(b)); \
+asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_2 src1_sel:BYTE_2" : "+v"(d) : "v"(a), "v"(b)); \
+asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3 src1_sel:BYTE_3" : "+v"(d) : "v"(a), "v"(b));
+
 // The step applied to every element of a 128-bit vector.
 template <typename T, int OP>
 __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
@@ -184,15 +193,14 @@ __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
     }
     return r;
   } else if constexpr (sizeof(T) == 1 && OP == ALAMD_PROD) {
-    // wrapping byte products as packed 16-bit products of the even and the odd bytes
-    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+    // wrapping byte products: the low byte of the 16-bit product of two bytes, one instruction per byte
     u32x4 r;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t a = in[j], b = inout[j];
-      const u16x2 pe = __builtin_bit_cast(u16x2, a & 0x00ff00ffu) * __builtin_bit_cast(u16x2, b & 0x00ff00ffu);
-      const u16x2 po = __builtin_bit_cast(u16x2, (a >> 8) & 0x00ff00ffu) * __builtin_bit_cast(u16x2, (b >> 8) & 0x00ff00ffu);
-      r[j] = (__builtin_bit_cast(uint32_t, pe) & 0x00ff00ffu) | ((__builtin_bit_cast(uint32_t, po) & 0x00ff00ffu) << 8);
+      uint32_t d;
+      ALAMD_PER_BYTE("v_mul_lo_u16_sdwa", "%1", "%2")
+      r[j] = d;
     }
     return r;
   } else if constexpr (sizeof(T) == 1 && (OP == ALAMD_MIN || OP == ALAMD_MAX)) {
@@ -205,19 +213,13 @@ __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
     for (int j = 0; j < 4; ++j) {
       const uint32_t a = in[j], b = inout[j];
       uint32_t d;
-#define ALAMD_BYTE_MINMAX(NAME, SRC0, SRC1)                                                                             \
-      asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0 src1_sel:BYTE_0" : "=v"(d) : "v"(a), "v"(b)); \
-      asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_1 src1_sel:BYTE_1" : "+v"(d) : "v"(a), "v"(b)); \
-      asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_2 src1_sel:BYTE_2" : "+v"(d) : "v"(a), "v"(b)); \
-      asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3 src1_sel:BYTE_3" : "+v"(d) : "v"(a), "v"(b));
       if constexpr (std::is_signed<T>::value) {
-        if constexpr (OP == ALAMD_MIN) { ALAMD_BYTE_MINMAX("v_min_i16_sdwa", "sext(%1)", "sext(%2)") }
-        else { ALAMD_BYTE_MINMAX("v_max_i16_sdwa", "sext(%1)", "sext(%2)") }
+        if constexpr (OP == ALAMD_MIN) { ALAMD_PER_BYTE("v_min_i16_sdwa", "sext(%1)", "sext(%2)") }
+        else { ALAMD_PER_BYTE("v_max_i16_sdwa", "sext(%1)", "sext(%2)") }
       } else {
-        if constexpr (OP == ALAMD_MIN) { ALAMD_BYTE_MINMAX("v_min_u16_sdwa", "%1", "%2") }
-        else { ALAMD_BYTE_MINMAX("v_max_u16_sdwa", "%1", "%2") }
+        if constexpr (OP == ALAMD_MIN) { ALAMD_PER_BYTE("v_min_u16_sdwa", "%1", "%2") }
+        else { ALAMD_PER_BYTE("v_max_u16_sdwa", "%1", "%2") }
       }
-#undef ALAMD_BYTE_MINMAX
       r[j] = d;
     }
     return r;
