@@ -147,6 +147,9 @@ inline unsigned stream_lds_bytes(int wgs_per_cu) {
 // 30832 tiles, six rounds: 79 us with 22, 83 us with 32; P = 8, 262144 tiles: 85 % with 22, 80 % with 32).  A tree, with twice the loads per wave, only goes from two
 // rounds to one where 22 or 26 per CU do that (64 ranks, 4528 tiles: 59 -> 46 us); more per CU cost it
 // more than the round saves.
+// (no launch of more streaming tiles than this has few rounds on any device, nor lies below the size
+// where the block shape ends: 384 MiB of 1 KiB tiles)
+constexpr size_t kFewRoundsTiles = (size_t)384 << 10;
 inline int stream_wgs_per_cu(bool tree, int streams, int outputs, size_t total_bytes, size_t tiles = 0, int cus = 0) {
   if (outputs >= 3) return 16;
   int n = tree ? 16 : 22;

@@ -264,7 +264,10 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
     const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + (p.seg.out_mode == OUT_ALL ? p.seg.nout : 1));
     constexpr size_t kBlockTile = Tile<Chained::U, Chained::THREADS>::BYTES;
     const size_t block_tiles = (size_t)nseg * ((max_len * sizeof(T) + kBlockTile - 1) / kBlockTile);
-    const bool block = !chain && use_block_shape(total_bytes, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, false, block_tiles, device_cus());
+    // (the number of CUs only matters to launches of few rounds: the others do not ask for it)
+    const size_t stream_tiles = (size_t)nseg * ((max_len * sizeof(T) + kStreamTileBytes - 1) / kStreamTileBytes);
+    const int cus = stream_tiles <= kFewRoundsTiles ? device_cus() : 0;
+    const bool block = !chain && use_block_shape(total_bytes, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, false, block_tiles, cus);
     const size_t tile_bytes = block ? kBlockTile : Tile<Stream::U, Stream::THREADS>::BYTES;
     const size_t tile_elems = tile_bytes / sizeof(T);
     FoldParams q = p;
@@ -329,7 +332,7 @@ int launch_fold_typed(const FoldParams &p, unsigned nseg, size_t max_len, bool r
     const size_t per_launch = launch_tiles(p.P, tile_bytes, tunables().launch_bytes);
     const size_t wgs = tunables().stream_wgs_per_cu;
     unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(false, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes,
-                                                                           (size_t)nseg * ((max_len * sizeof(T) + kStreamTileBytes - 1) / kStreamTileBytes), device_cus()));
+                                                                           stream_tiles, cus));
     unsigned threads = Stream::THREADS;
     if (block) {
       if constexpr (FP_MINMAX) kern = roles ? fold_vec_kernel<T, OP, true, 0, true, FOLD_BLOCK> : fold_vec_kernel<T, OP, false, 0, true, FOLD_BLOCK>;

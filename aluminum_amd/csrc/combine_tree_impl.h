@@ -349,7 +349,9 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   const size_t total_bytes = (size_t)nseg * max_len * sizeof(T) * (size_t)(p.P + (p.seg.out_mode == OUT_ALL ? p.seg.nout : 1));
   constexpr size_t kBlockTile = Tile<C::U, C::THREADS>::BYTES;
   const size_t block_tiles = (size_t)nseg * ((max_len * sizeof(T) + kBlockTile - 1) / kBlockTile);
-  const bool block = !chain.scratch && use_block_shape(total_bytes, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, true, block_tiles, device_cus(), kBlockTile);
+  const size_t stream_tiles = (size_t)nseg * ((max_len * sizeof(T) + kStreamTileBytes - 1) / kStreamTileBytes);
+  const int cus = stream_tiles <= kFewRoundsTiles ? device_cus() : 0;
+  const bool block = !chain.scratch && use_block_shape(total_bytes, p.P, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, true, block_tiles, cus, kBlockTile);
   const size_t tile_bytes = block ? kBlockTile : Tile<S::U, S::THREADS>::BYTES;
   const size_t tile_elems = tile_bytes / sizeof(T);
   const size_t per_launch = launch_tiles(p.P, tile_bytes, tunables().launch_bytes);
@@ -415,7 +417,7 @@ int launch_tree_mode(const TreeParams &p, unsigned nseg, size_t max_len, hipStre
   q.seg.simple = nseg == 1 && !q.seg.ragged && q.seg.seg_rem == 0 && !q.seg.in_blocked && q.seg.out_mode == OUT_ALL && q.seg.nout == 1;
   const size_t wgs = tunables().stream_wgs_per_cu;
   unsigned lds = stream_lds_bytes(wgs ? (int)wgs : stream_wgs_per_cu(true, SLOTS * HALVES, p.seg.out_mode == OUT_ALL ? p.seg.nout : 1, total_bytes,
-                                                                         (size_t)nseg * ((max_len * sizeof(T) + kStreamTileBytes - 1) / kStreamTileBytes), device_cus()));
+                                                                         stream_tiles, cus));
   unsigned threads = S::THREADS;
   void (*kern)(const TreeParams) =
       q.seg.any_head ? tree_vec_kernel<T, OP, SLOTS, MODE, true, HALVES> : tree_vec_kernel<T, OP, SLOTS, MODE, false, HALVES>;
