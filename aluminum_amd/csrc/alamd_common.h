@@ -168,8 +168,28 @@ asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0
 asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_2 src1_sel:BYTE_2" : "+v"(d) : "v"(a), "v"(b)); \
 asm(NAME " %0, " SRC0 ", " SRC1 " dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3 src1_sel:BYTE_3" : "+v"(d) : "v"(a), "v"(b));
 
+// A logical operator on 8- or 16-bit elements, which step_vec takes a dword at a time: its result holds 0
+// or 1 in every element, so a fold that has made its first operand so (truth_vec) can tell step_vec
+// that `inout` needs no looking at again (INOUT_IS_TRUTH): eleven instructions per dword become six.
+template <typename T, int OP> constexpr bool narrow_logical() {
+  return sizeof(T) <= 2 && (OP == ALAMD_LOR || OP == ALAMD_LAND || OP == ALAMD_LXOR);
+}
+// 1 in every 8- or 16-bit element that is nonzero, 0 in the others (the carry of low bits + all-ones
+// reaches the top bit iff a low bit is set).
+template <typename T> __device__ __forceinline__ uint32_t truth_dword(uint32_t x) {
+  constexpr uint32_t low = sizeof(T) == 1 ? 0x7f7f7f7fu : 0x7fff7fffu, top = ~low;
+  constexpr int shift = 8 * (int)sizeof(T) - 1;
+  return ((((x & low) + low) | x) & top) >> shift;
+}
+template <typename T> __device__ __forceinline__ u32x4 truth_vec(u32x4 v) {
+  u32x4 r;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) r[j] = truth_dword<T>(v[j]);
+  return r;
+}
+
 // The step applied to every element of a 128-bit vector.
-template <typename T, int OP>
+template <typename T, int OP, bool INOUT_IS_TRUTH = false>
 __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
   if constexpr (std::is_same<T, bf16_t>::value) {
     // two elements per dword: widen by shift / mask, one fp32 operation each,
@@ -223,18 +243,20 @@ __device__ __forceinline__ u32x4 step_vec(u32x4 in, u32x4 inout) {
       r[j] = d;
     }
     return r;
-  } else if constexpr (sizeof(T) <= 2 && (OP == ALAMD_LOR || OP == ALAMD_LAND || OP == ALAMD_LXOR)) {
-    // a whole dword of bytes or halfwords at a time: a 1 in every element that
-    // is nonzero (the carry of low-bits + all-ones reaches the top bit iff a
-    // low bit is set), then the bitwise operator
-    constexpr uint32_t low = sizeof(T) == 1 ? 0x7f7f7f7fu : 0x7fff7fffu, top = ~low;
-    constexpr int shift = 8 * (int)sizeof(T) - 1;
-    auto nonzero = [](uint32_t x) { return ((((x & low) + low) | x) & top) >> shift; };
+  } else if constexpr (narrow_logical<T, OP>()) {
+    // a whole dword of bytes or halfwords at a time: a 1 in every element that is nonzero, then the
+    // bitwise operator
     u32x4 r;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t a = in[j], b = inout[j];
-      r[j] = OP == ALAMD_LOR ? nonzero(b | a) : OP == ALAMD_LAND ? (nonzero(b) & nonzero(a)) : (nonzero(b) ^ nonzero(a));
+      if constexpr (INOUT_IS_TRUTH) {
+        const uint32_t ta = truth_dword<T>(a);
+        r[j] = OP == ALAMD_LOR ? (b | ta) : OP == ALAMD_LAND ? (b & ta) : (b ^ ta);
+      } else {
+        r[j] = OP == ALAMD_LOR ? truth_dword<T>(b | a) : OP == ALAMD_LAND ? (truth_dword<T>(b) & truth_dword<T>(a))
+                                                                           : (truth_dword<T>(b) ^ truth_dword<T>(a));
+      }
     }
     return r;
   } else {

@@ -114,6 +114,10 @@ fold_vec_kernel(const FoldParams p) {
     const size_t rem = vec_bytes - tb;
     const int nrec = rem > TL::BYTES ? (int)TL::BYTES : (int)rem;
     u32x4 acc[U];
+    // (a logical operator on 8- or 16-bit elements: the running result is made 0 / 1 per element once,
+    // and every step then only looks at the stream it adds; with one rank there is no step, and the
+    // result is the input as it is)
+    constexpr bool TRUTH = narrow_logical<T, OP>();
     if constexpr (!BLOCK) {
       static_assert(U == 1, "the streaming body holds one vector per lane and stream");
       // Stream k lives in x[k % FRONT].  A later load takes its offset from an empty asm statement that
@@ -139,12 +143,13 @@ fold_vec_kernel(const FoldParams p) {
         return __builtin_amdgcn_raw_buffer_load_b128(rs, vo, 0, kAuxLoadStream);
       };
       acc[0] = x[0];
+      if constexpr (TRUTH) { if (P >= 2) acc[0] = truth_vec<T>(acc[0]); }
       for (int base = 0; base < P; base += FRONT) {
 #pragma unroll
         for (int j = 0; j < FRONT; ++j) {
           const int k = base + j;
           if (k >= 1 && k < P) {
-            acc[0] = ACC_IS_IN ? step_vec<T, OP>(acc[0], x[j]) : step_vec<T, OP>(x[j], acc[0]);
+            acc[0] = ACC_IS_IN ? step_vec<T, OP>(acc[0], x[j]) : step_vec<T, OP, TRUTH>(x[j], acc[0]);
             if (k + FRONT - 1 < P) {
               x[(j + FRONT - 1) % FRONT] = load_after(TL::rsrc(next_in + vin + tb, nrec), acc[0]);
               req = next_rank(req, p.dir, P);
@@ -177,12 +182,18 @@ fold_vec_kernel(const FoldParams p) {
         if constexpr (FIRST) {
 #pragma unroll
           for (int u = 0; u < U; ++u) acc[u] = x[0][u];
+          if constexpr (TRUTH) {
+            if (P >= 2) {
+#pragma unroll
+              for (int u = 0; u < U; ++u) acc[u] = truth_vec<T>(acc[u]);
+            }
+          }
         }
 #pragma unroll
         for (int b = FIRST ? 1 : 0; b < R; ++b) {
 #pragma unroll
           for (int u = 0; u < U; ++u)
-            acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[b][u]) : step_vec<T, OP>(x[b][u], acc[u]);
+            acc[u] = ACC_IS_IN ? step_vec<T, OP>(acc[u], x[b][u]) : step_vec<T, OP, TRUTH>(x[b][u], acc[u]);
         }
       };
       using Yes = std::true_type;

@@ -57,6 +57,24 @@ def test_combine_all_ops_orders(al, dtype, shape):
                     assert_bits_equal(got, want, dtype, "%s %s P=%d %s n=%d" % (dtype, op, P, order, n))
 
 
+@pytest.mark.parametrize("dtype", ("u8", "i8", "u16", "i16", "i32"))
+def test_logical_operators_on_any_values(al, dtype, shape):
+    """lor / land / lxor see an element as true iff it is nonzero, whatever its value, and give 0 or 1; one
+    rank alone gets its input back as it is.  (The 8- and 16-bit kernels make the running result 0 / 1 once
+    and then only look at the stream each step adds.)"""
+    for P in (1, 2, 3, 8, 13):
+        for n in (5, 4099, 70001):
+            ins = [oracle.fill(n, dtype, "fullrange", 500 + r) for r in range(P)]
+            for a in ins[::2]:
+                a[::3] = 0  # enough zeros for land and lxor to give both answers
+            for op in ("lor", "land", "lxor"):
+                want = oracle.combine(ins, dtype, op, "rank_asc")
+                got = run_combine(al, ins, dtype, op, "rank_asc")[0]
+                assert_bits_equal(got, want, dtype, "%s %s P=%d n=%d" % (dtype, op, P, n))
+                if P == 1:
+                    assert got.tobytes() == ins[0].tobytes()
+
+
 @pytest.mark.parametrize("dtype", ("f32", "bf16", "i32"))
 @pytest.mark.parametrize("P", (4, 6, 7, 8, 13, 16, 31, 32, 33, 40, 48, 63, 64))
 def test_combine_many_ranks(al, dtype, P, shape):
